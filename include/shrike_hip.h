@@ -1,0 +1,270 @@
+/*
+ * libshrikehip — the routed-expert (MoE layer) hot path of Shrike on one AMD
+ * MI355X (gfx950), behind a plain C ABI in the style of the reference's
+ * ShrikeKernelsC target (sources/ShrikeKernelsC/include/shrike_kernels.h).
+ *
+ * Conventions (the reference's, sources/ShrikeKernelsC/include/shrike_expert_io.h:33-72):
+ *  - caller-owned memory; every pointer named `d_*` or documented "device" is a
+ *    device address; nothing on a per-layer call allocates;
+ *  - every enqueue-only call takes the HIP stream as `void *stream` (a hipStream_t;
+ *    NULL = the default stream) and returns at once: ordering is the stream's,
+ *    as it is the serial command encoder's in the reference;
+ *  - calls return 0 or an errno-style code (EINVAL for what the reference traps
+ *    as a precondition, ENOMEM, EIO for a HIP runtime failure);
+ *    shrike_hip_last_error() names the cause;
+ *  - opaque handles are created with `..._create(..., int *out_errno)` -> NULL on
+ *    failure and destroyed with no concurrent callers.
+ *
+ * Quantised layout (sources/ShrikeKernelsC/include/shrike_kernels.h:11-16,
+ * sources/Shrike/Infrastructure/ModelIO/Quantization.swift:30-45): 4-bit codes two
+ * per byte, element 2k in the low nibble of byte k; 8-bit codes one per byte; one
+ * 16-bit scale and one 16-bit bias per group of 64 along the row, row-major;
+ * w = code * scale + bias. The reference stores scale/bias as bf16; fp16 is
+ * accepted as well (`meta_dtype`).
+ */
+#ifndef SHRIKE_HIP_H
+#define SHRIKE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SHRIKE_GROUP_SIZE 64u
+#define SHRIKE_MAX_TOP_K 8u          /* MoE.maxStreamedExperts, MoE.swift:42 */
+#define SHRIKE_MAX_ROUTER_EXPERTS 256u /* MoE.swift:263 */
+#define SHRIKE_MAX_HIDDEN 4096u      /* staged activation ceiling (reference: 2880, moe.metal:11) */
+#define SHRIKE_POOL_MAX_CHUNKS 8u    /* ExpertCellArena.maxChunks, ExpertCellArena.swift:20 */
+#define SHRIKE_SLOT_SENTINEL 0xffffffffu /* ExpertResidencyEntry.notResidentSlot */
+#define SHRIKE_POOL_PAGE 16384u      /* .gturbo expert stride alignment, GTurboFormatV1.swift:7 */
+
+enum { SHRIKE_META_BF16 = 0, SHRIKE_META_F16 = 1 };
+enum { SHRIKE_ACT_GELU_TANH = 0, SHRIKE_ACT_SILU = 1, SHRIKE_ACT_CLAMPED_SWIGLU = 2 };
+enum { SHRIKE_RESIDENCY_EMPTY = 0, SHRIKE_RESIDENCY_LOADING = 1, SHRIKE_RESIDENCY_RESIDENT = 2 };
+
+const char *shrike_hip_last_error(void);
+/* 0 when a gfx950 device is present and the kernels' code object loaded. */
+int shrike_hip_init(int device);
+
+/* ---------------------------------------------------------------- layouts */
+
+/* MoEExpertOffsets, sources/Shrike/Kernels/MoE/MoE.swift:4-39 (field for field). */
+typedef struct {
+    uint32_t gate_w_off, gate_s_off, gate_b_off;
+    uint32_t up_w_off, up_s_off, up_b_off;
+    uint32_t down_w_off, down_s_off, down_b_off;
+    uint32_t gate_ab_off, up_ab_off, down_ab_off;
+} shrike_expert_offsets;
+
+/* CPUExpertFFN.Offsets(d:f:), sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:34-61,
+ * for 4- or 8-bit codes; additive biases (gpt-oss) are appended when asked for.
+ * Returns the packed blob size, 0 on invalid arguments. */
+uint64_t shrike_expert_offsets_make(uint32_t d, uint32_t f, uint32_t bits,
+                                    int additive_biases, shrike_expert_offsets *out);
+
+/* PoolBases, sources/Shrike/Metal/MoE/moe.metal:297-305: cell -> base[cell /
+ * cells_per_chunk] + (cell % cells_per_chunk) * stride. */
+typedef struct {
+    const void *base[SHRIKE_POOL_MAX_CHUNKS];
+    uint32_t cells_per_chunk;
+} shrike_pool_bases;
+
+/* SharedExpertProjection, sources/Shrike/Kernels/MoE/SharedExpertInt8.swift:9-31:
+ * one resident projection as three device tensors. */
+typedef struct {
+    const void *weights, *scales, *biases;
+} shrike_projection;
+
+/* ------------------------------------------------------ budget -> slot count */
+
+/* RuntimeConfiguration.parseBudgetBytes, sources/Shrike/Runtime/Configuration/
+ * RuntimeConfiguration.swift:111-129. Returns bytes, or -1 for what the reference
+ * maps to nil. */
+int64_t shrike_parse_budget_bytes(const char *text);
+/* RuntimeConfiguration.expertCacheSlots, RuntimeConfiguration.swift:77,:137-149. */
+int32_t shrike_expert_cache_slots(uint64_t expert_stride_bytes, int32_t layers,
+                                  int64_t budget_bytes);
+
+/* ------------------------------------------------------------ HBM slot pool */
+
+/* ExpertCellArena + the residency table of PreadExpertStreamer
+ * (sources/Shrike/Infrastructure/Streaming/ExpertCellArena.swift:16-133,
+ * PreadExpertStreamer.swift:283-352): `cells` cells of page-rounded stride in at
+ * most 8 device chunks, and one 64-bit residency word per expert in device memory
+ * (state << 32 | cell). */
+typedef struct shrike_hip_pool shrike_hip_pool;
+shrike_hip_pool *shrike_hip_pool_create(uint32_t cells, uint64_t expert_stride,
+                                        uint32_t num_experts, uint64_t chunk_bytes,
+                                        int *out_errno);
+void shrike_hip_pool_destroy(shrike_hip_pool *pool);
+uint64_t shrike_hip_pool_slot_stride(const shrike_hip_pool *pool);
+uint32_t shrike_hip_pool_cell_count(const shrike_hip_pool *pool);
+void *shrike_hip_pool_cell_ptr(const shrike_hip_pool *pool, uint32_t cell);
+const shrike_pool_bases *shrike_hip_pool_bases(const shrike_hip_pool *pool);
+/* device address of the u64[num_experts] residency table */
+void *shrike_hip_pool_residency_table(const shrike_hip_pool *pool);
+/* Copies one expert blob from host memory (pinned for a truly asynchronous copy)
+ * into a cell on `stream`; replaces the reader's pread into the slot
+ * (PreadExpertStreamer.swift:610-621). */
+int shrike_hip_pool_upload_async(shrike_hip_pool *pool, uint32_t cell, const void *host_src,
+                                 uint64_t bytes, void *stream);
+/* PreadExpertStreamer.publish, PreadExpertStreamer.swift:1143-1148: stream-ordered
+ * store of the expert's residency word; `cell` is ignored for EMPTY. The host
+ * shadow is updated at once. */
+int shrike_hip_pool_table_publish(shrike_hip_pool *pool, uint32_t expert, uint32_t cell,
+                                  uint32_t state, void *stream);
+uint64_t shrike_hip_pool_table_entry(const shrike_hip_pool *pool, uint32_t expert);
+
+/* ------------------------------------------------------------ MoE operators */
+
+/* MoE.init, sources/Shrike/Kernels/MoE/MoE.swift:94-216. */
+typedef struct {
+    uint32_t d, f, num_experts, top_k;
+    uint32_t routed_weight_bits;   /* 4 | 8 */
+    uint32_t router_weight_bits;   /* 0 = fp16 rows, 4 | 8 = group-affine */
+    uint32_t meta_dtype;           /* SHRIKE_META_* for every scale/bias tensor */
+    uint32_t activation;           /* SHRIKE_ACT_* */
+    uint32_t expert_additive_biases;
+    uint32_t sigmoid_router_scores;
+    float routed_scaling_factor;
+    uint32_t event_gated_io;       /* moe.metal:36-39: honour io_status words */
+} shrike_moe_desc;
+
+typedef struct shrike_hip_moe shrike_hip_moe;
+shrike_hip_moe *shrike_hip_moe_create(const shrike_moe_desc *desc, int *out_errno);
+void shrike_hip_moe_destroy(shrike_hip_moe *moe);
+
+/* MoE.encodeRouter, MoE.swift:249-316 (router_gemv_r4 + router_topk_select*,
+ * moe.metal:324-381, :419-582). hidden: fp16[d]; effective_scale: bf16[d];
+ * per_expert_scale, logit_bias: bf16[num_experts] (always read); out_indices:
+ * u32[top_k]; out_weights: fp16[top_k]. Router weights are fp16[num_experts, d]
+ * when router_weight_bits == 0 (scales/biases ignored). The fp32 logits land in
+ * the handle's own buffer (shrike_hip_moe_router_logits). */
+int shrike_hip_moe_router(shrike_hip_moe *moe, void *stream, const void *d_weights,
+                          const void *d_scales, const void *d_biases, const void *d_hidden,
+                          const void *d_effective_scale, const void *d_per_expert_scale,
+                          const void *d_logit_bias, uint32_t *d_out_indices,
+                          void *d_out_weights, uint32_t num_experts, uint32_t d,
+                          uint32_t top_k);
+const float *shrike_hip_moe_router_logits(const shrike_hip_moe *moe);
+
+/* MoE.encodeResidencyClassification, MoE.swift:552-610
+ * (moe_classify_expert_residency_spec, moe.metal:194-231). `full_grids` are the
+ * four full grids (12 words); d_spec_args receives the 12 published words: HIP
+ * has no indirect dispatch, so phase1/phase2 below read their grid word from it
+ * and return at once when it is zero. d_host_readback (2 + 5*top_k words, may be
+ * host-mapped pinned memory) is written when tag != 0. */
+int shrike_hip_moe_classify(shrike_hip_moe *moe, void *stream, const uint32_t *d_topk_indices,
+                            const uint64_t *d_residency, uint32_t *d_hit_count,
+                            uint32_t *d_hit_positions, uint32_t *d_miss_count,
+                            uint32_t *d_miss_positions, uint32_t *d_miss_experts,
+                            uint32_t *d_resolved_slots, uint32_t top_k, uint32_t num_experts,
+                            const uint32_t full_grids[12], uint32_t *d_spec_args,
+                            uint32_t *d_host_readback, uint32_t host_readback_tag,
+                            const void *d_topk_weights, const uint32_t *d_predicted_indices);
+
+/* MoE.encodeSpecPhase1U16Load, MoE.swift:906-951 (moe_phase1_gate_up_act_spec_u16load,
+ * moe.metal:950-999; 8-bit body moe.metal:650-672). x: fp16[d]; acts: fp16[top_k*f].
+ * A sentinel in d_resolved_slots skips that position. d_indirect (may be NULL) points
+ * at a 3-word grid; a zero first word dispatches nothing. d_io_status may be NULL. */
+int shrike_hip_moe_phase1_pool(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                               uint64_t pool_slot_stride, const uint32_t *d_resolved_slots,
+                               const shrike_expert_offsets *offsets, const void *d_x,
+                               void *d_acts, uint32_t d, uint32_t f, uint32_t top_k,
+                               const uint32_t *d_indirect, const uint32_t *d_io_status);
+
+/* MoE.encodeSpecPhase2Reduce, MoE.swift:992-1047 (moe_phase2_down_reduce_spec_k8,
+ * moe.metal:1008-1057): y = half(residual + sum_k half_w[k] * down_k . acts_k),
+ * hidden = half(hidden + y). A sentinel position takes d_fallback_cells[k] when that
+ * is given and contributes nothing otherwise. When event-gated and the status word
+ * is not ready, y = residual (moe.metal:918-921). */
+int shrike_hip_moe_phase2_pool(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                               uint64_t pool_slot_stride, const uint32_t *d_resolved_slots,
+                               const uint32_t *d_fallback_cells,
+                               const shrike_expert_offsets *offsets, const void *d_acts,
+                               const void *d_routing_weights, const void *d_residual,
+                               void *d_y, void *d_hidden, uint32_t d, uint32_t f,
+                               uint32_t top_k, const uint32_t *d_indirect,
+                               const uint32_t *d_io_status);
+
+/* SharedExpertInt4.encodeGateUp + encodeFusedDown / SharedExpertInt8
+ * (sources/Shrike/Kernels/MoE/SharedExpertInt4.swift:91-164, :251-342;
+ * dequant_int4.metal:206-331, dequant_int8.metal:109-164): h1 = half(down .
+ * half(glu(half(gate.x), half(up.x)))), optionally * sigmoid(scalar_gate[0]).
+ * d_scratch: fp16[2*f_shared] for the gate and up rows. */
+int shrike_hip_shared_expert(shrike_hip_moe *moe, void *stream, const shrike_projection *gate,
+                             const shrike_projection *up, const shrike_projection *down,
+                             uint32_t bits, const void *d_x, void *d_scratch, void *d_h1,
+                             const void *d_scalar_gate, uint32_t d, uint32_t f_shared);
+
+/* The whole decode layer as the runner encodes it
+ * (sources/Shrike/Runtime/Inference/RealForwardRunner.swift:2834-2901, :5520-5560):
+ * router -> select -> classify -> shared expert -> phase 1 -> phase 2 (+= hidden),
+ * in three launches. Same results as the calls above made one after another. */
+typedef struct {
+    /* router */
+    const void *router_weights, *router_scales, *router_biases;
+    const void *effective_scale, *per_expert_scale, *logit_bias;
+    /* pool */
+    const shrike_pool_bases *pool;
+    uint64_t pool_slot_stride;
+    const uint64_t *residency;
+    shrike_expert_offsets offsets;
+    /* shared expert (gate.weights == NULL: none, residual = 0) */
+    shrike_projection shared_gate, shared_up, shared_down;
+    uint32_t shared_bits, shared_f;
+    const void *shared_scalar_gate;
+    /* activations and outputs */
+    const void *x;          /* fp16[d] */
+    void *hidden;           /* fp16[d], += y */
+    void *y;                /* fp16[d] */
+    /* scratch the operator signatures assume (RealForwardRunner.swift:754-825) */
+    uint32_t *out_indices;  /* u32[top_k] */
+    void *out_weights;      /* fp16[top_k] */
+    uint32_t *resolved_slots, *hit_count, *hit_positions, *miss_count, *miss_positions,
+        *miss_experts;      /* u32[top_k] / u32[1] */
+    void *acts;             /* fp16[top_k*f] */
+    void *shared_scratch;   /* fp16[2*shared_f] */
+    void *h1;               /* fp16[d] */
+} shrike_decode_layer_args;
+int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
+                                const shrike_decode_layer_args *args);
+
+/* ----------------------------------------------------------------- plumbing
+ * Device memory, streams, events and graphs for hosts without a HIP binding of
+ * their own (the Python tests and benchmark). No counterpart in the reference,
+ * where Metal buffers and command queues play this part
+ * (sources/Shrike/Infrastructure/Metal/MetalContext.swift). Pointers returned are
+ * NULL on failure; int results are 0 or EIO. Streams are created at the default
+ * priority. */
+void *shrike_hip_malloc(uint64_t bytes);
+int shrike_hip_free(void *device_ptr);
+void *shrike_hip_host_alloc(uint64_t bytes);            /* pinned host memory */
+int shrike_hip_host_free(void *host_ptr);
+int shrike_hip_memcpy_h2d(void *dst, const void *src, uint64_t bytes);
+int shrike_hip_memcpy_d2h(void *dst, const void *src, uint64_t bytes);
+int shrike_hip_memcpy_d2d(void *dst, const void *src, uint64_t bytes);
+int shrike_hip_memcpy_h2d_async(void *dst, const void *src, uint64_t bytes, void *stream);
+int shrike_hip_memset(void *dst, int value, uint64_t bytes);
+int shrike_hip_device_synchronize(void);
+int shrike_hip_mem_info(uint64_t *free_bytes, uint64_t *total_bytes);
+void *shrike_hip_stream_create(void);
+int shrike_hip_stream_destroy(void *stream);
+int shrike_hip_stream_synchronize(void *stream);
+void *shrike_hip_event_create(void);
+int shrike_hip_event_destroy(void *event);
+int shrike_hip_event_record(void *event, void *stream);
+int shrike_hip_event_synchronize(void *event);
+int shrike_hip_stream_wait_event(void *stream, void *event);
+int shrike_hip_event_elapsed_ms(void *start, void *stop, float *ms);
+int shrike_hip_graph_begin_capture(void *stream);
+void *shrike_hip_graph_end_capture(void *stream);       /* -> executable graph */
+int shrike_hip_graph_launch(void *graph_exec, void *stream);
+int shrike_hip_graph_destroy(void *graph_exec);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

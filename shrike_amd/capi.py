@@ -1,0 +1,149 @@
+"""ctypes binding of libshrikehip.so (include/shrike_hip.h).
+
+The library is the product; this module only declares its entry points. There is
+no fallback: if the shared object is missing or a call fails, an exception says so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libshrikehip.so")
+
+MAX_TOP_K = 8
+POOL_MAX_CHUNKS = 8
+SENTINEL = 0xFFFFFFFF
+POOL_PAGE = 16384
+META_BF16, META_F16 = 0, 1
+ACT_GELU_TANH, ACT_SILU, ACT_CLAMPED_SWIGLU = 0, 1, 2
+EMPTY, LOADING, RESIDENT = 0, 1, 2
+
+
+class ShrikeError(RuntimeError):
+    pass
+
+
+class ExpertOffsets(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in (
+        "gate_w_off", "gate_s_off", "gate_b_off", "up_w_off", "up_s_off", "up_b_off",
+        "down_w_off", "down_s_off", "down_b_off", "gate_ab_off", "up_ab_off", "down_ab_off")]
+
+
+class PoolBases(C.Structure):
+    _fields_ = [("base", C.c_void_p * POOL_MAX_CHUNKS), ("cells_per_chunk", C.c_uint32)]
+
+
+class Projection(C.Structure):
+    _fields_ = [("weights", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p)]
+
+
+class MoEDesc(C.Structure):
+    _fields_ = [("d", C.c_uint32), ("f", C.c_uint32), ("num_experts", C.c_uint32),
+                ("top_k", C.c_uint32), ("routed_weight_bits", C.c_uint32),
+                ("router_weight_bits", C.c_uint32), ("meta_dtype", C.c_uint32),
+                ("activation", C.c_uint32), ("expert_additive_biases", C.c_uint32),
+                ("sigmoid_router_scores", C.c_uint32), ("routed_scaling_factor", C.c_float),
+                ("event_gated_io", C.c_uint32)]
+
+
+class DecodeLayerArgs(C.Structure):
+    _fields_ = [
+        ("router_weights", C.c_void_p), ("router_scales", C.c_void_p), ("router_biases", C.c_void_p),
+        ("effective_scale", C.c_void_p), ("per_expert_scale", C.c_void_p), ("logit_bias", C.c_void_p),
+        ("pool", C.POINTER(PoolBases)), ("pool_slot_stride", C.c_uint64), ("residency", C.c_void_p),
+        ("offsets", ExpertOffsets),
+        ("shared_gate", Projection), ("shared_up", Projection), ("shared_down", Projection),
+        ("shared_bits", C.c_uint32), ("shared_f", C.c_uint32), ("shared_scalar_gate", C.c_void_p),
+        ("x", C.c_void_p), ("hidden", C.c_void_p), ("y", C.c_void_p),
+        ("out_indices", C.c_void_p), ("out_weights", C.c_void_p),
+        ("resolved_slots", C.c_void_p), ("hit_count", C.c_void_p), ("hit_positions", C.c_void_p),
+        ("miss_count", C.c_void_p), ("miss_positions", C.c_void_p), ("miss_experts", C.c_void_p),
+        ("acts", C.c_void_p), ("shared_scratch", C.c_void_p), ("h1", C.c_void_p)]
+
+
+# name -> (restype, argtypes); every symbol include/shrike_hip.h declares
+_VP, _U32, _U64, _I32, _I64 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_int32, C.c_int64
+SIGNATURES = {
+    "shrike_hip_last_error": (C.c_char_p, []),
+    "shrike_hip_init": (C.c_int, [C.c_int]),
+    "shrike_expert_offsets_make": (_U64, [_U32, _U32, _U32, C.c_int, C.POINTER(ExpertOffsets)]),
+    "shrike_parse_budget_bytes": (_I64, [C.c_char_p]),
+    "shrike_expert_cache_slots": (_I32, [_U64, _I32, _I64]),
+    "shrike_hip_pool_create": (_VP, [_U32, _U64, _U32, _U64, C.POINTER(C.c_int)]),
+    "shrike_hip_pool_destroy": (None, [_VP]),
+    "shrike_hip_pool_slot_stride": (_U64, [_VP]),
+    "shrike_hip_pool_cell_count": (_U32, [_VP]),
+    "shrike_hip_pool_cell_ptr": (_VP, [_VP, _U32]),
+    "shrike_hip_pool_bases": (C.POINTER(PoolBases), [_VP]),
+    "shrike_hip_pool_residency_table": (_VP, [_VP]),
+    "shrike_hip_pool_upload_async": (C.c_int, [_VP, _U32, _VP, _U64, _VP]),
+    "shrike_hip_pool_table_publish": (C.c_int, [_VP, _U32, _U32, _U32, _VP]),
+    "shrike_hip_pool_table_entry": (_U64, [_VP, _U32]),
+    "shrike_hip_moe_create": (_VP, [C.POINTER(MoEDesc), C.POINTER(C.c_int)]),
+    "shrike_hip_moe_destroy": (None, [_VP]),
+    "shrike_hip_moe_router": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
+                                        _U32, _U32, _U32]),
+    "shrike_hip_moe_router_logits": (_VP, [_VP]),
+    "shrike_hip_moe_classify": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _U32, _U32,
+                                          C.POINTER(_U32), _VP, _VP, _U32, _VP, _VP]),
+    "shrike_hip_moe_phase1_pool": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, _VP,
+                                             C.POINTER(ExpertOffsets), _VP, _VP, _U32, _U32, _U32,
+                                             _VP, _VP]),
+    "shrike_hip_moe_phase2_pool": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, _VP, _VP,
+                                             C.POINTER(ExpertOffsets), _VP, _VP, _VP, _VP, _VP,
+                                             _U32, _U32, _U32, _VP, _VP]),
+    "shrike_hip_shared_expert": (C.c_int, [_VP, _VP, C.POINTER(Projection), C.POINTER(Projection),
+                                           C.POINTER(Projection), _U32, _VP, _VP, _VP, _VP, _U32, _U32]),
+    "shrike_hip_moe_decode_layer": (C.c_int, [_VP, _VP, C.POINTER(DecodeLayerArgs)]),
+    "shrike_hip_malloc": (_VP, [_U64]),
+    "shrike_hip_free": (C.c_int, [_VP]),
+    "shrike_hip_host_alloc": (_VP, [_U64]),
+    "shrike_hip_host_free": (C.c_int, [_VP]),
+    "shrike_hip_memcpy_h2d": (C.c_int, [_VP, _VP, _U64]),
+    "shrike_hip_memcpy_d2h": (C.c_int, [_VP, _VP, _U64]),
+    "shrike_hip_memcpy_d2d": (C.c_int, [_VP, _VP, _U64]),
+    "shrike_hip_memcpy_h2d_async": (C.c_int, [_VP, _VP, _U64, _VP]),
+    "shrike_hip_memset": (C.c_int, [_VP, C.c_int, _U64]),
+    "shrike_hip_device_synchronize": (C.c_int, []),
+    "shrike_hip_mem_info": (C.c_int, [C.POINTER(_U64), C.POINTER(_U64)]),
+    "shrike_hip_stream_create": (_VP, []),
+    "shrike_hip_stream_destroy": (C.c_int, [_VP]),
+    "shrike_hip_stream_synchronize": (C.c_int, [_VP]),
+    "shrike_hip_event_create": (_VP, []),
+    "shrike_hip_event_destroy": (C.c_int, [_VP]),
+    "shrike_hip_event_record": (C.c_int, [_VP, _VP]),
+    "shrike_hip_event_synchronize": (C.c_int, [_VP]),
+    "shrike_hip_stream_wait_event": (C.c_int, [_VP, _VP]),
+    "shrike_hip_event_elapsed_ms": (C.c_int, [_VP, _VP, C.POINTER(C.c_float)]),
+    "shrike_hip_graph_begin_capture": (C.c_int, [_VP]),
+    "shrike_hip_graph_end_capture": (_VP, [_VP]),
+    "shrike_hip_graph_launch": (C.c_int, [_VP, _VP]),
+    "shrike_hip_graph_destroy": (C.c_int, [_VP]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the built library; raise if it has not been built (no fallback exists)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ShrikeError(
+                f"{LIB_PATH} is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')")
+        lib = C.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+            fn.restype, fn.argtypes = restype, argtypes
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().shrike_hip_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise ShrikeError(f"{what} failed with {rc} ({os.strerror(rc)}): {last_error()}")

@@ -1,0 +1,171 @@
+// Device helpers shared by the gfx950 kernels: 16-bit float decoding, wave64
+// reductions over DPP, and the in-register dequant dot products.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+namespace shrike {
+
+constexpr uint32_t kGroup = 64;
+constexpr uint32_t kSentinel = 0xffffffffu;
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(uint32_t(b) << 16); }
+__device__ __forceinline__ float f16_to_f32(uint16_t b) {
+    return float(__builtin_bit_cast(_Float16, b));
+}
+__device__ __forceinline__ uint16_t f32_to_f16(float v) {
+    return __builtin_bit_cast(uint16_t, _Float16(v));  // round-to-nearest-even
+}
+template <int META>
+__device__ __forceinline__ float meta_to_f32(uint16_t b) {
+    return META == 1 ? f16_to_f32(b) : bf16_to_f32(b);
+}
+
+__device__ __forceinline__ h2_t as_h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
+__device__ __forceinline__ uint32_t as_u32(h2_t h) { return __builtin_bit_cast(uint32_t, h); }
+
+// ---- DPP lane exchange. Control codes: quad_perm = 0x00..0xff, row_mirror 0x140,
+// row_half_mirror 0x141, row_bcast15 0x142, row_bcast31 0x143.
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+    return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), CTRL, ROW_MASK, 0xf, false));
+}
+
+// Sum over aligned lane segments of `seg` lanes (seg in {1,2,4,8,16,32,64}); every
+// lane of a segment's last 16-lane row ends up holding the segment sum, and for
+// seg <= 16 every lane of the segment does. Callers read lane (segment end - 1).
+__device__ __forceinline__ float seg_sum(float v, uint32_t seg) {
+    if (seg >= 2) v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+    if (seg >= 4) v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+    if (seg >= 8) v += dpp_f32<0x141>(v);  // row_half_mirror
+    if (seg >= 16) v += dpp_f32<0x140>(v); // row_mirror
+    if (seg >= 32) v += dpp_f32<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+    if (seg >= 64) v += dpp_f32<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v = seg_sum(v, 64);
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// Max of a 64-bit key over the wave; result broadcast to every lane.
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t key) {
+    uint32_t lo = uint32_t(key), hi = uint32_t(key >> 32);
+#define SHRIKE_MAX_STEP(CTRL, MASK)                                             \
+    {                                                                            \
+        const uint32_t olo = dpp_u32<CTRL, MASK>(lo), ohi = dpp_u32<CTRL, MASK>(hi); \
+        const bool take = ohi > hi || (ohi == hi && olo > lo);                  \
+        lo = take ? olo : lo;                                                   \
+        hi = take ? ohi : hi;                                                   \
+    }
+    SHRIKE_MAX_STEP(0xB1, 0xf)
+    SHRIKE_MAX_STEP(0x4E, 0xf)
+    SHRIKE_MAX_STEP(0x141, 0xf)
+    SHRIKE_MAX_STEP(0x140, 0xf)
+    SHRIKE_MAX_STEP(0x142, 0xA)
+    SHRIKE_MAX_STEP(0x143, 0xC)
+#undef SHRIKE_MAX_STEP
+    lo = uint32_t(__builtin_amdgcn_readlane(int(lo), 63));
+    hi = uint32_t(__builtin_amdgcn_readlane(int(hi), 63));
+    return (uint64_t(hi) << 32) | lo;
+}
+
+// ---- 16-byte chunk of codes against the lane's activation slice.
+//
+// A chunk is 4 little-endian words. For 4-bit codes word j holds elements 8j..8j+7
+// (element i in bits 4i..4i+3). Codes become exact fp16 values in packed pairs with
+// the 0x6400 (=1024.0) exponent trick: (w & 0x000F000F) | 0x64006400 is the pair
+// {1024+q0, 1024+q4}; the pair taken from bits 4..7 / 20..23 is {1024+16*q1,
+// 1024+16*q5}, brought back by one packed fma with 1/16 and -64. The activation
+// slice is therefore kept as the pairs (e0,e4) (e1,e5) (e2,e6) (e3,e7) per word
+// (pairs_from_x8 below), and each pair costs one 2-way fp16 dot accumulated in fp32.
+struct XChunk4 { h2_t p[16]; };   // 32 activations of a 4-bit chunk, pair layout
+struct XChunk8 { h2_t p[8]; };    // 16 activations of an 8-bit chunk, natural pairs
+
+__device__ __forceinline__ void pairs_from_x8(const uint4 v, h2_t *p) {
+    // v = elements e0..e7 as (e0,e1)(e2,e3)(e4,e5)(e6,e7)
+    p[0] = as_h2(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u));  // (e0,e4)
+    p[1] = as_h2(__builtin_amdgcn_perm(v.z, v.x, 0x07060302u));  // (e1,e5)
+    p[2] = as_h2(__builtin_amdgcn_perm(v.w, v.y, 0x05040100u));  // (e2,e6)
+    p[3] = as_h2(__builtin_amdgcn_perm(v.w, v.y, 0x07060302u));  // (e3,e7)
+}
+
+__device__ __forceinline__ float sum_x8(const uint4 v) {
+    const h2_t a = as_h2(v.x), b = as_h2(v.y), c = as_h2(v.z), d = as_h2(v.w);
+    return ((float(a.x) + float(a.y)) + (float(b.x) + float(b.y)))
+         + ((float(c.x) + float(c.y)) + (float(d.x) + float(d.y)));
+}
+
+__device__ __forceinline__ float dot_word4(uint32_t w, const h2_t *p, float acc) {
+    const h2_t k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    const h2_t k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const h2_t k64 = {(_Float16)64.0f, (_Float16)64.0f};
+    const uint32_t w8 = w >> 8;
+    const h2_t q04 = as_h2((w & 0x000F000Fu) | 0x64006400u) - k1024;
+    const h2_t q15 = __builtin_elementwise_fma(as_h2((w & 0x00F000F0u) | 0x64006400u), k16th, -k64);
+    const h2_t q26 = as_h2((w8 & 0x000F000Fu) | 0x64006400u) - k1024;
+    const h2_t q37 = __builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x64006400u), k16th, -k64);
+    acc = __builtin_amdgcn_fdot2(q04, p[0], acc, false);
+    acc = __builtin_amdgcn_fdot2(q15, p[1], acc, false);
+    acc = __builtin_amdgcn_fdot2(q26, p[2], acc, false);
+    acc = __builtin_amdgcn_fdot2(q37, p[3], acc, false);
+    return acc;
+}
+
+__device__ __forceinline__ float dot_chunk4(const uint4 w, const XChunk4 &x) {
+    float acc = 0.0f;
+    acc = dot_word4(w.x, x.p + 0, acc);
+    acc = dot_word4(w.y, x.p + 4, acc);
+    acc = dot_word4(w.z, x.p + 8, acc);
+    acc = dot_word4(w.w, x.p + 12, acc);
+    return acc;
+}
+
+// 8-bit codes: bytes b0..b3 of a word are elements 4j..4j+3; a byte permute with a
+// register of 0x64 bytes builds the pairs {1024+b0, 1024+b1} and {1024+b2, 1024+b3}.
+__device__ __forceinline__ float dot_word8(uint32_t w, const h2_t *p, float acc) {
+    const h2_t k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    const uint32_t magic = 0x64646464u;
+    const h2_t q01 = as_h2(__builtin_amdgcn_perm(magic, w, 0x04010400u)) - k1024;
+    const h2_t q23 = as_h2(__builtin_amdgcn_perm(magic, w, 0x04030402u)) - k1024;
+    acc = __builtin_amdgcn_fdot2(q01, p[0], acc, false);
+    acc = __builtin_amdgcn_fdot2(q23, p[1], acc, false);
+    return acc;
+}
+
+__device__ __forceinline__ float dot_chunk8(const uint4 w, const XChunk8 &x) {
+    float acc = 0.0f;
+    acc = dot_word8(w.x, x.p + 0, acc);
+    acc = dot_word8(w.y, x.p + 2, acc);
+    acc = dot_word8(w.z, x.p + 4, acc);
+    acc = dot_word8(w.w, x.p + 6, acc);
+    return acc;
+}
+
+__device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float gelu_tanh(float v) {
+    const float cube = v * v * v;
+    float inner = 0.7978845608028654f * (v + 0.044715f * cube);
+    inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+    return 0.5f * v * (1.0f + tanhf(inner));
+}
+// moe.metal:280-288
+template <int ACT>
+__device__ __forceinline__ float glu(float gate, float up) {
+    if (ACT == 2) {
+        const float g = fminf(gate, 7.0f);
+        const float u = fminf(fmaxf(up, -7.0f), 7.0f);
+        return (g / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
+    }
+    return (ACT == 1 ? silu(gate) : gelu_tanh(gate)) * up;
+}
+
+}  // namespace shrike

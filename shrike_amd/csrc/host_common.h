@@ -1,0 +1,44 @@
+// Host-side plumbing shared by the C-ABI translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cerrno>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "../../include/shrike_hip.h"
+
+namespace shrike {
+
+void set_error(const char *fmt, ...);
+int hip_failed(hipError_t err, const char *what);  // records the error, returns EIO
+
+#define SHRIKE_REQUIRE(cond, ...)            \
+    do {                                     \
+        if (!(cond)) {                       \
+            ::shrike::set_error(__VA_ARGS__); \
+            return EINVAL;                   \
+        }                                    \
+    } while (0)
+
+#define SHRIKE_HIP(call)                                             \
+    do {                                                             \
+        hipError_t err__ = (call);                                   \
+        if (err__ != hipSuccess) return ::shrike::hip_failed(err__, #call); \
+    } while (0)
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+}  // namespace shrike
+
+// MoE.swift:41-216: the handle keeps the shape it was made for, the router's fp32
+// logits (routerLogits, MoE.swift:74) and the router's arrival counter.
+struct shrike_hip_moe {
+    shrike_moe_desc desc;
+    int device;
+    float *d_logits;        // fp32[SHRIKE_MAX_ROUTER_EXPERTS]
+    uint32_t *d_counter;    // u32[4], zero between launches
+};

@@ -1,0 +1,400 @@
+// Handles, the HBM slot pool and the small pure functions of the C ABI.
+#include "host_common.h"
+
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+namespace shrike {
+
+static thread_local std::string g_last_error;
+
+void set_error(const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+}
+
+int hip_failed(hipError_t err, const char *what) {
+    set_error("%s failed: %s", what, hipGetErrorString(err));
+    return EIO;
+}
+
+__global__ void k_store_u64(uint64_t *dst, uint64_t value) { *dst = value; }
+
+}  // namespace shrike
+
+using namespace shrike;
+
+// ExpertCellArena.swift:16-133 + the residency table of PreadExpertStreamer.swift:283-352.
+struct shrike_hip_pool {
+    uint32_t cells, num_experts, cells_per_chunk, chunk_count;
+    uint64_t stride;
+    void *chunks[SHRIKE_POOL_MAX_CHUNKS];
+    shrike_pool_bases bases;
+    uint64_t *d_table;
+    std::vector<uint64_t> shadow;  // host copy of the table, updated at publish
+};
+
+extern "C" {
+
+const char *shrike_hip_last_error(void) { return g_last_error.c_str(); }
+
+int shrike_hip_init(int device) {
+    int count = 0;
+    SHRIKE_HIP(hipGetDeviceCount(&count));
+    SHRIKE_REQUIRE(device >= 0 && device < count, "device %d of %d is not present", device, count);
+    SHRIKE_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    SHRIKE_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+        return ENODEV;
+    }
+    return 0;
+}
+
+uint64_t shrike_expert_offsets_make(uint32_t d, uint32_t f, uint32_t bits, int additive_biases,
+                                    shrike_expert_offsets *out) {
+    if (!out || (bits != 4 && bits != 8) || d == 0 || f == 0 || d % SHRIKE_GROUP_SIZE || f % SHRIKE_GROUP_SIZE) {
+        set_error("Offsets: d=%u and f=%u must be positive multiples of %u and bits=%u one of 4, 8", d, f,
+                  SHRIKE_GROUP_SIZE, bits);
+        return 0;
+    }
+    const uint64_t gate_codes = uint64_t(f) * d * bits / 8, gate_meta = uint64_t(f) * (d / SHRIKE_GROUP_SIZE) * 2;
+    const uint64_t down_codes = uint64_t(d) * f * bits / 8, down_meta = uint64_t(d) * (f / SHRIKE_GROUP_SIZE) * 2;
+    uint64_t at = 0;
+    auto take = [&at](uint64_t size) { const uint64_t here = at; at += size; return uint32_t(here); };
+    out->gate_w_off = take(gate_codes); out->gate_s_off = take(gate_meta); out->gate_b_off = take(gate_meta);
+    out->up_w_off = take(gate_codes); out->up_s_off = take(gate_meta); out->up_b_off = take(gate_meta);
+    out->down_w_off = take(down_codes); out->down_s_off = take(down_meta); out->down_b_off = take(down_meta);
+    out->gate_ab_off = out->up_ab_off = out->down_ab_off = 0;
+    if (additive_biases) {
+        out->gate_ab_off = take(uint64_t(f) * 2); out->up_ab_off = take(uint64_t(f) * 2);
+        out->down_ab_off = take(uint64_t(d) * 2);
+    }
+    return at;
+}
+
+// ------------------------------------------------------------------ budget
+
+// RuntimeConfiguration.swift:111-129
+int64_t shrike_parse_budget_bytes(const char *text) {
+    if (!text) return -1;
+    std::string raw(text);
+    auto trim = [](std::string &s) {
+        size_t a = 0, b = s.size();
+        while (a < b && (s[a] == ' ' || s[a] == '\t')) ++a;  // Swift's .whitespaces: space and tab
+        while (b > a && (s[b - 1] == ' ' || s[b - 1] == '\t')) --b;
+        s = s.substr(a, b - a);
+    };
+    trim(raw);
+    for (char &c : raw) c = char(toupper((unsigned char)c));
+    if (raw.empty()) return -1;
+    static const struct { const char *suffix; int64_t scale; } kMultipliers[] = {
+        {"GIB", int64_t(1) << 30}, {"MIB", int64_t(1) << 20}, {"KIB", int64_t(1) << 10},
+        {"GB", int64_t(1) << 30},  {"MB", int64_t(1) << 20},  {"KB", int64_t(1) << 10},
+        {"G", int64_t(1) << 30},   {"M", int64_t(1) << 20},   {"K", int64_t(1) << 10},
+    };
+    for (const auto &m : kMultipliers) {
+        const size_t n = strlen(m.suffix);
+        if (raw.size() < n || raw.compare(raw.size() - n, n, m.suffix) != 0) continue;
+        std::string number = raw.substr(0, raw.size() - n);
+        trim(number);
+        if (number.empty()) return -1;
+        // Swift's Double(String): the whole string must parse; no leading/trailing blanks
+        char *end = nullptr;
+        errno = 0;
+        const double value = strtod(number.c_str(), &end);
+        if (end == number.c_str() || *end != '\0' || isspace((unsigned char)number[0])) return -1;
+        if (!(value > 0)) return -1;
+        const double bytes = value * double(m.scale);
+        if (!std::isfinite(bytes) || bytes < 1 || !(bytes < 9223372036854775807.0)) return -1;
+        return int64_t(bytes);
+    }
+    if (raw.empty()) return -1;
+    size_t i = 0;
+    if (raw[0] == '+' || raw[0] == '-') i = 1;
+    if (i >= raw.size()) return -1;
+    for (size_t j = i; j < raw.size(); ++j)
+        if (raw[j] < '0' || raw[j] > '9') return -1;
+    errno = 0;
+    const long long plain = strtoll(raw.c_str(), nullptr, 10);
+    if (errno == ERANGE || plain <= 0) return -1;
+    return plain;
+}
+
+// RuntimeConfiguration.swift:77, :137-149
+int32_t shrike_expert_cache_slots(uint64_t expert_stride_bytes, int32_t layers, int64_t budget_bytes) {
+    static const int32_t kAllowed[] = {8, 16, 24, 32, 64, 96, 128, 160, 192, 224, 256};
+    if (expert_stride_bytes == 0 || layers <= 0) return kAllowed[0];
+    const double per_slot = double(expert_stride_bytes) * double(layers);
+    const double wanted = double(budget_bytes) / per_slot;
+    int32_t best = kAllowed[0];
+    for (int32_t slots : kAllowed)  // Swift's min(by:) keeps the first of equal elements
+        if (std::fabs(double(slots) - wanted) < std::fabs(double(best) - wanted)) best = slots;
+    return best;
+}
+
+// -------------------------------------------------------------------- pool
+
+shrike_hip_pool *shrike_hip_pool_create(uint32_t cells, uint64_t expert_stride, uint32_t num_experts,
+                                        uint64_t chunk_bytes, int *out_errno) {
+    auto fail = [&](int code) -> shrike_hip_pool * { if (out_errno) *out_errno = code; return nullptr; };
+    if (cells == 0 || expert_stride == 0 || num_experts == 0) {
+        set_error("invalid expert cell arena geometry: %u cells of %llu bytes for %u experts", cells,
+                  (unsigned long long)expert_stride, num_experts);
+        return fail(EINVAL);
+    }
+    // PreadExpertStreamer.swift:283-287: the slot stride is the expert stride rounded up to a page.
+    const uint64_t stride = (expert_stride + SHRIKE_POOL_PAGE - 1) / SHRIKE_POOL_PAGE * SHRIKE_POOL_PAGE;
+    // ExpertCellArena.swift:41-50
+    const uint64_t limit = chunk_bytes ? chunk_bytes : ~uint64_t(0);
+    uint64_t per_chunk = limit / stride;
+    if (per_chunk < 1) per_chunk = 1;
+    if (per_chunk > cells) per_chunk = cells;
+    const uint32_t chunk_count = uint32_t((cells + per_chunk - 1) / per_chunk);
+    if (chunk_count > SHRIKE_POOL_MAX_CHUNKS) {
+        set_error("expert cell arena of %u cells needs %u chunks of %llu; the kernels address at most %u", cells,
+                  chunk_count, (unsigned long long)per_chunk, SHRIKE_POOL_MAX_CHUNKS);
+        return fail(EINVAL);
+    }
+    shrike_hip_pool *pool = new shrike_hip_pool();
+    pool->cells = cells; pool->num_experts = num_experts; pool->stride = stride;
+    pool->cells_per_chunk = uint32_t(per_chunk); pool->chunk_count = chunk_count;
+    memset(pool->chunks, 0, sizeof(pool->chunks));
+    pool->d_table = nullptr;
+    for (uint32_t c = 0; c < chunk_count; ++c) {
+        const uint64_t n = std::min<uint64_t>(per_chunk, cells - uint64_t(c) * per_chunk);
+        if (hipMalloc(&pool->chunks[c], n * stride) != hipSuccess) {
+            set_error("hipMalloc of %llu bytes for pool chunk %u failed", (unsigned long long)(n * stride), c);
+            shrike_hip_pool_destroy(pool);
+            return fail(ENOMEM);
+        }
+    }
+    for (uint32_t i = 0; i < SHRIKE_POOL_MAX_CHUNKS; ++i)  // ExpertCellArena.swift:80-83
+        pool->bases.base[i] = pool->chunks[i < chunk_count ? i : chunk_count - 1];
+    pool->bases.cells_per_chunk = pool->cells_per_chunk;
+    pool->shadow.assign(num_experts, uint64_t(SHRIKE_RESIDENCY_EMPTY) << 32 | SHRIKE_SLOT_SENTINEL);
+    if (hipMalloc(reinterpret_cast<void **>(&pool->d_table), sizeof(uint64_t) * num_experts) != hipSuccess
+        || hipMemcpy(pool->d_table, pool->shadow.data(), sizeof(uint64_t) * num_experts, hipMemcpyHostToDevice)
+               != hipSuccess) {
+        set_error("residency table allocation failed");
+        shrike_hip_pool_destroy(pool);
+        return fail(ENOMEM);
+    }
+    if (out_errno) *out_errno = 0;
+    return pool;
+}
+
+void shrike_hip_pool_destroy(shrike_hip_pool *pool) {
+    if (!pool) return;
+    for (void *c : pool->chunks)
+        if (c) (void)hipFree(c);
+    if (pool->d_table) (void)hipFree(pool->d_table);
+    delete pool;
+}
+
+uint64_t shrike_hip_pool_slot_stride(const shrike_hip_pool *pool) { return pool ? pool->stride : 0; }
+uint32_t shrike_hip_pool_cell_count(const shrike_hip_pool *pool) { return pool ? pool->cells : 0; }
+
+void *shrike_hip_pool_cell_ptr(const shrike_hip_pool *pool, uint32_t cell) {
+    if (!pool || cell >= pool->cells) { set_error("expert cell out of range"); return nullptr; }
+    return static_cast<uint8_t *>(pool->chunks[cell / pool->cells_per_chunk])
+        + uint64_t(cell % pool->cells_per_chunk) * pool->stride;
+}
+
+const shrike_pool_bases *shrike_hip_pool_bases(const shrike_hip_pool *pool) { return pool ? &pool->bases : nullptr; }
+void *shrike_hip_pool_residency_table(const shrike_hip_pool *pool) { return pool ? pool->d_table : nullptr; }
+
+int shrike_hip_pool_upload_async(shrike_hip_pool *pool, uint32_t cell, const void *host_src, uint64_t bytes,
+                                 void *stream) {
+    SHRIKE_REQUIRE(pool && host_src, "pool or source is NULL");
+    SHRIKE_REQUIRE(cell < pool->cells, "expert cell %u out of range (%u cells)", cell, pool->cells);
+    SHRIKE_REQUIRE(bytes <= pool->stride, "%llu bytes do not fit a cell of %llu", (unsigned long long)bytes,
+                   (unsigned long long)pool->stride);
+    SHRIKE_HIP(hipMemcpyAsync(shrike_hip_pool_cell_ptr(pool, cell), host_src, bytes, hipMemcpyHostToDevice,
+                              as_stream(stream)));
+    return 0;
+}
+
+int shrike_hip_pool_table_publish(shrike_hip_pool *pool, uint32_t expert, uint32_t cell, uint32_t state,
+                                  void *stream) {
+    SHRIKE_REQUIRE(pool != nullptr, "pool is NULL");
+    if (expert >= pool->num_experts) return 0;  // PreadExpertStreamer.swift:1144: out-of-range experts are ignored
+    SHRIKE_REQUIRE(state <= SHRIKE_RESIDENCY_RESIDENT, "state %u is not a residency state", state);
+    SHRIKE_REQUIRE(state == SHRIKE_RESIDENCY_EMPTY || cell < pool->cells, "cell %u out of range", cell);
+    const uint32_t slot = state == SHRIKE_RESIDENCY_EMPTY ? SHRIKE_SLOT_SENTINEL : cell;
+    const uint64_t word = uint64_t(state) << 32 | slot;
+    pool->shadow[expert] = word;
+    hipLaunchKernelGGL(k_store_u64, dim3(1), dim3(1), 0, as_stream(stream), pool->d_table + expert, word);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+uint64_t shrike_hip_pool_table_entry(const shrike_hip_pool *pool, uint32_t expert) {
+    if (!pool || expert >= pool->num_experts) return uint64_t(SHRIKE_RESIDENCY_EMPTY) << 32 | SHRIKE_SLOT_SENTINEL;
+    return pool->shadow[expert];
+}
+
+// --------------------------------------------------------------------- moe
+
+shrike_hip_moe *shrike_hip_moe_create(const shrike_moe_desc *desc, int *out_errno) {
+    auto fail = [&](int code) -> shrike_hip_moe * { if (out_errno) *out_errno = code; return nullptr; };
+    if (!desc) { set_error("desc is NULL"); return fail(EINVAL); }
+    // MoE.swift:113-116
+    if (desc->routed_weight_bits != 4 && desc->routed_weight_bits != 8) {
+        set_error("routedWeightBits=%u not in {4, 8}", desc->routed_weight_bits); return fail(EINVAL);
+    }
+    if (desc->router_weight_bits != 0 && desc->router_weight_bits != 4 && desc->router_weight_bits != 8) {
+        set_error("routerWeightBits=%u not in {0 (fp16), 4, 8}", desc->router_weight_bits); return fail(EINVAL);
+    }
+    if (desc->top_k < 1 || desc->top_k > SHRIKE_MAX_TOP_K) {
+        set_error("topK=%u not in 1...%u", desc->top_k, SHRIKE_MAX_TOP_K); return fail(EINVAL);
+    }
+    if (desc->d == 0 || desc->d > SHRIKE_MAX_HIDDEN || desc->d % SHRIKE_GROUP_SIZE) {
+        set_error("d=%u must be a multiple of %u and at most %u", desc->d, SHRIKE_GROUP_SIZE, SHRIKE_MAX_HIDDEN);
+        return fail(EINVAL);
+    }
+    if (desc->f == 0 || desc->f % SHRIKE_GROUP_SIZE) {
+        set_error("f=%u must be a positive multiple of %u", desc->f, SHRIKE_GROUP_SIZE); return fail(EINVAL);
+    }
+    if (desc->num_experts < desc->top_k || desc->num_experts > SHRIKE_MAX_ROUTER_EXPERTS) {
+        set_error("numExperts=%u must be in topK...%u", desc->num_experts, SHRIKE_MAX_ROUTER_EXPERTS);
+        return fail(EINVAL);
+    }
+    if (desc->meta_dtype > SHRIKE_META_F16 || desc->activation > SHRIKE_ACT_CLAMPED_SWIGLU) {
+        set_error("metaDtype=%u or activation=%u is not a known value", desc->meta_dtype, desc->activation);
+        return fail(EINVAL);
+    }
+    shrike_hip_moe *moe = new shrike_hip_moe();
+    moe->desc = *desc;
+    moe->d_logits = nullptr; moe->d_counter = nullptr;
+    if (hipGetDevice(&moe->device) != hipSuccess
+        || hipMalloc(reinterpret_cast<void **>(&moe->d_logits), sizeof(float) * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess
+        || hipMalloc(reinterpret_cast<void **>(&moe->d_counter), sizeof(uint32_t) * 4) != hipSuccess
+        || hipMemset(moe->d_counter, 0, sizeof(uint32_t) * 4) != hipSuccess
+        || hipMemset(moe->d_logits, 0, sizeof(float) * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess) {
+        set_error("device allocation for the MoE handle failed: %s", hipGetErrorString(hipGetLastError()));
+        shrike_hip_moe_destroy(moe);
+        return fail(ENOMEM);
+    }
+    if (out_errno) *out_errno = 0;
+    return moe;
+}
+
+void shrike_hip_moe_destroy(shrike_hip_moe *moe) {
+    if (!moe) return;
+    if (moe->d_logits) (void)hipFree(moe->d_logits);
+    if (moe->d_counter) (void)hipFree(moe->d_counter);
+    delete moe;
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------- plumbing
+// Device memory, streams, events and graphs for hosts that have no HIP binding of
+// their own (the Python tests and benchmark). No counterpart in the reference: Metal
+// buffers and command queues play this part there (MetalContext.swift).
+extern "C" {
+
+void *shrike_hip_malloc(uint64_t bytes) {
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes ? bytes : 1) != hipSuccess) {
+        set_error("hipMalloc(%llu) failed: %s", (unsigned long long)bytes, hipGetErrorString(hipGetLastError()));
+        return nullptr;
+    }
+    return p;
+}
+int shrike_hip_free(void *p) { if (p) SHRIKE_HIP(hipFree(p)); return 0; }
+void *shrike_hip_host_alloc(uint64_t bytes) {
+    void *p = nullptr;
+    if (hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault) != hipSuccess) {
+        set_error("hipHostMalloc(%llu) failed: %s", (unsigned long long)bytes, hipGetErrorString(hipGetLastError()));
+        return nullptr;
+    }
+    return p;
+}
+int shrike_hip_host_free(void *p) { if (p) SHRIKE_HIP(hipHostFree(p)); return 0; }
+int shrike_hip_memcpy_h2d(void *dst, const void *src, uint64_t bytes) {
+    SHRIKE_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice)); return 0;
+}
+int shrike_hip_memcpy_d2h(void *dst, const void *src, uint64_t bytes) {
+    SHRIKE_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost)); return 0;
+}
+int shrike_hip_memcpy_d2d(void *dst, const void *src, uint64_t bytes) {
+    SHRIKE_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice)); return 0;
+}
+int shrike_hip_memcpy_h2d_async(void *dst, const void *src, uint64_t bytes, void *stream) {
+    SHRIKE_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream))); return 0;
+}
+int shrike_hip_memset(void *dst, int value, uint64_t bytes) { SHRIKE_HIP(hipMemset(dst, value, bytes)); return 0; }
+int shrike_hip_device_synchronize(void) { SHRIKE_HIP(hipDeviceSynchronize()); return 0; }
+int shrike_hip_mem_info(uint64_t *free_bytes, uint64_t *total_bytes) {
+    size_t f = 0, t = 0;
+    SHRIKE_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return 0;
+}
+
+void *shrike_hip_stream_create(void) {
+    hipStream_t s = nullptr;  // default priority only
+    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) {
+        set_error("hipStreamCreate failed: %s", hipGetErrorString(hipGetLastError()));
+        return nullptr;
+    }
+    return s;
+}
+int shrike_hip_stream_destroy(void *s) { if (s) SHRIKE_HIP(hipStreamDestroy(as_stream(s))); return 0; }
+int shrike_hip_stream_synchronize(void *s) { SHRIKE_HIP(hipStreamSynchronize(as_stream(s))); return 0; }
+
+void *shrike_hip_event_create(void) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+        set_error("hipEventCreate failed: %s", hipGetErrorString(hipGetLastError()));
+        return nullptr;
+    }
+    return e;
+}
+int shrike_hip_event_destroy(void *e) { if (e) SHRIKE_HIP(hipEventDestroy(static_cast<hipEvent_t>(e))); return 0; }
+int shrike_hip_event_record(void *e, void *stream) {
+    SHRIKE_HIP(hipEventRecord(static_cast<hipEvent_t>(e), as_stream(stream))); return 0;
+}
+int shrike_hip_event_synchronize(void *e) { SHRIKE_HIP(hipEventSynchronize(static_cast<hipEvent_t>(e))); return 0; }
+int shrike_hip_stream_wait_event(void *stream, void *e) {
+    SHRIKE_HIP(hipStreamWaitEvent(as_stream(stream), static_cast<hipEvent_t>(e), 0)); return 0;
+}
+int shrike_hip_event_elapsed_ms(void *start, void *stop, float *ms) {
+    SHRIKE_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop))); return 0;
+}
+
+int shrike_hip_graph_begin_capture(void *stream) {
+    SHRIKE_REQUIRE(stream != nullptr, "graph capture needs an explicit stream");
+    SHRIKE_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal)); return 0;
+}
+void *shrike_hip_graph_end_capture(void *stream) {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    if (hipStreamEndCapture(as_stream(stream), &graph) != hipSuccess || graph == nullptr) {
+        set_error("hipStreamEndCapture failed: %s", hipGetErrorString(hipGetLastError()));
+        return nullptr;
+    }
+    const hipError_t err = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (err != hipSuccess) { set_error("hipGraphInstantiate failed: %s", hipGetErrorString(err)); return nullptr; }
+    return exec;
+}
+int shrike_hip_graph_launch(void *exec, void *stream) {
+    SHRIKE_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(exec), as_stream(stream))); return 0;
+}
+int shrike_hip_graph_destroy(void *exec) {
+    if (exec) SHRIKE_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(exec))); return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,436 @@
+"""GPU parity: the decode kernels behind the C ABI against the CPU oracle on the same
+seeded bytes. Routing indices, residency lists and logits are compared bit for bit;
+FFN outputs within max-abs 2e-3 / relative 1e-3 (|a-b| <= 2e-3 + 1e-3*|b|)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from shrike_amd import capi
+from shrike_amd import synth as S
+from tests.helpers import Layer, assert_ffn_close, f16
+
+pytestmark = pytest.mark.gpu
+SENT = 0xFFFFFFFF
+
+
+class DeviceLayer:
+    """Uploads a Layer: every expert resident in a pool, cell = a permutation of the expert id."""
+
+    def __init__(self, rt, layer: Layer, cells=None, chunk_bytes=0, resident=None, moe_kwargs=None):
+        self.rt, self.L = rt, layer
+        L = layer
+        cells = cells or L.ne
+        self.pool = rt.ExpertPool(cells, L.stride, L.ne, chunk_bytes)
+        self.cell_of = {}
+        resident = range(L.ne) if resident is None else resident
+        for i, e in enumerate(resident):
+            cell = (i * 7 + 3) % cells if cells == L.ne and np.gcd(7, cells) == 1 else i
+            self.pool.upload(cell, L.blobs[e])
+            self.pool.publish(e, cell, capi.RESIDENT)
+            self.cell_of[e] = cell
+        self.off, stride = rt.expert_offsets(L.d, L.f, L.bits, L.additive)
+        assert stride == L.stride
+        kw = dict(routed_bits=L.bits, router_bits=L.router_bits, meta=L.meta)
+        kw.update(moe_kwargs or {})
+        self.moe = rt.MoE(L.d, L.f, L.ne, L.k, **kw)
+        dev = rt.dev
+        self.router_w = dev(L.router_w)
+        self.router_s = dev(L.router_s) if L.router_s is not None else None
+        self.router_b = dev(L.router_b) if L.router_b is not None else None
+        self.eff_scale, self.expert_scale, self.logit_bias = dev(L.eff_scale), dev(L.expert_scale), dev(L.logit_bias)
+        self.x, self.hidden = dev(L.x), dev(L.hidden)
+        self.out_idx, self.out_w = rt.empty(4 * 8), rt.empty(2 * 8)
+        self.resolved = rt.empty(4 * 8)
+        self.hit_count, self.miss_count = rt.empty(4), rt.empty(4)
+        self.hit_pos, self.miss_pos, self.miss_exp = rt.empty(32), rt.empty(32), rt.empty(32)
+        self.acts = rt.empty(2 * L.k * L.f)
+        self.y, self.h1 = rt.empty(2 * L.d), rt.empty(2 * L.d)
+        if L.shared_f:
+            self.shared = {n: tuple(dev(t) for t in L.shared[n]) for n in ("gate", "up", "down")}
+            self.shared_scratch = rt.empty(2 * 2 * L.shared_f)
+
+    def pool_blobs(self):
+        """cell -> blob, for the oracle."""
+        out = {}
+        for e, c in self.cell_of.items():
+            out[c] = self.L.blobs[e]
+        return out
+
+    def residency_words(self):
+        return np.array([self.pool.entry(e) for e in range(self.L.ne)], np.uint64)
+
+    def layer_args(self):
+        L = self.L
+        a = capi.DecodeLayerArgs()
+        a.router_weights = self.router_w.ptr
+        a.router_scales = self.router_s.ptr if self.router_s else None
+        a.router_biases = self.router_b.ptr if self.router_b else None
+        a.effective_scale, a.per_expert_scale, a.logit_bias = self.eff_scale.ptr, self.expert_scale.ptr, self.logit_bias.ptr
+        a.pool, a.pool_slot_stride, a.residency = self.pool.bases, self.pool.stride, self.pool.table
+        a.offsets = self.off
+        if L.shared_f:
+            for name in ("gate", "up", "down"):
+                w, s, b = self.shared[name]
+                setattr(a, f"shared_{name}", capi.Projection(w.ptr, s.ptr, b.ptr))
+            a.shared_bits, a.shared_f = L.shared_bits, L.shared_f
+            a.shared_scratch = self.shared_scratch.ptr
+        a.x, a.hidden, a.y = self.x.ptr, self.hidden.ptr, self.y.ptr
+        a.out_indices, a.out_weights = self.out_idx.ptr, self.out_w.ptr
+        a.resolved_slots, a.hit_count, a.hit_positions = self.resolved.ptr, self.hit_count.ptr, self.hit_pos.ptr
+        a.miss_count, a.miss_positions, a.miss_experts = self.miss_count.ptr, self.miss_pos.ptr, self.miss_exp.ptr
+        a.acts, a.h1 = self.acts.ptr, self.h1.ptr
+        return a
+
+
+def oracle_layer(L: Layer, dl: DeviceLayer, **kw):
+    shared = None
+    if L.shared_f:
+        shared = dict(gate=L.shared["gate"], up=L.shared["up"], down=L.shared["down"], f=L.shared_f,
+                      bits=L.shared_bits)
+    return O.moe_decode_layer(L.x, L.hidden, L.router_dict(), dl.pool_blobs(), dl.residency_words(),
+                              L.oracle_offsets(), L.d, L.f, L.k, shared=shared, bits=L.bits, meta=L.meta,
+                              additive_biases=L.additive, **kw)
+
+
+# --------------------------------------------------------------------------- router
+
+@pytest.mark.parametrize("router_bits", [0, 8, 4])
+@pytest.mark.parametrize("ne,d,k", [(256, 2048, 8), (32, 2880, 4), (256, 2304, 8), (16, 128, 8), (5, 64, 3)])
+def test_router_logits_and_indices_bit_exact(gpu, router_bits, ne, d, k):
+    L = Layer(0x5EED0002 + router_bits, d, 64, ne, k, router_bits=router_bits)
+    L.logit_bias = S.f32_to_bf16_bits(L.tree.key("bias").normal(ne, std=0.01))
+    L.expert_scale = S.f32_to_bf16_bits(L.tree.key("escale").uniform(0.6, 1.4, ne))
+    L.eff_scale = S.f32_to_bf16_bits(L.tree.key("eff").uniform(0.5, 1.5, d))
+    dl = DeviceLayer(gpu, L, resident=[])
+    dl.moe.encode_router(dl.router_w, dl.router_s, dl.router_b, dl.x, dl.eff_scale, dl.expert_scale,
+                         dl.logit_bias, dl.out_idx, dl.out_w, ne, d, k)
+    logits = dl.moe.logits(ne)
+    ref_logits = O.router_logits(L.router_w, L.router_s, L.router_b, router_bits, L.x, L.eff_scale, ne, d)
+    assert np.array_equal(logits.view(np.uint32), ref_logits.view(np.uint32)), "router logits differ in bits"
+    idx = dl.out_idx.download(np.uint32, k)
+    w = dl.out_w.download(np.uint16, k)
+    ref_idx, ref_w = O.router_select(ref_logits, L.expert_scale, L.logit_bias, k)
+    assert np.array_equal(idx, ref_idx)
+    assert np.max(np.abs(f16(w) - f16(ref_w))) <= 1e-3  # reference holds weights to 5e-3 (RouterTopKTests.swift:43)
+    # the select stage alone, on the device's own logits
+    idx2, _ = O.router_select(logits, L.expert_scale, L.logit_bias, k)
+    assert np.array_equal(idx, idx2)
+
+
+def test_router_ties_go_to_the_lower_index(gpu):
+    # identical rows -> identical logits: selection must be experts 0..k-1 in order
+    ne, d, k = 64, 256, 8
+    L = Layer(7, d, 64, ne, k)
+    L.router_w[:] = L.router_w[0]
+    dl = DeviceLayer(gpu, L, resident=[])
+    dl.moe.encode_router(dl.router_w, None, None, dl.x, dl.eff_scale, dl.expert_scale, dl.logit_bias,
+                         dl.out_idx, dl.out_w, ne, d, k)
+    assert dl.out_idx.download(np.uint32, k).tolist() == list(range(k))
+    assert np.allclose(f16(dl.out_w.download(np.uint16, k)), 1.0 / k, atol=1e-3)
+
+
+def test_router_sigmoid_scores(gpu):
+    ne, d, k = 256, 2304, 8
+    L = Layer(0x516, d, 64, ne, k, router_bits=8)
+    L.logit_bias = S.f32_to_bf16_bits(L.tree.key("corr").uniform(-0.2, 0.2, ne))
+    dl = DeviceLayer(gpu, L, resident=[], moe_kwargs=dict(sigmoid=True, scaling=2.446))
+    dl.moe.encode_router(dl.router_w, dl.router_s, dl.router_b, dl.x, dl.eff_scale, dl.expert_scale,
+                         dl.logit_bias, dl.out_idx, dl.out_w, ne, d, k)
+    logits = dl.moe.logits(ne)
+    ref_idx, ref_w = O.router_select(logits, L.expert_scale, L.logit_bias, k, sigmoid=True, scaling=2.446)
+    # sigmoid selection compares sigmoid(logit)+bias: device expf and libm expf may differ in the last
+    # bit, so the selection is checked on scores recomputed here with a gap guard.
+    idx = dl.out_idx.download(np.uint32, k)
+    s = 1.0 / (1.0 + np.exp(-logits.astype(np.float64))) + S.bf16_bits_to_f32(L.logit_bias)
+    order = np.lexsort((np.arange(ne), -s))
+    gap = s[order[k - 1]] - s[order[k]]
+    if gap > 1e-6:
+        assert np.array_equal(np.sort(idx), np.sort(order[:k].astype(np.uint32)))
+        assert np.array_equal(idx, ref_idx)
+    assert np.max(np.abs(f16(dl.out_w.download(np.uint16, k)) - f16(ref_w))) <= 2e-3
+
+
+# ------------------------------------------------------------------------- classify
+
+def test_classify_truth_table_and_spec_args(gpu):
+    ne, k = 16, 8
+    L = Layer(3, 64, 64, ne, k)
+    dl = DeviceLayer(gpu, L, resident=[])
+    words = np.full(ne, (0 << 32) | SENT, np.uint64)
+    words[2] = (2 << 32) | 5          # resident at cell 5
+    words[3] = (1 << 32) | 6          # loading: a miss
+    words[4] = (2 << 32) | SENT       # resident but no slot: a miss
+    words[9] = (2 << 32) | 0
+    table = gpu.dev(words)
+    topk = np.array([2, 3, 4, 9, 0, 200, 2, 9], np.uint32)  # 200 clamps to ne-1 (empty)
+    weights = S.f32_to_f16_bits(np.linspace(0.3, 0.05, k).astype(np.float32))
+    pred = np.arange(100, 100 + k, dtype=np.uint32)
+    spec, readback = gpu.empty(48), gpu.empty(4 * (2 + 5 * k))
+    full = [256, 1, 1, 13, 7, 1, 256, 1, 1, 13, 7, 1]
+    dl.moe.encode_residency_classification(gpu.dev(topk), table, dl.hit_count, dl.hit_pos, dl.miss_count,
+                                           dl.miss_pos, dl.miss_exp, dl.resolved, k, ne, full_grids=full,
+                                           spec_args=spec, host_readback=readback, tag=0x1234,
+                                           topk_weights=gpu.dev(weights), predicted=gpu.dev(pred))
+    ref = O.classify(topk, words, ne)
+    hits, misses = dl.hit_count.download(np.uint32, 1)[0], dl.miss_count.download(np.uint32, 1)[0]
+    assert (hits, misses) == (ref["hit_count"], ref["miss_count"]) == (4, 4)
+    assert np.array_equal(dl.hit_pos.download(np.uint32, hits), ref["hit_positions"])
+    assert np.array_equal(dl.miss_pos.download(np.uint32, misses), ref["miss_positions"])
+    assert np.array_equal(dl.miss_exp.download(np.uint32, misses), ref["miss_experts"])
+    assert np.array_equal(dl.resolved.download(np.uint32, k), ref["resolved_slots"])
+    # a miss: phase 1 keeps the full grid, phase 2 gets a zero-width grid, the fixup the full ones
+    # (GPUExpertResidencyTests.swift:16-22)
+    assert spec.download(np.uint32, 12).tolist() == [256, 1, 1, 0, 1, 1, 256, 1, 1, 13, 7, 1]
+    rb = readback.download(np.uint32, 2 + 5 * k)
+    t = 0x1234 << 16
+    assert rb[0] == t | 4 and rb[1] == t | 4
+    assert rb[2:2 + k].tolist() == [t | min(int(e), ne - 1) for e in topk]
+    assert rb[2 + k:2 + 2 * k].tolist() == [t | int(b) for b in weights]
+    assert rb[2 + 2 * k:2 + 3 * k].tolist() == [t | int(p) for p in ref["hit_positions"]] + [t] * 4
+    assert rb[2 + 3 * k:2 + 4 * k].tolist() == [t | int(p) for p in ref["miss_positions"]] + [t] * 4
+    assert rb[2 + 4 * k:].tolist() == [t | int(p) for p in pred]
+    # all hit
+    topk2 = np.array([2, 9, 2, 9, 2, 9, 2, 9], np.uint32)
+    dl.moe.encode_residency_classification(gpu.dev(topk2), table, dl.hit_count, dl.hit_pos, dl.miss_count,
+                                           dl.miss_pos, dl.miss_exp, dl.resolved, k, ne, full_grids=full,
+                                           spec_args=spec)
+    assert spec.download(np.uint32, 12).tolist() == [256, 1, 1, 13, 7, 1, 0, 1, 1, 0, 1, 1]
+    assert dl.resolved.download(np.uint32, k).tolist() == [5, 0, 5, 0, 5, 0, 5, 0]
+
+
+# --------------------------------------------------------------------- phase 1 / 2
+
+SHAPES = [  # d, f
+    (2048, 512), (128, 64), (192, 320), (704, 192), (2880, 2880), (2304, 1024), (4096, 256)]
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("meta", [S.META_BF16, S.META_F16])
+@pytest.mark.parametrize("d,f", SHAPES)
+def test_phase1_phase2_against_oracle(gpu, bits, meta, d, f):
+    if d * bits // 128 > 256:
+        pytest.skip("row longer than four wave loads")
+    k, ne = 8, 8
+    if d * f > 4_000_000:
+        k, ne = 4, 4
+    L = Layer(0x5EED0000 + d + f + bits, d, f, ne, k, bits=bits, meta=meta)
+    dl = DeviceLayer(gpu, L)
+    resolved = np.array([dl.cell_of[e] for e in range(k)], np.uint32)
+    resolved[k - 1] = SENT  # one sentinel position: its acts must stay untouched, its partial must be zero
+    d_res = gpu.dev(resolved)
+    acts0 = S.f32_to_f16_bits(np.full(k * f, 0.25, np.float32))
+    dl.acts.upload(acts0)
+    dl.moe.encode_spec_phase1(dl.pool, d_res, dl.off, dl.x, dl.acts, d, f, k)
+    acts = dl.acts.download(np.uint16, k * f)
+    blobs = [None if s == SENT else dl.pool_blobs()[int(s)] for s in resolved]
+    ref_acts = O.moe_phase1(blobs, L.oracle_offsets(), L.x, d, f, bits=bits, meta=meta, acts=acts0.copy())
+    assert np.array_equal(acts[(k - 1) * f:], acts0[(k - 1) * f:]), "sentinel position was written"
+    assert_ffn_close(acts, ref_acts, "phase-1 acts")
+
+    w = S.f32_to_f16_bits(L.tree.key("w").uniform(0.05, 0.3, k))
+    residual = S.activations_f16(L.tree, "residual", d)
+    hidden = L.hidden.copy()
+    # phase 2 from the ORACLE's acts so the comparison isolates the down matvec + combine
+    dl.acts.upload(ref_acts)
+    dl.moe.encode_spec_phase2(dl.pool, d_res, dl.off, dl.acts, gpu.dev(w), gpu.dev(residual), dl.y,
+                              dl.hidden, d, f, k)
+    ref_y = O.moe_phase2(blobs, L.oracle_offsets(), ref_acts, w, residual, d, f, bits=bits, meta=meta,
+                         hidden_f16=hidden)
+    y = dl.y.download(np.uint16, d)
+    assert_ffn_close(y, ref_y, "phase-2 y")
+    # hidden += y is exact given y (moe.metal:889-893)
+    got_hidden = dl.hidden.download(np.uint16, d)
+    expect_hidden = O.residual_add_f16(L.hidden.copy(), y)
+    assert np.array_equal(got_hidden, expect_hidden)
+
+
+def test_phase2_fallback_cells_and_indirect_zero_grid(gpu):
+    d, f, k = 256, 128, 4
+    L = Layer(11, d, f, k, k)
+    dl = DeviceLayer(gpu, L)
+    cells = np.array([dl.cell_of[e] for e in range(k)], np.uint32)
+    resolved = cells.copy()
+    resolved[1] = SENT
+    acts = O.moe_phase1([dl.pool_blobs()[int(c)] for c in cells], L.oracle_offsets(), L.x, d, f)
+    dl.acts.upload(acts)
+    w = S.f32_to_f16_bits(np.full(k, 0.25, np.float32))
+    residual = np.zeros(d, np.uint16)
+    dw, dr = gpu.dev(w), gpu.dev(residual)
+    # fallback supplies the missing cell (moe.metal:1037-1038)
+    dl.moe.encode_spec_phase2(dl.pool, gpu.dev(resolved), dl.off, dl.acts, dw, dr, dl.y, None, d, f, k,
+                              fallback_cells=gpu.dev(cells))
+    ref = O.moe_phase2([dl.pool_blobs()[int(c)] for c in cells], L.oracle_offsets(), acts, w, residual, d, f)
+    assert_ffn_close(dl.y.download(np.uint16, d), ref, "fallback")
+    # zero-width indirect grid: nothing is written
+    dl.y.upload(np.full(d, 0x3C00, np.uint16))
+    dl.moe.encode_spec_phase2(dl.pool, gpu.dev(cells), dl.off, dl.acts, dw, dr, dl.y, None, d, f, k,
+                              indirect=gpu.dev(np.array([0, 1, 1], np.uint32)))
+    assert np.all(dl.y.download(np.uint16, d) == 0x3C00)
+
+
+def test_event_gated_status_word(gpu):
+    d, f, k = 128, 64, 2
+    L = Layer(12, d, f, k, k)
+    dl = DeviceLayer(gpu, L, moe_kwargs=dict(event_gated=True))
+    cells = gpu.dev(np.array([dl.cell_of[e] for e in range(k)], np.uint32))
+    residual = S.activations_f16(L.tree, "r", d)
+    w = gpu.dev(S.f32_to_f16_bits(np.full(k, 0.5, np.float32)))
+    failed = gpu.dev(np.array([2], np.uint32))  # a failed batch (moe.metal:36-39)
+    acts0 = np.full(k * f, 0x1234, np.uint16)
+    dl.acts.upload(acts0)
+    dl.moe.encode_spec_phase1(dl.pool, cells, dl.off, dl.x, dl.acts, d, f, k, io_status=failed)
+    assert np.array_equal(dl.acts.download(np.uint16, k * f), acts0)
+    dl.moe.encode_spec_phase2(dl.pool, cells, dl.off, dl.acts, w, gpu.dev(residual), dl.y, dl.hidden, d, f, k,
+                              io_status=failed)
+    assert np.array_equal(dl.y.download(np.uint16, d), residual)  # residual written through (:918-921)
+    assert np.array_equal(dl.hidden.download(np.uint16, d), O.residual_add_f16(L.hidden.copy(), residual))
+
+
+def test_closed_form_ffn(gpu):
+    """q=0, scale=0: gate = bias*sum(x) = 1, up = 0.5, act = 0.5*silu(1); down bias 1/64 over F=64
+    -> each expert returns act; eight experts at 0.125 -> silu(1)*0.5... scaled as the reference's
+    known-answer test (MoEFusedFFNTests.swift:17-55, :868-900): gate bias 1/64, up bias 0.5/64,
+    down bias 1/64, x = 1, D=128, F=64 -> every output 2/(1+e^-2) within 0.01."""
+    d, f, k = 128, 64, 8
+    off, stride = S.expert_offsets(d, f, 4)
+    blob = np.zeros(stride, np.uint8)
+
+    def put(name, value, count):
+        blob[off[name]:off[name] + 2 * count] = np.full(count, S.f32_to_bf16_bits(np.array([value], np.float32))[0],
+                                                        np.uint16).view(np.uint8)
+    put("gate_b", 1.0 / 64.0, f * (d // 64))
+    put("up_b", 0.5 / 64.0, f * (d // 64))
+    put("down_b", 1.0 / 64.0, d * (f // 64))
+    pool = gpu.ExpertPool(k, stride, k)
+    for c in range(k):
+        pool.upload(c, blob)
+    moe = gpu.MoE(d, f, k, k)
+    o, _ = gpu.expert_offsets(d, f, 4)
+    x = gpu.dev(S.f32_to_f16_bits(np.ones(d, np.float32)))
+    acts, y = gpu.empty(2 * k * f), gpu.empty(2 * d)
+    res = gpu.dev(np.arange(k, dtype=np.uint32))
+    moe.encode_spec_phase1(pool, res, o, x, acts, d, f, k)
+    moe.encode_spec_phase2(pool, res, o, acts, gpu.dev(S.f32_to_f16_bits(np.full(k, 0.125, np.float32))),
+                           gpu.dev(np.zeros(d, np.uint16)), y, None, d, f, k)
+    # gate = (1/64)*128 = 2, up = (0.5/64)*128 = 1, act = silu(2)*1 = 2/(1+e^-2); down = (1/64)*64*act
+    expect = 2.0 / (1.0 + np.exp(-2.0))
+    assert np.all(np.abs(f16(y.download(np.uint16, d)) - expect) <= 0.01)
+    assert np.all(np.abs(f16(acts.download(np.uint16, k * f)) - expect) <= 2e-3)
+
+
+# --------------------------------------------------------------------- shared expert
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("d,fs", [(2048, 512), (2304, 1024), (128, 64), (192, 320)])
+def test_shared_expert_against_oracle(gpu, bits, d, fs):
+    L = Layer(0x5EED0100 + d + bits, d, 64, 2, 1, shared_f=fs, shared_bits=bits)
+    dl = DeviceLayer(gpu, L, resident=[])
+    dl.moe.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, dl.x,
+                                dl.shared_scratch, dl.h1, d, fs)
+    ref = O.shared_expert(L.shared["gate"], L.shared["up"], L.shared["down"], L.x, d, fs, bits=bits)
+    assert_ffn_close(dl.h1.download(np.uint16, d), ref, "shared expert h1")
+    gate = S.f32_to_f16_bits(np.array([0.3], np.float32))
+    dl.moe.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, dl.x,
+                                dl.shared_scratch, dl.h1, d, fs, scalar_gate=gpu.dev(gate))
+    ref = O.shared_expert(L.shared["gate"], L.shared["up"], L.shared["down"], L.x, d, fs, bits=bits,
+                          scalar_gate_f16=gate)
+    # two fp16 roundings in a row (the GEMV's, then the gate's: dequant_int4.metal:322-329): a
+    # last-bit difference before the first can move the result by two fp16 steps, 2 * 2^-10
+    assert_ffn_close(dl.h1.download(np.uint16, d), ref, "gated shared expert h1", rel=2e-3)
+
+
+# ------------------------------------------------------------------------ whole layer
+
+CONFIGS = [
+    # name, d, f, E, K, bits, meta, router_bits, shared_f
+    ("q35b-a3b-int4-f16meta", 2048, 512, 256, 8, 4, S.META_F16, 0, 512),
+    ("q35b-a3b-int4-bf16meta-affine8-router", 2048, 512, 256, 8, 4, S.META_BF16, 8, 512),
+    ("gpt-oss-int4", 2880, 2880, 32, 4, 4, S.META_BF16, 0, 0),
+    ("gpt-oss-int8", 2880, 2880, 32, 4, 8, S.META_BF16, 0, 0),
+    ("kimi-int8", 2304, 1024, 64, 8, 8, S.META_BF16, 8, 1024),
+    ("toy", 128, 64, 16, 8, 4, S.META_BF16, 0, 64),
+]
+
+
+@pytest.mark.parametrize("cfg", CONFIGS, ids=[c[0] for c in CONFIGS])
+def test_decode_layer_matches_oracle_and_split_calls(gpu, cfg):
+    name, d, f, ne, k, bits, meta, rbits, fs = cfg
+    n_blobs = ne if d * f * ne < 600_000_000 else 8
+    L = Layer(0x5EED0002, d, f, ne, k, bits=bits, meta=meta, router_bits=rbits, shared_f=fs)
+    dl = DeviceLayer(gpu, L)
+    dl.moe.encode_decode_layer(dl.layer_args())
+    ref = oracle_layer(L, dl)
+    idx = dl.out_idx.download(np.uint32, k)
+    assert np.array_equal(idx, ref["indices"]), "routing indices differ"
+    assert np.array_equal(dl.moe.logits(ne).view(np.uint32), ref["logits"].view(np.uint32))
+    assert np.array_equal(dl.resolved.download(np.uint32, k), ref["classify"]["resolved_slots"])
+    assert dl.hit_count.download(np.uint32, 1)[0] == k and dl.miss_count.download(np.uint32, 1)[0] == 0
+    assert np.max(np.abs(f16(dl.out_w.download(np.uint16, k)) - f16(ref["weights"]))) <= 1e-3
+    if fs:
+        assert_ffn_close(dl.h1.download(np.uint16, d), ref["h1"], "h1")
+    assert_ffn_close(dl.acts.download(np.uint16, k * f), ref["acts"], "acts")
+    y = dl.y.download(np.uint16, d)
+    assert_ffn_close(y, ref["y"], "y")
+    assert np.array_equal(dl.hidden.download(np.uint16, d), O.residual_add_f16(L.hidden.copy(), y))
+
+    # the operators called one after another give the same bytes as the fused entry point
+    y_fused, acts_fused = y.copy(), dl.acts.download(np.uint16, k * f)
+    dl.hidden.upload(L.hidden)
+    dl.moe.encode_router(dl.router_w, dl.router_s, dl.router_b, dl.x, dl.eff_scale, dl.expert_scale,
+                         dl.logit_bias, dl.out_idx, dl.out_w, ne, d, k)
+    dl.moe.encode_residency_classification(dl.out_idx, dl.pool.table, dl.hit_count, dl.hit_pos, dl.miss_count,
+                                           dl.miss_pos, dl.miss_exp, dl.resolved, k, ne)
+    residual = dl.h1
+    if fs:
+        dl.moe.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], L.shared_bits, dl.x,
+                                    dl.shared_scratch, dl.h1, d, fs)
+    else:
+        dl.h1.fill(0)
+    dl.moe.encode_spec_phase1(dl.pool, dl.resolved, dl.off, dl.x, dl.acts, d, f, k)
+    dl.moe.encode_spec_phase2(dl.pool, dl.resolved, dl.off, dl.acts, dl.out_w, residual, dl.y, dl.hidden, d, f, k)
+    assert np.array_equal(dl.acts.download(np.uint16, k * f), acts_fused)
+    assert np.array_equal(dl.y.download(np.uint16, d), y_fused)
+
+
+def test_decode_layer_is_deterministic(gpu):
+    L = Layer(0x5EED0002, 2048, 512, 256, 8, shared_f=512)
+    dl = DeviceLayer(gpu, L)
+    outs = []
+    for _ in range(3):
+        dl.hidden.upload(L.hidden)
+        dl.moe.encode_decode_layer(dl.layer_args())
+        outs.append((dl.y.download(np.uint16, 2048), dl.hidden.download(np.uint16, 2048),
+                     dl.out_idx.download(np.uint32, 8)))
+    for o in outs[1:]:
+        assert all(np.array_equal(a, b) for a, b in zip(o, outs[0]))
+
+
+def test_multi_chunk_pool_addressing(gpu):
+    """The same cells through a pool split into several chunks (ExpertCellArena chunking)."""
+    d, f, k, ne = 256, 128, 4, 12
+    L = Layer(21, d, f, ne, k)
+    one = DeviceLayer(gpu, L)
+    padded = (L.stride + capi.POOL_PAGE - 1) // capi.POOL_PAGE * capi.POOL_PAGE
+    many = DeviceLayer(gpu, L, chunk_bytes=5 * padded + 100)  # 5 cells per chunk -> 3 chunks
+    assert many.pool.bases.contents.cells_per_chunk == 5
+    outs = []
+    for dl in (one, many):
+        dl.moe.encode_decode_layer(dl.layer_args())
+        outs.append(dl.y.download(np.uint16, d))
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_argument_errors_are_reported_not_trapped(gpu):
+    moe = gpu.MoE(128, 64, 16, 8)
+    with pytest.raises(capi.ShrikeError, match="topK"):
+        moe.encode_router(gpu.empty(16), None, None, gpu.empty(16), gpu.empty(16), gpu.empty(16), gpu.empty(16),
+                          gpu.empty(64), gpu.empty(32), 16, 128, 9)
+    with pytest.raises(capi.ShrikeError, match="multiple"):
+        moe.encode_router(gpu.empty(16), None, None, gpu.empty(16), gpu.empty(16), gpu.empty(16), gpu.empty(16),
+                          gpu.empty(64), gpu.empty(32), 16, 100, 8)
+    with pytest.raises(capi.ShrikeError):
+        gpu.MoE(128, 64, 16, 9)
+    with pytest.raises(capi.ShrikeError):
+        gpu.ExpertPool(0, 4096, 4)
