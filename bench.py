@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the routed-expert decode layer on one MI355X.
+
+A step is one MoE-layer decode for one token at the 35B-A3B int4 shape (hidden 2048,
+256 routed experts of intermediate 512, top-8, one shared expert of intermediate 512,
+fp16 router, group-64 affine int4 with 16-bit scale/bias): router -> top-k -> slot
+resolve -> shared expert -> gate/up matvec + SiLU-multiply -> down matvec + weighted
+combine. Consecutive steps walk a stack of layers whose expert pools sit at distinct
+addresses and together exceed the 256 MB Infinity Cache, so every step streams its
+experts from HBM. The stack is captured once in a HIP graph and replayed.
+
+Prints ONE JSON line. `value` is expert bytes read per second (8 routed + 1 shared
+expert = 15,925,248 B per step) with all inputs resident in HBM; `ms_per_step` carries
+the per-layer time. `roofline` prices the dominant kernel (phase 1) against 8 TB/s;
+`cpu_baseline` times the CPU oracle's fp32 port of the same layer on this host.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+D, F, NE, K, FS, BITS = 2048, 512, 256, 8, 512, 4
+HBM_PEAK_GBPS = 8000.0
+
+
+def build_layers(rt, capi, S, n_layers, meta):
+    """Layer 0's pool comes from the seeded generator; the other layers hold byte copies of it at
+    their own addresses (cache behaviour follows addresses, not values). Routers, shared experts
+    and activations are distinct per layer."""
+    tree = S.SeedTree(0x5EED0002)
+    off, stride = rt.expert_offsets(D, F, BITS)
+    t0 = time.time()
+    blobs = [S.expert_blob(tree, f"layer.0.expert.{e}", D, F, BITS, meta) for e in range(NE)]
+    layers = []
+    ones_d = rt.dev(S.f32_to_bf16_bits(np.ones(D, np.float32)))
+    ones_e = rt.dev(S.f32_to_bf16_bits(np.ones(NE, np.float32)))
+    zeros_e = rt.dev(np.zeros(NE, np.uint16))
+    hidden = rt.dev(S.activations_f16(tree, "hidden", D))
+    first_pool = None
+    for l in range(n_layers):
+        pool = rt.ExpertPool(NE, stride, NE)
+        if l == 0:
+            for e in range(NE):
+                capi.check(capi.load().shrike_hip_memcpy_h2d(pool.cell_ptr(e), blobs[e].ctypes.data, blobs[e].nbytes), "h2d")
+            first_pool = pool
+        else:
+            capi.check(capi.load().shrike_hip_memcpy_d2d(pool.cell_ptr(0), first_pool.cell_ptr(0), NE * pool.stride), "d2d")
+        for e in range(NE):
+            pool.publish(e, e, capi.RESIDENT)
+        lay = dict(pool=pool)
+        lay["router"] = rt.dev(S.router_f16(tree, f"layer.{l}.router.w", NE, D))
+        lay["x"] = rt.dev(S.activations_f16(tree, f"layer.{l}.x", D))
+        lay["shared"] = {n: tuple(rt.dev(t) for t in S.affine_matrix(tree.key(f"layer.{l}.shared.{n}"), r, c, BITS, meta))
+                         for n, r, c in (("gate", FS, D), ("up", FS, D), ("down", D, FS))}
+        for name, size in dict(idx=32, w=16, res=32, hc=4, hp=32, mc=4, mp=32, me=32, acts=2 * K * F,
+                               ss=4 * FS, h1=2 * D, y=2 * D).items():
+            lay[name] = rt.empty(size)
+        a = capi.DecodeLayerArgs()
+        a.router_weights, a.effective_scale, a.per_expert_scale, a.logit_bias = lay["router"].ptr, ones_d.ptr, ones_e.ptr, zeros_e.ptr
+        a.pool, a.pool_slot_stride, a.residency, a.offsets = pool.bases, pool.stride, pool.table, off
+        for n in ("gate", "up", "down"):
+            setattr(a, f"shared_{n}", capi.Projection(*(t.ptr for t in lay["shared"][n])))
+        a.shared_bits, a.shared_f = BITS, FS
+        a.x, a.hidden, a.y = lay["x"].ptr, hidden.ptr, lay["y"].ptr
+        a.out_indices, a.out_weights, a.resolved_slots = lay["idx"].ptr, lay["w"].ptr, lay["res"].ptr
+        a.hit_count, a.hit_positions, a.miss_count = lay["hc"].ptr, lay["hp"].ptr, lay["mc"].ptr
+        a.miss_positions, a.miss_experts = lay["mp"].ptr, lay["me"].ptr
+        a.acts, a.shared_scratch, a.h1 = lay["acts"].ptr, lay["ss"].ptr, lay["h1"].ptr
+        lay["args"] = a
+        layers.append(lay)
+    rt.synchronize()
+    keep = (ones_d, ones_e, zeros_e, hidden, blobs)
+    return layers, off, stride, keep, time.time() - t0
+
+
+def capture(rt, capi, stream, body):
+    capi.check(capi.load().shrike_hip_graph_begin_capture(stream.handle), "graph_begin_capture")
+    body()
+    g = capi.load().shrike_hip_graph_end_capture(stream.handle)
+    if not g:
+        raise capi.ShrikeError(capi.last_error())
+    return g
+
+
+def time_graph(rt, capi, stream, graph, launches):
+    start, stop = rt.Event(), rt.Event()
+    stream.synchronize()
+    rt.synchronize()
+    start.record(stream)
+    for _ in range(launches):
+        capi.check(capi.load().shrike_hip_graph_launch(graph, stream.handle), "graph_launch")
+    stop.record(stream)
+    stop.synchronize()
+    rt.synchronize()
+    return start.elapsed_ms(stop)
+
+
+def cpu_baseline(S, blobs, sample_layers, meta):
+    """The oracle's fp32 port of the layer (one task per expert, as
+    sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:10-14 describes) on this host's cores."""
+    from oracle import oracle as O
+    off, _ = O.expert_offsets(D, F, BITS)
+    cores = min(K + 1, len(os.sched_getaffinity(0)))
+    tree = S.SeedTree(0xC0FFEE)
+    x = tree.key("x").normal(D)
+    rng = np.random.default_rng(0)
+    weights = np.full(K + 1, 1.0 / K, np.float32)
+    t0 = time.perf_counter()
+    for i in range(sample_layers):
+        picks = rng.choice(NE, K + 1, replace=False)
+        O.cpu_layer_fp32([blobs[int(e)] for e in picks], weights, off, x, D, F, cores, bits=BITS, meta=meta)
+    dt = time.perf_counter() - t0
+    per_layer = dt / sample_layers
+    expert_bytes = (K + 1) * 1_769_472
+    return {"value": round(expert_bytes / per_layer / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "us_per_layer": round(per_layer * 1e6, 1),
+            "sample": f"{sample_layers} layer evaluations of 9 experts (8 routed + 1 shared-sized) drawn from the "
+                      f"256-expert pool, fp32 scalar C port of shrike_int4_affine_gemv + CPUExpertFFN.accumulate, "
+                      f"{cores} threads, gcc -O2"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--layers", type=int, default=40, help="stacked layers with their own pools (40 x 453 MB)")
+    ap.add_argument("--meta", choices=["f16", "bf16"], default="f16")
+    ap.add_argument("--cpu-sample", type=int, default=60, help="layer evaluations timed on the CPU (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path is built and measured on a single MI355X "
+              "(--gpus N with N > 1 is not supported)", file=sys.stderr)
+        sys.exit(2)
+
+    from shrike_amd import capi, runtime as rt
+    from shrike_amd import synth as S
+
+    rt.init(0)
+    meta = S.META_F16 if args.meta == "f16" else S.META_BF16
+    n_layers = args.layers
+    layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta)
+    moe = rt.MoE(D, F, NE, K, routed_bits=BITS, router_bits=0, meta=meta)
+    stream = rt.Stream()
+    moe.stream = stream
+
+    def all_layers():
+        for lay in layers:
+            moe.encode_decode_layer(lay["args"])
+
+    all_layers()  # eager pass: fills every layer's routing scratch
+    stream.synchronize()
+    g_layer = capture(rt, capi, stream, all_layers)
+
+    def phase1_only():
+        for lay in layers:
+            moe.encode_spec_phase1(lay["pool"], lay["res"], off, lay["x"], lay["acts"], D, F, K)
+
+    def phase2_only():
+        for lay in layers:
+            moe.encode_spec_phase2(lay["pool"], lay["res"], off, lay["acts"], lay["w"], lay["h1"], lay["y"], None, D, F, K)
+
+    def router_only():
+        a0 = layers[0]["args"]
+        for lay in layers:
+            a = lay["args"]
+            moe.encode_router(a.router_weights, None, None, a.x, a.effective_scale, a.per_expert_scale, a.logit_bias,
+                              a.out_indices, a.out_weights, NE, D, K)
+
+    def shared_only():
+        for lay in layers:
+            sh = lay["shared"]
+            moe.encode_shared_expert(sh["gate"], sh["up"], sh["down"], BITS, lay["x"], lay["ss"], lay["h1"], D, FS)
+
+    g_p1 = capture(rt, capi, stream, phase1_only)
+    g_p2 = capture(rt, capi, stream, phase2_only)
+    g_rt = capture(rt, capi, stream, router_only)
+    g_sh = capture(rt, capi, stream, shared_only)
+
+    steps = max(n_layers, args.steps // n_layers * n_layers)
+    warm = max(n_layers, args.warmup // n_layers * n_layers)
+    time_graph(rt, capi, stream, g_layer, warm // n_layers)
+    ms = time_graph(rt, capi, stream, g_layer, steps // n_layers)
+    ms_per_step = ms / steps
+
+    reps = max(1, steps // n_layers // 2)
+    parts = {}
+    for name, g, launches_per_layer in (("phase1", g_p1, 1), ("phase2", g_p2, 1), ("router_select_classify", g_rt, 1),
+                                        ("shared_expert(2 launches)", g_sh, 1)):
+        time_graph(rt, capi, stream, g, 2)
+        parts[name] = time_graph(rt, capi, stream, g, reps) / (reps * n_layers) * 1e3  # us per layer
+
+    expert_bytes = (K + 1) * stride  # 15,925,248
+    total_bytes = expert_bytes + NE * D * 2 + 2 * D * 2
+    p1_bytes = K * 2 * (F * D // 2 + 2 * F * (D // 64) * 2)  # gate+up codes, scales and biases of 8 experts
+    p1_us = parts["phase1"]
+    value = expert_bytes / (ms_per_step * 1e-3) / 1e9
+    out = {
+        "metric": "MoE-layer decode: HBM GB/s on expert bytes (us per layer in ms_per_step), 35B-A3B int4 shape",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": round(ms_per_step, 6), "us_per_layer": round(ms_per_step * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (seeded SplitMix64: uniform int4 codes, |N(0,0.02)| scales, N(0,1) fp16 activations)",
+        "config": {"workload": "config 2: full MoE layer decode, 1 token, hidden 2048, top-8 of 256 int4 experts "
+                               "(intermediate 512, group 64) + 1 shared expert, fp16 router, all slots resident",
+                   "stacked_layers": n_layers, "pool_bytes_total": n_layers * NE * stride,
+                   "meta_dtype": args.meta, "launches_per_layer": 3, "hip_graph": True},
+        "hbm_peak_frac_on_expert_bytes": round(value / HBM_PEAK_GBPS, 4),
+        "expert_bytes_per_step": expert_bytes, "total_bytes_per_step": total_bytes,
+        "kernel_us_per_layer": {k: round(v, 3) for k, v in parts.items()},
+        "roofline": {"bound": "hbm", "kernel": "k_phase1<4,1,2> (routed gate/up matvec + SiLU-multiply)",
+                     "achieved": round(p1_bytes / (p1_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(p1_bytes / (p1_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "bytes_per_launch": p1_bytes, "us_per_launch": round(p1_us, 3), "traffic": None},
+        "setup_seconds": round(gen_s, 1),
+    }
+    if args.cpu_sample > 0:
+        out["cpu_baseline"] = cpu_baseline(S, keep[4], args.cpu_sample, meta)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -168,6 +168,23 @@ def shared_expert(gate, up, down, x_f16, d, f, bits=4, meta=META_BF16, act=ACT_S
     return h1
 
 
+def shared_gate_up(gate, up, x_f16, d, f, bits=4, meta=META_BF16):
+    g = Proj(gate[0].ctypes.data, gate[1].ctypes.data, gate[2].ctypes.data)
+    u = Proj(up[0].ctypes.data, up[1].ctypes.data, up[2].ctypes.data)
+    go, uo = np.empty(f, np.uint16), np.empty(f, np.uint16)
+    lib().orc_shared_gate_up(C.byref(g), C.byref(u), C.c_int(meta), C.c_int(bits), _p(x_f16),
+                             C.c_uint32(d), C.c_uint32(f), _p(go), _p(uo))
+    return go, uo
+
+
+def shared_down(down, gate_f16, up_f16, d, f, bits=4, meta=META_BF16, act=ACT_SILU, scalar_gate_f16=None):
+    dn = Proj(down[0].ctypes.data, down[1].ctypes.data, down[2].ctypes.data)
+    h1 = np.empty(d, np.uint16)
+    lib().orc_shared_down(C.byref(dn), C.c_int(meta), C.c_int(bits), C.c_int(act), _p(gate_f16),
+                          _p(up_f16), C.c_uint32(d), C.c_uint32(f), _p(scalar_gate_f16), _p(h1))
+    return h1
+
+
 def router_logits(weights, scales, biases, kind, hidden_f16, eff_scale_bf16, num_experts, d,
                   meta=META_BF16):
     out = np.empty(num_experts, np.float32)

@@ -306,24 +306,30 @@ void orc_moe_phase2(const uint8_t *const *expert_base, const orc_offsets *off,
 
 /* ------------------------------------------------------------ shared expert */
 
-void orc_shared_expert(const orc_proj *gate, const orc_proj *up, const orc_proj *down,
-                       int meta, int bits, int act, const uint16_t *x_f16, uint32_t d,
-                       uint32_t f, const uint16_t *scalar_gate_f16, uint16_t *h1_f16) {
+void orc_shared_gate_up(const orc_proj *gate, const orc_proj *up, int meta, int bits,
+                        const uint16_t *x_f16, uint32_t d, uint32_t f, uint16_t *gate_f16,
+                        uint16_t *up_f16) {
     float *x = (float *)malloc(sizeof(float) * d);
     float *g = (float *)malloc(sizeof(float) * f);
     float *u = (float *)malloc(sizeof(float) * f);
-    float *y = (float *)malloc(sizeof(float) * d);
     for (uint32_t i = 0; i < d; ++i) x[i] = orc_f16_to_f32(x_f16[i]);
     orc_affine_gemv(gate->w, gate->s, gate->b, meta, bits, x, f, d, g);
     orc_affine_gemv(up->w, up->s, up->b, meta, bits, x, f, d, u);
-    for (uint32_t i = 0; i < f; ++i) {
-        /* dequant_int4.metal:177-179 (GEMV writes half), :283-287 (act from the halves);
-         * dequant_int8.metal:159-163 (same roundings inside the fused kernel). */
-        const float gh = orc_f16_to_f32(orc_f32_to_f16(g[i]));
-        const float uh = orc_f16_to_f32(orc_f32_to_f16(u[i]));
-        g[i] = orc_f16_to_f32(orc_f32_to_f16(orc_glu(gh, uh, act)));
+    for (uint32_t i = 0; i < f; ++i) { /* dequant_int4.metal:177-179: the GEMV writes half */
+        gate_f16[i] = orc_f32_to_f16(g[i]);
+        up_f16[i] = orc_f32_to_f16(u[i]);
     }
-    orc_affine_gemv(down->w, down->s, down->b, meta, bits, g, d, f, y);
+    free(x); free(g); free(u);
+}
+
+void orc_shared_down(const orc_proj *down, int meta, int bits, int act, const uint16_t *gate_f16,
+                     const uint16_t *up_f16, uint32_t d, uint32_t f,
+                     const uint16_t *scalar_gate_f16, uint16_t *h1_f16) {
+    float *a = (float *)malloc(sizeof(float) * f);
+    float *y = (float *)malloc(sizeof(float) * d);
+    for (uint32_t i = 0; i < f; ++i) /* dequant_int4.metal:283-287; dequant_int8.metal:159-163 */
+        a[i] = orc_f16_to_f32(orc_f32_to_f16(orc_glu(orc_f16_to_f32(gate_f16[i]), orc_f16_to_f32(up_f16[i]), act)));
+    orc_affine_gemv(down->w, down->s, down->b, meta, bits, a, d, f, y);
     for (uint32_t r = 0; r < d; ++r) {
         uint16_t yh = orc_f32_to_f16(y[r]);
         if (scalar_gate_f16) { /* dequant_int4.metal:322-329 */
@@ -332,7 +338,17 @@ void orc_shared_expert(const orc_proj *gate, const orc_proj *up, const orc_proj 
         }
         h1_f16[r] = yh;
     }
-    free(x); free(g); free(u); free(y);
+    free(a); free(y);
+}
+
+void orc_shared_expert(const orc_proj *gate, const orc_proj *up, const orc_proj *down,
+                       int meta, int bits, int act, const uint16_t *x_f16, uint32_t d,
+                       uint32_t f, const uint16_t *scalar_gate_f16, uint16_t *h1_f16) {
+    uint16_t *g = (uint16_t *)malloc(sizeof(uint16_t) * f);
+    uint16_t *u = (uint16_t *)malloc(sizeof(uint16_t) * f);
+    orc_shared_gate_up(gate, up, meta, bits, x_f16, d, f, g, u);
+    orc_shared_down(down, meta, bits, act, g, u, d, f, scalar_gate_f16, h1_f16);
+    free(g); free(u);
 }
 
 /* ------------------------------------------------------------------- router */

@@ -93,6 +93,12 @@ void orc_moe_phase2(const uint8_t *const *expert_base, const orc_offsets *off,
 typedef struct {
     const uint8_t *w; const uint16_t *s; const uint16_t *b;
 } orc_proj;
+void orc_shared_gate_up(const orc_proj *gate, const orc_proj *up, int meta, int bits,
+                        const uint16_t *x_f16, uint32_t d, uint32_t f, uint16_t *gate_f16,
+                        uint16_t *up_f16);
+void orc_shared_down(const orc_proj *down, int meta, int bits, int act, const uint16_t *gate_f16,
+                     const uint16_t *up_f16, uint32_t d, uint32_t f,
+                     const uint16_t *scalar_gate_f16, uint16_t *h1_f16);
 void orc_shared_expert(const orc_proj *gate, const orc_proj *up, const orc_proj *down,
                        int meta, int bits, int act, const uint16_t *x_f16, uint32_t d,
                        uint32_t f, const uint16_t *scalar_gate_f16 /* NULL = ungated */,

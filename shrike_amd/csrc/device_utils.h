@@ -81,12 +81,14 @@ __device__ __forceinline__ uint64_t wave_max_u64(uint64_t key) {
 // ---- 16-byte chunk of codes against the lane's activation slice.
 //
 // A chunk is 4 little-endian words. For 4-bit codes word j holds elements 8j..8j+7
-// (element i in bits 4i..4i+3). Codes become exact fp16 values in packed pairs with
-// the 0x6400 (=1024.0) exponent trick: (w & 0x000F000F) | 0x64006400 is the pair
-// {1024+q0, 1024+q4}; the pair taken from bits 4..7 / 20..23 is {1024+16*q1,
-// 1024+16*q5}, brought back by one packed fma with 1/16 and -64. The activation
-// slice is therefore kept as the pairs (e0,e4) (e1,e5) (e2,e6) (e3,e7) per word
-// (pairs_from_x8 below), and each pair costs one 2-way fp16 dot accumulated in fp32.
+// (element i in bits 4i..4i+3). A code needs no conversion to enter the fp16 dot: the
+// bit pattern 0x000q is the fp16 subnormal q * 2^-24 and 0x00q0 is q * 2^-20, both exact,
+// and the 2-way fp16 dot of gfx950 takes subnormal inputs at full precision (products are
+// exact in fp32, the sum is kept in fp32). So (w & 0x000F000F) is the pair {q0, q4} * 2^-24
+// and (w & 0x00F000F0) the pair {q1, q5} * 2^-20; after one shift by 8 the same two masks
+// give {q2, q6} and {q3, q7}. The two scalings go to two accumulators that are joined once
+// per chunk: dot = (lo * 16 + hi) * 2^20. The activation slice is therefore kept as the
+// pairs (e0,e4) (e1,e5) (e2,e6) (e3,e7) per word (pairs_from_x8 below).
 struct XChunk4 { h2_t p[16]; };   // 32 activations of a 4-bit chunk, pair layout
 struct XChunk8 { h2_t p[8]; };    // 16 activations of an 8-bit chunk, natural pairs
 
@@ -98,46 +100,38 @@ __device__ __forceinline__ void pairs_from_x8(const uint4 v, h2_t *p) {
     p[3] = as_h2(__builtin_amdgcn_perm(v.w, v.y, 0x07060302u));  // (e3,e7)
 }
 
+// fp32 sum of 8 fp16 activations: four 2-way dots against (1, 1).
 __device__ __forceinline__ float sum_x8(const uint4 v) {
-    const h2_t a = as_h2(v.x), b = as_h2(v.y), c = as_h2(v.z), d = as_h2(v.w);
-    return ((float(a.x) + float(a.y)) + (float(b.x) + float(b.y)))
-         + ((float(c.x) + float(c.y)) + (float(d.x) + float(d.y)));
+    const h2_t one = {(_Float16)1.0f, (_Float16)1.0f};
+    float s = __builtin_amdgcn_fdot2(as_h2(v.x), one, 0.0f, false);
+    s = __builtin_amdgcn_fdot2(as_h2(v.y), one, s, false);
+    s = __builtin_amdgcn_fdot2(as_h2(v.z), one, s, false);
+    s = __builtin_amdgcn_fdot2(as_h2(v.w), one, s, false);
+    return s;
 }
 
-__device__ __forceinline__ float dot_word4(uint32_t w, const h2_t *p, float acc) {
-    const h2_t k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
-    const h2_t k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
-    const h2_t k64 = {(_Float16)64.0f, (_Float16)64.0f};
+__device__ __forceinline__ void dot_word4(uint32_t w, const h2_t *p, float &lo, float &hi) {
     const uint32_t w8 = w >> 8;
-    const h2_t q04 = as_h2((w & 0x000F000Fu) | 0x64006400u) - k1024;
-    const h2_t q15 = __builtin_elementwise_fma(as_h2((w & 0x00F000F0u) | 0x64006400u), k16th, -k64);
-    const h2_t q26 = as_h2((w8 & 0x000F000Fu) | 0x64006400u) - k1024;
-    const h2_t q37 = __builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x64006400u), k16th, -k64);
-    acc = __builtin_amdgcn_fdot2(q04, p[0], acc, false);
-    acc = __builtin_amdgcn_fdot2(q15, p[1], acc, false);
-    acc = __builtin_amdgcn_fdot2(q26, p[2], acc, false);
-    acc = __builtin_amdgcn_fdot2(q37, p[3], acc, false);
-    return acc;
+    lo = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), p[0], lo, false);
+    hi = __builtin_amdgcn_fdot2(as_h2(w & 0x00F000F0u), p[1], hi, false);
+    lo = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), p[2], lo, false);
+    hi = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), p[3], hi, false);
 }
 
 __device__ __forceinline__ float dot_chunk4(const uint4 w, const XChunk4 &x) {
-    float acc = 0.0f;
-    acc = dot_word4(w.x, x.p + 0, acc);
-    acc = dot_word4(w.y, x.p + 4, acc);
-    acc = dot_word4(w.z, x.p + 8, acc);
-    acc = dot_word4(w.w, x.p + 12, acc);
-    return acc;
+    float lo = 0.0f, hi = 0.0f;
+    dot_word4(w.x, x.p + 0, lo, hi);
+    dot_word4(w.y, x.p + 4, lo, hi);
+    dot_word4(w.z, x.p + 8, lo, hi);
+    dot_word4(w.w, x.p + 12, lo, hi);
+    return fmaf(lo, 16.0f, hi) * 1048576.0f;
 }
 
-// 8-bit codes: bytes b0..b3 of a word are elements 4j..4j+3; a byte permute with a
-// register of 0x64 bytes builds the pairs {1024+b0, 1024+b1} and {1024+b2, 1024+b3}.
+// 8-bit codes: bytes b0..b3 of a word are elements 4j..4j+3; a byte permute spreads two
+// of them over the low bytes of the two halves: {b0, b1} * 2^-24 as fp16 subnormals.
 __device__ __forceinline__ float dot_word8(uint32_t w, const h2_t *p, float acc) {
-    const h2_t k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
-    const uint32_t magic = 0x64646464u;
-    const h2_t q01 = as_h2(__builtin_amdgcn_perm(magic, w, 0x04010400u)) - k1024;
-    const h2_t q23 = as_h2(__builtin_amdgcn_perm(magic, w, 0x04030402u)) - k1024;
-    acc = __builtin_amdgcn_fdot2(q01, p[0], acc, false);
-    acc = __builtin_amdgcn_fdot2(q23, p[1], acc, false);
+    acc = __builtin_amdgcn_fdot2(as_h2(__builtin_amdgcn_perm(0u, w, 0x0c010c00u)), p[0], acc, false);
+    acc = __builtin_amdgcn_fdot2(as_h2(__builtin_amdgcn_perm(0u, w, 0x0c030c02u)), p[1], acc, false);
     return acc;
 }
 
@@ -147,7 +141,7 @@ __device__ __forceinline__ float dot_chunk8(const uint4 w, const XChunk8 &x) {
     acc = dot_word8(w.y, x.p + 2, acc);
     acc = dot_word8(w.z, x.p + 4, acc);
     acc = dot_word8(w.w, x.p + 6, acc);
-    return acc;
+    return acc * 16777216.0f;
 }
 
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }

@@ -27,6 +27,16 @@ def assert_ffn_close(dev_bits: np.ndarray, ref_bits: np.ndarray, what: str = "",
         f"(|diff| {err[worst]:.3e} > {bound[worst]:.3e}); {int(np.sum(err > bound))} of {a.size} out of tolerance")
 
 
+def assert_rel_close(dev_bits: np.ndarray, ref_bits: np.ndarray, what: str = "", tol: float = REL_TOL):
+    """The reference's own metric (sources/ShrikeValidation/Support/Tolerance/RelError.swift:7-19):
+    max |a - b| / max(max |b|, 1e-6). Used end to end, where fp16 roundings between the stages
+    (gate/up -> act -> down) make single elements of a cancelling sum move by more than 2e-3."""
+    a, b = f16(dev_bits).astype(np.float64), f16(ref_bits).astype(np.float64)
+    assert np.all(np.isfinite(b)), f"{what}: the oracle's output is not finite"
+    rel = np.max(np.abs(a - b)) / max(np.max(np.abs(b)), 1e-6)
+    assert rel <= tol, f"{what}: relative error {rel:.3e} > {tol:.1e}"
+
+
 class Layer:
     """One synthetic MoE layer: E routed expert blobs, router, optional shared expert."""
 

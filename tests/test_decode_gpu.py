@@ -9,7 +9,7 @@ import pytest
 from oracle import oracle as O
 from shrike_amd import capi
 from shrike_amd import synth as S
-from tests.helpers import Layer, assert_ffn_close, f16
+from tests.helpers import Layer, assert_ffn_close, assert_rel_close, f16
 
 pytestmark = pytest.mark.gpu
 SENT = 0xFFFFFFFF
@@ -327,18 +327,32 @@ def test_closed_form_ffn(gpu):
 def test_shared_expert_against_oracle(gpu, bits, d, fs):
     L = Layer(0x5EED0100 + d + bits, d, 64, 2, 1, shared_f=fs, shared_bits=bits)
     dl = DeviceLayer(gpu, L, resident=[])
-    dl.moe.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, dl.x,
-                                dl.shared_scratch, dl.h1, d, fs)
-    ref = O.shared_expert(L.shared["gate"], L.shared["up"], L.shared["down"], L.x, d, fs, bits=bits)
-    assert_ffn_close(dl.h1.download(np.uint16, d), ref, "shared expert h1")
-    gate = S.f32_to_f16_bits(np.array([0.3], np.float32))
-    dl.moe.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, dl.x,
-                                dl.shared_scratch, dl.h1, d, fs, scalar_gate=gpu.dev(gate))
-    ref = O.shared_expert(L.shared["gate"], L.shared["up"], L.shared["down"], L.x, d, fs, bits=bits,
-                          scalar_gate_f16=gate)
-    # two fp16 roundings in a row (the GEMV's, then the gate's: dequant_int4.metal:322-329): a
-    # last-bit difference before the first can move the result by two fp16 steps, 2 * 2^-10
-    assert_ffn_close(dl.h1.download(np.uint16, d), ref, "gated shared expert h1", rel=2e-3)
+    sh = L.shared
+    for gate in (None, S.f32_to_f16_bits(np.array([0.3], np.float32))):
+        dl.moe.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, dl.x,
+                                    dl.shared_scratch, dl.h1, d, fs,
+                                    scalar_gate=None if gate is None else gpu.dev(gate))
+        check_shared_stages(dl, L, gate)
+
+
+def check_shared_stages(dl, L, gate=None):
+    """Each stage against the oracle fed with the device's previous stage (one fp16 rounding per
+    comparison), then the whole chain with the reference's relative metric."""
+    d, fs, bits, sh = L.d, L.shared_f, L.shared_bits, L.shared
+    halves = dl.shared_scratch.download(np.uint16, 2 * fs)
+    g_dev, u_dev = halves[:fs].copy(), halves[fs:].copy()
+    g_ref, u_ref = O.shared_gate_up(sh["gate"], sh["up"], L.x, d, fs, bits=bits, meta=L.meta)
+    assert_ffn_close(g_dev, g_ref, "shared gate rows")
+    assert_ffn_close(u_dev, u_ref, "shared up rows")
+    h1 = dl.h1.download(np.uint16, d)
+    # a gated output is rounded to fp16 twice in a row (dequant_int4.metal:322-329): two fp16 steps
+    assert_ffn_close(h1, O.shared_down(sh["down"], g_dev, u_dev, d, fs, bits=bits, meta=L.meta,
+                                       scalar_gate_f16=gate), "shared down from the device's gate/up",
+                     rel=1e-3 if gate is None else 2e-3)
+    assert_rel_close(h1, O.shared_expert(sh["gate"], sh["up"], sh["down"], L.x, d, fs, bits=bits, meta=L.meta,
+                                         scalar_gate_f16=gate), "shared expert end to end",
+                     tol=1e-3 if gate is None else 2e-3)
+    return h1
 
 
 # ------------------------------------------------------------------------ whole layer
@@ -368,11 +382,16 @@ def test_decode_layer_matches_oracle_and_split_calls(gpu, cfg):
     assert np.array_equal(dl.resolved.download(np.uint32, k), ref["classify"]["resolved_slots"])
     assert dl.hit_count.download(np.uint32, 1)[0] == k and dl.miss_count.download(np.uint32, 1)[0] == 0
     assert np.max(np.abs(f16(dl.out_w.download(np.uint16, k)) - f16(ref["weights"]))) <= 1e-3
-    if fs:
-        assert_ffn_close(dl.h1.download(np.uint16, d), ref["h1"], "h1")
-    assert_ffn_close(dl.acts.download(np.uint16, k * f), ref["acts"], "acts")
+    h1 = check_shared_stages(dl, L) if fs else np.zeros(d, np.uint16)
+    acts = dl.acts.download(np.uint16, k * f)
+    assert_ffn_close(acts, ref["acts"], "acts")
     y = dl.y.download(np.uint16, d)
-    assert_ffn_close(y, ref["y"], "y")
+    # phase 2 against the oracle fed with the device's own acts, weights and h1 (one rounding),
+    # then the whole layer with the reference's relative metric
+    blobs = [dl.pool_blobs()[int(c)] for c in dl.resolved.download(np.uint32, k)]
+    assert_ffn_close(y, O.moe_phase2(blobs, L.oracle_offsets(), acts, dl.out_w.download(np.uint16, k), h1, d, f,
+                                     bits=bits, meta=meta), "y from the device's acts")
+    assert_rel_close(y, ref["y"], "y end to end")
     assert np.array_equal(dl.hidden.download(np.uint16, d), O.residual_add_f16(L.hidden.copy(), y))
 
     # the operators called one after another give the same bytes as the fused entry point
