@@ -33,7 +33,7 @@ D, F, NE, K, FS, BITS = 2048, 512, 256, 8, 512, 4
 HBM_PEAK_GBPS = 8000.0
 
 
-def build_layers(rt, capi, S, n_layers, meta):
+def build_layers(rt, capi, S, n_layers, meta, shared=True):
     """Layer 0's pool comes from the seeded generator; the other layers hold byte copies of it at
     their own addresses (cache behaviour follows addresses, not values). Routers, shared experts
     and activations are distinct per layer."""
@@ -47,6 +47,11 @@ def build_layers(rt, capi, S, n_layers, meta):
     zeros_e = rt.dev(np.zeros(NE, np.uint16))
     hidden = rt.dev(S.activations_f16(tree, "hidden", D))
     first_pool = None
+    # the decode scratch is one set of buffers for all layers, as in the reference's runner
+    # (sources/Shrike/Runtime/Inference/RealForwardRunner.swift:754-825)
+    scratch = {name: rt.empty(size) for name, size in dict(idx=32, w=16, res=32, hc=4, hp=32, mc=4, mp=32, me=32,
+                                                           acts=2 * K * F, ss=4 * FS, h1=2 * D, y=2 * D).items()}
+    x = rt.dev(S.activations_f16(tree, "layer.x", D))
     for l in range(n_layers):
         pool = rt.ExpertPool(NE, stride, NE)
         if l == 0:
@@ -57,19 +62,16 @@ def build_layers(rt, capi, S, n_layers, meta):
             capi.check(capi.load().shrike_hip_memcpy_d2d(pool.cell_ptr(0), first_pool.cell_ptr(0), NE * pool.stride), "d2d")
         for e in range(NE):
             pool.publish(e, e, capi.RESIDENT)
-        lay = dict(pool=pool)
+        lay = dict(pool=pool, x=x, **scratch)
         lay["router"] = rt.dev(S.router_f16(tree, f"layer.{l}.router.w", NE, D))
-        lay["x"] = rt.dev(S.activations_f16(tree, f"layer.{l}.x", D))
         lay["shared"] = {n: tuple(rt.dev(t) for t in S.affine_matrix(tree.key(f"layer.{l}.shared.{n}"), r, c, BITS, meta))
                          for n, r, c in (("gate", FS, D), ("up", FS, D), ("down", D, FS))}
-        for name, size in dict(idx=32, w=16, res=32, hc=4, hp=32, mc=4, mp=32, me=32, acts=2 * K * F,
-                               ss=4 * FS, h1=2 * D, y=2 * D).items():
-            lay[name] = rt.empty(size)
         a = capi.DecodeLayerArgs()
         a.router_weights, a.effective_scale, a.per_expert_scale, a.logit_bias = lay["router"].ptr, ones_d.ptr, ones_e.ptr, zeros_e.ptr
         a.pool, a.pool_slot_stride, a.residency, a.offsets = pool.bases, pool.stride, pool.table, off
         for n in ("gate", "up", "down"):
-            setattr(a, f"shared_{n}", capi.Projection(*(t.ptr for t in lay["shared"][n])))
+            if shared:
+                setattr(a, f"shared_{n}", capi.Projection(*(t.ptr for t in lay["shared"][n])))
         a.shared_bits, a.shared_f = BITS, FS
         a.x, a.hidden, a.y = lay["x"].ptr, hidden.ptr, lay["y"].ptr
         a.out_indices, a.out_weights, a.resolved_slots = lay["idx"].ptr, lay["w"].ptr, lay["res"].ptr
@@ -137,6 +139,7 @@ def main():
     ap.add_argument("--layers", type=int, default=40, help="stacked layers with their own pools (40 x 453 MB)")
     ap.add_argument("--meta", choices=["f16", "bf16"], default="f16")
     ap.add_argument("--cpu-sample", type=int, default=60, help="layer evaluations timed on the CPU (0 = skip)")
+    ap.add_argument("--no-shared", action="store_true", help="diagnostic: leave the shared expert out of the layer")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path is built and measured on a single MI355X "
@@ -149,7 +152,7 @@ def main():
     rt.init(0)
     meta = S.META_F16 if args.meta == "f16" else S.META_BF16
     n_layers = args.layers
-    layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta)
+    layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta, shared=not args.no_shared)
     moe = rt.MoE(D, F, NE, K, routed_bits=BITS, router_bits=0, meta=meta)
     stream = rt.Stream()
     moe.stream = stream
@@ -182,6 +185,12 @@ def main():
             sh = lay["shared"]
             moe.encode_shared_expert(sh["gate"], sh["up"], sh["down"], BITS, lay["x"], lay["ss"], lay["h1"], D, FS)
 
+    def phase12():
+        for lay in layers:
+            moe.encode_spec_phase1(lay["pool"], lay["res"], off, lay["x"], lay["acts"], D, F, K)
+            moe.encode_spec_phase2(lay["pool"], lay["res"], off, lay["acts"], lay["w"], lay["h1"], lay["y"], None, D, F, K)
+
+    g_p12 = capture(rt, capi, stream, phase12)
     g_p1 = capture(rt, capi, stream, phase1_only)
     g_p2 = capture(rt, capi, stream, phase2_only)
     g_rt = capture(rt, capi, stream, router_only)
@@ -195,7 +204,7 @@ def main():
 
     reps = max(1, steps // n_layers // 2)
     parts = {}
-    for name, g, launches_per_layer in (("phase1", g_p1, 1), ("phase2", g_p2, 1), ("router_select_classify", g_rt, 1),
+    for name, g, launches_per_layer in (("phase1+phase2 alternating", g_p12, 2), ("phase1", g_p1, 1), ("phase2", g_p2, 1), ("router_select_classify", g_rt, 1),
                                         ("shared_expert(2 launches)", g_sh, 1)):
         time_graph(rt, capi, stream, g, 2)
         parts[name] = time_graph(rt, capi, stream, g, reps) / (reps * n_layers) * 1e3  # us per layer

@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libshrikehip.so")
+# SHRIKE_HIP_LIBRARY names another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("SHRIKE_HIP_LIBRARY") or os.path.join(_HERE, "libshrikehip.so")
 
 MAX_TOP_K = 8
 POOL_MAX_CHUNKS = 8

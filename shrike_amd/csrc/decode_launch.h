@@ -1,0 +1,63 @@
+// Argument blocks and launchers of the decode kernels, shared by the translation units
+// that define them and by the fused-layer entry point.
+#pragma once
+
+#include "gemv_common.h"
+
+namespace shrike {
+
+struct RouterArgs {
+    const void *weights;
+    const uint16_t *scales, *biases;
+    const uint16_t *hidden, *effective_scale;
+    uint32_t d, meta;
+    uint32_t *counter;
+    float *logits_out;
+    SelectArgs sel;
+    RouteLists lists;  // out_indices == nullptr: logits only
+};
+
+struct Phase1Args {
+    PoolArg pool;
+    uint64_t stride;
+    const uint32_t *resolved;
+    shrike_expert_offsets off;
+    const uint16_t *x;
+    uint16_t *acts;
+    uint32_t d, f, top_k, meta, act, ebias;
+    const uint32_t *indirect, *io_status;
+    // fused layer only: route from the logits of the previous launch (sel.logits != nullptr),
+    // and run the shared expert's down projection in workgroups past `routed_blocks`
+    SelectArgs sel;
+    RouteLists lists;
+    uint32_t routed_blocks;
+    GemvArgs shared_down;
+};
+
+struct Phase2Args {
+    PoolArg pool;
+    uint64_t stride;
+    const uint32_t *resolved, *fallback;
+    shrike_expert_offsets off;
+    const uint16_t *acts, *routing_w, *residual;
+    uint16_t *y, *hidden;
+    uint32_t d, f, top_k, meta, ebias;
+    const uint32_t *indirect, *io_status;
+};
+
+int launch_router(const RouterArgs &a, uint32_t router_bits, hipStream_t s);
+// router logit rows + the shared expert's gate/up rows in one grid
+int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, hipStream_t s);
+uint32_t phase1_blocks(uint32_t top_k, uint32_t f);
+// shared_down_bits: 0 = none, else the shared down rows ride in the same grid (one chunk
+// column per lane only: nch_for(shared_f, bits) == 1)
+int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t shared_down_bits, hipStream_t s);
+int launch_phase2(const Phase2Args &a, uint32_t bits, hipStream_t s);
+int launch_gemv(const GemvArgs &a, uint32_t bits, hipStream_t s);
+
+int check_offsets(const shrike_expert_offsets *o, uint32_t d, uint32_t f, uint32_t bits);
+int check_router(const shrike_hip_moe *moe, uint32_t num_experts, uint32_t d, uint32_t top_k);
+int check_shared(const shrike_projection *gate, const shrike_projection *up, const shrike_projection *down,
+                 uint32_t bits, uint32_t d, uint32_t f_shared);
+
+}  // namespace shrike

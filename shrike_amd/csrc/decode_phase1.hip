@@ -1,0 +1,168 @@
+// Phase 1 of the routed decode layer for gfx950: gate and up matvecs of the selected
+// experts against one activation vector, GLU, fp16 activations out
+// (moe.metal:950-999 for 4-bit codes, the :650-672 body for 8-bit, pool addressing
+// :297-305). In the fused layer the same launch routes (select + classify in the prologue
+// of every workgroup, from the logits of the previous launch) and carries the shared
+// expert's down projection in extra workgroups.
+#include "decode_launch.h"
+
+namespace shrike {
+
+constexpr int kPhase1RowPairs = 4;  // (gate, up) row pairs per wave
+
+// A wave owns RP consecutive f of one routed position: RP gate rows and RP up rows, each a
+// run of 16-byte chunks across the lanes. The lane's slice of x comes straight from global
+// memory (L2-resident) ahead of the row loads, so in-order load return never holds it back.
+template <int BITS, int NCH, int RP, bool ROUTE, int SBITS>
+__global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
+    typedef Chunk<BITS> C;
+    __shared__ uint32_t s_cell[SHRIKE_MAX_TOP_K];
+    if (SBITS != 0 && blockIdx.x >= a.routed_blocks) {
+        gemv_job<SBITS == 0 ? 4 : SBITS, 1>(a.shared_down, blockIdx.x - a.routed_blocks);
+        return;
+    }
+    if (a.indirect && a.indirect[0] == 0u) return;
+    if (!io_ready(a.io_status)) return;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t cpr = a.d * BITS / 128u, groups = a.d / kGroup, row_bytes = cpr * 16u;
+    const uint32_t pair0 = (blockIdx.x * 4u + wave) * RP;
+    const bool in_range = pair0 < a.top_k * a.f;
+    const uint32_t k = in_range ? pair0 / a.f : 0u;
+    const uint32_t f0 = pair0 - k * a.f;
+
+    SliceRegs<BITS, NCH> xr;
+    load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(a.x), cpr, lane, true);
+
+    uint32_t cell = kSentinel;
+    if (ROUTE) {
+        if (wave == 0) {
+            uint32_t my_cell;
+            route_wave<false>(a.sel, a.lists, lane, blockIdx.x == 0, my_cell);
+            if (lane < a.top_k) s_cell[lane] = my_cell;
+        }
+        __syncthreads();
+        if (in_range) cell = s_cell[k];
+    } else if (in_range) {
+        cell = a.resolved[k];
+    }
+    if (cell == kSentinel) return;  // moe.metal:986, and waves past the last row
+    const uint8_t *base = cell_base(a.pool, cell, a.stride);
+
+    RowRegs<BITS, NCH> rows[2 * RP];
+#pragma unroll
+    for (int r = 0; r < 2 * RP; ++r) {
+        const bool up = r >= RP;
+        const uint32_t f = f0 + uint32_t(r % RP);
+        const uint8_t *w = base + (up ? a.off.up_w_off : a.off.gate_w_off) + size_t(f) * row_bytes;
+        const uint16_t *s = reinterpret_cast<const uint16_t *>(base + (up ? a.off.up_s_off : a.off.gate_s_off)) + size_t(f) * groups;
+        const uint16_t *b = reinterpret_cast<const uint16_t *>(base + (up ? a.off.up_b_off : a.off.gate_b_off)) + size_t(f) * groups;
+        load_row<BITS, NCH>(rows[r], w, s, b, cpr, lane, true);
+    }
+    float gab = 0.0f, uab = 0.0f;
+    if (a.ebias && lane < uint32_t(RP)) {  // moe.metal:261-269
+        gab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.gate_ab_off)[f0 + lane]);
+        uab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.up_ab_off)[f0 + lane]);
+    }
+
+    typename C::X x[NCH];
+    float xs[NCH];
+    unpack_slices<BITS, NCH>(xr, x, xs);
+    float res[2 * RP];
+#pragma unroll
+    for (int r = 0; r < 2 * RP; ++r) res[r] = wave_sum(row_partial<BITS, NCH>(rows[r], x, xs, a.meta));
+    // lane p < RP finishes row pair p
+    float g = res[0], u = res[RP];
+#pragma unroll
+    for (int p = 1; p < RP; ++p) {
+        g = lane == uint32_t(p) ? res[p] : g;
+        u = lane == uint32_t(p) ? res[RP + p] : u;
+    }
+    const uint16_t act = f32_to_f16(glu_rt(g + gab, u + uab, a.act));
+    if (lane < uint32_t(RP)) a.acts[size_t(k) * a.f + f0 + lane] = act;
+}
+
+uint32_t phase1_blocks(uint32_t top_k, uint32_t f) {
+    const uint32_t waves = (top_k * f + kPhase1RowPairs - 1) / kPhase1RowPairs;
+    return (waves + 3) / 4;
+}
+
+template <int BITS, bool ROUTE, int SBITS>
+static void launch_phase1_nch(const Phase1Args &a, dim3 grid, hipStream_t s) {
+    constexpr int RP = kPhase1RowPairs;
+    const dim3 block(256);
+    switch (nch_for(a.d, BITS)) {
+        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, RP, ROUTE, SBITS>), grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, RP, ROUTE, SBITS>), grid, block, 0, s, a); break;
+        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RP, ROUTE, SBITS>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RP, ROUTE, SBITS>), grid, block, 0, s, a); break;
+    }
+}
+
+int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t shared_down_bits, hipStream_t s) {
+    SHRIKE_REQUIRE(a.f % kPhase1RowPairs == 0, "phase1: f=%u must be a multiple of %d", a.f, kPhase1RowPairs);
+    uint32_t extra = 0;
+    if (shared_down_bits) {
+        SHRIKE_REQUIRE(routing && nch_for(a.shared_down.n, shared_down_bits) == 1,
+                       "phase1: the shared down rows ride along only in the routed launch and with one chunk column per lane");
+        extra = gemv_blocks(a.shared_down.rows, a.shared_down.n, shared_down_bits);
+    }
+    const dim3 grid(a.routed_blocks + extra);
+    if (bits == 4) {
+        if (!routing) launch_phase1_nch<4, false, 0>(a, grid, s);
+        else if (shared_down_bits == 0) launch_phase1_nch<4, true, 0>(a, grid, s);
+        else if (shared_down_bits == 4) launch_phase1_nch<4, true, 4>(a, grid, s);
+        else launch_phase1_nch<4, true, 8>(a, grid, s);
+    } else {
+        if (!routing) launch_phase1_nch<8, false, 0>(a, grid, s);
+        else if (shared_down_bits == 0) launch_phase1_nch<8, true, 0>(a, grid, s);
+        else if (shared_down_bits == 4) launch_phase1_nch<8, true, 4>(a, grid, s);
+        else launch_phase1_nch<8, true, 8>(a, grid, s);
+    }
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int check_offsets(const shrike_expert_offsets *o, uint32_t d, uint32_t f, uint32_t bits) {
+    SHRIKE_REQUIRE(o != nullptr, "offsets is NULL");
+    SHRIKE_REQUIRE(d % SHRIKE_GROUP_SIZE == 0 && f % SHRIKE_GROUP_SIZE == 0,
+                   "d=%u and f=%u must be multiples of %u", d, f, SHRIKE_GROUP_SIZE);
+    SHRIKE_REQUIRE(d <= SHRIKE_MAX_HIDDEN, "d=%u exceeds the activation ceiling %u", d, SHRIKE_MAX_HIDDEN);
+    SHRIKE_REQUIRE(nch_for(d, bits) <= 4 && nch_for(f, bits) <= 4, "row of %u/%u %u-bit codes is too long", d, f, bits);
+    // 128-bit code loads need 16-byte aligned code tensors; metadata needs 2 bytes
+    SHRIKE_REQUIRE((o->gate_w_off | o->up_w_off | o->down_w_off) % 16u == 0,
+                   "code sub-tensors must be 16-byte aligned inside the blob");
+    SHRIKE_REQUIRE((o->gate_s_off | o->gate_b_off | o->up_s_off | o->up_b_off | o->down_s_off | o->down_b_off
+                    | o->gate_ab_off | o->up_ab_off | o->down_ab_off) % 2u == 0,
+                   "metadata sub-tensors must be 2-byte aligned");
+    SHRIKE_REQUIRE((d * bits / 8u) % 16u == 0 && (f * bits / 8u) % 16u == 0, "row bytes must be a multiple of 16");
+    return 0;
+}
+
+}  // namespace shrike
+
+using namespace shrike;
+
+extern "C" {
+
+int shrike_hip_moe_phase1_pool(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                               uint64_t pool_slot_stride, const uint32_t *d_resolved_slots,
+                               const shrike_expert_offsets *offsets, const void *d_x, void *d_acts, uint32_t d,
+                               uint32_t f, uint32_t top_k, const uint32_t *d_indirect, const uint32_t *d_io_status) {
+    SHRIKE_REQUIRE(moe != nullptr && pool != nullptr, "moe handle or pool is NULL");
+    SHRIKE_REQUIRE(top_k >= 1 && top_k <= SHRIKE_MAX_TOP_K, "phase1: topK=%u not in 1...8", top_k);  // MoE.swift:925
+    const uint32_t bits = moe->desc.routed_weight_bits;
+    if (int rc = check_offsets(offsets, d, f, bits)) return rc;
+    SHRIKE_REQUIRE(d_resolved_slots && d_x && d_acts, "phase1: resolvedSlots, x and acts must be bound");
+    SHRIKE_REQUIRE(pool_slot_stride % 16u == 0, "phase1: pool slot stride must be a multiple of 16");
+    Phase1Args a = {};
+    fill_pool(a.pool, pool);
+    a.stride = pool_slot_stride; a.resolved = d_resolved_slots; a.off = *offsets;
+    a.x = static_cast<const uint16_t *>(d_x); a.acts = static_cast<uint16_t *>(d_acts);
+    a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.act = moe->desc.activation;
+    a.ebias = moe->desc.expert_additive_biases;
+    a.indirect = d_indirect; a.io_status = moe->desc.event_gated_io ? d_io_status : nullptr;
+    a.routed_blocks = phase1_blocks(top_k, f);
+    return launch_phase1(a, bits, false, 0, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,299 @@
+// Phase 2 of the routed decode layer for gfx950 (down matvec per selected expert, weighted
+// combine, residual, hidden += y: moe.metal:889-941, :1008-1057), the dense group-affine
+// GEMV of the shared expert, and the fused-layer entry point.
+#include "decode_launch.h"
+
+namespace shrike {
+
+constexpr uint32_t kPhase2Rows = 8;  // output rows per workgroup
+
+// moe.metal:889-893
+__device__ __forceinline__ void phase2_finish(uint16_t *y, uint16_t *hidden, uint32_t d, uint16_t value,
+                                              uint16_t hidden_old) {
+    y[d] = value;
+    if (hidden) hidden[d] = f32_to_f16(f16_to_f32(hidden_old) + f16_to_f32(value));
+}
+
+// One wave per routed position (blockDim = 64 * top_k); a workgroup owns kPhase2Rows output
+// rows. When a down row is shorter than a wave's 1 KiB load, the wave covers 64/cpr rows per
+// load and reduces over lane segments. BATCH row groups are in flight per wave.
+template <int BITS, int NCH, int BATCH>
+__global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
+    typedef Chunk<BITS> C;
+    __shared__ float partial[SHRIKE_MAX_TOP_K][kPhase2Rows];
+    if (a.indirect && a.indirect[0] == 0u) return;
+    const uint32_t lane = threadIdx.x & 63u, k = threadIdx.x >> 6;
+    const uint32_t d0 = blockIdx.x * kPhase2Rows;
+    // the epilogue's operands do not depend on anything computed here: fetch them first
+    const bool finisher = threadIdx.x < kPhase2Rows && d0 + threadIdx.x < a.d;
+    uint16_t res_bits = 0, hid_bits = 0;
+    if (finisher) {
+        if (a.residual) res_bits = a.residual[d0 + threadIdx.x];
+        if (a.hidden) hid_bits = a.hidden[d0 + threadIdx.x];
+    }
+    if (!io_ready(a.io_status)) {  // moe.metal:1032-1035
+        if (finisher) phase2_finish(a.y, a.hidden, d0 + threadIdx.x, res_bits, hid_bits);
+        return;
+    }
+    const uint32_t cpr = a.f * BITS / 128u, groups = a.f / kGroup, row_bytes = cpr * 16u;
+    const bool packed = cpr < 64u && (64u % cpr) == 0u;
+    const uint32_t rpl = packed ? min(64u / cpr, kPhase2Rows) : 1u;  // rows per wave load
+    const uint32_t seg = packed ? cpr : 64u;
+    const uint32_t sub = packed ? lane / cpr : 0u, col = packed ? lane % cpr : lane;
+    const bool lane_on = sub < rpl;
+
+    SliceRegs<BITS, NCH> xr;
+    load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(a.acts + size_t(k) * a.f), cpr, col, lane_on);
+    uint32_t cell = a.resolved[k];
+    const float wk = f16_to_f32(a.routing_w[k]);
+    if (cell == kSentinel && a.fallback) cell = a.fallback[k];  // moe.metal:1037-1038
+    const bool live = cell != kSentinel;
+    const uint8_t *base = cell_base(a.pool, live ? cell : 0u, a.stride);
+    const uint16_t *s_all = reinterpret_cast<const uint16_t *>(base + a.off.down_s_off);
+    const uint16_t *b_all = reinterpret_cast<const uint16_t *>(base + a.off.down_b_off);
+
+    if (live) {
+        const uint32_t n_groups = kPhase2Rows / rpl;
+        typename C::X x[NCH];
+        float xs[NCH];
+        for (uint32_t g0 = 0; g0 < n_groups; g0 += BATCH) {
+            RowRegs<BITS, NCH> rows[BATCH];
+            uint32_t row[BATCH];
+            bool on[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                row[j] = d0 + (g0 + j) * rpl + sub;
+                on[j] = lane_on && (g0 + j) < n_groups && row[j] < a.d;
+                const uint32_t rr = on[j] ? row[j] : 0u;
+                load_row<BITS, NCH>(rows[j], base + a.off.down_w_off + size_t(rr) * row_bytes,
+                                    s_all + size_t(rr) * groups, b_all + size_t(rr) * groups, cpr, col, on[j]);
+            }
+            if (g0 == 0) unpack_slices<BITS, NCH>(xr, x, xs);
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                float v = seg_sum(row_partial<BITS, NCH>(rows[j], x, xs, a.meta), seg);
+                const bool writer = on[j] && (lane % seg) == seg - 1u;
+                if (writer) {
+                    if (a.ebias) v += bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[row[j]]);
+                    partial[k][row[j] - d0] = wk * v;  // moe.metal:1049
+                }
+            }
+        }
+    } else if (lane < kPhase2Rows) {
+        partial[k][lane] = 0.0f;
+    }
+    __syncthreads();
+    if (finisher) {
+        float acc = a.residual ? f16_to_f32(res_bits) : 0.0f;
+        for (uint32_t i = 0; i < a.top_k; ++i) acc += partial[i][threadIdx.x];
+        phase2_finish(a.y, a.hidden, d0 + threadIdx.x, f32_to_f16(acc), hid_bits);
+    }
+}
+
+template <int BITS, int NCH>
+__global__ __launch_bounds__(256) void k_gemv(GemvArgs a) { gemv_job<BITS, NCH>(a, blockIdx.x); }
+
+template <int BITS, int NCH>
+static void launch_phase2_batch(const Phase2Args &a, dim3 grid, dim3 block, hipStream_t s) {
+    const uint32_t cpr = a.f * BITS / 128u;
+    const uint32_t rpl = (cpr < 64u && 64u % cpr == 0u) ? (64u / cpr < kPhase2Rows ? 64u / cpr : kPhase2Rows) : 1u;
+    const uint32_t n_groups = kPhase2Rows / rpl;  // row groups per wave; up to 4 in flight
+    if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4>), grid, block, 0, s, a);
+    else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1>), grid, block, 0, s, a);
+}
+
+template <int BITS>
+static void launch_phase2_bits(const Phase2Args &a, hipStream_t s) {
+    const dim3 grid((a.d + kPhase2Rows - 1) / kPhase2Rows), block(64 * a.top_k);
+    switch (nch_for(a.f, BITS)) {
+        case 1: launch_phase2_batch<BITS, 1>(a, grid, block, s); break;
+        case 2: launch_phase2_batch<BITS, 2>(a, grid, block, s); break;
+        case 3: launch_phase2_batch<BITS, 3>(a, grid, block, s); break;
+        default: launch_phase2_batch<BITS, 4>(a, grid, block, s); break;
+    }
+}
+
+int launch_phase2(const Phase2Args &a, uint32_t bits, hipStream_t s) {
+    if (bits == 4) launch_phase2_bits<4>(a, s); else launch_phase2_bits<8>(a, s);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int BITS>
+static void launch_gemv_bits(const GemvArgs &a, hipStream_t s) {
+    const dim3 grid(gemv_blocks(a.rows + a.rows_b, a.n, BITS)), block(256);
+    switch (nch_for(a.n, BITS)) {
+        case 1: hipLaunchKernelGGL((k_gemv<BITS, 1>), grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL((k_gemv<BITS, 2>), grid, block, 0, s, a); break;
+        case 3: hipLaunchKernelGGL((k_gemv<BITS, 3>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((k_gemv<BITS, 4>), grid, block, 0, s, a); break;
+    }
+}
+
+int launch_gemv(const GemvArgs &a, uint32_t bits, hipStream_t s) {
+    if (bits == 4) launch_gemv_bits<4>(a, s); else launch_gemv_bits<8>(a, s);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+static void fill_gemv_gate_up(GemvArgs &a, const shrike_projection *gate, const shrike_projection *up,
+                              uint16_t *gate_out, uint16_t *up_out, uint32_t rows, uint32_t n, uint32_t meta,
+                              const void *x) {
+    a.w_a = static_cast<const uint8_t *>(gate->weights); a.s_a = static_cast<const uint16_t *>(gate->scales);
+    a.b_a = static_cast<const uint16_t *>(gate->biases); a.y_a = gate_out;
+    a.w_b = static_cast<const uint8_t *>(up->weights); a.s_b = static_cast<const uint16_t *>(up->scales);
+    a.b_b = static_cast<const uint16_t *>(up->biases); a.y_b = up_out;
+    a.rows = rows; a.rows_b = rows; a.n = n; a.meta = meta;
+    a.x = static_cast<const uint16_t *>(x);
+}
+
+static void fill_gemv_down(GemvArgs &b, const shrike_projection *down, const uint16_t *gate_in,
+                           const uint16_t *up_in, void *h1, uint32_t d, uint32_t f_shared, uint32_t meta,
+                           uint32_t act, const void *scalar_gate) {
+    b.w_a = static_cast<const uint8_t *>(down->weights); b.s_a = static_cast<const uint16_t *>(down->scales);
+    b.b_a = static_cast<const uint16_t *>(down->biases); b.y_a = static_cast<uint16_t *>(h1);
+    b.rows = d; b.rows_b = 0; b.n = f_shared; b.meta = meta;
+    b.gate_in = gate_in; b.up_in = up_in; b.act = act;
+    b.scalar_gate = static_cast<const uint16_t *>(scalar_gate);
+}
+
+int check_shared(const shrike_projection *gate, const shrike_projection *up, const shrike_projection *down,
+                 uint32_t bits, uint32_t d, uint32_t f_shared) {
+    SHRIKE_REQUIRE(gate && up && down && gate->weights && up->weights && down->weights && gate->scales && gate->biases
+                   && up->scales && up->biases && down->scales && down->biases,
+                   "sharedExpert: gate, up and down projections must be bound");
+    SHRIKE_REQUIRE(bits == 4 || bits == 8, "sharedExpert: bits=%u not in {4, 8}", bits);
+    SHRIKE_REQUIRE(d % SHRIKE_GROUP_SIZE == 0 && f_shared % SHRIKE_GROUP_SIZE == 0 && f_shared > 0,
+                   "sharedExpert: d=%u and f=%u must be multiples of %u", d, f_shared, SHRIKE_GROUP_SIZE);
+    SHRIKE_REQUIRE(nch_for(d, bits) <= 4 && nch_for(f_shared, bits) <= 4, "sharedExpert: rows too long");
+    return 0;
+}
+
+}  // namespace shrike
+
+using namespace shrike;
+
+extern "C" {
+
+int shrike_hip_moe_phase2_pool(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                               uint64_t pool_slot_stride, const uint32_t *d_resolved_slots,
+                               const uint32_t *d_fallback_cells, const shrike_expert_offsets *offsets,
+                               const void *d_acts, const void *d_routing_weights, const void *d_residual, void *d_y,
+                               void *d_hidden, uint32_t d, uint32_t f, uint32_t top_k, const uint32_t *d_indirect,
+                               const uint32_t *d_io_status) {
+    SHRIKE_REQUIRE(moe != nullptr && pool != nullptr, "moe handle or pool is NULL");
+    SHRIKE_REQUIRE(top_k >= 1 && top_k <= SHRIKE_MAX_TOP_K, "phase2: topK=%u not in 1...8", top_k);  // MoE.swift:1015
+    const uint32_t bits = moe->desc.routed_weight_bits;
+    if (int rc = check_offsets(offsets, d, f, bits)) return rc;
+    SHRIKE_REQUIRE(d_resolved_slots && d_acts && d_routing_weights && d_residual && d_y,
+                   "phase2: resolvedSlots, acts, routingWeights, residual and y must be bound");
+    SHRIKE_REQUIRE(pool_slot_stride % 16u == 0, "phase2: pool slot stride must be a multiple of 16");
+    Phase2Args a = {};
+    fill_pool(a.pool, pool);
+    a.stride = pool_slot_stride; a.resolved = d_resolved_slots; a.fallback = d_fallback_cells; a.off = *offsets;
+    a.acts = static_cast<const uint16_t *>(d_acts); a.routing_w = static_cast<const uint16_t *>(d_routing_weights);
+    a.residual = static_cast<const uint16_t *>(d_residual);
+    a.y = static_cast<uint16_t *>(d_y); a.hidden = static_cast<uint16_t *>(d_hidden);
+    a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.ebias = moe->desc.expert_additive_biases;
+    a.indirect = d_indirect; a.io_status = moe->desc.event_gated_io ? d_io_status : nullptr;
+    return launch_phase2(a, bits, as_stream(stream));
+}
+
+int shrike_hip_shared_expert(shrike_hip_moe *moe, void *stream, const shrike_projection *gate,
+                             const shrike_projection *up, const shrike_projection *down, uint32_t bits,
+                             const void *d_x, void *d_scratch, void *d_h1, const void *d_scalar_gate, uint32_t d,
+                             uint32_t f_shared) {
+    SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
+    if (int rc = check_shared(gate, up, down, bits, d, f_shared)) return rc;
+    SHRIKE_REQUIRE(d_x && d_scratch && d_h1, "sharedExpert: x, scratch and h1 must be bound");
+    uint16_t *gate_out = static_cast<uint16_t *>(d_scratch), *up_out = gate_out + f_shared;
+    GemvArgs a = {};
+    fill_gemv_gate_up(a, gate, up, gate_out, up_out, f_shared, d, moe->desc.meta_dtype, d_x);
+    if (int rc = launch_gemv(a, bits, as_stream(stream))) return rc;
+    GemvArgs b = {};
+    fill_gemv_down(b, down, gate_out, up_out, d_h1, d, f_shared, moe->desc.meta_dtype, moe->desc.activation,
+                   d_scalar_gate);
+    return launch_gemv(b, bits, as_stream(stream));
+}
+
+// Three launches: (1) router logit rows + shared gate/up rows; (2) select + classify in the
+// prologue of every phase-1 workgroup, the routed gate/up rows, and the shared down rows;
+// (3) phase 2 with the shared expert's output as the residual.
+int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *g) {
+    SHRIKE_REQUIRE(moe != nullptr && g != nullptr, "moe handle or args is NULL");
+    const shrike_moe_desc &m = moe->desc;
+    if (int rc = check_router(moe, m.num_experts, m.d, m.top_k)) return rc;
+    if (int rc = check_offsets(&g->offsets, m.d, m.f, m.routed_weight_bits)) return rc;
+    SHRIKE_REQUIRE(g->router_weights && g->effective_scale && g->per_expert_scale && g->logit_bias,
+                   "decodeLayer: router operands must be bound");
+    SHRIKE_REQUIRE(m.router_weight_bits == 0 || (g->router_scales && g->router_biases),
+                   "decodeLayer: affine router needs scales and biases");
+    SHRIKE_REQUIRE(g->pool && g->residency && g->x && g->y && g->out_indices && g->out_weights && g->resolved_slots
+                   && g->hit_count && g->hit_positions && g->miss_count && g->miss_positions && g->miss_experts
+                   && g->acts, "decodeLayer: pool, residency, x, y and the scratch buffers must be bound");
+    SHRIKE_REQUIRE(g->pool_slot_stride % 16u == 0, "decodeLayer: pool slot stride must be a multiple of 16");
+    hipStream_t s = as_stream(stream);
+    const bool shared = g->shared_gate.weights != nullptr;
+    const uint32_t sbits = g->shared_bits ? g->shared_bits : m.routed_weight_bits;
+    if (shared) {
+        if (int rc = check_shared(&g->shared_gate, &g->shared_up, &g->shared_down, sbits, m.d, g->shared_f)) return rc;
+        SHRIKE_REQUIRE(g->shared_scratch && g->h1, "decodeLayer: sharedScratch and h1 must be bound");
+    }
+    uint16_t *gate_out = static_cast<uint16_t *>(g->shared_scratch), *up_out = gate_out ? gate_out + g->shared_f : nullptr;
+
+    RouterArgs r = {};
+    r.weights = g->router_weights; r.scales = static_cast<const uint16_t *>(g->router_scales);
+    r.biases = static_cast<const uint16_t *>(g->router_biases);
+    r.hidden = static_cast<const uint16_t *>(g->x);
+    r.effective_scale = static_cast<const uint16_t *>(g->effective_scale);
+    r.d = m.d; r.meta = m.meta_dtype; r.counter = moe->d_counter; r.logits_out = moe->d_logits;
+    r.sel.logits = moe->d_logits;
+    r.sel.per_expert_scale = static_cast<const uint16_t *>(g->per_expert_scale);
+    r.sel.logit_bias = static_cast<const uint16_t *>(g->logit_bias);
+    r.sel.num_experts = m.num_experts; r.sel.top_k = m.top_k;
+    r.sel.sigmoid = m.sigmoid_router_scores; r.sel.scaling = m.routed_scaling_factor;
+    // r.lists stays empty: launch 1 writes logits only
+
+    Phase1Args p1 = {};
+    fill_pool(p1.pool, g->pool);
+    p1.stride = g->pool_slot_stride; p1.resolved = g->resolved_slots; p1.off = g->offsets;
+    p1.x = static_cast<const uint16_t *>(g->x); p1.acts = static_cast<uint16_t *>(g->acts);
+    p1.d = m.d; p1.f = m.f; p1.top_k = m.top_k; p1.meta = m.meta_dtype; p1.act = m.activation;
+    p1.ebias = m.expert_additive_biases;
+    p1.sel = r.sel;
+    p1.lists.out_indices = g->out_indices; p1.lists.out_weights = static_cast<uint16_t *>(g->out_weights);
+    p1.lists.residency = g->residency; p1.lists.hit_count = g->hit_count; p1.lists.hit_positions = g->hit_positions;
+    p1.lists.miss_count = g->miss_count; p1.lists.miss_positions = g->miss_positions;
+    p1.lists.miss_experts = g->miss_experts; p1.lists.resolved_slots = g->resolved_slots;
+    p1.routed_blocks = phase1_blocks(m.top_k, m.f);
+
+    const void *residual = nullptr;
+    bool down_fused = false;
+    if (shared) {
+        GemvArgs gu = {};
+        fill_gemv_gate_up(gu, &g->shared_gate, &g->shared_up, gate_out, up_out, g->shared_f, m.d, m.meta_dtype, g->x);
+        if (int rc = launch_head(r, m.router_weight_bits, gu, sbits, s)) return rc;
+        fill_gemv_down(p1.shared_down, &g->shared_down, gate_out, up_out, g->h1, m.d, g->shared_f, m.meta_dtype,
+                       m.activation, g->shared_scalar_gate);
+        down_fused = nch_for(g->shared_f, sbits) == 1;
+        residual = g->h1;
+    } else {
+        if (int rc = launch_router(r, m.router_weight_bits, s)) return rc;
+    }
+    if (int rc = launch_phase1(p1, m.routed_weight_bits, true, down_fused ? sbits : 0u, s)) return rc;
+    if (shared && !down_fused) {
+        if (int rc = launch_gemv(p1.shared_down, sbits, s)) return rc;
+    }
+
+    Phase2Args p = {};
+    fill_pool(p.pool, g->pool);
+    p.stride = g->pool_slot_stride; p.resolved = g->resolved_slots; p.off = g->offsets;
+    p.acts = static_cast<const uint16_t *>(g->acts); p.routing_w = static_cast<const uint16_t *>(g->out_weights);
+    p.residual = static_cast<const uint16_t *>(residual);
+    p.y = static_cast<uint16_t *>(g->y); p.hidden = static_cast<uint16_t *>(g->hidden);
+    p.d = m.d; p.f = m.f; p.top_k = m.top_k; p.meta = m.meta_dtype; p.ebias = m.expert_additive_biases;
+    return launch_phase2(p, m.routed_weight_bits, s);
+}
+
+}  // extern "C"

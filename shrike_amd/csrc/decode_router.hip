@@ -1,0 +1,297 @@
+// Router logits, top-k select and residency classification for gfx950, and the head
+// launch of the fused layer (router rows beside the shared expert's gate/up rows).
+#include "decode_launch.h"
+
+namespace shrike {
+
+// One expert row of the router GEMV (moe.metal:324-364), RK: 0 = fp16 rows, 8 / 4 =
+// group-affine codes. The per-lane fused-multiply-add order and the xor butterfly are
+// fixed so that the fp32 logits are reproducible bit for bit (lane l takes chunks
+// l, l+64, ...).
+template <int RK>
+__device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint32_t lane) {
+    constexpr int E = RK == 0 ? 8 : RK == 8 ? 16 : 32;  // elements per 16-byte weight chunk
+    constexpr int PIECES = E / 8;
+    constexpr int MAXI = RK == 0 ? 8 : 4;
+    const uint32_t chunks = a.d / E;
+    const uint32_t groups = a.d / kGroup;
+    const uint32_t row_bytes = chunks * 16u;
+    const uint8_t *row = static_cast<const uint8_t *>(a.weights) + size_t(e) * row_bytes;
+    uint4 w[MAXI], xv[MAXI][PIECES], ev[MAXI][PIECES];
+    uint16_t sc[MAXI], bi[MAXI];
+#pragma unroll
+    for (int i = 0; i < MAXI; ++i) {
+        const uint32_t c = lane + 64u * i;
+        const uint32_t cc = c < chunks ? c : 0u;
+        w[i] = *reinterpret_cast<const uint4 *>(row + 16u * cc);
+#pragma unroll
+        for (int j = 0; j < PIECES; ++j) {
+            xv[i][j] = reinterpret_cast<const uint4 *>(a.hidden)[cc * PIECES + j];
+            ev[i][j] = reinterpret_cast<const uint4 *>(a.effective_scale)[cc * PIECES + j];
+        }
+        if (RK != 0) {
+            sc[i] = a.scales[size_t(e) * groups + cc * E / kGroup];
+            bi[i] = a.biases[size_t(e) * groups + cc * E / kGroup];
+        }
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MAXI; ++i) {
+        const uint32_t c = lane + 64u * i;
+        if (c < chunks) {
+            float xs[E];
+#pragma unroll
+            for (int j = 0; j < PIECES; ++j) {
+                const uint32_t xw[4] = {xv[i][j].x, xv[i][j].y, xv[i][j].z, xv[i][j].w};
+                const uint32_t ew[4] = {ev[i][j].x, ev[i][j].y, ev[i][j].z, ev[i][j].w};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {  // moe.metal:357-358 (exact product)
+                    xs[8 * j + 2 * t] = __fmul_rn(f16_to_f32(uint16_t(xw[t])), bf16_to_f32(uint16_t(ew[t])));
+                    xs[8 * j + 2 * t + 1] = __fmul_rn(f16_to_f32(uint16_t(xw[t] >> 16)), bf16_to_f32(uint16_t(ew[t] >> 16)));
+                }
+            }
+            const uint32_t ww[4] = {w[i].x, w[i].y, w[i].z, w[i].w};
+            if (RK == 0) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    acc = fmaf(f16_to_f32(uint16_t(ww[t])), xs[2 * t], acc);
+                    acc = fmaf(f16_to_f32(uint16_t(ww[t] >> 16)), xs[2 * t + 1], acc);
+                }
+            } else {
+                float qx = 0.0f, sum = 0.0f;
+#pragma unroll
+                for (int t = 0; t < E; ++t) {
+                    const uint32_t q = RK == 8 ? (ww[t / 4] >> (8 * (t % 4))) & 0xffu
+                                               : (ww[t / 8] >> (4 * (t % 8))) & 0xfu;
+                    qx = fmaf(float(q), xs[t], qx);
+                    sum = __fadd_rn(sum, xs[t]);
+                }
+                acc = fmaf(meta_f32(sc[i], a.meta), qx, acc);
+                acc = fmaf(meta_f32(bi[i], a.meta), sum, acc);
+            }
+        }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, o));
+    if (lane == 0) a.logits_out[e] = acc;
+}
+
+// MoE.encodeRouter as one launch: four expert rows per workgroup, and the workgroup that
+// finishes last runs select (+ classify when a residency table is bound).
+template <int RK>
+__global__ __launch_bounds__(256) void k_router(RouterArgs a) {
+    __shared__ uint32_t s_last;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t e = blockIdx.x * 4u + wave;
+    if (e < a.sel.num_experts) {
+        router_row<RK>(a, e, lane);
+        if (lane == 0) __threadfence();
+    }
+    if (!a.lists.out_indices) return;  // logits only
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __threadfence();
+        s_last = atomicAdd(a.counter, 1u) == gridDim.x - 1u ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!s_last || wave != 0) return;
+    __threadfence();
+    uint32_t cell;
+    route_wave<true>(a.sel, a.lists, lane, true, cell);
+    if (lane == 0) *a.counter = 0u;
+}
+
+// The head of the fused layer: the router's logit rows and, beside them in the same grid,
+// the shared expert's gate and up rows. Neither depends on the other.
+template <int RK, int BITS, int NCH>
+__global__ __launch_bounds__(256) void k_head(RouterArgs r, GemvArgs g, uint32_t router_blocks) {
+    if (blockIdx.x < router_blocks) {
+        const uint32_t e = blockIdx.x * 4u + (threadIdx.x >> 6);
+        if (e < r.sel.num_experts) router_row<RK>(r, e, threadIdx.x & 63u);
+    } else {
+        gemv_job<BITS, NCH>(g, blockIdx.x - router_blocks);
+    }
+}
+
+struct ClassifyArgs {
+    const uint32_t *topk;
+    const uint64_t *residency;
+    uint32_t *hit_count, *hit_positions, *miss_count, *miss_positions, *miss_experts, *resolved_slots;
+    uint32_t top_k, num_experts;
+    uint32_t full_grids[12];
+    uint32_t *spec_args;
+    uint32_t *host_readback;
+    uint32_t tag;
+    const uint16_t *topk_weights;
+    const uint32_t *predicted;
+};
+
+// moe.metal:194-231 with the readback of :158-181; lane p classifies position p.
+__global__ __launch_bounds__(64) void k_classify(ClassifyArgs a) {
+    __shared__ uint32_t s_hit[SHRIKE_MAX_TOP_K], s_miss[SHRIKE_MAX_TOP_K];
+    const uint32_t lane = threadIdx.x;
+    const bool on = lane < a.top_k;
+    uint32_t expert = 0, slot = kSentinel, state = 0;
+    if (on) {
+        expert = min(a.topk[lane], a.num_experts - 1u);
+        const uint64_t word = a.residency[expert];
+        slot = uint32_t(word);
+        state = uint32_t(word >> 32);
+    }
+    const bool hit = on && state == SHRIKE_RESIDENCY_RESIDENT && slot != kSentinel;
+    const uint64_t hit_mask = __ballot(hit), miss_mask = __ballot(on && !hit);
+    const uint64_t below = (uint64_t(1) << lane) - 1u;
+    const uint32_t hits = __popcll(hit_mask), misses = __popcll(miss_mask);
+    const uint32_t my_hit_at = __popcll(hit_mask & below), my_miss_at = __popcll(miss_mask & below);
+    if (hit) {
+        a.hit_positions[my_hit_at] = lane;
+        a.resolved_slots[lane] = slot;
+        s_hit[my_hit_at] = lane;
+    } else if (on) {
+        a.miss_positions[my_miss_at] = lane;
+        a.miss_experts[my_miss_at] = expert;
+        a.resolved_slots[lane] = kSentinel;
+        s_miss[my_miss_at] = lane;
+    }
+    if (lane == 0) {
+        a.hit_count[0] = hits;
+        a.miss_count[0] = misses;
+    }
+    const bool all_hit = misses == 0u;
+    if (a.spec_args && lane < 3) {
+        const uint32_t zero_grid = lane == 0 ? 0u : 1u;
+        a.spec_args[lane] = a.full_grids[lane];
+        a.spec_args[3 + lane] = all_hit ? a.full_grids[3 + lane] : zero_grid;
+        a.spec_args[6 + lane] = all_hit ? zero_grid : a.full_grids[6 + lane];
+        a.spec_args[9 + lane] = all_hit ? zero_grid : a.full_grids[9 + lane];
+    }
+    __syncthreads();
+    if (a.tag != 0u && a.host_readback) {
+        const uint32_t t = a.tag << 16, K = a.top_k;
+        if (lane == 0) {
+            a.host_readback[0] = t | hits;
+            a.host_readback[1] = t | misses;
+        }
+        if (on) {
+            a.host_readback[2 + lane] = t | expert;
+            a.host_readback[2 + K + lane] = t | uint32_t(a.topk_weights[lane]);
+            a.host_readback[2 + 2 * K + lane] = t | (lane < hits ? s_hit[lane] : 0u);
+            a.host_readback[2 + 3 * K + lane] = t | (lane < misses ? s_miss[lane] : 0u);
+            a.host_readback[2 + 4 * K + lane] = t | (a.predicted[lane] & 0xffffu);
+        }
+    }
+}
+
+int launch_router(const RouterArgs &a, uint32_t router_bits, hipStream_t s) {
+    const dim3 grid((a.sel.num_experts + 3) / 4), block(256);
+    if (router_bits == 0) hipLaunchKernelGGL((k_router<0>), grid, block, 0, s, a);
+    else if (router_bits == 8) hipLaunchKernelGGL((k_router<8>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((k_router<4>), grid, block, 0, s, a);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int RK, int BITS>
+static void launch_head_nch(const RouterArgs &r, const GemvArgs &g, uint32_t router_blocks, dim3 grid, hipStream_t s) {
+    const dim3 block(256);
+    switch (nch_for(g.n, BITS)) {
+        case 1: hipLaunchKernelGGL((k_head<RK, BITS, 1>), grid, block, 0, s, r, g, router_blocks); break;
+        case 2: hipLaunchKernelGGL((k_head<RK, BITS, 2>), grid, block, 0, s, r, g, router_blocks); break;
+        case 3: hipLaunchKernelGGL((k_head<RK, BITS, 3>), grid, block, 0, s, r, g, router_blocks); break;
+        default: hipLaunchKernelGGL((k_head<RK, BITS, 4>), grid, block, 0, s, r, g, router_blocks); break;
+    }
+}
+
+int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, hipStream_t s) {
+    const uint32_t router_blocks = (r.sel.num_experts + 3) / 4;
+    const dim3 grid(router_blocks + gemv_blocks(g.rows + g.rows_b, g.n, shared_bits));
+    if (shared_bits == 4) {
+        if (router_bits == 0) launch_head_nch<0, 4>(r, g, router_blocks, grid, s);
+        else if (router_bits == 8) launch_head_nch<8, 4>(r, g, router_blocks, grid, s);
+        else launch_head_nch<4, 4>(r, g, router_blocks, grid, s);
+    } else {
+        if (router_bits == 0) launch_head_nch<0, 8>(r, g, router_blocks, grid, s);
+        else if (router_bits == 8) launch_head_nch<8, 8>(r, g, router_blocks, grid, s);
+        else launch_head_nch<4, 8>(r, g, router_blocks, grid, s);
+    }
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int check_router(const shrike_hip_moe *moe, uint32_t num_experts, uint32_t d, uint32_t top_k) {
+    // MoE.swift:262-277
+    SHRIKE_REQUIRE(d % SHRIKE_GROUP_SIZE == 0, "encodeRouter: d=%u must be a multiple of %u", d, SHRIKE_GROUP_SIZE);
+    SHRIKE_REQUIRE(num_experts >= 1 && num_experts <= SHRIKE_MAX_ROUTER_EXPERTS, "encodeRouter: numExperts=%u not in 1...256", num_experts);
+    SHRIKE_REQUIRE(top_k >= 1 && top_k <= SHRIKE_MAX_TOP_K, "encodeRouter: topK=%u not in 1...8", top_k);
+    SHRIKE_REQUIRE(top_k <= num_experts, "encodeRouter: topK=%u exceeds numExperts=%u", top_k, num_experts);
+    const uint32_t bits = moe->desc.router_weight_bits;
+    const uint32_t chunks = bits == 0 ? d / 8u : d * bits / 128u;
+    SHRIKE_REQUIRE(chunks <= (bits == 0 ? 512u : 256u), "encodeRouter: d=%u is too long for the router kernel", d);
+    return 0;
+}
+
+}  // namespace shrike
+
+using namespace shrike;
+
+extern "C" {
+
+int shrike_hip_moe_router(shrike_hip_moe *moe, void *stream, const void *d_weights, const void *d_scales,
+                          const void *d_biases, const void *d_hidden, const void *d_effective_scale,
+                          const void *d_per_expert_scale, const void *d_logit_bias, uint32_t *d_out_indices,
+                          void *d_out_weights, uint32_t num_experts, uint32_t d, uint32_t top_k) {
+    SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
+    if (int rc = check_router(moe, num_experts, d, top_k)) return rc;
+    SHRIKE_REQUIRE(d_weights && d_hidden && d_effective_scale && d_per_expert_scale && d_logit_bias,
+                   "encodeRouter: weights, hidden, effectiveScale, perExpertScale and logitBias must all be bound");
+    SHRIKE_REQUIRE(moe->desc.router_weight_bits == 0 || (d_scales && d_biases), "encodeRouter: affine router needs scales and biases");
+    SHRIKE_REQUIRE(d_out_indices && d_out_weights, "encodeRouter: outputs must be bound");
+    RouterArgs a = {};
+    a.weights = d_weights;
+    a.scales = static_cast<const uint16_t *>(d_scales);
+    a.biases = static_cast<const uint16_t *>(d_biases);
+    a.hidden = static_cast<const uint16_t *>(d_hidden);
+    a.effective_scale = static_cast<const uint16_t *>(d_effective_scale);
+    a.d = d; a.meta = moe->desc.meta_dtype;
+    a.counter = moe->d_counter; a.logits_out = moe->d_logits;
+    a.sel.logits = moe->d_logits;
+    a.sel.per_expert_scale = static_cast<const uint16_t *>(d_per_expert_scale);
+    a.sel.logit_bias = static_cast<const uint16_t *>(d_logit_bias);
+    a.sel.num_experts = num_experts; a.sel.top_k = top_k;
+    a.sel.sigmoid = moe->desc.sigmoid_router_scores; a.sel.scaling = moe->desc.routed_scaling_factor;
+    a.lists.out_indices = d_out_indices;
+    a.lists.out_weights = static_cast<uint16_t *>(d_out_weights);
+    return launch_router(a, moe->desc.router_weight_bits, as_stream(stream));
+}
+
+const float *shrike_hip_moe_router_logits(const shrike_hip_moe *moe) { return moe ? moe->d_logits : nullptr; }
+
+int shrike_hip_moe_classify(shrike_hip_moe *moe, void *stream, const uint32_t *d_topk_indices,
+                            const uint64_t *d_residency, uint32_t *d_hit_count, uint32_t *d_hit_positions,
+                            uint32_t *d_miss_count, uint32_t *d_miss_positions, uint32_t *d_miss_experts,
+                            uint32_t *d_resolved_slots, uint32_t top_k, uint32_t num_experts,
+                            const uint32_t full_grids[12], uint32_t *d_spec_args, uint32_t *d_host_readback,
+                            uint32_t host_readback_tag, const void *d_topk_weights,
+                            const uint32_t *d_predicted_indices) {
+    SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
+    SHRIKE_REQUIRE(top_k >= 1 && top_k <= SHRIKE_MAX_TOP_K, "classify: topK=%u not in 1...8", top_k);  // MoE.swift:567
+    SHRIKE_REQUIRE(num_experts >= 1, "classify: numExperts must be positive");
+    SHRIKE_REQUIRE(d_topk_indices && d_residency && d_hit_count && d_hit_positions && d_miss_count
+                   && d_miss_positions && d_miss_experts && d_resolved_slots, "classify: every list must be bound");
+    SHRIKE_REQUIRE(host_readback_tag == 0 || (d_host_readback && d_topk_weights && d_predicted_indices),
+                   "classify: a tagged readback needs its buffer, the weights and the predicted ids");  // MoE.swift:569-575
+    SHRIKE_REQUIRE(host_readback_tag <= 0xffffu, "classify: the readback tag is 16 bits");
+    ClassifyArgs a = {};
+    a.topk = d_topk_indices; a.residency = d_residency;
+    a.hit_count = d_hit_count; a.hit_positions = d_hit_positions; a.miss_count = d_miss_count;
+    a.miss_positions = d_miss_positions; a.miss_experts = d_miss_experts; a.resolved_slots = d_resolved_slots;
+    a.top_k = top_k; a.num_experts = num_experts;
+    for (int i = 0; i < 12; ++i) a.full_grids[i] = full_grids ? full_grids[i] : 1u;
+    a.spec_args = d_spec_args; a.host_readback = d_host_readback; a.tag = host_readback_tag;
+    a.topk_weights = static_cast<const uint16_t *>(d_topk_weights); a.predicted = d_predicted_indices;
+    hipLaunchKernelGGL(k_classify, dim3(1), dim3(64), 0, as_stream(stream), a);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // extern "C"

@@ -56,6 +56,56 @@ __device__ __forceinline__ float wave_sum(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Wave-wide float max / unsigned min, broadcast to every lane. Rows a step does not
+// write keep their own value (old = self), so the partial results stay valid operands.
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_keep_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ uint32_t dpp_keep_u32(uint32_t v) {
+    return uint32_t(__builtin_amdgcn_update_dpp(int(v), int(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+    v = fmaxf(v, dpp_keep_f32<0xB1>(v));
+    v = fmaxf(v, dpp_keep_f32<0x4E>(v));
+    v = fmaxf(v, dpp_keep_f32<0x141>(v));
+    v = fmaxf(v, dpp_keep_f32<0x140>(v));
+    v = fmaxf(v, dpp_keep_f32<0x142, 0xA>(v));
+    v = fmaxf(v, dpp_keep_f32<0x143, 0xC>(v));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+// Written out in assembly so that each step is one DPP-fused max (rows a step's row mask
+// leaves out keep their value); a DPP read of a register needs two wait states after the
+// write before it.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_max_u32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_u32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_u32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_u32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_u32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(v));
+    return uint32_t(__builtin_amdgcn_readlane(int(v), 63));
+}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+    v = min(v, dpp_keep_u32<0xB1>(v));
+    v = min(v, dpp_keep_u32<0x4E>(v));
+    v = min(v, dpp_keep_u32<0x141>(v));
+    v = min(v, dpp_keep_u32<0x140>(v));
+    v = min(v, dpp_keep_u32<0x142, 0xA>(v));
+    v = min(v, dpp_keep_u32<0x143, 0xC>(v));
+    return uint32_t(__builtin_amdgcn_readlane(int(v), 63));
+}
+
 // Max of a 64-bit key over the wave; result broadcast to every lane.
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t key) {
     uint32_t lo = uint32_t(key), hi = uint32_t(key >> 32);

@@ -1,0 +1,430 @@
+// The group-affine matvec building blocks every decode kernel is made of.
+//
+// A row of codes is a run of 16-byte chunks; lane l of a 64-wide wave owns column
+// chunks l, l+64, ... of every row it touches, so its slice of the activation vector
+// sits in registers once (already in the pair layout the fp16 dot wants) and each row
+// costs one 128-bit load per chunk. The kernels are bound by memory latency and
+// bandwidth: all of a wave's row loads are issued before the first is consumed, and
+// out-of-range chunks are clamped to a valid address and zeroed rather than predicated,
+// so the loads stay back to back.
+#pragma once
+
+#include "device_utils.h"
+#include "host_common.h"
+
+namespace shrike {
+
+struct PoolArg {
+    const uint8_t *base[SHRIKE_POOL_MAX_CHUNKS];
+    uint32_t cells_per_chunk;
+};
+
+// moe.metal:302-305
+__device__ __forceinline__ const uint8_t *cell_base(const PoolArg &pool, uint32_t cell, uint64_t stride) {
+    return pool.base[cell / pool.cells_per_chunk] + uint64_t(cell % pool.cells_per_chunk) * stride;
+}
+
+__device__ __forceinline__ float meta_f32(uint16_t b, uint32_t meta) {
+    return meta == SHRIKE_META_F16 ? f16_to_f32(b) : bf16_to_f32(b);
+}
+
+// moe.metal:280-288; `act` is uniform, so this is one scalar branch
+__device__ __forceinline__ float glu_rt(float g, float u, uint32_t act) {
+    if (act == SHRIKE_ACT_SILU) return glu<1>(g, u);
+    if (act == SHRIKE_ACT_CLAMPED_SWIGLU) return glu<2>(g, u);
+    return glu<0>(g, u);
+}
+
+// moe.metal:36-39
+__device__ __forceinline__ bool io_ready(const uint32_t *io_status) {
+    if (!io_status) return true;
+    const uint32_t st = io_status[0];
+    return st == 1u || st == 3u;
+}
+
+template <int BITS> struct Chunk;
+template <> struct Chunk<4> {
+    static constexpr int E = 32, PIECES = 4;
+    typedef XChunk4 X;
+    static __device__ __forceinline__ void fill(X &x, int piece, const uint4 v) { pairs_from_x8(v, x.p + 4 * piece); }
+    static __device__ __forceinline__ float dot(const uint4 w, const X &x) { return dot_chunk4(w, x); }
+};
+template <> struct Chunk<8> {
+    static constexpr int E = 16, PIECES = 2;
+    typedef XChunk8 X;
+    static __device__ __forceinline__ void fill(X &x, int piece, const uint4 v) {
+        x.p[4 * piece + 0] = as_h2(v.x);
+        x.p[4 * piece + 1] = as_h2(v.y);
+        x.p[4 * piece + 2] = as_h2(v.z);
+        x.p[4 * piece + 3] = as_h2(v.w);
+    }
+    static __device__ __forceinline__ float dot(const uint4 w, const X &x) { return dot_chunk8(w, x); }
+};
+
+__device__ __forceinline__ uint4 zero4() { return make_uint4(0u, 0u, 0u, 0u); }
+
+// Raw 16-byte pieces of the lane's activation slices for column chunks col + 64*i.
+template <int BITS, int NCH>
+struct SliceRegs {
+    uint4 v[NCH][Chunk<BITS>::PIECES];
+};
+
+template <int BITS, int NCH>
+__device__ __forceinline__ void load_slice_regs(SliceRegs<BITS, NCH> &r, const uint4 *vec, uint32_t cpr,
+                                                uint32_t col, bool lane_on) {
+    typedef Chunk<BITS> C;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const uint32_t c = col + 64u * i;
+        const bool on = lane_on && c < cpr;
+        const uint32_t cc = on ? c : 0u;
+#pragma unroll
+        for (int j = 0; j < C::PIECES; ++j) {
+            uint4 v = vec[cc * C::PIECES + j];
+            if (!on) v = zero4();
+            r.v[i][j] = v;
+        }
+    }
+}
+
+// Pieces -> the dot's pair layout plus the fp32 sum of each slice (for the bias term).
+template <int BITS, int NCH>
+__device__ __forceinline__ void unpack_slices(const SliceRegs<BITS, NCH> &r, typename Chunk<BITS>::X (&x)[NCH],
+                                              float (&xs)[NCH]) {
+    typedef Chunk<BITS> C;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < C::PIECES; ++j) {
+            C::fill(x[i], j, r.v[i][j]);
+            s += sum_x8(r.v[i][j]);
+        }
+        xs[i] = s;
+    }
+}
+
+template <int BITS, int NCH>
+__device__ __forceinline__ void load_slices(const uint4 *vec, uint32_t cpr, uint32_t col, bool lane_on,
+                                            typename Chunk<BITS>::X (&x)[NCH], float (&xs)[NCH]) {
+    SliceRegs<BITS, NCH> r;
+    load_slice_regs<BITS, NCH>(r, vec, cpr, col, lane_on);
+    unpack_slices<BITS, NCH>(r, x, xs);
+}
+
+// One row's codes and metadata for the lane's column chunks.
+template <int BITS, int NCH>
+struct RowRegs {
+    uint4 w[NCH];
+    uint16_t s[NCH], b[NCH];
+};
+
+template <int BITS, int NCH>
+__device__ __forceinline__ void load_row(RowRegs<BITS, NCH> &r, const uint8_t *w_row, const uint16_t *s_row,
+                                         const uint16_t *b_row, uint32_t cpr, uint32_t col, bool lane_on) {
+    typedef Chunk<BITS> C;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const uint32_t c = col + 64u * i;
+        const bool on = lane_on && c < cpr;
+        const uint32_t cc = on ? c : 0u;
+        const uint32_t g = cc * C::E / kGroup;
+        uint4 w = *reinterpret_cast<const uint4 *>(w_row + 16u * cc);
+        uint16_t s = s_row[g], b = b_row[g];
+        if (!on) { w = zero4(); s = 0; b = 0; }
+        r.w[i] = w; r.s[i] = s; r.b[i] = b;
+    }
+}
+
+template <int BITS, int NCH>
+__device__ __forceinline__ float row_partial(const RowRegs<BITS, NCH> &r, const typename Chunk<BITS>::X (&x)[NCH],
+                                             const float (&xs)[NCH], uint32_t meta) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        acc = fmaf(meta_f32(r.s[i], meta), Chunk<BITS>::dot(r.w[i], x[i]), acc);
+        acc = fmaf(meta_f32(r.b[i], meta), xs[i], acc);
+    }
+    return acc;
+}
+
+// ------------------------------------------------- dense group-affine GEMV
+
+struct GemvArgs {
+    // two row sets of one shape over the same input (gate rows then up rows):
+    // dequant_int4.metal:206-235; set B unused when rows_b == 0.
+    const uint8_t *w_a; const uint16_t *s_a, *b_a; uint16_t *y_a;
+    const uint8_t *w_b; const uint16_t *s_b, *b_b; uint16_t *y_b;
+    uint32_t rows, rows_b, n, meta;
+    // input: x (fp16[n]) or, when gate_in != nullptr, act = half(glu(gate_in, up_in))
+    // computed on the fly (dequant_int4.metal:247-287).
+    const uint16_t *x, *gate_in, *up_in;
+    uint32_t act;
+    const uint16_t *scalar_gate;  // dequant_int4.metal:322-329
+};
+
+constexpr uint32_t kGemvRowsPerWave = 4;
+
+// dequant_int4.metal:101-199 / dequant_int8.metal:66-107: y[row] = half(W[row,:] . x), the
+// work of workgroup `block` of a grid of 256-thread workgroups.
+template <int BITS, int NCH>
+__device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block) {
+    typedef Chunk<BITS> C;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t cpr = a.n * BITS / 128u, groups = a.n / kGroup, row_bytes = cpr * 16u;
+    const bool packed = cpr < 64u && (64u % cpr) == 0u;
+    const uint32_t rpl = packed ? 64u / cpr : 1u;
+    const uint32_t seg = packed ? cpr : 64u;
+    const uint32_t sub = packed ? lane / cpr : 0u, col = packed ? lane % cpr : lane;
+    const uint32_t total = a.rows + a.rows_b;
+    const uint32_t first = (block * 4u + wave) * kGemvRowsPerWave * rpl;
+    const bool active = first < total;
+
+    // the input slice first: in-order load return must not hold it behind the rows
+    SliceRegs<BITS, NCH> xin;
+    if (!a.gate_in && active) load_slice_regs<BITS, NCH>(xin, reinterpret_cast<const uint4 *>(a.x), cpr, col, true);
+    uint16_t gate_bits = 0;
+    if (a.scalar_gate) gate_bits = a.scalar_gate[0];
+
+    RowRegs<BITS, NCH> rows[kGemvRowsPerWave];
+    uint32_t row[kGemvRowsPerWave];
+    bool on[kGemvRowsPerWave];
+    if (active) {
+#pragma unroll
+        for (uint32_t j = 0; j < kGemvRowsPerWave; ++j) {
+            row[j] = first + j * rpl + sub;
+            on[j] = row[j] < total;
+            const uint32_t rr = on[j] ? row[j] : 0u;
+            const bool second = rr >= a.rows;
+            const uint32_t local = second ? rr - a.rows : rr;
+            load_row<BITS, NCH>(rows[j], (second ? a.w_b : a.w_a) + size_t(local) * row_bytes,
+                                (second ? a.s_b : a.s_a) + size_t(local) * groups,
+                                (second ? a.b_b : a.b_a) + size_t(local) * groups, cpr, col, on[j]);
+        }
+    }
+    if (a.gate_in) {
+        // dequant_int4.metal:283-287: act = half(glu(gate, up)) once per workgroup, staged in LDS
+        __shared__ uint4 act_l[SHRIKE_MAX_HIDDEN / 8];
+        for (uint32_t p = threadIdx.x; p < a.n / 8u; p += 256u) {
+            const uint4 gv = reinterpret_cast<const uint4 *>(a.gate_in)[p];
+            const uint4 uv = reinterpret_cast<const uint4 *>(a.up_in)[p];
+            const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+            uint32_t o[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint16_t lo = f32_to_f16(glu_rt(f16_to_f32(uint16_t(gw[t])), f16_to_f32(uint16_t(uw[t])), a.act));
+                const uint16_t hi = f32_to_f16(glu_rt(f16_to_f32(uint16_t(gw[t] >> 16)), f16_to_f32(uint16_t(uw[t] >> 16)), a.act));
+                o[t] = uint32_t(lo) | (uint32_t(hi) << 16);
+            }
+            act_l[p] = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+        __syncthreads();
+        if (active) load_slice_regs<BITS, NCH>(xin, act_l, cpr, col, true);
+    }
+    if (!active) return;
+    typename C::X x[NCH];
+    float xs[NCH];
+    unpack_slices<BITS, NCH>(xin, x, xs);
+#pragma unroll
+    for (uint32_t j = 0; j < kGemvRowsPerWave; ++j) {
+        const float v = seg_sum(row_partial<BITS, NCH>(rows[j], x, xs, a.meta), seg);
+        if (on[j] && (lane % seg) == seg - 1u) {
+            const bool second = row[j] >= a.rows;
+            uint16_t yh = f32_to_f16(v);
+            if (a.scalar_gate) yh = f32_to_f16(f16_to_f32(yh) / (1.0f + expf(-f16_to_f32(gate_bits))));
+            (second ? a.y_b : a.y_a)[second ? row[j] - a.rows : row[j]] = yh;
+        }
+    }
+}
+
+inline uint32_t nch_for(uint32_t n, uint32_t bits) { return (n * bits / 128u + 63u) / 64u; }
+
+inline uint32_t gemv_blocks(uint32_t total_rows, uint32_t n, uint32_t bits) {
+    const uint32_t cpr = n * bits / 128u;
+    const uint32_t rpl = (cpr < 64u && 64u % cpr == 0u) ? 64u / cpr : 1u;
+    const uint32_t per_wave = kGemvRowsPerWave * rpl;
+    return ((total_rows + per_wave - 1) / per_wave + 3) / 4;
+}
+
+inline void fill_pool(PoolArg &p, const shrike_pool_bases *pool) {
+    for (uint32_t i = 0; i < SHRIKE_POOL_MAX_CHUNKS; ++i) p.base[i] = static_cast<const uint8_t *>(pool->base[i]);
+    p.cells_per_chunk = pool->cells_per_chunk ? pool->cells_per_chunk : 1u;
+}
+
+// ------------------------------------------------------------ routing
+
+struct SelectArgs {
+    const float *logits;
+    const uint16_t *per_expert_scale, *logit_bias;
+    uint32_t num_experts, top_k, sigmoid;
+    float scaling;
+};
+
+struct RouteLists {  // outputs of select + classify; residency == nullptr: select only
+    uint32_t *out_indices;
+    uint16_t *out_weights;
+    const uint64_t *residency;
+    uint32_t *hit_count, *hit_positions, *miss_count, *miss_positions, *miss_experts, *resolved_slots;
+};
+
+__device__ __forceinline__ float sigmoidf_(float v) { return 1.0f / (1.0f + expf(-v)); }
+template <bool COHERENT>
+__device__ __forceinline__ float load_logit(const float *p) {
+    return COHERENT ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *p;
+}
+
+// moe.metal:419-491 and :121-151, run by one wave. Lane l holds experts l, l+64, l+128,
+// l+192 with their bias, scale and residency word (all fetched up front, so nothing that
+// follows waits on memory). Each of the top_k rounds takes the wave-wide maximum score and,
+// among the experts that hold it, the lowest index (moe.metal:443-449); a NaN score is never
+// taken, and -inf scores are never taken either (the reference's slots start at -inf, index
+// 0). On return lane p < top_k holds position p's resolved cell (sentinel on a miss).
+// COHERENT reads the logits past the non-coherent caches (they were written by other
+// workgroups of the same launch); otherwise they come from an earlier launch.
+template <bool COHERENT>
+__device__ void route_wave(const SelectArgs &a, const RouteLists &out, uint32_t lane, bool write_lists,
+                           uint32_t &my_cell) {
+    // key = the score's bits mapped to an unsigned order (larger score, larger key); 0 marks
+    // what can never be taken: NaN, -inf and experts past num_experts
+    uint32_t key[4], cellv[4], gainv[4];
+    float raw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t e = lane + 64u * j;
+        const bool on = e < a.num_experts;
+        const uint32_t ee = on ? e : 0u;
+        raw[j] = load_logit<COHERENT>(a.logits + ee);
+        const float bias = bf16_to_f32(a.logit_bias[ee]);
+        gainv[j] = a.per_expert_scale[ee];
+        const uint64_t word = out.residency ? out.residency[ee] : 0;
+        // moe.metal:136-146: a hit names its cell, anything else is the sentinel
+        cellv[j] = (uint32_t(word >> 32) == SHRIKE_RESIDENCY_RESIDENT) ? uint32_t(word) : kSentinel;
+        float s = (a.sigmoid ? sigmoidf_(raw[j]) : raw[j]) + bias;
+        s = s + 0.0f;  // -0 and +0 tie
+        const uint32_t u = __float_as_uint(s);
+        const uint32_t ord = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+        key[j] = (on && s == s && s > -INFINITY) ? ord : 0u;
+    }
+    const uint32_t K = a.top_k;
+    // Every lane parks its four candidates in LDS; after the rounds lane p fetches position
+    // p's full key, gain, cell (and raw logit) by expert index with one read each.
+    __shared__ uint32_t s_key[256], s_gain[256], s_cellv[256];
+    __shared__ float s_raw[256];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        s_key[lane + 64u * j] = key[j];
+        s_gain[lane + 64u * j] = gainv[j];
+        s_cellv[lane + 64u * j] = cellv[j];
+        if (a.sigmoid) s_raw[lane + 64u * j] = raw[j];
+    }
+    // Fast rounds on a 32-bit composite key: the score key's upper 24 bits over 255 - index.
+    // One wave-wide max per round names the winner (higher score, lower index on equal
+    // scores). The composite order is the true order unless two candidates agree in those 24
+    // bits and differ below them; that is checked once after the rounds, and the exact rounds
+    // further down run instead if it can have mattered.
+    uint32_t ck[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ck[j] = key[j] ? ((key[j] & 0xffffff00u) | (255u - (lane + 64u * j))) : 0u;
+    uint32_t fast_top = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        if (uint32_t(r) < K) {
+            const uint32_t best = max(max(ck[0], ck[1]), max(ck[2], ck[3]));
+            const uint32_t top = wave_max_u32(best);  // 0: nothing left to take
+#pragma unroll
+            for (int j = 0; j < 4; ++j) ck[j] = ck[j] == top ? 0u : ck[j];
+            fast_top = lane == uint32_t(r) ? top : fast_top;
+        }
+    }
+    // The fast result is the true one when (a) the winners' prefixes fall strictly from rank
+    // to rank (equal prefixes are fine only for equal full keys, where the index decided), and
+    // (b) no candidate left behind shares the last winner's prefix with a different full key.
+    uint32_t mine = fast_top ? 255u - (fast_top & 255u) : 0u;
+    uint32_t my_key = fast_top ? s_key[mine] : 0u;
+    const uint32_t next_top = __shfl_down(fast_top, 1), next_key = __shfl_down(my_key, 1);
+    const bool pair_clash = lane + 1u < K && next_top != 0u && (fast_top >> 8) == (next_top >> 8) && my_key != next_key;
+    const uint32_t last_top = uint32_t(__builtin_amdgcn_readlane(int(fast_top), int(K) - 1));
+    const uint32_t last_key = uint32_t(__builtin_amdgcn_readlane(int(my_key), int(K) - 1));
+    bool left_clash = false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) left_clash |= ck[j] != 0u && last_top != 0u && (ck[j] >> 8) == (last_top >> 8) && key[j] != last_key;
+    if (__ballot(pair_clash || left_clash) != 0) {
+        // exact rounds: wave-wide max of the full key, then the lowest index among its holders
+        mine = 0; my_key = 0;
+#pragma unroll 1
+        for (uint32_t r = 0; r < K; ++r) {
+            uint32_t best = key[0], bj = 0;
+#pragma unroll
+            for (int j = 1; j < 4; ++j) {
+                const bool better = key[j] > best;  // strict: the lower index of equals stays
+                best = better ? key[j] : best;
+                bj = better ? uint32_t(j) : bj;
+            }
+            const uint32_t top = wave_max_u32(best);
+            uint32_t win = 0;
+            if (top != 0u) {
+                const bool holds = best == top;
+                win = wave_min_u32(holds ? lane + 64u * bj : 0xffffffffu);
+                const bool me = lane == (win & 63u);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) key[j] = (me && (win >> 6) == uint32_t(j)) ? 0u : key[j];
+            }
+            if (lane == r) { mine = win; my_key = top; }
+        }
+    }
+    const float my_score = my_key == 0u ? -INFINITY
+        : __uint_as_float((my_key & 0x80000000u) ? (my_key & 0x7fffffffu) : ~my_key);
+    const bool on = lane < K;
+    const float my_gain = bf16_to_f32(uint16_t(s_gain[mine]));
+    const uint32_t cell_of_mine = s_cellv[mine];
+    float weight;
+    if (a.sigmoid) {  // moe.metal:460-474
+        const float orig = on ? sigmoidf_(s_raw[mine]) : 0.0f;
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {  // rank order, as the reference adds them
+            const float o = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(orig), r));
+            if (uint32_t(r) < K) sum += o;
+        }
+        weight = orig * (a.scaling / (sum + 1e-20f));
+    } else {  // moe.metal:477-490
+        const float top = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_score), 0));
+        const float ex = on ? expf(my_score - top) : 0.0f;
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const float o = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ex), r));
+            if (uint32_t(r) < K) sum += o;
+        }
+        weight = ex / sum;
+    }
+    const uint16_t wbits = f32_to_f16(weight * my_gain);
+    if (write_lists && on) {
+        out.out_indices[lane] = mine;
+        out.out_weights[lane] = wbits;
+    }
+    my_cell = kSentinel;
+    if (!out.residency) return;
+    // moe.metal:121-151 (the select above never yields an index past num_experts - 1, so
+    // the reference's clamp is the identity here)
+    const bool hit = on && cell_of_mine != kSentinel;
+    if (hit) my_cell = cell_of_mine;
+    if (!write_lists) return;
+    const uint64_t hit_mask = __ballot(hit), miss_mask = __ballot(on && !hit);
+    const uint64_t below = (uint64_t(1) << lane) - 1u;
+    if (hit) {
+        out.hit_positions[__popcll(hit_mask & below)] = lane;
+        out.resolved_slots[lane] = cell_of_mine;
+    } else if (on) {
+        const uint32_t at = __popcll(miss_mask & below);
+        out.miss_positions[at] = lane;
+        out.miss_experts[at] = mine;
+        out.resolved_slots[lane] = kSentinel;
+    }
+    if (lane == 0) {
+        out.hit_count[0] = __popcll(hit_mask);
+        out.miss_count[0] = __popcll(miss_mask);
+    }
+}
+
+}  // namespace shrike
