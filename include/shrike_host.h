@@ -1,0 +1,216 @@
+/*
+ * libshrikehip, host side: the integer bookkeeping around the routed-expert path —
+ * token/expert pair records, the grouping permutation, the expert sweep order, the
+ * staging-wave planner and the slot cache. Plain C ABI, caller-owned memory, no
+ * device calls (the functions here run without a GPU); same conventions as
+ * shrike_hip.h. Where the reference throws a Swift error the call returns a
+ * nonzero code and shrike_hip_last_error() carries the reference's message.
+ */
+#ifndef SHRIKE_HOST_H
+#define SHRIKE_HOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------ pair records */
+
+/* PrefillTokenExpertPair, sources/Shrike/Kernels/Prefill/MoE/PrefillRouter.swift:5-28
+ * (16 bytes; the fp16 weight's bits sit in the low half of the fourth word). */
+typedef struct {
+    uint32_t token, expert, rank, weight_bits_and_reserved;
+} shrike_token_expert_pair;
+
+/* PrefillRouter.makeTokenExpertPairs, PrefillRouter.swift:160-180: token-major
+ * records from the router's [query_count * top_k] indices and fp16 weights. */
+int shrike_make_token_expert_pairs(const uint32_t *indices, const uint16_t *weights_f16,
+                                   uint32_t query_count, uint32_t top_k,
+                                   shrike_token_expert_pair *out_pairs);
+
+/* ---------------------------------------------------------------- grouping */
+
+/* PrefillMoEGroup / PrefillMoETile, PrefillMoEGrouping.swift:4-30. */
+typedef struct {
+    uint32_t expert, pair_start, pair_count;
+} shrike_moe_group;
+typedef struct {
+    uint32_t group_start, group_count, pair_start, pair_count;
+} shrike_moe_tile;
+
+/* PrefillMoEGroupingError, PrefillMoEGrouping.swift:52-89, in declaration order. */
+enum {
+    SHRIKE_GROUPING_OK = 0,
+    SHRIKE_GROUPING_INVALID_QUERY_COUNT = 1,
+    SHRIKE_GROUPING_INVALID_TOP_K = 2,
+    SHRIKE_GROUPING_INVALID_NUM_EXPERTS = 3,
+    SHRIKE_GROUPING_INVALID_TILE_EXPERT_COUNT = 4,
+    SHRIKE_GROUPING_PAIR_COUNT_MISMATCH = 5,
+    SHRIKE_GROUPING_TOKEN_OUT_OF_RANGE = 6,
+    SHRIKE_GROUPING_RANK_OUT_OF_RANGE = 7,
+    SHRIKE_GROUPING_EXPERT_OUT_OF_RANGE = 8,
+    SHRIKE_GROUPING_DUPLICATE_TOKEN_RANK = 9,
+    SHRIKE_GROUPING_EXPERT_SORT_KEY_COUNT_MISMATCH = 10
+};
+
+/* PrefillMoEGroupedRoutes, PrefillMoEGrouping.swift:32-50. The caller provides
+ * sorted_pairs[pair_count], per_expert_offsets[num_experts], per_expert_counts
+ * [num_experts], groups and tiles [min(num_experts, pair_count)]; the counts and
+ * maxima are written by the call. */
+typedef struct {
+    shrike_token_expert_pair *sorted_pairs;
+    uint32_t *per_expert_offsets; /* UINT32_MAX where the expert has no pair */
+    uint32_t *per_expert_counts;
+    shrike_moe_group *groups;
+    shrike_moe_tile *tiles;
+    uint32_t group_count, tile_count;
+    uint32_t max_pairs_per_expert, max_pairs_per_tile, max_live_experts_per_tile;
+    /* the two values of the reference's error case (0 where it has fewer) */
+    int64_t error_value[2];
+} shrike_grouped_routes;
+
+/* PrefillMoEGrouping.groupTokenExpertPairs, PrefillMoEGrouping.swift:269-370;
+ * called at RealForwardRunner.swift:4352. expert_sort_keys may be NULL (then
+ * sort_key_count is ignored). Returns a SHRIKE_GROUPING_* code. */
+int shrike_group_pairs(const shrike_token_expert_pair *pairs, size_t pair_count,
+                       int64_t query_count, int64_t top_k, int64_t num_experts,
+                       int64_t tile_expert_count, const uint64_t *expert_sort_keys,
+                       size_t sort_key_count, shrike_grouped_routes *out);
+
+/* -------------------------------------------------------------- sweep order */
+
+/* PrefillSweepOrder.residentFirstBalanced, PrefillMoEGrouping.swift:131-177. The
+ * chunk's routed experts come as parallel arrays (expert id, rows, last row; ids
+ * distinct); resident[e] != 0 marks an expert the pool holds (ids past
+ * resident_count count as absent). out_order has room for `count` ids. */
+int shrike_sweep_order_resident_first_balanced(const uint32_t *experts, const int64_t *rows,
+                                               const int64_t *last_row, size_t count,
+                                               const uint8_t *resident, size_t resident_count,
+                                               int64_t slots, int64_t tile_width,
+                                               uint32_t *out_order, size_t *out_count);
+
+/* PrefillSweepOrder.expertSortKeys, PrefillMoEGrouping.swift:196-202. */
+void shrike_expert_sort_keys(const uint32_t *order, size_t count, size_t num_experts,
+                             uint64_t *out_keys);
+
+/* -------------------------------------------------------------- wave planner */
+
+/* PrefillExpertPairRange, PrefillGroupedRoutedMoE.swift:33-43. */
+typedef struct {
+    uint32_t expert;
+    int64_t pair_start, pair_count;
+} shrike_expert_pair_range;
+
+/* PrefillRoutedExpertBlock, PrefillGroupedRoutedMoE.swift:71-77 (5 x u32, the
+ * layout the kernels read). */
+typedef struct {
+    uint32_t slot, pair_start, rows, staging_row, row_tile_start;
+} shrike_routed_expert_block;
+
+/* PrefillRoutedExpertWave, PrefillGroupedRoutedMoE.swift:83-89, with its blocks
+ * as a range of the flat block array. */
+typedef struct {
+    uint32_t block_start, block_count, padded_rows, tail_rows;
+} shrike_routed_expert_wave;
+
+/* PrefillGroupedRoutedMoE.planExpertWaves, PrefillGroupedRoutedMoE.swift:104-241;
+ * called at RealForwardRunner.swift:4910. An expert's slot is its position in
+ * bound_experts (PrefillStreamedTileBinding.localSlot). row_tile 64 (or 32 with
+ * tail_tile 0); tail_tile 0 or 32. EINVAL for what the reference throws
+ * (staging rows, unbound expert, tile combination), ENOSPC when blocks/waves
+ * are too small (the counts needed are still written). */
+int shrike_plan_expert_waves(const shrike_expert_pair_range *ranges, size_t range_count,
+                             const uint32_t *bound_experts, size_t bound_count,
+                             int64_t staging_rows, int64_t row_tile, int64_t tail_tile,
+                             shrike_routed_expert_block *blocks, size_t block_capacity,
+                             size_t *block_count, shrike_routed_expert_wave *waves,
+                             size_t wave_capacity, size_t *wave_count);
+
+/* rowTileTable, PrefillGroupedRoutedMoE.swift:272-283: table[t] = index (within the
+ * wave) of the block that owns row tile t; padded_rows / row_tile entries. */
+int shrike_row_tile_table(const shrike_routed_expert_block *blocks, size_t block_count,
+                          uint32_t padded_rows, uint32_t row_tile, uint32_t *table);
+
+/* rowTileTables, PrefillGroupedRoutedMoE.swift:247-269: gather (padded_rows / 32),
+ * body ((padded_rows - tail_rows) / 64) and tail (tail_rows / 32) tables. */
+int shrike_row_tile_tables(const shrike_routed_expert_block *blocks, size_t block_count,
+                           uint32_t padded_rows, uint32_t tail_rows, uint32_t *gather,
+                           uint32_t *body, uint32_t *tail);
+
+/* ---------------------------------------------------------------- slot cache */
+
+/* The slot bookkeeping of PreadExpertStreamer
+ * (sources/Shrike/Infrastructure/Streaming/PreadExpertStreamer.swift:405-543,
+ * :676-767, :1085-1148): hit lookup, victim choice, loading/resident states, cell
+ * generations, pins, statistics and the residency words. One lock guards it, as
+ * in the reference. Slot s is pool cell first_cell + s. */
+typedef struct shrike_slot_cache shrike_slot_cache;
+
+/* ExpertEvictionPolicy, sources/Shrike/Runtime/Inference/Model.swift:22-41. */
+enum { SHRIKE_EVICT_AGING_LFU = 0, SHRIKE_EVICT_SLRU = 1 };
+
+shrike_slot_cache *shrike_slot_cache_create(uint32_t slot_count, uint32_t experts_per_layer,
+                                            uint32_t first_cell, int policy,
+                                            double slru_protected_share, int *out_errno);
+void shrike_slot_cache_destroy(shrike_slot_cache *cache);
+
+/* ExpertCachePlan. Arrays are caller-provided with room for expert_count entries;
+ * experts is copied in by the plan call. */
+typedef struct {
+    uint32_t expert_count;
+    int32_t layer;
+    int32_t *experts;
+    int32_t *assigned_slots;
+    uint64_t *assigned_generations;
+    uint32_t *misses; /* indices into experts */
+    uint32_t miss_count;
+    uint32_t hits;
+} shrike_expert_cache_plan;
+
+/* makeExpertCachePlan, PreadExpertStreamer.swift:405-543 (planExpertsCached /
+ * planExpertsCachedIfPossible). avoiding_slots and protected_experts may be NULL;
+ * misses_counted < 0 counts the plan's own misses. Returns 0, ENOSPC when the
+ * experts cannot be placed (the reference's nil / expertCacheUnplaceable), EINVAL
+ * when expert_count exceeds the slot count. */
+int shrike_slot_cache_plan(shrike_slot_cache *cache, const int32_t *experts, uint32_t expert_count,
+                           int32_t layer, const int32_t *avoiding_slots, uint32_t avoiding_count,
+                           const uint8_t *protected_experts, uint32_t protected_count,
+                           int64_t misses_counted, shrike_expert_cache_plan *plan);
+/* markPlanMissesResident + the success leg of finishPlanExecution
+ * (PreadExpertStreamer.swift:1085-1105, :1070-1083): the plan's misses become
+ * resident and are counted as one load batch. EIO when a generation changed. */
+int shrike_slot_cache_complete(shrike_slot_cache *cache, const shrike_expert_cache_plan *plan,
+                               uint64_t elapsed_nanos, uint64_t fetch_nanos);
+/* abandonExpertCachePlan, PreadExpertStreamer.swift:1110-1128. */
+void shrike_slot_cache_abandon(shrike_slot_cache *cache, const shrike_expert_cache_plan *plan);
+/* pin / unpin, PreadExpertStreamer.swift:744-778. pin returns EIO on a stale plan. */
+int shrike_slot_cache_pin(shrike_slot_cache *cache, const shrike_expert_cache_plan *plan);
+void shrike_slot_cache_unpin(shrike_slot_cache *cache, const int32_t *slots,
+                             const uint64_t *generations, uint32_t count);
+
+/* ExpertStreamingStatistics, PreadExpertStreamer.swift:40-71 (the fields this
+ * library maintains). */
+typedef struct {
+    uint64_t plans, requested_experts, hits, misses, bytes_read, read_operations;
+    uint64_t evictions, reloads, load_batches, total_load_nanos, fetch_nanos, maximum_load_nanos;
+    uint64_t latency_histogram[17];
+    uint32_t resident_slots, loading_slots, pinned_slots, peak_loading_slots;
+} shrike_streaming_statistics;
+void shrike_slot_cache_statistics(shrike_slot_cache *cache, uint64_t expert_stride_bytes,
+                                  shrike_streaming_statistics *out);
+/* residentExperts, PreadExpertStreamer.swift:807-813: ascending ids; returns the count. */
+size_t shrike_slot_cache_resident_experts(shrike_slot_cache *cache, int32_t *out, size_t capacity);
+/* residencyEntry, PreadExpertStreamer.swift:663-670: state << 32 | cell. */
+uint64_t shrike_slot_cache_entry(shrike_slot_cache *cache, uint32_t expert);
+/* Entries whose word changed since the last drain, oldest first (an expert appears
+ * once, with its latest word): what a caller mirrors into the device table with
+ * shrike_hip_pool_table_publish. Returns the number written. */
+size_t shrike_slot_cache_drain_publications(shrike_slot_cache *cache, uint32_t *experts,
+                                            uint64_t *words, size_t capacity);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SHRIKE_HOST_H */

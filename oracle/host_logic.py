@@ -1,0 +1,684 @@
+"""CPU restatement of the reference's host-side integer logic around the routed-expert
+path. TEST INFRASTRUCTURE ONLY: imported by tests/ (and nothing in the product);
+the shipped implementation is the C++ in shrike_amd/csrc/host_logic.cpp and
+slot_cache.cpp, which the tests compare against these functions.
+
+Every function follows one reference function (cited in its docstring) and is pinned
+in tests/test_host_logic.py by the vectors the reference's own unit tests hold.
+All arithmetic here is integer; results are compared for equality.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+U32_MAX = 0xFFFFFFFF
+
+ALLOWED_SLOTS = [8, 16, 24, 32, 64, 96, 128, 160, 192, 224, 256]
+DEFAULT_BUDGET = 8 << 30
+
+
+# ----------------------------------------------------------------------- budget
+
+def parse_budget_bytes(text: str):
+    """RuntimeConfiguration.parseBudgetBytes,
+    sources/Shrike/Runtime/Configuration/RuntimeConfiguration.swift:111-129."""
+    raw = text.strip(" ").upper()
+    if not raw:
+        return None
+    for suffix, scale in (("GIB", 1 << 30), ("MIB", 1 << 20), ("KIB", 1 << 10), ("GB", 1 << 30),
+                          ("MB", 1 << 20), ("KB", 1 << 10), ("G", 1 << 30), ("M", 1 << 20), ("K", 1 << 10)):
+        if raw.endswith(suffix):
+            number = raw[: -len(suffix)].strip(" ")
+            value = _swift_double(number)
+            if value is None or not value > 0:
+                return None
+            b = value * scale
+            if b != b or b in (float("inf"), float("-inf")) or b < 1 or not b < float(2**63 - 1):
+                return None
+            return int(b)
+    if not _is_swift_int(raw):
+        return None
+    plain = int(raw)
+    if plain <= 0 or plain > 2**63 - 1:
+        return None
+    return plain
+
+
+def _is_swift_int(s: str) -> bool:
+    body = s[1:] if s[:1] in "+-" else s
+    return body.isascii() and body.isdigit()
+
+
+def _swift_double(s: str):
+    # Swift's Double(String) accepts what strtod accepts when the whole string is consumed
+    # and it holds no whitespace; "abc", "" and "2X" give nil.
+    if not s or any(c.isspace() for c in s):
+        return None
+    allowed = set("0123456789+-.EINFATYXP")
+    if any(c not in allowed for c in s.upper()):
+        return None
+    try:
+        return float.fromhex(s) if s.upper().lstrip("+-").startswith("0X") else float(s)
+    except ValueError:
+        return None
+
+
+def expert_cache_slots(expert_stride_bytes: int, layers: int, budget_bytes: int = DEFAULT_BUDGET) -> int:
+    """RuntimeConfiguration.expertCacheSlots, RuntimeConfiguration.swift:137-149: the allowed
+    count nearest to budget / (stride * layers); `min` keeps the first of equals."""
+    if expert_stride_bytes <= 0 or layers <= 0:
+        return ALLOWED_SLOTS[0]
+    wanted = float(budget_bytes) / (float(expert_stride_bytes) * float(layers))
+    best = ALLOWED_SLOTS[0]
+    for s in ALLOWED_SLOTS[1:]:
+        if abs(float(s) - wanted) < abs(float(best) - wanted):
+            best = s
+    return best
+
+
+# ------------------------------------------------------------- pairs and grouping
+
+@dataclass(frozen=True, order=False)
+class Pair:
+    """PrefillTokenExpertPair, sources/Shrike/Kernels/Prefill/MoE/PrefillRouter.swift:5-28."""
+    token: int
+    expert: int
+    rank: int
+    weight_bits: int
+
+    def as_tuple(self):
+        return (self.token, self.expert, self.rank, self.weight_bits)
+
+
+def make_token_expert_pairs(indices, weight_bits, query_count: int, top_k: int):
+    """PrefillRouter.makeTokenExpertPairs, PrefillRouter.swift:160-180 (token-major)."""
+    assert len(indices) == query_count * top_k and len(weight_bits) == query_count * top_k
+    return [Pair(t, int(indices[t * top_k + r]), r, int(weight_bits[t * top_k + r]))
+            for t in range(query_count) for r in range(top_k)]
+
+
+class GroupingError(Exception):
+    def __init__(self, case: str, *values):
+        super().__init__(case, *values)
+        self.case = case
+        self.values = values
+
+
+@dataclass
+class GroupedRoutes:
+    sorted_pairs: list
+    per_expert_offsets: list
+    per_expert_counts: list
+    groups: list  # (expert, pair_start, pair_count)
+    tiles: list   # (group_start, group_count, pair_start, pair_count)
+    query_count: int
+
+    @property
+    def max_pairs_per_expert(self):
+        return max((g[2] for g in self.groups), default=0)
+
+    @property
+    def max_pairs_per_tile(self):
+        return max((t[3] for t in self.tiles), default=0)
+
+    @property
+    def max_live_experts_per_tile(self):
+        return max((t[1] for t in self.tiles), default=0)
+
+
+def group_token_expert_pairs(pairs, query_count, top_k, num_experts, tile_expert_count=16,
+                             expert_sort_keys=None) -> GroupedRoutes:
+    """PrefillMoEGrouping.groupTokenExpertPairs,
+    sources/Shrike/Kernels/Prefill/MoE/PrefillMoEGrouping.swift:269-370: checks in the
+    reference's order, sort by (sort key, expert, token, rank), offsets (U32_MAX when absent),
+    counts, groups, tiles of at most tile_expert_count groups."""
+    if query_count < 0:
+        raise GroupingError("invalidQueryCount", query_count)
+    if top_k <= 0:
+        raise GroupingError("invalidTopK", top_k)
+    if num_experts <= 0:
+        raise GroupingError("invalidNumExperts", num_experts)
+    if not 1 <= tile_expert_count <= 16:
+        raise GroupingError("invalidTileExpertCount", tile_expert_count)
+    if expert_sort_keys is not None and len(expert_sort_keys) != num_experts:
+        raise GroupingError("expertSortKeyCountMismatch", num_experts, len(expert_sort_keys))
+    if len(pairs) != query_count * top_k:
+        raise GroupingError("pairCountMismatch", query_count * top_k, len(pairs))
+    seen = set()
+    for p in pairs:
+        if not p.token < query_count:
+            raise GroupingError("tokenOutOfRange", p.token)
+        if not p.rank < top_k:
+            raise GroupingError("rankOutOfRange", p.rank)
+        if not p.expert < num_experts:
+            raise GroupingError("expertOutOfRange", p.expert)
+        if (p.token, p.rank) in seen:
+            raise GroupingError("duplicateTokenRank", p.token, p.rank)
+        seen.add((p.token, p.rank))
+
+    def key(p):
+        lead = (expert_sort_keys[p.expert],) if expert_sort_keys is not None else ()
+        return lead + (p.expert, p.token, p.rank)
+
+    s = sorted(pairs, key=key)  # (token, rank) is unique, so the order is total
+    offsets = [U32_MAX] * num_experts
+    counts = [0] * num_experts
+    groups = []
+    i = 0
+    while i < len(s):
+        e, start = s[i].expert, i
+        while i < len(s) and s[i].expert == e:
+            i += 1
+        offsets[e], counts[e] = start, i - start
+        groups.append((e, start, i - start))
+    tiles = []
+    g = 0
+    while g < len(groups):
+        end = min(len(groups), g + tile_expert_count)
+        first, last = groups[g], groups[end - 1]
+        tiles.append((g, end - g, first[1], last[1] + last[2] - first[1]))
+        g = end
+    return GroupedRoutes(s, offsets, counts, groups, tiles, query_count)
+
+
+# ---------------------------------------------------------------------- sweep order
+
+HEAD_FACTOR = 6      # PrefillMoEGrouping.swift:96
+FALLBACK_TAIL = 96   # PrefillMoEGrouping.swift:101
+
+
+def _ranked(rows, last_row):
+    """PrefillSweepOrder.residentFirstRanked, PrefillMoEGrouping.swift:107-119."""
+    return sorted(last_row.keys(), key=lambda e: (last_row.get(e, 0), rows.get(e, 0), e))
+
+
+def _heaviest_first(experts, rows):
+    return sorted(experts, key=lambda e: (-rows.get(e, 0), e))
+
+
+def _pack_by_rows(experts, rows, tile_width):
+    """packByRows, PrefillMoEGrouping.swift:203-226: heaviest first into the lightest bin
+    that still has room, ties to the lower bin."""
+    if not experts:
+        return []
+    n = (len(experts) + tile_width - 1) // tile_width
+    totals, bins = [0] * n, [[] for _ in range(n)]
+    for e in _heaviest_first(experts, rows):
+        best, best_total = -1, None
+        for i in range(n):
+            if len(bins[i]) < tile_width and (best_total is None or totals[i] < best_total):
+                best, best_total = i, totals[i]
+        if best < 0:
+            break
+        bins[best].append(e)
+        totals[best] += rows.get(e, 0)
+    return [e for b in bins for e in b]
+
+
+def _pack_by_rows_into(experts, preseeded, rows, tile_width):
+    """packByRows(_:into:), PrefillMoEGrouping.swift:234-261."""
+    bins = [list(b) for b in preseeded]
+    weights = [sum(rows.get(e, 0) for e in b) for b in bins]
+    for e in _heaviest_first(experts, rows):
+        best, best_w = -1, None
+        for i in range(len(bins)):
+            if len(bins[i]) < tile_width and (best_w is None or weights[i] < best_w):
+                best, best_w = i, weights[i]
+        if best < 0:
+            break
+        bins[best].append(e)
+        weights[best] += rows.get(e, 0)
+    return bins
+
+
+def _fallback_order(resident_group, absent_group, rows, tile_width):
+    """residentFirstFallbackOrder, PrefillMoEGrouping.swift:179-190."""
+    tail = min(FALLBACK_TAIL, len(absent_group))
+    head = len(absent_group) - tail
+    return (_pack_by_rows(resident_group, rows, tile_width)
+            + _pack_by_rows(absent_group[:head], rows, tile_width)
+            + _pack_by_rows(absent_group[head:], rows, tile_width))
+
+
+def resident_first_balanced(rows: dict, last_row: dict, resident, slots: int, tile_width: int):
+    """PrefillSweepOrder.residentFirstBalanced, PrefillMoEGrouping.swift:131-177."""
+    ranked = _ranked(rows, last_row)
+    res = [e for e in ranked if e < len(resident) and resident[e]]
+    absent = [e for e in ranked if not (e < len(resident) and resident[e])]
+    if not res or not absent:
+        return _fallback_order(res, absent, rows, tile_width)
+    tile_count = (len(res) + len(absent) + tile_width - 1) // tile_width
+    head = 0
+    while head < tile_count:
+        remaining = tile_count - head
+        mixed_misses = (len(absent) + remaining - 1) // remaining
+        if len(res) - tile_width * head <= slots - HEAD_FACTOR * mixed_misses:
+            break
+        head += 1
+    head_res, rest_res = res[: tile_width * head], res[tile_width * head:]
+    mixed = tile_count - head
+    if mixed <= 0:
+        return _fallback_order(res, absent, rows, tile_width)
+    bins = []
+    for t in range(mixed):
+        lo, hi = (t * len(absent)) // mixed, ((t + 1) * len(absent)) // mixed
+        bins.append(absent[lo:hi] if lo < hi else [])
+    filled = _pack_by_rows_into(rest_res, bins, rows, tile_width)
+    return head_res + [e for b in filled for e in b]
+
+
+def expert_sort_keys(order, num_experts: int):
+    """PrefillSweepOrder.expertSortKeys, PrefillMoEGrouping.swift:196-202."""
+    keys = [len(order)] * num_experts
+    for rank, e in enumerate(order):
+        if e < num_experts:
+            keys[e] = rank
+    return keys
+
+
+# --------------------------------------------------------------------- wave planner
+
+ROW_TILE = 64   # MPPPrefillInt4QMM.tileM
+TAIL_TILE = 32
+
+
+class PlanError(Exception):
+    pass
+
+
+@dataclass
+class Wave:
+    blocks: list  # (slot, pair_start, rows, staging_row, row_tile_start)
+    padded_rows: int
+    tail_rows: int = 0
+
+    @property
+    def body_padded_rows(self):
+        return self.padded_rows - self.tail_rows
+
+
+def plan_expert_waves(ranges, bound_experts, staging_rows, row_tile=ROW_TILE, tail_tile=0):
+    """PrefillGroupedRoutedMoE.planExpertWaves,
+    sources/Shrike/Kernels/Prefill/MoE/PrefillGroupedRoutedMoE.swift:104-150 (and the tail
+    variant :160-241). `ranges` are (expert, pair_start, pair_count); an expert's local slot
+    is its position in `bound_experts`."""
+    slot_of = {}
+    for i, e in enumerate(bound_experts):
+        slot_of.setdefault(e, i)
+    if tail_tile != 0:
+        if row_tile != ROW_TILE:
+            raise PlanError("a tail tile packs 64-row bodies")
+        return _plan_with_tail(ranges, slot_of, staging_rows, tail_tile)
+    tile = row_tile
+    if not (staging_rows >= tile and staging_rows % tile == 0):
+        raise PlanError("stagingTooSmall")
+    waves, blocks, cursor = [], [], 0
+
+    def close():
+        nonlocal blocks, cursor
+        if blocks:
+            waves.append(Wave(blocks, cursor))
+            blocks, cursor = [], 0
+
+    for expert, pair_start, pair_count in ranges:
+        if pair_count <= 0:
+            continue
+        if expert not in slot_of:
+            raise PlanError("expert %d is not bound in the tile" % expert)
+        consumed = 0
+        while consumed < pair_count:
+            if cursor == staging_rows:
+                close()
+            rows = min(pair_count - consumed, staging_rows - cursor)
+            blocks.append((slot_of[expert], pair_start + consumed, rows, cursor, cursor // tile))
+            cursor += (rows + tile - 1) // tile * tile
+            consumed += rows
+    close()
+    return waves
+
+
+def _plan_with_tail(ranges, slot_of, staging_rows, tail_tile):
+    body = ROW_TILE
+    if tail_tile != TAIL_TILE:
+        raise PlanError("tail tile is not 32")
+    if not (staging_rows >= body and staging_rows % body == 0):
+        raise PlanError("stagingTooSmall")
+    waves, body_pieces, tail_pieces = [], [], []
+    used = 0
+
+    def close():
+        nonlocal body_pieces, tail_pieces, used
+        if not body_pieces and not tail_pieces:
+            return
+        blocks, cursor = [], 0
+        for slot, ps, rows in body_pieces:
+            blocks.append((slot, ps, rows, cursor, cursor // body))
+            cursor += (rows + body - 1) // body * body
+        body_padded = cursor
+        for i, (slot, ps, rows) in enumerate(tail_pieces):
+            blocks.append((slot, ps, rows, cursor, i))
+            cursor += tail_tile
+        waves.append(Wave(blocks, cursor, cursor - body_padded))
+        body_pieces, tail_pieces, used = [], [], 0
+
+    def padded_cost(rows):
+        rem = rows % body
+        return rows - rem + (0 if rem == 0 else tail_tile if rem <= tail_tile else body)
+
+    def place(slot, ps, rows):
+        nonlocal used
+        rem = rows % body
+        body_rows = rows if rem > tail_tile else rows - rem
+        if body_rows > 0:
+            body_pieces.append((slot, ps, body_rows))
+        if 0 < rem <= tail_tile:
+            tail_pieces.append((slot, ps + body_rows, rem))
+        used += padded_cost(rows)
+
+    for expert, pair_start, pair_count in ranges:
+        if pair_count <= 0:
+            continue
+        if expert not in slot_of:
+            raise PlanError("expert %d is not bound in the tile" % expert)
+        consumed = 0
+        while consumed < pair_count:
+            remaining = pair_count - consumed
+            available = staging_rows - used
+            if used + padded_cost(remaining) <= staging_rows:
+                place(slot_of[expert], pair_start + consumed, remaining)
+                consumed += remaining
+                continue
+            cut = available // body * body + (tail_tile if available % body >= tail_tile else 0)
+            if cut > 0:
+                place(slot_of[expert], pair_start + consumed, cut)
+                consumed += cut
+            close()
+    close()
+    return waves
+
+
+def row_tile_table(wave: Wave, row_tile=ROW_TILE):
+    """rowTileTable, PrefillGroupedRoutedMoE.swift:272-283."""
+    table = [0] * (wave.padded_rows // row_tile)
+    for i, b in enumerate(wave.blocks):
+        first, count = b[4], (b[2] + row_tile - 1) // row_tile
+        for t in range(first, first + count):
+            table[t] = i
+    return table
+
+
+def row_tile_tables(wave: Wave):
+    """rowTileTables, PrefillGroupedRoutedMoE.swift:247-269: (gather, body, tail)."""
+    body, tail = ROW_TILE, TAIL_TILE
+    gather = [0] * (wave.padded_rows // tail)
+    body_t = [0] * (wave.body_padded_rows // body)
+    tail_t = [0] * (wave.tail_rows // tail)
+    for i, b in enumerate(wave.blocks):
+        start = b[3]
+        is_tail = start >= wave.body_padded_rows
+        padded = tail if is_tail else (b[2] + body - 1) // body * body
+        for row in range(start, start + padded, tail):
+            gather[row // tail] = i
+        if is_tail:
+            tail_t[b[4]] = i
+        else:
+            for t in range(start // body, (start + padded) // body):
+                body_t[t] = i
+    return gather, body_t, tail_t
+
+
+# ----------------------------------------------------------------------- slot pool
+
+EMPTY, LOADING, RESIDENT = 0, 1, 2
+
+
+def residency_word(state: int, cell: int) -> int:
+    """ExpertResidencyEntry as the 64-bit word the kernels read,
+    sources/Shrike/Infrastructure/Streaming/ExpertResidencyTable.swift:4-18 and the publish
+    rule of PreadExpertStreamer.swift:1143-1148 (an empty entry names the sentinel cell)."""
+    slot = U32_MAX if state == EMPTY else cell & U32_MAX
+    return (state << 32) | slot
+
+
+@dataclass
+class CachePlan:
+    experts: list
+    assigned_slots: list
+    assigned_generations: list
+    misses: list  # indices into experts
+    hits: int
+    layer: int = 0
+
+
+@dataclass
+class SlotCache:
+    """The slot bookkeeping of PreadExpertStreamer (PreadExpertStreamer.swift:405-543,
+    :676-767, :1085-1148) without the file reads: hits, victim choice (aging LFU then LRU, or
+    SLRU), loading/resident states, per-cell generations, pins, statistics and the residency
+    words. Landings, the prefetch ring and overflow slots are not modelled."""
+    slot_count: int
+    experts_per_layer: int
+    first_cell: int = 0
+    slru_share: float | None = None  # None = aging LFU
+
+    def __post_init__(self):
+        n, e = self.slot_count, max(1, self.experts_per_layer)
+        self.slot_expert = [-1] * n
+        self.slot_last_use = [0] * n
+        self.slot_state = [EMPTY] * n
+        self.slot_pins = [0] * n
+        self.slot_protected = [False] * n
+        self.protected_count = 0
+        # ExpertEvictionPolicy.protectedCapacity, Model.swift:26-33 (rounds half away from zero)
+        self.protected_capacity = 0 if self.slru_share is None else max(1, int(self.slru_share * n + 0.5))
+        self.use_count = [0] * e
+        self.load_count = [0] * e
+        self.generation = [0] * n
+        self.generation_clock = 0  # ExpertCellArena.bumpCellGeneration, ExpertCellArena.swift:99-104
+        self.use_clock = 0
+        self.words = [residency_word(EMPTY, 0)] * self.experts_per_layer
+        self.stats = dict(plans=0, requested=0, hits=0, misses=0, evictions=0, reloads=0,
+                          read_operations=0, load_batches=0, peak_loading=0)
+
+    def cell(self, slot):
+        return self.first_cell + slot
+
+    def _publish(self, expert, cell, state):
+        if 0 <= expert < self.experts_per_layer:
+            self.words[expert] = residency_word(state, cell)
+
+    def _should_evict(self, lhs, rhs):
+        """shouldEvictSlot, PreadExpertStreamer.swift:728-742."""
+        le, re = self.slot_expert[lhs], self.slot_expert[rhs]
+        if le < 0 or re < 0:
+            return le < re
+        if self.slru_share is not None:
+            if self.slot_protected[lhs] != self.slot_protected[rhs]:
+                return not self.slot_protected[lhs]
+            return self.slot_last_use[lhs] < self.slot_last_use[rhs]
+        lc = self.use_count[le] if le < len(self.use_count) else 0
+        rc = self.use_count[re] if re < len(self.use_count) else 0
+        if lc != rc:
+            return lc < rc
+        return self.slot_last_use[lhs] < self.slot_last_use[rhs]
+
+    def _select_victims(self, miss_count, reserved, protected=None):
+        """selectVictimSlots, PreadExpertStreamer.swift:676-705."""
+        victims, eligible = [], 0
+        for slot in range(self.slot_count):
+            if reserved[slot] or self.slot_state[slot] == LOADING or self.slot_pins[slot] != 0:
+                continue
+            e = self.slot_expert[slot]
+            if protected is not None and 0 <= e < len(protected) and protected[e]:
+                continue
+            eligible += 1
+            if len(victims) < miss_count:
+                at = len(victims)
+                victims.append(slot)
+                while at > 0 and self._should_evict(slot, victims[at - 1]):
+                    victims[at] = victims[at - 1]
+                    at -= 1
+                victims[at] = slot
+            elif victims and self._should_evict(slot, victims[-1]):
+                at = len(victims) - 1
+                while at > 0 and self._should_evict(slot, victims[at - 1]):
+                    victims[at] = victims[at - 1]
+                    at -= 1
+                victims[at] = slot
+        return victims if miss_count <= eligible else None
+
+    def _promote(self, slot, clock):
+        """promoteToProtected, PreadExpertStreamer.swift:708-720."""
+        self.slot_protected[slot] = True
+        self.protected_count += 1
+        if self.protected_count <= self.protected_capacity:
+            return
+        oldest = -1
+        for c in range(self.slot_count):
+            if self.slot_protected[c] and c != slot:
+                if oldest < 0 or self.slot_last_use[c] < self.slot_last_use[oldest]:
+                    oldest = c
+        if oldest < 0:
+            return
+        self.slot_protected[oldest] = False
+        self.protected_count -= 1
+        self.slot_last_use[oldest] = clock
+
+    def plan(self, experts, layer=0, avoiding_slots=(), protected_experts=None, misses_counted=None):
+        """makeExpertCachePlan, PreadExpertStreamer.swift:405-543; None when unplaceable."""
+        assert len(experts) <= self.slot_count
+        avoiding = {s for s in avoiding_slots if 0 <= s < self.slot_count}
+        reserved = [False] * self.slot_count
+        clock = self.use_clock + 1
+        if self.stats["plans"] > 0 and self.stats["plans"] % 1024 == 0:
+            self.use_count = [c >> 1 for c in self.use_count]
+        for s in range(self.slot_count):
+            if self.slot_state[s] == LOADING:
+                reserved[s] = True
+        assigned = [-1] * len(experts)
+        miss_count = 0
+        for i, e in enumerate(experts):
+            for s in range(self.slot_count):
+                if not reserved[s] and self.slot_state[s] == RESIDENT and self.slot_expert[s] == e:
+                    assigned[i] = s
+                    reserved[s] = True
+                    break
+            if assigned[i] == -1:
+                miss_count += 1
+        for s in avoiding:
+            reserved[s] = True
+        victims = []
+        if miss_count > 0:
+            victims = self._select_victims(miss_count, reserved, protected_experts) if protected_experts is not None else None
+            if victims is None:
+                victims = self._select_victims(miss_count, reserved)
+                if victims is None:
+                    return None
+        self.use_clock = clock
+        for e in experts:
+            if 0 <= e < len(self.use_count):
+                self.use_count[e] += 1
+        for s in assigned:
+            if s >= 0:
+                self.slot_last_use[s] = clock
+        if self.slru_share is not None:
+            for s in assigned:
+                if s >= 0 and not self.slot_protected[s]:
+                    self._promote(s, clock)
+        misses, v = [], 0
+        for i, e in enumerate(experts):
+            if assigned[i] != -1:
+                continue
+            slot = victims[v]
+            v += 1
+            if self.slot_state[slot] == RESIDENT:
+                self.stats["evictions"] += 1
+            previous = self.slot_expert[slot]
+            assigned[i] = slot
+            reserved[slot] = True
+            if self.slot_protected[slot]:
+                self.slot_protected[slot] = False
+                self.protected_count -= 1
+            self.generation_clock += 1
+            self.generation[slot] = self.generation_clock
+            if previous >= 0:
+                self._publish(previous, self.cell(slot), EMPTY)
+            self.slot_expert[slot] = e
+            self.slot_last_use[slot] = clock
+            self.slot_state[slot] = LOADING
+            self._publish(e, self.cell(slot), LOADING)
+            misses.append(i)
+        counted = len(misses) if misses_counted is None else misses_counted
+        self.stats["plans"] += 1
+        self.stats["requested"] += len(experts)
+        self.stats["hits"] += len(experts) - counted
+        self.stats["misses"] += counted
+        self.stats["peak_loading"] = max(self.stats["peak_loading"], self.slot_state.count(LOADING))
+        return CachePlan(list(experts), assigned, [self.generation[s] for s in assigned], misses,
+                         len(experts) - len(misses), layer)
+
+    def complete(self, plan: CachePlan):
+        """markPlanMissesResident + the success leg of finishPlanExecution,
+        PreadExpertStreamer.swift:1085-1105, :1070-1083, :1150-1179."""
+        for i in plan.misses:
+            if self.generation[plan.assigned_slots[i]] != plan.assigned_generations[i]:
+                raise RuntimeError("expert-cache cell generation changed during expert load")
+        for i in plan.misses:
+            s = plan.assigned_slots[i]
+            self.slot_state[s] = RESIDENT
+            self.slot_expert[s] = plan.experts[i]
+            self.slot_last_use[s] = self.use_clock
+            self._publish(plan.experts[i], self.cell(s), RESIDENT)
+        if plan.misses:
+            self.stats["read_operations"] += len(plan.misses)
+            self.stats["load_batches"] += 1
+            for i in plan.misses:
+                e = plan.experts[i]
+                if 0 <= e < len(self.load_count):
+                    if self.load_count[e] > 0:
+                        self.stats["reloads"] += 1
+                    self.load_count[e] += 1
+
+    def abandon(self, plan: CachePlan):
+        """abandonExpertCachePlan / resetLoadingMissesUnlocked, PreadExpertStreamer.swift:1110-1128."""
+        for i in plan.misses:
+            s = plan.assigned_slots[i]
+            if not (0 <= s < self.slot_count and self.generation[s] == plan.assigned_generations[i]
+                    and self.slot_state[s] == LOADING):
+                continue
+            self.slot_state[s] = EMPTY
+            self.slot_expert[s] = -1
+            self._publish(plan.experts[i], self.cell(s), EMPTY)
+
+    def load(self, experts, **kw):
+        """loadExpertsCached, PreadExpertStreamer.swift:355-358."""
+        p = self.plan(experts, **kw)
+        if p is None:
+            raise RuntimeError("unplaceable")
+        self.complete(p)
+        return p
+
+    def pin(self, plan: CachePlan):
+        """pin, PreadExpertStreamer.swift:744-767; raises on a stale plan."""
+        for i, e in enumerate(plan.experts):
+            s = plan.assigned_slots[i]
+            if not (0 <= s < self.slot_count and self.generation[s] == plan.assigned_generations[i]
+                    and self.slot_expert[s] == e and self.slot_state[s] != EMPTY):
+                raise RuntimeError("expert-cache plan became stale before GPU pin")
+        for s in plan.assigned_slots:
+            self.slot_pins[s] += 1
+
+    def unpin(self, slots, generations):
+        """unpin, PreadExpertStreamer.swift:769-778."""
+        for s, g in zip(slots, generations):
+            if 0 <= s < self.slot_count and self.generation[s] == g:
+                assert self.slot_pins[s] > 0
+                self.slot_pins[s] -= 1
+
+    def resident_experts(self):
+        """residentExperts, PreadExpertStreamer.swift:807-813."""
+        return sorted(e for e, st in zip(self.slot_expert, self.slot_state) if st == RESIDENT and e >= 0)
+
+    def counts(self):
+        return dict(resident=self.slot_state.count(RESIDENT), loading=self.slot_state.count(LOADING),
+                    pinned=sum(1 for p in self.slot_pins if p > 0))

@@ -65,6 +65,54 @@ class DecodeLayerArgs(C.Structure):
 
 # name -> (restype, argtypes); every symbol include/shrike_hip.h declares
 _VP, _U32, _U64, _I32, _I64 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_int32, C.c_int64
+# ---- include/shrike_host.h ----------------------------------------------------------
+
+class TokenExpertPair(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("token", "expert", "rank", "weight_bits_and_reserved")]
+
+
+class MoEGroup(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("expert", "pair_start", "pair_count")]
+
+
+class MoETile(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("group_start", "group_count", "pair_start", "pair_count")]
+
+
+class GroupedRoutes(C.Structure):
+    _fields_ = [("sorted_pairs", C.POINTER(TokenExpertPair)), ("per_expert_offsets", C.POINTER(C.c_uint32)),
+                ("per_expert_counts", C.POINTER(C.c_uint32)), ("groups", C.POINTER(MoEGroup)),
+                ("tiles", C.POINTER(MoETile)), ("group_count", C.c_uint32), ("tile_count", C.c_uint32),
+                ("max_pairs_per_expert", C.c_uint32), ("max_pairs_per_tile", C.c_uint32),
+                ("max_live_experts_per_tile", C.c_uint32), ("error_value", C.c_int64 * 2)]
+
+
+class ExpertPairRange(C.Structure):
+    _fields_ = [("expert", C.c_uint32), ("pair_start", C.c_int64), ("pair_count", C.c_int64)]
+
+
+class RoutedExpertBlock(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("slot", "pair_start", "rows", "staging_row", "row_tile_start")]
+
+
+class RoutedExpertWave(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("block_start", "block_count", "padded_rows", "tail_rows")]
+
+
+class ExpertCachePlan(C.Structure):
+    _fields_ = [("expert_count", C.c_uint32), ("layer", C.c_int32), ("experts", C.POINTER(C.c_int32)),
+                ("assigned_slots", C.POINTER(C.c_int32)), ("assigned_generations", C.POINTER(C.c_uint64)),
+                ("misses", C.POINTER(C.c_uint32)), ("miss_count", C.c_uint32), ("hits", C.c_uint32)]
+
+
+class StreamingStatistics(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in (
+        "plans", "requested_experts", "hits", "misses", "bytes_read", "read_operations", "evictions",
+        "reloads", "load_batches", "total_load_nanos", "fetch_nanos", "maximum_load_nanos")] + [
+        ("latency_histogram", C.c_uint64 * 17)] + [(n, C.c_uint32) for n in (
+            "resident_slots", "loading_slots", "pinned_slots", "peak_loading_slots")]
+
+
 SIGNATURES = {
     "shrike_hip_last_error": (C.c_char_p, []),
     "shrike_hip_init": (C.c_int, [C.c_int]),
@@ -121,6 +169,29 @@ SIGNATURES = {
     "shrike_hip_graph_end_capture": (_VP, [_VP]),
     "shrike_hip_graph_launch": (C.c_int, [_VP, _VP]),
     "shrike_hip_graph_destroy": (C.c_int, [_VP]),
+    # include/shrike_host.h
+    "shrike_make_token_expert_pairs": (C.c_int, [_VP, _VP, _U32, _U32, C.POINTER(TokenExpertPair)]),
+    "shrike_group_pairs": (C.c_int, [C.POINTER(TokenExpertPair), C.c_size_t, _I64, _I64, _I64, _I64, _VP,
+                                     C.c_size_t, C.POINTER(GroupedRoutes)]),
+    "shrike_sweep_order_resident_first_balanced": (C.c_int, [_VP, _VP, _VP, C.c_size_t, _VP, C.c_size_t, _I64, _I64,
+                                                             _VP, C.POINTER(C.c_size_t)]),
+    "shrike_expert_sort_keys": (None, [_VP, C.c_size_t, C.c_size_t, _VP]),
+    "shrike_plan_expert_waves": (C.c_int, [C.POINTER(ExpertPairRange), C.c_size_t, _VP, C.c_size_t, _I64, _I64, _I64,
+                                           C.POINTER(RoutedExpertBlock), C.c_size_t, C.POINTER(C.c_size_t),
+                                           C.POINTER(RoutedExpertWave), C.c_size_t, C.POINTER(C.c_size_t)]),
+    "shrike_row_tile_table": (C.c_int, [C.POINTER(RoutedExpertBlock), C.c_size_t, _U32, _U32, _VP]),
+    "shrike_row_tile_tables": (C.c_int, [C.POINTER(RoutedExpertBlock), C.c_size_t, _U32, _U32, _VP, _VP, _VP]),
+    "shrike_slot_cache_create": (_VP, [_U32, _U32, _U32, C.c_int, C.c_double, C.POINTER(C.c_int)]),
+    "shrike_slot_cache_destroy": (None, [_VP]),
+    "shrike_slot_cache_plan": (C.c_int, [_VP, _VP, _U32, _I32, _VP, _U32, _VP, _U32, _I64, C.POINTER(ExpertCachePlan)]),
+    "shrike_slot_cache_complete": (C.c_int, [_VP, C.POINTER(ExpertCachePlan), _U64, _U64]),
+    "shrike_slot_cache_abandon": (None, [_VP, C.POINTER(ExpertCachePlan)]),
+    "shrike_slot_cache_pin": (C.c_int, [_VP, C.POINTER(ExpertCachePlan)]),
+    "shrike_slot_cache_unpin": (None, [_VP, _VP, _VP, _U32]),
+    "shrike_slot_cache_statistics": (None, [_VP, _U64, C.POINTER(StreamingStatistics)]),
+    "shrike_slot_cache_resident_experts": (C.c_size_t, [_VP, _VP, C.c_size_t]),
+    "shrike_slot_cache_entry": (_U64, [_VP, _U32]),
+    "shrike_slot_cache_drain_publications": (C.c_size_t, [_VP, _VP, _VP, C.c_size_t]),
 }
 
 _lib = None

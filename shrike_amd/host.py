@@ -1,0 +1,267 @@
+"""Host-side mirror of the reference's prefill bookkeeping and slot cache over the C ABI
+(include/shrike_host.h). Names follow the reference's Swift types; every function calls
+into libshrikehip.so — nothing here computes a result in Python."""
+from __future__ import annotations
+
+import ctypes as C
+import errno
+
+import numpy as np
+
+from . import capi
+from .capi import ShrikeError
+
+PAIR_DTYPE = np.dtype([("token", "<u4"), ("expert", "<u4"), ("rank", "<u4"), ("weight_bits", "<u4")])
+GROUP_DTYPE = np.dtype([("expert", "<u4"), ("pair_start", "<u4"), ("pair_count", "<u4")])
+TILE_DTYPE = np.dtype([("group_start", "<u4"), ("group_count", "<u4"), ("pair_start", "<u4"), ("pair_count", "<u4")])
+BLOCK_DTYPE = np.dtype([("slot", "<u4"), ("pair_start", "<u4"), ("rows", "<u4"), ("staging_row", "<u4"),
+                        ("row_tile_start", "<u4")])
+WAVE_DTYPE = np.dtype([("block_start", "<u4"), ("block_count", "<u4"), ("padded_rows", "<u4"), ("tail_rows", "<u4")])
+
+GROUPING_ERRORS = {
+    1: "invalidQueryCount", 2: "invalidTopK", 3: "invalidNumExperts", 4: "invalidTileExpertCount",
+    5: "pairCountMismatch", 6: "tokenOutOfRange", 7: "rankOutOfRange", 8: "expertOutOfRange",
+    9: "duplicateTokenRank", 10: "expertSortKeyCountMismatch",
+}
+_ERROR_ARITY = {5: 2, 9: 2, 10: 2}
+
+
+def _vp(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _as(a, struct):
+    return a.ctypes.data_as(C.POINTER(struct))
+
+
+class GroupingError(ShrikeError):
+    """PrefillMoEGroupingError (PrefillMoEGrouping.swift:52-89): `case` names the Swift case,
+    `values` its associated values."""
+
+    def __init__(self, code, values, message):
+        super().__init__(message)
+        self.code, self.case = code, GROUPING_ERRORS.get(code, "invalidArgument")
+        self.values = tuple(values[: _ERROR_ARITY.get(code, 1)])
+
+
+class GroupedRoutes:
+    """PrefillMoEGroupedRoutes (PrefillMoEGrouping.swift:32-50) as numpy arrays."""
+
+    def __init__(self, sorted_pairs, offsets, counts, groups, tiles, maxima, query_count):
+        self.sorted_pairs, self.per_expert_offsets, self.per_expert_counts = sorted_pairs, offsets, counts
+        self.groups, self.tiles, self.query_count = groups, tiles, query_count
+        self.max_pairs_per_expert, self.max_pairs_per_tile, self.max_live_experts_per_tile = maxima
+
+
+def make_token_expert_pairs(indices, weights_f16_bits, query_count: int, top_k: int) -> np.ndarray:
+    """PrefillRouter.makeTokenExpertPairs (PrefillRouter.swift:160-180)."""
+    idx = np.ascontiguousarray(indices, dtype=np.uint32)
+    w = np.ascontiguousarray(weights_f16_bits, dtype=np.uint16)
+    if idx.size != query_count * top_k or w.size != query_count * top_k:
+        raise ShrikeError("indices/weights count mismatch")  # the reference's precondition
+    out = np.zeros(query_count * top_k, dtype=PAIR_DTYPE)
+    capi.check(capi.load().shrike_make_token_expert_pairs(_vp(idx), _vp(w), query_count, top_k,
+                                                          _as(out, capi.TokenExpertPair)), "makeTokenExpertPairs")
+    return out
+
+
+def group_token_expert_pairs(pairs: np.ndarray, query_count: int, top_k: int, num_experts: int,
+                             tile_expert_count: int = 16, expert_sort_keys=None) -> GroupedRoutes:
+    """PrefillMoEGrouping.groupTokenExpertPairs (PrefillMoEGrouping.swift:269-370)."""
+    pairs = np.ascontiguousarray(pairs, dtype=PAIR_DTYPE)
+    n, e = pairs.size, max(int(num_experts), 0)
+    cap = max(1, min(e, n))
+    sorted_pairs = np.zeros(max(n, 1), dtype=PAIR_DTYPE)
+    offsets, counts = np.zeros(max(e, 1), np.uint32), np.zeros(max(e, 1), np.uint32)
+    groups, tiles = np.zeros(cap, GROUP_DTYPE), np.zeros(cap, TILE_DTYPE)
+    out = capi.GroupedRoutes(_as(sorted_pairs, capi.TokenExpertPair), _as(offsets, C.c_uint32), _as(counts, C.c_uint32),
+                             _as(groups, capi.MoEGroup), _as(tiles, capi.MoETile))
+    keys = None if expert_sort_keys is None else np.ascontiguousarray(expert_sort_keys, dtype=np.uint64)
+    rc = capi.load().shrike_group_pairs(_as(pairs, capi.TokenExpertPair), n, query_count, top_k, num_experts,
+                                        tile_expert_count, _vp(keys), 0 if keys is None else keys.size, C.byref(out))
+    if rc != 0:
+        raise GroupingError(rc, list(out.error_value), capi.last_error())
+    return GroupedRoutes(sorted_pairs[:n], offsets[:e], counts[:e], groups[: out.group_count], tiles[: out.tile_count],
+                         (out.max_pairs_per_expert, out.max_pairs_per_tile, out.max_live_experts_per_tile), query_count)
+
+
+def resident_first_balanced(rows_by_expert: dict, last_row_by_expert: dict, resident, slots: int,
+                            tile_width: int) -> list:
+    """PrefillSweepOrder.residentFirstBalanced (PrefillMoEGrouping.swift:131-177)."""
+    experts = np.array(list(last_row_by_expert.keys()), dtype=np.uint32)
+    rows = np.array([rows_by_expert.get(int(e), 0) for e in experts], dtype=np.int64)
+    last = np.array([last_row_by_expert[int(e)] for e in experts], dtype=np.int64)
+    res = np.ascontiguousarray(np.asarray(resident, dtype=np.uint8))
+    out = np.zeros(max(1, experts.size), np.uint32)
+    count = C.c_size_t(0)
+    capi.check(capi.load().shrike_sweep_order_resident_first_balanced(
+        _vp(experts), _vp(rows), _vp(last), experts.size, _vp(res), res.size, slots, tile_width, _vp(out),
+        C.byref(count)), "residentFirstBalanced")
+    return out[: count.value].tolist()
+
+
+def expert_sort_keys(order, num_experts: int) -> np.ndarray:
+    """PrefillSweepOrder.expertSortKeys (PrefillMoEGrouping.swift:196-202)."""
+    o = np.ascontiguousarray(order, dtype=np.uint32)
+    keys = np.zeros(max(1, num_experts), np.uint64)
+    capi.load().shrike_expert_sort_keys(_vp(o), o.size, num_experts, _vp(keys))
+    return keys[:num_experts]
+
+
+class PlanError(ShrikeError):
+    pass
+
+
+def plan_expert_waves(ranges, bound_experts, staging_rows: int, row_tile: int = 64, tail_tile: int = 0):
+    """PrefillGroupedRoutedMoE.planExpertWaves (PrefillGroupedRoutedMoE.swift:104-241).
+    `ranges`: (expert, pair_start, pair_count). Returns (blocks, waves) structured arrays."""
+    r = (capi.ExpertPairRange * max(1, len(ranges)))(*[capi.ExpertPairRange(*x) for x in ranges])
+    bound = np.ascontiguousarray(bound_experts, dtype=np.uint32)
+    lib = capi.load()
+    cap_b, cap_w = 64, 16
+    while True:
+        blocks, waves = np.zeros(cap_b, BLOCK_DTYPE), np.zeros(cap_w, WAVE_DTYPE)
+        nb, nw = C.c_size_t(0), C.c_size_t(0)
+        rc = lib.shrike_plan_expert_waves(r, len(ranges), _vp(bound), bound.size, staging_rows, row_tile, tail_tile,
+                                          _as(blocks, capi.RoutedExpertBlock), cap_b, C.byref(nb),
+                                          _as(waves, capi.RoutedExpertWave), cap_w, C.byref(nw))
+        if rc == errno.ENOSPC:
+            cap_b, cap_w = max(cap_b, nb.value), max(cap_w, nw.value)
+            continue
+        if rc != 0:
+            raise PlanError(capi.last_error())
+        return blocks[: nb.value], waves[: nw.value]
+
+
+def row_tile_table(blocks: np.ndarray, wave, row_tile: int = 64) -> list:
+    """rowTileTable (PrefillGroupedRoutedMoE.swift:272-283) for one wave of `blocks`."""
+    b = np.ascontiguousarray(blocks[int(wave["block_start"]): int(wave["block_start"]) + int(wave["block_count"])])
+    table = np.zeros(max(1, int(wave["padded_rows"]) // row_tile), np.uint32)
+    capi.check(capi.load().shrike_row_tile_table(_as(b, capi.RoutedExpertBlock), b.size, int(wave["padded_rows"]),
+                                                 row_tile, _vp(table)), "rowTileTable")
+    return table[: int(wave["padded_rows"]) // row_tile].tolist()
+
+
+def row_tile_tables(blocks: np.ndarray, wave):
+    """rowTileTables (PrefillGroupedRoutedMoE.swift:247-269): (gather, body, tail)."""
+    b = np.ascontiguousarray(blocks[int(wave["block_start"]): int(wave["block_start"]) + int(wave["block_count"])])
+    padded, tail_rows = int(wave["padded_rows"]), int(wave["tail_rows"])
+    ng, nb, nt = padded // 32, (padded - tail_rows) // 64, tail_rows // 32
+    g, bo, t = (np.zeros(max(1, n), np.uint32) for n in (ng, nb, nt))
+    capi.check(capi.load().shrike_row_tile_tables(_as(b, capi.RoutedExpertBlock), b.size, padded, tail_rows,
+                                                  _vp(g), _vp(bo), _vp(t)), "rowTileTables")
+    return g[:ng].tolist(), bo[:nb].tolist(), t[:nt].tolist()
+
+
+class CachePlan:
+    """ExpertCachePlan (PreadExpertStreamer.swift:17-38)."""
+
+    def __init__(self, n: int):
+        self.experts_a = np.zeros(max(1, n), np.int32)
+        self.slots_a = np.zeros(max(1, n), np.int32)
+        self.gens_a = np.zeros(max(1, n), np.uint64)
+        self.misses_a = np.zeros(max(1, n), np.uint32)
+        self.c = capi.ExpertCachePlan(0, 0, _as(self.experts_a, C.c_int32), _as(self.slots_a, C.c_int32),
+                                      _as(self.gens_a, C.c_uint64), _as(self.misses_a, C.c_uint32), 0, 0)
+
+    @property
+    def experts(self):
+        return self.experts_a[: self.c.expert_count].tolist()
+
+    @property
+    def assigned_slots(self):
+        return self.slots_a[: self.c.expert_count].tolist()
+
+    @property
+    def assigned_generations(self):
+        return self.gens_a[: self.c.expert_count].tolist()
+
+    @property
+    def misses(self):
+        return self.misses_a[: self.c.miss_count].tolist()
+
+    @property
+    def hits(self):
+        return self.c.hits
+
+    @property
+    def layer(self):
+        return self.c.layer
+
+
+class SlotCache:
+    """The slot bookkeeping of PreadExpertStreamer (PreadExpertStreamer.swift:405-543, :676-767)."""
+
+    def __init__(self, slot_count: int, experts_per_layer: int, first_cell: int = 0, slru_share=None):
+        err = C.c_int(0)
+        self.slot_count, self.experts_per_layer = slot_count, experts_per_layer
+        self._h = capi.load().shrike_slot_cache_create(slot_count, experts_per_layer, first_cell,
+                                                       0 if slru_share is None else 1,
+                                                       0.0 if slru_share is None else float(slru_share), C.byref(err))
+        if not self._h:
+            raise ShrikeError(f"slot cache: {capi.last_error()}")
+
+    def close(self):
+        if self._h:
+            capi.load().shrike_slot_cache_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def plan(self, experts, layer=0, avoiding_slots=(), protected_experts=None, misses_counted=None):
+        """planExpertsCachedIfPossible: None when the experts cannot be placed."""
+        e = np.ascontiguousarray(experts, dtype=np.int32)
+        avoid = np.ascontiguousarray(sorted(avoiding_slots), dtype=np.int32)
+        prot = None if protected_experts is None else np.ascontiguousarray(np.asarray(protected_experts, dtype=np.uint8))
+        plan = CachePlan(e.size)
+        rc = capi.load().shrike_slot_cache_plan(self._h, _vp(e), e.size, layer, _vp(avoid) if avoid.size else None,
+                                                avoid.size, _vp(prot), 0 if prot is None else prot.size,
+                                                -1 if misses_counted is None else misses_counted, C.byref(plan.c))
+        if rc == errno.ENOSPC:
+            return None
+        capi.check(rc, "planExpertsCached")
+        return plan
+
+    def complete(self, plan: CachePlan, elapsed_nanos: int = 0, fetch_nanos: int = 0):
+        capi.check(capi.load().shrike_slot_cache_complete(self._h, C.byref(plan.c), elapsed_nanos, fetch_nanos),
+                   "markPlanMissesResident")
+
+    def abandon(self, plan: CachePlan):
+        capi.load().shrike_slot_cache_abandon(self._h, C.byref(plan.c))
+
+    def load(self, experts, **kw):
+        """loadExpertsCached without the reads: plan, then mark the misses resident."""
+        plan = self.plan(experts, **kw)
+        if plan is None:
+            raise ShrikeError(capi.last_error())  # ModelError.expertCacheUnplaceable
+        self.complete(plan)
+        return plan
+
+    def pin(self, plan: CachePlan):
+        capi.check(capi.load().shrike_slot_cache_pin(self._h, C.byref(plan.c)), "pin")
+
+    def unpin(self, slots, generations):
+        s, g = np.ascontiguousarray(slots, np.int32), np.ascontiguousarray(generations, np.uint64)
+        capi.load().shrike_slot_cache_unpin(self._h, _vp(s), _vp(g), s.size)
+
+    def statistics(self, expert_stride_bytes: int = 0) -> capi.StreamingStatistics:
+        st = capi.StreamingStatistics()
+        capi.load().shrike_slot_cache_statistics(self._h, expert_stride_bytes, C.byref(st))
+        return st
+
+    def resident_experts(self) -> list:
+        out = np.zeros(max(1, self.slot_count), np.int32)
+        n = capi.load().shrike_slot_cache_resident_experts(self._h, _vp(out), out.size)
+        return out[:n].tolist()
+
+    def entry(self, expert: int) -> int:
+        return int(capi.load().shrike_slot_cache_entry(self._h, expert))
+
+    def drain_publications(self):
+        e, w = np.zeros(max(1, self.experts_per_layer), np.uint32), np.zeros(max(1, self.experts_per_layer), np.uint64)
+        n = capi.load().shrike_slot_cache_drain_publications(self._h, _vp(e), _vp(w), e.size)
+        return list(zip(e[:n].tolist(), w[:n].tolist()))
