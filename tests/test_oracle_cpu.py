@@ -1,0 +1,309 @@
+"""The arithmetic oracle (oracle/shrike_oracle.c) against what pins it without a GPU: the
+reference's own C kernel compiled in place (oracle/_ref, when it was built), the reference
+tests' known answers, closed forms, and fp64 / brute-force restatements written here from the
+format's definition rather than from the oracle's code."""
+import math
+import os
+
+import numpy as np
+import pytest
+
+from oracle import host_logic as H
+from oracle import oracle as O
+from shrike_amd import synth as S
+
+
+def f16(bits):
+    return np.asarray(bits, np.uint16).view(np.float16).astype(np.float32)
+
+
+# ------------------------------------------------------------------------------ conversions
+
+def test_conversions_exhaustive_against_numpy():
+    L = O.lib()
+    for h in range(0, 65536, 1):
+        v = np.uint16(h).view(np.float16)
+        got = L.orc_f16_to_f32(h)
+        if np.isnan(v):
+            assert math.isnan(got)
+        else:
+            assert got == float(v)
+    rng = np.random.default_rng(1)
+    xs = np.concatenate([rng.standard_normal(20000).astype(np.float32) * 10.0 ** rng.integers(-8, 6, 20000),
+                         np.array([0.0, -0.0, 65504.0, 65520.0, 65519.99, 5.96e-8, 2.98e-8, 2.9802325e-8, 1e-10,
+                                   np.inf, -np.inf], np.float32)]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want16 = xs.astype(np.float16).view(np.uint16)
+    for x, w16 in zip(xs, want16):
+        assert L.orc_f32_to_f16(float(x)) == int(w16), x
+    # bf16: round to nearest even on the upper 16 bits (Quantization.swift:17-28)
+    for x in xs:
+        u = int(np.float32(x).view(np.uint32))
+        want = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF
+        assert L.orc_f32_to_bf16(float(x)) == want
+        assert L.orc_bf16_to_f32(want) == float(np.uint32(want << 16).view(np.float32))
+
+
+# ---------------------------------------------------------------------------- blob layout
+
+def test_offsets_known_answers():  # CPUExpertFFNTests.swift:56-67, ExpertCacheBudgetTests.swift:16-18
+    o, stride = O.expert_offsets(2048, 512, 4)
+    assert stride == 1_769_472
+    assert (o.gate_w, o.gate_s, o.up_w, o.down_w) == (0, 524_288, 589_824, 1_179_648)
+    t = o.as_tuple()[:9]
+    assert list(t) == sorted(t)
+    assert O.expert_offsets(2048, 512, 8)[1] == 3_342_336
+    assert O.expert_offsets(2880, 2880, 4)[1] == 13_996_800
+    assert O.expert_offsets(2880, 2880, 8)[1] == 26_438_400
+    assert O.expert_offsets(2880, 2880, 8, additive_biases=True)[1] == 26_438_400 + 17_280
+    assert O.expert_offsets(2304, 1024, 8)[1] == 7_520_256
+    so, sstride = S.expert_offsets(2048, 512, 4)
+    assert sstride == stride and tuple(so[n] for n, _ in O.Offsets._fields_) == o.as_tuple()
+
+
+# --------------------------------------------------------------------------- affine GEMV
+
+def brute_gemv(w, s, b, x, rows, n, bits, meta):
+    """w = q * scale + bias per element, in fp64, from the format's definition."""
+    out = np.zeros(rows, np.float64)
+    w, s, b = (np.ascontiguousarray(a).reshape(-1) for a in (w, s, b))
+    sf, bf = S.meta_to_f32(s, meta).astype(np.float64), S.meta_to_f32(b, meta).astype(np.float64)
+    for r in range(rows):
+        row = w[r * n * bits // 8:(r + 1) * n * bits // 8]
+        q = np.stack([row & 0xF, row >> 4], axis=1).reshape(-1) if bits == 4 else row
+        g = np.arange(n) // 64
+        out[r] = np.sum((q.astype(np.float64) * sf[r * (n // 64) + g] + bf[r * (n // 64) + g]) * x.astype(np.float64))
+    return out
+
+
+@pytest.mark.parametrize("rows,n", [(128, 64), (64, 512), (32, 2880)])
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("meta", [S.META_BF16, S.META_F16])
+def test_gemv_against_brute_force(rows, n, bits, meta):
+    rng = S.SeedTree(0x5EED0001).key(f"gemv.{rows}.{n}.{bits}.{meta}")
+    w, s, b = S.affine_matrix(rng, rows, n, bits, meta)
+    x = rng.normal(n).astype(np.float32)
+    ref = brute_gemv(w, s, b, x, rows, n, bits, meta)
+    got = O.affine_gemv(w, s, b, x, rows, n, bits, meta)
+    got64 = O.affine_gemv_f64(w, s, b, x, rows, n, bits, meta)
+    scale = np.abs(ref).max()
+    assert np.abs(got64 - ref).max() <= 1e-9 * scale
+    assert np.abs(got - ref).max() <= 1e-5 * scale  # DequantInt4GEMVReferenceTests.swift:32-53
+    if bits == 4:
+        assert np.array_equal(O.int4_affine_gemv(w, s, b, x, rows, n, meta), got)
+
+
+@pytest.mark.skipif(O.ref_lib() is None, reason="oracle/_ref was not built (no reference checkout at build time)")
+@pytest.mark.parametrize("rows,n", [(2048, 512), (512, 2048), (128, 64), (2880, 2880), (1024, 2304)])
+def test_int4_gemv_bit_equal_to_the_reference_c(rows, n):
+    rng = S.SeedTree(0x5EED0001).key(f"ref.{rows}.{n}")
+    w, s, b = S.affine_matrix(rng, rows, n, 4, S.META_BF16)
+    x = rng.normal(n).astype(np.float32)
+    ours = O.int4_affine_gemv(w, s, b, x, rows, n, S.META_BF16)
+    theirs = O.ref_int4_affine_gemv(w, s, b, x, rows, n)
+    assert ours.view(np.uint32).tolist() == theirs.view(np.uint32).tolist()
+
+
+def test_nibble_layout_low_even_high_odd():  # QuantizationTests.swift:36-50
+    row = (np.arange(64, dtype=np.float32) - 31.5)[None, :]
+    w, s, b = (a.reshape(-1) for a in S.quantize_affine(row, 4))
+    lo, hi = int(w[0] & 0xF), int(w[0] >> 4)
+    sc, bi = float(S.bf16_bits_to_f32(s)[0]), float(S.bf16_bits_to_f32(b)[0])
+    assert abs(lo * sc + bi - row[0, 0]) <= sc + 1e-3 and abs(hi * sc + bi - row[0, 1]) <= sc + 1e-3
+    e = np.zeros(64, np.float32)
+    e[1] = 1.0  # picks element 1: the high nibble of byte 0
+    assert abs(O.affine_gemv(w, s, b, e, 1, 64, 4)[0] - (hi * sc + bi)) < 1e-6
+
+
+def test_quantiser_round_trip_bound():  # QuantizationTests.swift:8-34
+    rng = S.SeedTree(0x51A71001).key("int4-affine-round-trip")
+    row = rng.uniform(-1.0, 1.0, 256).astype(np.float32)[None, :]
+    w, s, b = (a.reshape(-1) for a in S.quantize_affine(row, 4))
+    q = np.stack([w & 0xF, w >> 4], axis=1).reshape(-1).astype(np.float32)
+    rec = q * np.repeat(S.bf16_bits_to_f32(s), 64) + np.repeat(S.bf16_bits_to_f32(b), 64)
+    for g in range(4):
+        seg = slice(64 * g, 64 * g + 64)
+        assert np.all(np.abs(rec[seg] - row[0, seg]) <= np.abs(row[0, seg]).max() / 7.0 + 1e-3)
+
+
+# --------------------------------------------------------------------------- expert FFN
+
+def closed_form_blob(d, f, meta=S.META_BF16):
+    """q = 0, scale = 0, gate bias 1/64... (MoEFusedFFNTests.swift:17-55): every weight equals its
+    group's bias, so gate = D/64 * 1/64 * ... reduces to sums of ones."""
+    o, stride = O.expert_offsets(d, f, 4)
+    blob = np.zeros(stride, np.uint8)
+
+    def put(off, rows, n, value):
+        vals = np.full(rows * (n // 64), value, np.float32)
+        blob[off:off + vals.size * 2] = S.meta_bits(vals, meta).view(np.uint8)
+    put(o.gate_b, f, d, 1.0 / 64)
+    put(o.up_b, f, d, 0.5 / 64)
+    put(o.down_b, d, f, 1.0 / 64)
+    return blob, o
+
+
+def test_ffn_closed_form():  # MoEFusedFFNTests.swift:868-900: D=128, F=64, 8 experts x 0.125 -> 2/(1+e^-2)
+    d, f = 128, 64
+    blob, o = closed_form_blob(d, f)
+    x = S.f32_to_f16_bits(np.ones(d, np.float32))
+    acts = O.moe_phase1([blob] * 8, o, x, d, f)
+    # gate = 128/64 = 2, up = 1, act = silu(2) * 1
+    assert np.allclose(f16(acts), 2.0 / (1.0 + math.exp(-2.0)), atol=1e-3)
+    w = S.f32_to_f16_bits(np.full(8, 0.125, np.float32))
+    zero = S.f32_to_f16_bits(np.zeros(d, np.float32))
+    hidden = zero.copy()
+    y = O.moe_phase2([blob] * 8, o, acts, w, zero, d, f, hidden_f16=hidden)
+    # down = sum_f act / 64 = act
+    assert np.allclose(f16(y), 2.0 / (1.0 + math.exp(-2.0)), atol=1e-2)
+    assert np.array_equal(hidden, y)
+
+
+def test_cpu_ffn_matches_fp64_chain_and_accumulates():  # CPUExpertFFNTests.swift:69-152
+    d, f = 256, 128
+    tree = S.SeedTree(0x5EED0001)
+    blob = S.expert_blob(tree, "cpu.ffn", d, f, 4)
+    o, _ = O.expert_offsets(d, f, 4)
+    v = S.blob_views(blob, d, f, 4)
+    x = tree.key("cpu.x").normal(d).astype(np.float32)
+    gate = brute_gemv(*v["gate"], x, f, d, 4, S.META_BF16)
+    up = brute_gemv(*v["up"], x, f, d, 4, S.META_BF16)
+    act = gate / (1.0 + np.exp(-gate)) * up
+    down = brute_gemv(*v["down"], act.astype(np.float32), d, f, 4, S.META_BF16)
+    out = np.zeros(d, np.float32)
+    O.cpu_expert_ffn_accumulate(blob, o, x, d, f, 0.75, out)
+    assert np.abs(out - 0.75 * down).max() <= 2e-4 * max(1.0, np.abs(down).max())
+    once = out.copy()
+    O.cpu_expert_ffn_accumulate(blob, o, x, d, f, 0.75, out)
+    assert np.allclose(out, 2 * once, rtol=1e-6, atol=1e-6)
+
+
+def test_glu_variants():  # moe.metal:98-105, :257-288
+    L = O.lib()
+    g, u = 0.7, -1.3
+    assert abs(L.orc_glu(g, u, O.ACT_SILU) - g / (1 + math.exp(-g)) * u) < 1e-6
+    gelu = 0.5 * g * (1 + math.tanh(0.7978845608 * (g + 0.044715 * g ** 3)))
+    assert abs(L.orc_glu(g, u, O.ACT_GELU_TANH) - gelu * u) < 1e-6
+    # gpt-oss: gate clamped above at 7, up to [-7, 7], gate * sigmoid(1.702 gate) * (up + 1)
+    for g, u in ((9.0, 9.0), (-9.0, -9.0), (0.5, 0.25)):
+        gc, uc = min(g, 7.0), max(-7.0, min(7.0, u))
+        want = gc / (1 + math.exp(-1.702 * gc)) * (uc + 1)
+        assert abs(L.orc_glu(g, u, O.ACT_CLAMPED_SWIGLU) - want) < 1e-5 * max(1, abs(want))
+
+
+# --------------------------------------------------------------------------------- router
+
+def softmax_reference(logits, expert_scale, k):
+    """RouterTopKTests.swift:594-620: sort by (score desc, index asc), exp(s - max) / sum, x scale."""
+    order = sorted(range(len(logits)), key=lambda e: (-float(logits[e]), e))[:k]
+    ex = [math.exp(float(logits[e]) - float(logits[order[0]])) for e in order]
+    return order, [v / sum(ex) * float(expert_scale[e]) for v, e in zip(ex, order)]
+
+
+def test_router_select_against_sorted_reference():
+    rng = np.random.default_rng(7)
+    ones = S.f32_to_bf16_bits(np.ones(256, np.float32))
+    zeros = S.f32_to_bf16_bits(np.zeros(256, np.float32))
+    for trial in range(50):
+        n, k = int(rng.choice([32, 64, 128, 256])), int(rng.choice([1, 4, 8]))
+        logits = rng.standard_normal(n).astype(np.float32)
+        if trial % 5 == 0:
+            logits[rng.integers(0, n, 6)] = logits[0]  # exact ties: the lower index wins
+        scale = S.f32_to_bf16_bits((1 + rng.random(n)).astype(np.float32))
+        idx, w = O.router_select(logits, scale, zeros[:n], k)
+        order, weights = softmax_reference(logits, S.bf16_bits_to_f32(scale), k)
+        assert idx.tolist() == order
+        assert np.abs(f16(w) - np.array(weights)).max() < 5e-3  # RouterTopKTests.swift:43
+    # additive bias shifts the selection (RouterTopKTests.swift:75-99)
+    logits = np.linspace(-1, 1, 64).astype(np.float32)
+    bias = np.zeros(64, np.float32)
+    bias[0] = 100.0
+    idx0, _ = O.router_select(logits, ones[:64], zeros[:64], 4)
+    idx1, w1 = O.router_select(logits, ones[:64], S.f32_to_bf16_bits(bias), 4)
+    assert 0 not in idx0.tolist() and idx1[0] == 0 and f16(w1)[0] > 0.99
+
+
+def test_router_near_tie_resolves_like_the_sorted_reference():  # RouterTopKTests.swift:101-125
+    d, e = 512, 64
+    rng = S.SplitMix64(0x71E0F4A)
+    pattern = rng.uniform(0.2, 1.0, d)
+    hidden = rng.uniform(0.5, 1.5, d)
+    gains = np.zeros(e, np.float32)
+    gains[:7] = 1.0 - np.arange(7) * 0.05
+    gains[7], gains[8] = 0.5, 0.5 * (1.0 + 1e-4)
+    gains[9:] = 0.4 - np.arange(e - 9) * 0.02
+    w = (gains[:, None] * pattern[None, :]).astype(np.float32)
+    wq, ws, wb = S.quantize_affine(w, 8)
+    x = S.f32_to_f16_bits(hidden.astype(np.float32))
+    ones = S.f32_to_bf16_bits(np.ones(d, np.float32))
+    logits = O.router_logits(wq, ws, wb, O.ROUTER_AFFINE8, x, ones, e, d)
+    ref = brute_gemv(wq, ws, wb, f16(x), e, d, 8, S.META_BF16)
+    assert np.abs(logits - ref).max() <= 1e-4 * np.abs(ref).max()
+    idx, _ = O.router_select(logits, S.f32_to_bf16_bits(np.ones(e, np.float32)), S.f32_to_bf16_bits(np.zeros(e, np.float32)), 8)
+    assert idx.tolist() == softmax_reference(ref.astype(np.float32), np.ones(e), 8)[0]
+    assert idx.tolist()[7] == 8  # the 1e-4 gap is resolved, not tied
+
+
+def test_sigmoid_router():  # RouterTopKTests.swift:343-368: select on sigmoid + bias, weigh by sigmoid, x 2.446
+    rng = np.random.default_rng(11)
+    n, k, scaling = 256, 8, 2.446
+    logits = rng.standard_normal(n).astype(np.float32)
+    corr = S.bf16_bits_to_f32(S.f32_to_bf16_bits((rng.standard_normal(n) * 0.1).astype(np.float32)))
+    sig = 1 / (1 + np.exp(-logits.astype(np.float64)))
+    order = sorted(range(n), key=lambda e: (-(np.float32(sig[e]) + np.float32(corr[e])), e))[:k]
+    orig = [sig[e] for e in order]
+    want = [v / (sum(orig) + 1e-20) * scaling for v in orig]
+    idx, w = O.router_select(logits, S.f32_to_bf16_bits(np.ones(n, np.float32)), S.f32_to_bf16_bits(corr), k,
+                             sigmoid=True, scaling=scaling)
+    assert idx.tolist() == order
+    assert np.abs(f16(w) - np.array(want)).max() < 5e-3
+
+
+def test_fp16_router_logits_against_fp64():
+    tree = S.SeedTree(0x5EED0002)
+    e, d = 256, 2048
+    w = S.router_f16(tree, "router.w", e, d)
+    x = S.activations_f16(tree, "x", d)
+    eff = S.f32_to_bf16_bits(np.ones(d, np.float32))
+    got = O.router_logits(w, None, None, O.ROUTER_F16, x, eff, e, d)
+    ref = f16(w).astype(np.float64).reshape(e, d) @ f16(x).astype(np.float64)
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-6
+
+
+# ---------------------------------------------------------------------- residency classify
+
+def classify_with(cache: H.SlotCache, experts):
+    table = np.array(cache.words, np.uint64)
+    return O.classify(np.array(experts, np.uint32), table, cache.experts_per_layer)
+
+
+def test_classify_follows_the_slot_cache_states():  # GPUExpertResidencyTests.swift:24-70
+    c = H.SlotCache(2, 4)
+    loading = c.plan([0])
+    r = classify_with(c, [0, 1, 2, 3])
+    assert r["hit_count"] == 0 and r["miss_positions"].tolist() == [0, 1, 2, 3]
+    c.complete(loading)
+    c.load([2])
+    r = classify_with(c, [0, 1, 2, 3])
+    assert r["hit_positions"].tolist() == [0, 2] and r["miss_positions"].tolist() == [1, 3]
+    assert r["miss_experts"].tolist() == [1, 3]
+    assert r["resolved_slots"][0] != H.U32_MAX and r["resolved_slots"][2] != H.U32_MAX
+    assert r["resolved_slots"][1] == H.U32_MAX
+    c.load([1, 3])
+    r = classify_with(c, [0, 1, 2, 3])
+    assert r["hit_positions"].tolist() == [1, 3] and r["miss_positions"].tolist() == [0, 2]
+    assert c.words[0] >> 32 == H.EMPTY
+
+
+def test_prefill_reduce_and_residual():  # PrefillMoETests.swift:8-64
+    rng = np.random.default_rng(3)
+    t, k, d = 5, 4, 64
+    partials = S.f32_to_f16_bits(rng.standard_normal(t * k * d).astype(np.float32))
+    weights = S.f32_to_f16_bits(rng.random(t * k).astype(np.float32))
+    h2 = O.prefill_reduce(partials, weights, t, k, d)
+    ref = np.einsum("tkd,tk->td", f16(partials).reshape(t, k, d).astype(np.float64), f16(weights).reshape(t, k).astype(np.float64))
+    assert np.abs(f16(h2).reshape(t, d) - ref).max() <= 2e-3 * max(1.0, np.abs(ref).max())
+    hidden = S.f32_to_f16_bits(rng.standard_normal(t * d).astype(np.float32))
+    want = (f16(hidden) + f16(h2)).astype(np.float16)
+    got = O.residual_add_f16(hidden.copy(), h2)
+    assert np.array_equal(got.view(np.float16), want)
