@@ -232,6 +232,82 @@ typedef struct {
 int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
                                 const shrike_decode_layer_args *args);
 
+/* ------------------------------------------------------- prefill operators */
+
+/* PrefillRouter.encodeBlock, sources/Shrike/Kernels/Prefill/MoE/PrefillRouter.swift:75-152
+ * (prefill_router_block_tiled, sources/Shrike/Metal/Prefill/prefill.metal:369-563):
+ * the router for query_count tokens. hidden: fp16[query_count, hidden_stride_elements]
+ * (row t at t * stride); out_indices: u32[query_count * top_k]; out_weights:
+ * fp16[query_count * top_k], token-major. Every token's logits and selection are
+ * bit-identical to shrike_hip_moe_router on that token alone. d_logits_workspace:
+ * fp32[query_count * num_experts], caller-owned. */
+int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_weights,
+                              const void *d_scales, const void *d_biases, const void *d_hidden,
+                              const void *d_effective_scale, const void *d_per_expert_scale,
+                              const void *d_logit_bias, uint32_t *d_out_indices,
+                              void *d_out_weights, float *d_logits_workspace,
+                              uint32_t query_count, uint32_t num_experts, uint32_t d,
+                              uint32_t top_k, uint32_t hidden_stride_elements);
+
+/* One 64-row tile of one expert's pairs: the unit the grouped FFN's workgroups take
+ * (the device form of PrefillRoutedExpertBlock + rowTileTable,
+ * PrefillGroupedRoutedMoE.swift:71-77, :272-283). `cell` is the expert's pool cell,
+ * SHRIKE_SLOT_SENTINEL when the residency table does not hold it. */
+typedef struct {
+    uint32_t cell, pair_start, rows, expert;
+} shrike_row_tile;
+
+/* Device outputs of the grouping (PrefillMoEGroupedRoutes,
+ * PrefillMoEGrouping.swift:32-50): sorted_pairs are 16-byte PrefillTokenExpertPair
+ * records (token, expert, rank, fp16 weight bits); per_expert_offsets is UINT32_MAX
+ * where an expert has no pair. row_tiles has room for
+ * shrike_hip_group_max_row_tiles() entries; row_tile_count is one word. */
+typedef struct {
+    void *sorted_pairs;
+    uint32_t *per_expert_offsets;
+    uint32_t *per_expert_counts;
+    shrike_row_tile *row_tiles;
+    uint32_t *row_tile_count;
+} shrike_hip_grouped_routes;
+
+uint32_t shrike_hip_group_max_row_tiles(uint64_t pair_count, uint32_t num_experts);
+
+/* PrefillMoEGrouping.groupTokenExpertPairs (PrefillMoEGrouping.swift:269-370) on the
+ * device, for the router's token-major output: a stable counting sort by expert, so the
+ * order is (sort key, expert, token, rank) exactly as the host function's. Experts are
+ * laid out by (d_expert_sort_keys[e], e) when keys are given (u64[num_experts]), by id
+ * otherwise. d_residency (u64[num_experts], may be NULL) resolves each expert's cell;
+ * with NULL the cell is the expert id. num_experts <= 256. */
+int shrike_hip_group_pairs(void *stream, const uint32_t *d_indices, const void *d_weights,
+                           uint32_t query_count, uint32_t top_k, uint32_t num_experts,
+                           const uint64_t *d_expert_sort_keys, const uint64_t *d_residency,
+                           const shrike_hip_grouped_routes *out);
+
+/* PrefillGroupedRoutedMoE.encodeGroupedExpertGEMMs (PrefillGroupedRoutedMoE.swift:925-1126;
+ * gather, mpp_prefill_affine_grouped_f16 x3, silu_mul_fp16, scatter —
+ * sources/Shrike/Metal/TensorCore/tensorops.metal:61-248, prefill.metal:749-790) for all
+ * row tiles in two MFMA launches: route_partials[(token * top_k + rank) * d ..] =
+ * fp16(down . fp16(glu(gate . x, up . x))) for every pair of a resident expert.
+ * hidden: fp16[query_count, hidden_stride_elements]. d_workspace: caller-owned, at least
+ * shrike_hip_prefill_ffn_workspace_bytes(). Tiles of absent experts are skipped (their
+ * partial rows are left untouched). */
+size_t shrike_hip_prefill_ffn_workspace_bytes(uint32_t query_count, uint32_t max_row_tiles,
+                                              uint32_t d, uint32_t f);
+int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                   uint64_t pool_slot_stride, const shrike_expert_offsets *offsets,
+                                   const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles,
+                                   const void *d_hidden, uint32_t hidden_stride_elements,
+                                   void *d_route_partials, void *d_workspace, size_t workspace_bytes,
+                                   uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k);
+
+/* PrefillMoE.encodeReduceTokenMajor, sources/Shrike/Kernels/Prefill/MoE/PrefillMoE.swift:11-40
+ * (prefill_moe_reduce_token_major, prefill.metal:624-645): h2[t, :] =
+ * fp16(sum over ranks, in rank order, of weight[t, r] * partial[t, r, :]). */
+int shrike_hip_prefill_reduce(void *stream, const void *d_route_partials, const void *d_route_weights,
+                              void *d_h2, uint32_t query_count, uint32_t top_k, uint32_t d);
+/* residual_add_fp16 (RealForwardRunner.swift:4658-4665): hidden[i] = fp16(hidden[i] + delta[i]). */
+int shrike_hip_residual_add_f16(void *stream, void *d_hidden, const void *d_delta, uint64_t count);
+
 /* ----------------------------------------------------------------- plumbing
  * Device memory, streams, events and graphs for hosts without a HIP binding of
  * their own (the Python tests and benchmark). No counterpart in the reference,

@@ -4,7 +4,7 @@ the shipped implementation is the C++ in shrike_amd/csrc/host_logic.cpp and
 slot_cache.cpp, which the tests compare against these functions.
 
 Every function follows one reference function (cited in its docstring) and is pinned
-in tests/test_host_logic.py by the vectors the reference's own unit tests hold.
+in tests/test_host_logic_oracle.py by the vectors the reference's own unit tests hold.
 All arithmetic here is integer; results are compared for equality.
 """
 from __future__ import annotations

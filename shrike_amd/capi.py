@@ -65,6 +65,15 @@ class DecodeLayerArgs(C.Structure):
 
 # name -> (restype, argtypes); every symbol include/shrike_hip.h declares
 _VP, _U32, _U64, _I32, _I64 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_int32, C.c_int64
+class RowTile(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("cell", "pair_start", "rows", "expert")]
+
+
+class HipGroupedRoutes(C.Structure):
+    _fields_ = [("sorted_pairs", C.c_void_p), ("per_expert_offsets", C.c_void_p), ("per_expert_counts", C.c_void_p),
+                ("row_tiles", C.c_void_p), ("row_tile_count", C.c_void_p)]
+
+
 # ---- include/shrike_host.h ----------------------------------------------------------
 
 class TokenExpertPair(C.Structure):
@@ -169,6 +178,17 @@ SIGNATURES = {
     "shrike_hip_graph_end_capture": (_VP, [_VP]),
     "shrike_hip_graph_launch": (C.c_int, [_VP, _VP]),
     "shrike_hip_graph_destroy": (C.c_int, [_VP]),
+    # prefill operators
+    "shrike_hip_prefill_router": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
+                                            _U32, _U32, _U32, _U32, _U32]),
+    "shrike_hip_group_max_row_tiles": (_U32, [_U64, _U32]),
+    "shrike_hip_group_pairs": (C.c_int, [_VP, _VP, _VP, _U32, _U32, _U32, _VP, _VP, C.POINTER(HipGroupedRoutes)]),
+    "shrike_hip_prefill_ffn_workspace_bytes": (C.c_size_t, [_U32, _U32, _U32, _U32]),
+    "shrike_hip_prefill_grouped_ffn": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, C.POINTER(ExpertOffsets),
+                                                 C.POINTER(HipGroupedRoutes), _U32, _VP, _U32, _VP, _VP, C.c_size_t,
+                                                 _U32, _U32, _U32, _U32]),
+    "shrike_hip_prefill_reduce": (C.c_int, [_VP, _VP, _VP, _VP, _U32, _U32, _U32]),
+    "shrike_hip_residual_add_f16": (C.c_int, [_VP, _VP, _VP, _U64]),
     # include/shrike_host.h
     "shrike_make_token_expert_pairs": (C.c_int, [_VP, _VP, _U32, _U32, C.POINTER(TokenExpertPair)]),
     "shrike_group_pairs": (C.c_int, [C.POINTER(TokenExpertPair), C.c_size_t, _I64, _I64, _I64, _I64, _VP,

@@ -36,8 +36,9 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     uint32_t cell = kSentinel;
     if (ROUTE) {
         if (wave == 0) {
+            __shared__ RouteScratch s_route;
             uint32_t my_cell;
-            route_wave<false>(a.sel, a.lists, lane, blockIdx.x == 0, my_cell);
+            route_wave<false>(a.sel, a.lists, lane, blockIdx.x == 0, my_cell, s_route);
             if (lane < a.top_k) s_cell[lane] = my_cell;
         }
         __syncthreads();

@@ -1,80 +1,9 @@
 // Router logits, top-k select and residency classification for gfx950, and the head
 // launch of the fused layer (router rows beside the shared expert's gate/up rows).
 #include "decode_launch.h"
+#include "router_row.h"
 
 namespace shrike {
-
-// One expert row of the router GEMV (moe.metal:324-364), RK: 0 = fp16 rows, 8 / 4 =
-// group-affine codes. The per-lane fused-multiply-add order and the xor butterfly are
-// fixed so that the fp32 logits are reproducible bit for bit (lane l takes chunks
-// l, l+64, ...).
-template <int RK>
-__device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint32_t lane) {
-    constexpr int E = RK == 0 ? 8 : RK == 8 ? 16 : 32;  // elements per 16-byte weight chunk
-    constexpr int PIECES = E / 8;
-    constexpr int MAXI = RK == 0 ? 8 : 4;
-    const uint32_t chunks = a.d / E;
-    const uint32_t groups = a.d / kGroup;
-    const uint32_t row_bytes = chunks * 16u;
-    const uint8_t *row = static_cast<const uint8_t *>(a.weights) + size_t(e) * row_bytes;
-    uint4 w[MAXI], xv[MAXI][PIECES], ev[MAXI][PIECES];
-    uint16_t sc[MAXI], bi[MAXI];
-#pragma unroll
-    for (int i = 0; i < MAXI; ++i) {
-        const uint32_t c = lane + 64u * i;
-        const uint32_t cc = c < chunks ? c : 0u;
-        w[i] = *reinterpret_cast<const uint4 *>(row + 16u * cc);
-#pragma unroll
-        for (int j = 0; j < PIECES; ++j) {
-            xv[i][j] = reinterpret_cast<const uint4 *>(a.hidden)[cc * PIECES + j];
-            ev[i][j] = reinterpret_cast<const uint4 *>(a.effective_scale)[cc * PIECES + j];
-        }
-        if (RK != 0) {
-            sc[i] = a.scales[size_t(e) * groups + cc * E / kGroup];
-            bi[i] = a.biases[size_t(e) * groups + cc * E / kGroup];
-        }
-    }
-    float acc = 0.0f;
-#pragma unroll
-    for (int i = 0; i < MAXI; ++i) {
-        const uint32_t c = lane + 64u * i;
-        if (c < chunks) {
-            float xs[E];
-#pragma unroll
-            for (int j = 0; j < PIECES; ++j) {
-                const uint32_t xw[4] = {xv[i][j].x, xv[i][j].y, xv[i][j].z, xv[i][j].w};
-                const uint32_t ew[4] = {ev[i][j].x, ev[i][j].y, ev[i][j].z, ev[i][j].w};
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {  // moe.metal:357-358 (exact product)
-                    xs[8 * j + 2 * t] = __fmul_rn(f16_to_f32(uint16_t(xw[t])), bf16_to_f32(uint16_t(ew[t])));
-                    xs[8 * j + 2 * t + 1] = __fmul_rn(f16_to_f32(uint16_t(xw[t] >> 16)), bf16_to_f32(uint16_t(ew[t] >> 16)));
-                }
-            }
-            const uint32_t ww[4] = {w[i].x, w[i].y, w[i].z, w[i].w};
-            if (RK == 0) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    acc = fmaf(f16_to_f32(uint16_t(ww[t])), xs[2 * t], acc);
-                    acc = fmaf(f16_to_f32(uint16_t(ww[t] >> 16)), xs[2 * t + 1], acc);
-                }
-            } else {
-                float qx = 0.0f, sum = 0.0f;
-#pragma unroll
-                for (int t = 0; t < E; ++t) {
-                    const uint32_t q = RK == 8 ? (ww[t / 4] >> (8 * (t % 4))) & 0xffu
-                                               : (ww[t / 8] >> (4 * (t % 8))) & 0xfu;
-                    qx = fmaf(float(q), xs[t], qx);
-                    sum = __fadd_rn(sum, xs[t]);
-                }
-                acc = fmaf(meta_f32(sc[i], a.meta), qx, acc);
-                acc = fmaf(meta_f32(bi[i], a.meta), sum, acc);
-            }
-        }
-    }
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, o));
-    if (lane == 0) a.logits_out[e] = acc;
-}
 
 // MoE.encodeRouter as one launch: four expert rows per workgroup, and the workgroup that
 // finishes last runs select (+ classify when a residency table is bound).
@@ -96,8 +25,9 @@ __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
     __syncthreads();
     if (!s_last || wave != 0) return;
     __threadfence();
+    __shared__ RouteScratch s_route;
     uint32_t cell;
-    route_wave<true>(a.sel, a.lists, lane, true, cell);
+    route_wave<true>(a.sel, a.lists, lane, true, cell, s_route);
     if (lane == 0) *a.counter = 0u;
 }
 

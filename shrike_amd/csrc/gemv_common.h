@@ -281,9 +281,16 @@ __device__ __forceinline__ float load_logit(const float *p) {
 // 0). On return lane p < top_k holds position p's resolved cell (sentinel on a miss).
 // COHERENT reads the logits past the non-coherent caches (they were written by other
 // workgroups of the same launch); otherwise they come from an earlier launch.
+// One wave's table of candidates in LDS for route_wave (a workgroup whose waves route side
+// by side gives each its own).
+struct RouteScratch {
+    uint32_t key[256], gain[256], cellv[256];
+    float raw[256];
+};
+
 template <bool COHERENT>
 __device__ void route_wave(const SelectArgs &a, const RouteLists &out, uint32_t lane, bool write_lists,
-                           uint32_t &my_cell) {
+                           uint32_t &my_cell, RouteScratch &lds) {
     // key = the score's bits mapped to an unsigned order (larger score, larger key); 0 marks
     // what can never be taken: NaN, -inf and experts past num_experts
     uint32_t key[4], cellv[4], gainv[4];
@@ -308,8 +315,8 @@ __device__ void route_wave(const SelectArgs &a, const RouteLists &out, uint32_t 
     const uint32_t K = a.top_k;
     // Every lane parks its four candidates in LDS; after the rounds lane p fetches position
     // p's full key, gain, cell (and raw logit) by expert index with one read each.
-    __shared__ uint32_t s_key[256], s_gain[256], s_cellv[256];
-    __shared__ float s_raw[256];
+    uint32_t *s_key = lds.key, *s_gain = lds.gain, *s_cellv = lds.cellv;
+    float *s_raw = lds.raw;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         s_key[lane + 64u * j] = key[j];

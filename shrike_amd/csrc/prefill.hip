@@ -1,0 +1,335 @@
+// The prefill side of the routed path for gfx950, except the grouped FFN: the router for a
+// block of tokens, the token->expert grouping as a stable counting sort, the per-row group
+// sums the grouped FFN folds the affine biases with, the token-major reduce and the
+// residual add.
+#include "prefill_common.h"
+#include "router_row.h"
+
+#include "../../include/shrike_host.h"
+
+namespace shrike {
+
+constexpr uint32_t kRouterTokenBlock = 4;  // tokens a wave runs one expert row against
+
+// prefill.metal:369-439: logits of every (token, expert). A wave holds one expert and walks
+// kRouterTokenBlock tokens, so the row comes from HBM once and from L1 afterwards. The row
+// arithmetic is the decode router's, operand for operand.
+template <int RK>
+__global__ __launch_bounds__(256) void k_prefill_logits(RouterArgs a, uint32_t query_count, uint32_t stride, float *ws) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t e = blockIdx.x * 4u + wave;
+    if (e >= a.sel.num_experts) return;
+#pragma unroll 1
+    for (uint32_t i = 0; i < kRouterTokenBlock; ++i) {
+        const uint32_t t = blockIdx.y * kRouterTokenBlock + i;
+        if (t >= query_count) break;
+        RouterArgs b = a;
+        b.hidden = a.hidden + size_t(t) * stride;
+        b.logits_out = ws + size_t(t) * a.sel.num_experts;
+        router_row<RK>(b, e, lane);
+    }
+}
+
+// prefill.metal:441-563: one wave selects for one token.
+__global__ __launch_bounds__(256) void k_prefill_select(SelectArgs sel, const float *ws, uint32_t *out_indices,
+                                                        uint16_t *out_weights, uint32_t query_count) {
+    __shared__ RouteScratch s_route[4];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t t = blockIdx.x * 4u + wave;
+    if (t >= query_count) return;
+    sel.logits = ws + size_t(t) * sel.num_experts;
+    RouteLists lists = {};
+    lists.out_indices = out_indices + size_t(t) * sel.top_k;
+    lists.out_weights = out_weights + size_t(t) * sel.top_k;
+    uint32_t cell;
+    route_wave<false>(sel, lists, lane, true, cell, s_route[wave]);
+}
+
+// ---- grouping ---------------------------------------------------------------------------
+
+struct GroupArgs {
+    const uint32_t *indices;
+    const uint16_t *weights;
+    uint32_t pairs, top_k, num_experts;
+    const uint64_t *sort_keys, *residency;
+    shrike_token_expert_pair *sorted;
+    uint32_t *offsets, *counts;
+    shrike_row_tile *tiles;
+    uint32_t *tile_count;
+};
+
+// pass 1: pairs per expert; one wave per expert
+__global__ __launch_bounds__(256) void k_group_count(GroupArgs a) {
+    const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (e >= a.num_experts) return;
+    uint32_t n = 0;
+    for (uint32_t i = lane; i < a.pairs; i += 64u) n += a.indices[i] == e ? 1u : 0u;
+    n = wave_sum_u32(n);
+    if (lane == 0) a.counts[e] = n;
+}
+
+// pass 2: the expert's first position (the pairs of every expert ordered before it), its
+// row tiles, and its pairs written in (token, rank) order. The pairs arrive token-major, so
+// walking them in index order keeps that order within the expert: the permutation equals
+// the reference's sort by (sort key, expert, token, rank) (PrefillMoEGrouping.swift:323-332).
+__global__ __launch_bounds__(256) void k_group_place(GroupArgs a) {
+    const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (e >= a.num_experts) return;
+    const uint64_t key = a.sort_keys ? a.sort_keys[e] : 0u;
+    uint32_t offset = 0, tiles_before = 0, tiles_total = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < SHRIKE_MAX_ROUTER_EXPERTS / 64u; ++j) {
+        const uint32_t other = lane + 64u * j;
+        if (other >= a.num_experts) continue;
+        const uint32_t c = a.counts[other];
+        const uint64_t k2 = a.sort_keys ? a.sort_keys[other] : 0u;
+        const bool before = k2 < key || (k2 == key && other < e);
+        const uint32_t t = (c + kRowTile - 1u) / kRowTile;
+        offset += before ? c : 0u;
+        tiles_before += before ? t : 0u;
+        tiles_total += t;
+    }
+    offset = wave_sum_u32(offset);
+    tiles_before = wave_sum_u32(tiles_before);
+    tiles_total = wave_sum_u32(tiles_total);
+    const uint32_t count = a.counts[e];
+    if (lane == 0) {
+        a.offsets[e] = count ? offset : 0xffffffffu;
+        if (e == 0) *a.tile_count = tiles_total;
+    }
+    uint32_t cell = e;
+    if (a.residency) {  // moe.metal:136-146
+        const uint64_t word = a.residency[e];
+        cell = uint32_t(word >> 32) == SHRIKE_RESIDENCY_RESIDENT ? uint32_t(word) : kSentinel;
+    }
+    const uint32_t my_tiles = (count + kRowTile - 1u) / kRowTile;
+    for (uint32_t j = lane; j < my_tiles; j += 64u) {
+        shrike_row_tile t;
+        t.cell = cell;
+        t.pair_start = offset + j * kRowTile;
+        t.rows = min(kRowTile, count - j * kRowTile);
+        t.expert = e;
+        a.tiles[tiles_before + j] = t;
+    }
+    if (count == 0) return;
+    uint32_t running = 0;
+    const uint64_t below = (uint64_t(1) << lane) - 1u;
+    for (uint32_t base = 0; base < a.pairs; base += 64u) {
+        const uint32_t i = base + lane;
+        const bool mine = i < a.pairs && a.indices[i] == e;
+        const uint64_t mask = __ballot(mine);
+        if (mine) {
+            shrike_token_expert_pair p;
+            p.token = i / a.top_k;
+            p.expert = e;
+            p.rank = i - p.token * a.top_k;
+            p.weight_bits_and_reserved = a.weights[i];
+            a.sorted[offset + running + __popcll(mask & below)] = p;
+        }
+        running += __popcll(mask);
+    }
+}
+
+// ---- group sums -------------------------------------------------------------------------
+
+// For every row of an fp16 matrix [rows, n] (row r at r * stride), the sum of each group of
+// 64 elements, accumulated in fp32 in a fixed order and stored as two fp16 halves (hi, lo):
+// the operand that turns the affine bias term sum_g bias[g] * (sum of x over g) into one
+// more matrix product. Eight lanes share a group; a lane sums its eight elements in order,
+// then the eight partials fold pairwise.
+__global__ __launch_bounds__(256) void k_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uint32_t n,
+                                                        uint32_t *out, const uint32_t *row_limit_tiles) {
+    const uint32_t groups = n / kGroup;
+    const size_t slot = size_t(blockIdx.x) * 256u + threadIdx.x;  // (row, group, eighth)
+    const size_t per_row = size_t(groups) * 8u;
+    const uint32_t row = uint32_t(slot / per_row);
+    uint32_t live_rows = rows;
+    if (row_limit_tiles) live_rows = min(rows, *row_limit_tiles * kRowTile);
+    const bool on = row < live_rows;
+    const uint32_t rest = uint32_t(slot - size_t(row) * per_row);
+    float s = 0.0f;
+    if (on) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(src + size_t(row) * stride + size_t(rest) * 8u);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            s = __fadd_rn(s, f16_to_f32(uint16_t(w[t])));
+            s = __fadd_rn(s, f16_to_f32(uint16_t(w[t] >> 16)));
+        }
+    }
+    s = __fadd_rn(s, __shfl_xor(s, 1));
+    s = __fadd_rn(s, __shfl_xor(s, 2));
+    s = __fadd_rn(s, __shfl_xor(s, 4));
+    if (on && (rest & 7u) == 0u) out[size_t(row) * groups + rest / 8u] = split_hi_lo(s);
+}
+
+// ---- reduce and residual ----------------------------------------------------------------
+
+// prefill.metal:624-645: a thread owns eight neighbouring d of one token; fp32 fma in rank order
+__global__ __launch_bounds__(256) void k_prefill_reduce(const uint16_t *partials, const uint16_t *weights, uint16_t *h2,
+                                                        uint32_t query_count, uint32_t top_k, uint32_t d) {
+    const uint32_t per_row = d / 8u;
+    const size_t slot = size_t(blockIdx.x) * 256u + threadIdx.x;
+    const uint32_t t = uint32_t(slot / per_row);
+    if (t >= query_count) return;
+    const uint32_t c = uint32_t(slot - size_t(t) * per_row);
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (uint32_t r = 0; r < top_k; ++r) {
+        const float w = f16_to_f32(weights[size_t(t) * top_k + r]);
+        const uint4 v = *reinterpret_cast<const uint4 *>(partials + (size_t(t) * top_k + r) * d + size_t(c) * 8u);
+        const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[2 * j] = fmaf(w, f16_to_f32(uint16_t(p[j])), acc[2 * j]);
+            acc[2 * j + 1] = fmaf(w, f16_to_f32(uint16_t(p[j] >> 16)), acc[2 * j + 1]);
+        }
+    }
+    uint4 o;
+    o.x = uint32_t(f32_to_f16(acc[0])) | uint32_t(f32_to_f16(acc[1])) << 16;
+    o.y = uint32_t(f32_to_f16(acc[2])) | uint32_t(f32_to_f16(acc[3])) << 16;
+    o.z = uint32_t(f32_to_f16(acc[4])) | uint32_t(f32_to_f16(acc[5])) << 16;
+    o.w = uint32_t(f32_to_f16(acc[6])) | uint32_t(f32_to_f16(acc[7])) << 16;
+    *reinterpret_cast<uint4 *>(h2 + size_t(t) * d + size_t(c) * 8u) = o;
+}
+
+__global__ __launch_bounds__(256) void k_residual_add(uint16_t *hidden, const uint16_t *delta, uint64_t count) {
+    const uint64_t i = (uint64_t(blockIdx.x) * 256u + threadIdx.x) * 8u;
+    if (i >= count) return;
+    if (i + 8u <= count) {
+        uint4 h = *reinterpret_cast<const uint4 *>(hidden + i);
+        const uint4 dl = *reinterpret_cast<const uint4 *>(delta + i);
+        uint32_t hw[4] = {h.x, h.y, h.z, h.w};
+        const uint32_t dw[4] = {dl.x, dl.y, dl.z, dl.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint16_t lo = f32_to_f16(__fadd_rn(f16_to_f32(uint16_t(hw[j])), f16_to_f32(uint16_t(dw[j]))));
+            const uint16_t hi = f32_to_f16(__fadd_rn(f16_to_f32(uint16_t(hw[j] >> 16)), f16_to_f32(uint16_t(dw[j] >> 16))));
+            hw[j] = uint32_t(lo) | uint32_t(hi) << 16;
+        }
+        h.x = hw[0]; h.y = hw[1]; h.z = hw[2]; h.w = hw[3];
+        *reinterpret_cast<uint4 *>(hidden + i) = h;
+    } else {
+        for (uint64_t j = i; j < count; ++j) hidden[j] = f32_to_f16(__fadd_rn(f16_to_f32(hidden[j]), f16_to_f32(delta[j])));
+    }
+}
+
+int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uint32_t n, uint32_t *out,
+                          const uint32_t *row_limit_tiles, hipStream_t s) {
+    const size_t slots = size_t(rows) * (n / kGroup) * 8u;
+    if (slots == 0) return 0;
+    hipLaunchKernelGGL(k_row_group_sums, dim3(uint32_t((slots + 255u) / 256u)), dim3(256), 0, s, src, stride, rows, n, out,
+                       row_limit_tiles);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace shrike
+
+using namespace shrike;
+
+extern "C" {
+
+int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_weights, const void *d_scales,
+                              const void *d_biases, const void *d_hidden, const void *d_effective_scale,
+                              const void *d_per_expert_scale, const void *d_logit_bias, uint32_t *d_out_indices,
+                              void *d_out_weights, float *d_logits_workspace, uint32_t query_count, uint32_t num_experts,
+                              uint32_t d, uint32_t top_k, uint32_t hidden_stride_elements) {
+    SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
+    SHRIKE_REQUIRE(query_count > 0, "queryCount must be positive");  // PrefillRouter.swift:99
+    if (int rc = check_router(moe, num_experts, d, top_k)) return rc;
+    SHRIKE_REQUIRE(hidden_stride_elements >= d, "hidden stride is too small");  // PrefillRouter.swift:104
+    SHRIKE_REQUIRE(hidden_stride_elements % 8u == 0, "hidden stride must keep rows 16-byte aligned");
+    SHRIKE_REQUIRE(d_weights && d_hidden && d_effective_scale && d_per_expert_scale && d_logit_bias,
+                   "prefill router: weights, hidden, effectiveScale, perExpertScale and logitBias must all be bound");
+    SHRIKE_REQUIRE(moe->desc.router_weight_bits == 0 || (d_scales && d_biases), "prefill router: affine router needs scales and biases");
+    SHRIKE_REQUIRE(d_out_indices && d_out_weights && d_logits_workspace, "prefill router: outputs and the logits workspace must be bound");
+    RouterArgs a = {};
+    a.weights = d_weights;
+    a.scales = static_cast<const uint16_t *>(d_scales);
+    a.biases = static_cast<const uint16_t *>(d_biases);
+    a.hidden = static_cast<const uint16_t *>(d_hidden);
+    a.effective_scale = static_cast<const uint16_t *>(d_effective_scale);
+    a.d = d;
+    a.meta = moe->desc.meta_dtype;
+    a.sel.per_expert_scale = static_cast<const uint16_t *>(d_per_expert_scale);
+    a.sel.logit_bias = static_cast<const uint16_t *>(d_logit_bias);
+    a.sel.num_experts = num_experts;
+    a.sel.top_k = top_k;
+    a.sel.sigmoid = moe->desc.sigmoid_router_scores;
+    a.sel.scaling = moe->desc.routed_scaling_factor;
+    hipStream_t s = as_stream(stream);
+    const dim3 grid((num_experts + 3u) / 4u, (query_count + kRouterTokenBlock - 1u) / kRouterTokenBlock);
+    switch (moe->desc.router_weight_bits) {
+        case 0: hipLaunchKernelGGL(k_prefill_logits<0>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;
+        case 8: hipLaunchKernelGGL(k_prefill_logits<8>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;
+        default: hipLaunchKernelGGL(k_prefill_logits<4>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;
+    }
+    SHRIKE_HIP(hipGetLastError());
+    hipLaunchKernelGGL(k_prefill_select, dim3((query_count + 3u) / 4u), dim3(256), 0, s, a.sel, d_logits_workspace, d_out_indices,
+                       static_cast<uint16_t *>(d_out_weights), query_count);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+uint32_t shrike_hip_group_max_row_tiles(uint64_t pair_count, uint32_t num_experts) {
+    return max_row_tiles(pair_count, num_experts);
+}
+
+int shrike_hip_group_pairs(void *stream, const uint32_t *d_indices, const void *d_weights, uint32_t query_count,
+                           uint32_t top_k, uint32_t num_experts, const uint64_t *d_expert_sort_keys,
+                           const uint64_t *d_residency, const shrike_hip_grouped_routes *out) {
+    SHRIKE_REQUIRE(top_k > 0, "topK must be positive, got %u", top_k);                    // PrefillMoEGrouping.swift:280
+    SHRIKE_REQUIRE(num_experts > 0, "numExperts must be positive, got %u", num_experts);  // :283
+    SHRIKE_REQUIRE(num_experts <= SHRIKE_MAX_ROUTER_EXPERTS, "numExperts > 256 is not supported");
+    SHRIKE_REQUIRE(uint64_t(query_count) * top_k <= 0x7fffffffull, "too many route pairs");
+    SHRIKE_REQUIRE(out && out->sorted_pairs && out->per_expert_offsets && out->per_expert_counts && out->row_tiles && out->row_tile_count,
+                   "group pairs: an output is NULL");
+    SHRIKE_REQUIRE(query_count == 0 || (d_indices && d_weights), "group pairs: indices and weights must be bound");
+    GroupArgs a = {};
+    a.indices = d_indices;
+    a.weights = static_cast<const uint16_t *>(d_weights);
+    a.pairs = query_count * top_k;
+    a.top_k = top_k;
+    a.num_experts = num_experts;
+    a.sort_keys = d_expert_sort_keys;
+    a.residency = d_residency;
+    a.sorted = static_cast<shrike_token_expert_pair *>(out->sorted_pairs);
+    a.offsets = out->per_expert_offsets;
+    a.counts = out->per_expert_counts;
+    a.tiles = out->row_tiles;
+    a.tile_count = out->row_tile_count;
+    hipStream_t s = as_stream(stream);
+    const dim3 grid((num_experts + 3u) / 4u);
+    hipLaunchKernelGGL(k_group_count, grid, dim3(256), 0, s, a);
+    SHRIKE_HIP(hipGetLastError());
+    hipLaunchKernelGGL(k_group_place, grid, dim3(256), 0, s, a);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int shrike_hip_prefill_reduce(void *stream, const void *d_route_partials, const void *d_route_weights, void *d_h2,
+                              uint32_t query_count, uint32_t top_k, uint32_t d) {
+    SHRIKE_REQUIRE(d_route_partials && d_route_weights && d_h2, "prefill reduce: NULL buffer");
+    SHRIKE_REQUIRE(d % 8u == 0 && top_k > 0, "prefill reduce: D must be a multiple of 8 and topK positive");
+    const size_t slots = size_t(query_count) * (d / 8u);
+    if (slots == 0) return 0;
+    hipLaunchKernelGGL(k_prefill_reduce, dim3(uint32_t((slots + 255u) / 256u)), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint16_t *>(d_route_partials), static_cast<const uint16_t *>(d_route_weights),
+                       static_cast<uint16_t *>(d_h2), query_count, top_k, d);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int shrike_hip_residual_add_f16(void *stream, void *d_hidden, const void *d_delta, uint64_t count) {
+    SHRIKE_REQUIRE(d_hidden && d_delta, "residual add: NULL buffer");
+    SHRIKE_REQUIRE((reinterpret_cast<uintptr_t>(d_hidden) | reinterpret_cast<uintptr_t>(d_delta)) % 16u == 0,
+                   "residual add: buffers must be 16-byte aligned");
+    if (count == 0) return 0;
+    const uint64_t threads = (count + 7u) / 8u;
+    hipLaunchKernelGGL(k_residual_add, dim3(uint32_t((threads + 255u) / 256u)), dim3(256), 0, as_stream(stream),
+                       static_cast<uint16_t *>(d_hidden), static_cast<const uint16_t *>(d_delta), count);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,387 @@
+// The grouped expert FFN of prefill for gfx950 (PrefillGroupedRoutedMoE.encodeGroupedExpertGEMMs,
+// PrefillGroupedRoutedMoE.swift:925-1126): for every 64-row tile of one expert's pairs,
+// act = fp16(glu(gate . X, up . X)) and partial = fp16(down . act), on the matrix cores.
+//
+// The quantised weights never become fp16 weights. With w = q * s + b per group of 64,
+//   sum_k x_k w_k = sum_g s_g (sum_{k in g} x_k q_k) + sum_g b_g (sum_{k in g} x_k),
+// the codes enter v_mfma_f32_32x32x16_f16 as they are: a 4- or 8-bit code placed in the low
+// bits of an fp16 is the subnormal q * 2^-24, which the matrix core multiplies exactly, so
+// the per-group product sum_k x_k q_k comes out of four chained MFMAs in fp32 and is scaled
+// by s_g * 2^24 on the vector ALU. The bias term is one more short matrix product between
+// the per-row group sums of X (fp32 sums carried as fp16 hi + lo, see k_row_group_sums) and
+// the group biases.
+#include "decode_launch.h"
+#include "prefill_common.h"
+
+#include "../../include/shrike_host.h"
+
+namespace shrike {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr uint32_t kChunkK = 256;                 // k staged in LDS per step: four groups
+constexpr uint32_t kLdsRow = kChunkK + 8;         // halves per staged row; the pad spreads the banks
+constexpr uint32_t kMaxMT = kRowTile / 32;        // 32-row MFMA tiles per row tile
+constexpr float kTwo24 = 16777216.0f;
+
+struct FfnArgs {
+    PoolArg pool;
+    uint64_t stride;
+    shrike_expert_offsets off;
+    const shrike_row_tile *tiles;
+    const uint32_t *tile_count;
+    const shrike_token_expert_pair *pairs;
+    const uint16_t *hidden;       // fp16[T, hidden_stride]
+    uint32_t hidden_stride;
+    const uint32_t *hidden_sums;  // (hi, lo)[T, d / 64]
+    uint16_t *act;                // fp16[tiles * 64, f]
+    const uint32_t *act_sums;     // (hi, lo)[tiles * 64, f / 64]
+    uint16_t *partials;           // fp16[T * top_k, d]
+    uint32_t d, f, top_k, meta, act_kind, ebias;
+};
+
+union Frag {
+    half8 h;
+    uint32_t u[4];
+    uint4 v;
+};
+
+// 4-bit: the eight codes of one word as fp16 subnormals in the order (0,4,1,5,2,6,3,7),
+// which is the order the staged A rows are permuted to.
+__device__ __forceinline__ half8 codes4(uint32_t w) {
+    Frag f;
+    f.u[0] = w & 0x000f000fu;
+    f.u[1] = (w >> 4) & 0x000f000fu;
+    f.u[2] = (w >> 8) & 0x000f000fu;
+    f.u[3] = (w >> 12) & 0x000f000fu;
+    return f.h;
+}
+// 8-bit: eight codes of two words, in order
+__device__ __forceinline__ half8 codes8(uint32_t w0, uint32_t w1) {
+    Frag f;
+    f.u[0] = __builtin_amdgcn_perm(0u, w0, 0x0c010c00u);
+    f.u[1] = __builtin_amdgcn_perm(0u, w0, 0x0c030c02u);
+    f.u[2] = __builtin_amdgcn_perm(0u, w1, 0x0c010c00u);
+    f.u[3] = __builtin_amdgcn_perm(0u, w1, 0x0c030c02u);
+    return f.h;
+}
+
+template <int BITS>
+struct BRegs {  // one lane's codes of one weight row for one group: its 32 k
+    uint4 w[BITS / 4];
+    uint16_t scale;
+};
+
+template <int BITS>
+__device__ __forceinline__ void load_b(BRegs<BITS> &r, const uint8_t *row_w, const uint16_t *row_s, uint32_t g, uint32_t kb) {
+    const uint4 *p = reinterpret_cast<const uint4 *>(row_w + size_t(g) * (kGroup * BITS / 8) + kb * (4 * BITS));
+#pragma unroll
+    for (int i = 0; i < BITS / 4; ++i) r.w[i] = p[i];
+    r.scale = row_s[g];
+}
+
+template <int BITS>
+__device__ __forceinline__ half8 b_step(const BRegs<BITS> &r, int s) {
+    if (BITS == 4) {
+        const uint32_t w[4] = {r.w[0].x, r.w[0].y, r.w[0].z, r.w[0].w};
+        return codes4(w[s]);
+    } else {
+        const uint32_t w[8] = {r.w[0].x, r.w[0].y, r.w[0].z, r.w[0].w, r.w[BITS / 4 - 1].x, r.w[BITS / 4 - 1].y, r.w[BITS / 4 - 1].z, r.w[BITS / 4 - 1].w};
+        return codes8(w[2 * s], w[2 * s + 1]);
+    }
+}
+
+// MODE 0: gate and up rows n0..n0+31 of one expert against the gathered token rows, GLU,
+// fp16 activations out. MODE 1: down rows n0..n0+63 against the activations, fp16 partials
+// scattered to (token, rank).
+template <int BITS, int MODE>
+__global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
+    __shared__ __align__(16) uint16_t s_a[2][kRowTile][kLdsRow];
+    const uint32_t tile_index = blockIdx.x;
+    if (tile_index >= *a.tile_count) return;
+    const shrike_row_tile tile = a.tiles[tile_index];
+    if (tile.cell == kSentinel || tile.rows == 0) return;
+
+    const uint32_t K = MODE == 0 ? a.d : a.f, N = MODE == 0 ? a.f : a.d;
+    const uint32_t G = K / kGroup;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t col = lane & 31u, kb = lane >> 5;
+    const uint32_t mt_count = (tile.rows + 31u) / 32u;
+    const uint32_t n0 = (blockIdx.y * 4u + wave) * (MODE == 0 ? 32u : 64u);
+    const bool active = n0 < N;
+
+    // ---- A staging: thread -> (row = tid / 32 + 8 i, 16-byte piece = tid % 32)
+    const uint32_t piece = threadIdx.x & 31u, row0 = threadIdx.x >> 5;
+    const uint16_t *src_row[kMaxMT * 4];
+#pragma unroll
+    for (uint32_t i = 0; i < kMaxMT * 4; ++i) {
+        const uint32_t r = min(row0 + 8u * i, tile.rows - 1u);  // rows past the tile repeat its last row
+        if (MODE == 0) {
+            src_row[i] = a.hidden + size_t(a.pairs[tile.pair_start + r].token) * a.hidden_stride;
+        } else {
+            src_row[i] = a.act + (size_t(tile_index) * kRowTile + r) * a.f;
+        }
+    }
+    uint4 stage[kMaxMT * 4];
+    auto fetch = [&](uint32_t chunk) {
+        const uint32_t k = chunk * kChunkK + piece * 8u;
+#pragma unroll
+        for (uint32_t i = 0; i < kMaxMT * 4; ++i)
+            if (i < mt_count * 4u && k < K) stage[i] = *reinterpret_cast<const uint4 *>(src_row[i] + k);
+    };
+    auto commit = [&](uint32_t buf) {
+#pragma unroll
+        for (uint32_t i = 0; i < kMaxMT * 4; ++i) {
+            if (i >= mt_count * 4u) continue;
+            uint4 v = stage[i];
+            if (BITS == 4) {  // (0,1,2,3,4,5,6,7) -> (0,4,1,5,2,6,3,7), to meet codes4
+                uint4 p;
+                p.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+                p.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+                p.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+                p.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+                v = p;
+            }
+            *reinterpret_cast<uint4 *>(&s_a[buf][row0 + 8u * i][piece * 8u]) = v;
+        }
+    };
+
+    // ---- B rows of this lane
+    const uint8_t *base = cell_base(a.pool, tile.cell, a.stride);
+    const uint32_t row_bytes = K * BITS / 8u;
+    const uint8_t *bw[2];
+    const uint16_t *bs[2], *bb[2];
+    {
+        const uint32_t n = active ? n0 + col : 0u;
+        if (MODE == 0) {
+            bw[0] = base + a.off.gate_w_off + size_t(n) * row_bytes;
+            bw[1] = base + a.off.up_w_off + size_t(n) * row_bytes;
+            bs[0] = reinterpret_cast<const uint16_t *>(base + a.off.gate_s_off) + size_t(n) * G;
+            bs[1] = reinterpret_cast<const uint16_t *>(base + a.off.up_s_off) + size_t(n) * G;
+            bb[0] = reinterpret_cast<const uint16_t *>(base + a.off.gate_b_off) + size_t(n) * G;
+            bb[1] = reinterpret_cast<const uint16_t *>(base + a.off.up_b_off) + size_t(n) * G;
+        } else {
+            const uint32_t n1 = n + 32u;
+            bw[0] = base + a.off.down_w_off + size_t(n) * row_bytes;
+            bw[1] = base + a.off.down_w_off + size_t(n1) * row_bytes;
+            bs[0] = reinterpret_cast<const uint16_t *>(base + a.off.down_s_off) + size_t(n) * G;
+            bs[1] = reinterpret_cast<const uint16_t *>(base + a.off.down_s_off) + size_t(n1) * G;
+            bb[0] = reinterpret_cast<const uint16_t *>(base + a.off.down_b_off) + size_t(n) * G;
+            bb[1] = reinterpret_cast<const uint16_t *>(base + a.off.down_b_off) + size_t(n1) * G;
+        }
+    }
+
+    f32x16 total[2][kMaxMT];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (uint32_t mt = 0; mt < kMaxMT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) total[nt][mt][i] = 0.0f;
+
+    BRegs<BITS> cur[2], nxt[2];
+    if (active) {
+        load_b<BITS>(cur[0], bw[0], bs[0], 0, kb);
+        load_b<BITS>(cur[1], bw[1], bs[1], 0, kb);
+    }
+    const uint32_t chunks = (K + kChunkK - 1u) / kChunkK;
+    fetch(0);
+    commit(0);
+    __syncthreads();
+    for (uint32_t c = 0; c < chunks; ++c) {
+        const uint32_t buf = c & 1u;
+        if (c + 1u < chunks) fetch(c + 1u);
+        const uint32_t groups_here = min(4u, G - 4u * c);
+        if (active) {
+            for (uint32_t gi = 0; gi < groups_here; ++gi) {
+                const uint32_t g = 4u * c + gi;
+                const uint32_t gn = min(g + 1u, G - 1u);
+                load_b<BITS>(nxt[0], bw[0], bs[0], gn, kb);
+                load_b<BITS>(nxt[1], bw[1], bs[1], gn, kb);
+                half8 af[kMaxMT][4];
+#pragma unroll
+                for (uint32_t mt = 0; mt < kMaxMT; ++mt)
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        if (mt < mt_count)
+                            af[mt][s] = *reinterpret_cast<const half8 *>(&s_a[buf][mt * 32u + col][gi * 64u + kb * 32u + s * 8u]);
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) {
+                    half8 bf[4];
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) bf[s] = b_step<BITS>(cur[nt], s);
+                    const float sc = meta_f32(cur[nt].scale, a.meta) * kTwo24;
+#pragma unroll
+                    for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+                        if (mt < mt_count) {
+                            f32x16 p = {0};
+#pragma unroll
+                            for (int s = 0; s < 4; ++s) p = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt][s], bf[s], p, 0, 0, 0);
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) total[nt][mt][i] = fmaf(sc, p[i], total[nt][mt][i]);
+                        }
+                    }
+                }
+                cur[0] = nxt[0];
+                cur[1] = nxt[1];
+            }
+        }
+        if (c + 1u < chunks) commit(buf ^ 1u);
+        __syncthreads();
+    }
+    if (!active) return;
+
+    // ---- bias term: (group sums of the rows) x (group biases), sixteen k' = eight groups a step
+    {
+        const uint32_t *sums = MODE == 0 ? a.hidden_sums : a.act_sums;
+        const uint32_t *sum_row[kMaxMT];
+#pragma unroll
+        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+            const uint32_t r = min(mt * 32u + col, tile.rows - 1u);
+            sum_row[mt] = MODE == 0 ? sums + size_t(a.pairs[tile.pair_start + r].token) * G
+                                    : sums + (size_t(tile_index) * kRowTile + r) * G;
+        }
+        for (uint32_t g0 = 0; g0 < G; g0 += 8u) {
+            const uint32_t gl = g0 + 4u * kb;  // this lane's four groups
+            Frag bfr[2], afr[kMaxMT];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool on = gl + j < G;
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) {
+                    uint16_t bits = on ? bb[nt][gl + j] : uint16_t(0);
+                    if (a.meta == SHRIKE_META_BF16) bits = f32_to_f16(bf16_to_f32(bits));
+                    bfr[nt].u[j] = uint32_t(bits) * 0x00010001u;  // against (hi, lo)
+                }
+#pragma unroll
+                for (uint32_t mt = 0; mt < kMaxMT; ++mt) afr[mt].u[j] = (on && mt < mt_count) ? sum_row[mt][gl + j] : 0u;
+            }
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (uint32_t mt = 0; mt < kMaxMT; ++mt)
+                    if (mt < mt_count) total[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[mt].h, bfr[nt].h, total[nt][mt], 0, 0, 0);
+        }
+    }
+
+    // ---- epilogue: lane holds (m = 32 mt + 8 (i / 4) + 4 kb + i % 4, n = n0 + col)
+    const uint32_t n = n0 + col;
+    if (MODE == 0) {
+        float gab = 0.0f, uab = 0.0f;
+        if (a.ebias) {  // moe.metal:261-269
+            gab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.gate_ab_off)[n]);
+            uab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.up_ab_off)[n]);
+        }
+#pragma unroll
+        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
+                if (mt < mt_count && m < tile.rows) {
+                    const float act = glu_rt(total[0][mt][i] + gab, total[1][mt][i] + uab, a.act_kind);
+                    a.act[(size_t(tile_index) * kRowTile + m) * a.f + n] = f32_to_f16(act);
+                }
+            }
+        }
+    } else {
+        float dab[2] = {0.0f, 0.0f};
+        if (a.ebias) {
+            dab[0] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n]);
+            dab[1] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n + 32u]);
+        }
+#pragma unroll
+        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
+                if (mt < mt_count && m < tile.rows) {
+                    const shrike_token_expert_pair p = a.pairs[tile.pair_start + m];
+                    uint16_t *dst = a.partials + (size_t(p.token) * a.top_k + p.rank) * a.d + n;
+                    dst[0] = f32_to_f16(total[0][mt][i] + dab[0]);
+                    dst[32] = f32_to_f16(total[1][mt][i] + dab[1]);
+                }
+            }
+        }
+    }
+}
+
+int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uint32_t n, uint32_t *out,
+                          const uint32_t *row_limit_tiles, hipStream_t s);
+
+template <int BITS>
+static int launch_ffn(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
+    const dim3 block(256);
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0>), dim3(max_tiles, (a.f + 127u) / 128u), block, 0, s, a);
+    SHRIKE_HIP(hipGetLastError());
+    if (int rc = launch_row_group_sums(a.act, a.f, max_tiles * kRowTile, a.f, const_cast<uint32_t *>(a.act_sums), a.tile_count, s)) return rc;
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1>), dim3(max_tiles, (a.d + 255u) / 256u), block, 0, s, a);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+struct Workspace {
+    size_t hidden_sums, act, act_sums, total;
+};
+static Workspace workspace_layout(uint32_t query_count, uint32_t max_tiles, uint32_t d, uint32_t f) {
+    auto round = [](size_t v) { return (v + 255u) & ~size_t(255); };
+    Workspace w;
+    w.hidden_sums = 0;
+    w.act = round(size_t(query_count) * (d / kGroup) * 4u);
+    w.act_sums = w.act + round(size_t(max_tiles) * kRowTile * f * 2u);
+    w.total = w.act_sums + round(size_t(max_tiles) * kRowTile * (f / kGroup) * 4u);
+    return w;
+}
+
+}  // namespace shrike
+
+using namespace shrike;
+
+extern "C" {
+
+size_t shrike_hip_prefill_ffn_workspace_bytes(uint32_t query_count, uint32_t max_row_tiles, uint32_t d, uint32_t f) {
+    return workspace_layout(query_count, max_row_tiles, d, f).total;
+}
+
+int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                   uint64_t pool_slot_stride, const shrike_expert_offsets *offsets,
+                                   const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles, const void *d_hidden,
+                                   uint32_t hidden_stride_elements, void *d_route_partials, void *d_workspace,
+                                   size_t workspace_bytes, uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k) {
+    SHRIKE_REQUIRE(moe && pool && offsets && routes, "grouped FFN: NULL argument");
+    SHRIKE_REQUIRE(d == moe->desc.d && f == moe->desc.f, "grouped FFN: shape %ux%u differs from the handle's %ux%u", d, f, moe->desc.d, moe->desc.f);
+    SHRIKE_REQUIRE(d % kGroup == 0 && f % kGroup == 0 && d > 0 && f > 0, "D and F must be positive multiples of 64");
+    SHRIKE_REQUIRE(top_k > 0, "topK must be positive");
+    SHRIKE_REQUIRE(hidden_stride_elements >= d && hidden_stride_elements % 8u == 0, "hidden stride is too small or leaves rows unaligned");
+    SHRIKE_REQUIRE(routes->sorted_pairs && routes->row_tiles && routes->row_tile_count, "grouped FFN: routes are not bound");
+    SHRIKE_REQUIRE(d_hidden && d_route_partials && d_workspace, "grouped FFN: NULL buffer");
+    SHRIKE_REQUIRE(reinterpret_cast<uintptr_t>(d_workspace) % 256u == 0, "grouped FFN: workspace must be 256-byte aligned");
+    SHRIKE_REQUIRE(pool->cells_per_chunk > 0 && pool_slot_stride % 16u == 0, "grouped FFN: bad pool geometry");
+    if (int rc = check_offsets(offsets, d, f, moe->desc.routed_weight_bits)) return rc;
+    if (max_row_tiles == 0 || query_count == 0) return 0;
+    const Workspace w = workspace_layout(query_count, max_row_tiles, d, f);
+    SHRIKE_REQUIRE(workspace_bytes >= w.total, "grouped FFN: workspace of %zu bytes, %zu needed", workspace_bytes, w.total);
+    uint8_t *ws = static_cast<uint8_t *>(d_workspace);
+    FfnArgs a = {};
+    fill_pool(a.pool, pool);
+    a.stride = pool_slot_stride;
+    a.off = *offsets;
+    a.tiles = routes->row_tiles;
+    a.tile_count = routes->row_tile_count;
+    a.pairs = static_cast<const shrike_token_expert_pair *>(routes->sorted_pairs);
+    a.hidden = static_cast<const uint16_t *>(d_hidden);
+    a.hidden_stride = hidden_stride_elements;
+    a.hidden_sums = reinterpret_cast<uint32_t *>(ws + w.hidden_sums);
+    a.act = reinterpret_cast<uint16_t *>(ws + w.act);
+    a.act_sums = reinterpret_cast<uint32_t *>(ws + w.act_sums);
+    a.partials = static_cast<uint16_t *>(d_route_partials);
+    a.d = d; a.f = f; a.top_k = top_k;
+    a.meta = moe->desc.meta_dtype;
+    a.act_kind = moe->desc.activation;
+    a.ebias = moe->desc.expert_additive_biases;
+    hipStream_t s = as_stream(stream);
+    if (int rc = launch_row_group_sums(a.hidden, hidden_stride_elements, query_count, d, const_cast<uint32_t *>(a.hidden_sums), nullptr, s)) return rc;
+    return moe->desc.routed_weight_bits == 8 ? launch_ffn<8>(a, max_row_tiles, s) : launch_ffn<4>(a, max_row_tiles, s);
+}
+
+}  // extern "C"
