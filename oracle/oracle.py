@@ -268,3 +268,34 @@ def moe_decode_layer(x_f16, hidden_f16, router, pool_blobs, residency_u64, off, 
                    additive_biases=additive_biases, hidden_f16=hidden)
     return dict(logits=logits, indices=idx, weights=w, classify=cls, h1=h1, acts=acts, y=y,
                 hidden=hidden)
+
+
+# ------------------------------------------------------------------ prefill (composition)
+
+def prefill_router(router, hidden_f16, query_count, d, top_k, stride=None, sigmoid=False, scaling=1.0):
+    """The router for query_count tokens, token by token with the decode functions
+    (sources/Shrike/Metal/Prefill/prefill.metal:369-563 computes the same per token).
+    Returns (indices u32[T*K], weights f16 bits[T*K], logits f32[T, E])."""
+    stride = d if stride is None else stride
+    ne = router["expert_scale"].shape[0]
+    idx = np.empty(query_count * top_k, np.uint32)
+    w = np.empty(query_count * top_k, np.uint16)
+    logits = np.empty((query_count, ne), np.float32)
+    for t in range(query_count):
+        x = np.ascontiguousarray(hidden_f16[t * stride:t * stride + d])
+        logits[t] = router_logits(router["weights"], router.get("scales"), router.get("biases"), router["kind"], x,
+                                  router["eff_scale"], ne, d, meta=router.get("meta", META_BF16))
+        i, ww = router_select(logits[t], router["expert_scale"], router["bias"], top_k, sigmoid, scaling)
+        idx[t * top_k:(t + 1) * top_k], w[t * top_k:(t + 1) * top_k] = i, ww
+    return idx, w, logits
+
+
+def prefill_pair_partial(blob, off, x_f16, d, f, bits=4, meta=META_BF16, act=ACT_SILU, additive_biases=False):
+    """One (token, expert) pair's partial row as the reference's scalar model computes it
+    (tests/Shrike/Core/Kernels/Prefill/PrefillGroupedRoutedMoETests.swift:368-473): gate and up
+    in fp32, act rounded to fp16, down in fp32, the row rounded to fp16. A phase-2 pass with
+    weight 1 and residual 0 gives exactly that rounding."""
+    acts = moe_phase1([blob], off, x_f16, d, f, bits, meta, act, additive_biases)
+    one = np.array([0x3C00], np.uint16)
+    zero = np.zeros(d, np.uint16)
+    return moe_phase2([blob], off, acts, one, zero, d, f, bits, meta, additive_biases)

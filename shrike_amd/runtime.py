@@ -260,3 +260,72 @@ class MoE:
     def encode_decode_layer(self, args: DecodeLayerArgs):
         check(capi.load().shrike_hip_moe_decode_layer(self.handle, self._s(), C.byref(args)),
               "shrike_hip_moe_decode_layer")
+
+
+class GroupedRoutesDevice:
+    """Device buffers of shrike_hip_grouped_routes for up to `pairs` pairs over `num_experts`."""
+
+    def __init__(self, pairs: int, num_experts: int):
+        self.pairs, self.num_experts = pairs, num_experts
+        self.max_row_tiles = capi.load().shrike_hip_group_max_row_tiles(pairs, num_experts)
+        self.sorted_pairs = empty(max(1, pairs) * 16)
+        self.offsets = empty(num_experts * 4)
+        self.counts = empty(num_experts * 4)
+        self.row_tiles = empty(max(1, self.max_row_tiles) * 16)
+        self.row_tile_count = empty(4).fill(0)
+        self.c = capi.HipGroupedRoutes(ptr(self.sorted_pairs), ptr(self.offsets), ptr(self.counts),
+                                       ptr(self.row_tiles), ptr(self.row_tile_count))
+
+    def download(self):
+        n = int(self.row_tile_count.download(np.uint32, 1)[0])
+        return dict(sorted_pairs=self.sorted_pairs.download(np.uint32, self.pairs * 4).reshape(-1, 4),
+                    offsets=self.offsets.download(np.uint32, self.num_experts),
+                    counts=self.counts.download(np.uint32, self.num_experts),
+                    row_tiles=self.row_tiles.download(np.uint32, n * 4).reshape(-1, 4), row_tile_count=n)
+
+
+class Prefill:
+    """The prefill operators of the routed path with the reference's names: PrefillRouter.encodeBlock,
+    PrefillMoEGrouping on the device, PrefillGroupedRoutedMoE.encodeGroupedExpertGEMMs,
+    PrefillMoE.encodeReduceTokenMajor."""
+
+    def __init__(self, moe: MoE):
+        self.moe = moe
+
+    def _s(self):
+        return self.moe._s()
+
+    def encode_block(self, weights, scales, biases, hidden, effective_scale, per_expert_scale, logit_bias,
+                     out_indices, out_weights, logits_workspace, query_count, num_experts, d, top_k,
+                     hidden_stride_elements):
+        check(capi.load().shrike_hip_prefill_router(
+            self.moe.handle, self._s(), ptr(weights), ptr(scales), ptr(biases), ptr(hidden), ptr(effective_scale),
+            ptr(per_expert_scale), ptr(logit_bias), ptr(out_indices), ptr(out_weights), ptr(logits_workspace),
+            query_count, num_experts, d, top_k, hidden_stride_elements), "shrike_hip_prefill_router")
+
+    def group_pairs(self, indices, weights, query_count, top_k, num_experts, routes: GroupedRoutesDevice,
+                    expert_sort_keys=None, residency=None):
+        check(capi.load().shrike_hip_group_pairs(self._s(), ptr(indices), ptr(weights), query_count, top_k, num_experts,
+                                                 ptr(expert_sort_keys), ptr(residency), C.byref(routes.c)),
+              "shrike_hip_group_pairs")
+
+    def ffn_workspace_bytes(self, query_count, max_row_tiles):
+        return capi.load().shrike_hip_prefill_ffn_workspace_bytes(query_count, max_row_tiles, self.moe.desc.d,
+                                                                  self.moe.desc.f)
+
+    def encode_grouped_expert_gemms(self, pool: ExpertPool, offsets, routes: GroupedRoutesDevice, hidden,
+                                    hidden_stride_elements, route_partials, workspace: DeviceBuffer, query_count,
+                                    top_k, max_row_tiles=None):
+        check(capi.load().shrike_hip_prefill_grouped_ffn(
+            self.moe.handle, self._s(), pool.bases, pool.stride, C.byref(offsets), C.byref(routes.c),
+            routes.max_row_tiles if max_row_tiles is None else max_row_tiles, ptr(hidden), hidden_stride_elements,
+            ptr(route_partials), ptr(workspace), workspace.nbytes, query_count, self.moe.desc.d, self.moe.desc.f, top_k),
+            "shrike_hip_prefill_grouped_ffn")
+
+    def encode_reduce_token_major(self, route_partials, route_weights, h2, query_count, top_k, d):
+        check(capi.load().shrike_hip_prefill_reduce(self._s(), ptr(route_partials), ptr(route_weights), ptr(h2),
+                                                    query_count, top_k, d), "shrike_hip_prefill_reduce")
+
+    def residual_add(self, hidden, delta, count):
+        check(capi.load().shrike_hip_residual_add_f16(self._s(), ptr(hidden), ptr(delta), count),
+              "shrike_hip_residual_add_f16")

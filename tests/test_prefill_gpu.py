@@ -1,0 +1,300 @@
+"""GPU parity of the prefill operators behind the C ABI: the router for a token block, the
+device grouping, the grouped expert FFN on the matrix cores, the token-major reduce and the
+residual add. Indices, permutations, tables and the reduce are compared bit for bit; FFN
+partial rows within max-abs 2e-3 / relative 1e-3 (|a-b| <= 2e-3 + 1e-3*|b|)."""
+import numpy as np
+import pytest
+
+from oracle import host_logic as H
+from oracle import oracle as O
+from shrike_amd import capi
+from shrike_amd import host as HL
+from shrike_amd import synth as S
+from tests.helpers import Layer, assert_ffn_close, assert_rel_close, f16
+from tests.test_decode_gpu import DeviceLayer
+
+pytestmark = pytest.mark.gpu
+SENT = 0xFFFFFFFF
+
+
+def token_rows(L: Layer, t: int, stride: int, label="prefill.x"):
+    """fp16[T, stride] activations; the tail of each row past d is filler that must not be read."""
+    x = S.activations_f16(L.tree, label, t * stride).reshape(t, stride).copy()
+    x[:, L.d:] = 0x7E00  # NaN: any use shows
+    return x.reshape(-1)
+
+
+def run_router(gpu, dl, L, hidden, t, stride):
+    pf = gpu.Prefill(dl.moe)
+    idx, w = gpu.empty(4 * t * L.k), gpu.empty(2 * t * L.k)
+    ws = gpu.empty(4 * t * L.ne)
+    pf.encode_block(dl.router_w, dl.router_s, dl.router_b, hidden, dl.eff_scale, dl.expert_scale, dl.logit_bias,
+                    idx, w, ws, t, L.ne, L.d, L.k, stride)
+    gpu.synchronize()
+    return pf, idx, w, ws
+
+
+@pytest.mark.parametrize("router_bits,ne,d,k,t,pad", [(0, 256, 2048, 8, 48, 0), (0, 256, 2048, 8, 5, 64), (8, 32, 2880, 4, 9, 8),
+                                                      (4, 64, 512, 8, 33, 0), (8, 256, 2304, 8, 1, 0)])
+def test_prefill_router_bit_exact_and_equal_to_decode(gpu, router_bits, ne, d, k, t, pad):
+    L = Layer(0x5EED0003 + router_bits, d, 64, ne, k, router_bits=router_bits)
+    L.logit_bias = S.f32_to_bf16_bits(L.tree.key("bias").normal(ne, std=0.01))
+    L.expert_scale = S.f32_to_bf16_bits(L.tree.key("escale").uniform(0.6, 1.4, ne))
+    dl = DeviceLayer(gpu, L, resident=[])
+    stride = d + pad
+    x = token_rows(L, t, stride)
+    hidden = gpu.dev(x)
+    pf, idx, w, ws = run_router(gpu, dl, L, hidden, t, stride)
+    ref_idx, ref_w, ref_logits = O.prefill_router(L.router_dict(), x, t, d, k, stride=stride)
+    logits = ws.download(np.float32, t * ne).reshape(t, ne)
+    assert np.array_equal(logits.view(np.uint32), ref_logits.view(np.uint32)), "prefill logits differ in bits"
+    got_idx, got_w = idx.download(np.uint32, t * k), w.download(np.uint16, t * k)
+    assert np.array_equal(got_idx, ref_idx)
+    assert np.max(np.abs(f16(got_w) - f16(ref_w))) <= 1e-3
+    # the decode router on the same token gives the same bytes
+    for tok in sorted({0, t // 2, t - 1}):
+        one = gpu.dev(np.ascontiguousarray(x[tok * stride:tok * stride + d]))
+        dl.moe.encode_router(dl.router_w, dl.router_s, dl.router_b, one, dl.eff_scale, dl.expert_scale, dl.logit_bias,
+                             dl.out_idx, dl.out_w, ne, d, k)
+        assert np.array_equal(dl.out_idx.download(np.uint32, k), got_idx[tok * k:(tok + 1) * k])
+        assert np.array_equal(dl.out_w.download(np.uint16, k), got_w[tok * k:(tok + 1) * k])
+
+
+def random_routes(seed, t, k, ne, skew=1.2):
+    rng = np.random.default_rng(seed)
+    p = 1.0 / np.arange(1, ne + 1) ** skew
+    p = rng.permutation(p / p.sum())
+    idx = np.concatenate([rng.choice(ne, size=k, replace=False, p=p) for _ in range(t)]).astype(np.uint32) if t else np.zeros(0, np.uint32)
+    w = rng.integers(0, 0x3C00, size=t * k).astype(np.uint16)
+    return idx, w
+
+
+def expected_row_tiles(groups, cell_of):
+    tiles = []
+    for e, start, count in groups:
+        for j in range(0, count, 64):
+            tiles.append((cell_of(e), start + j, min(64, count - j), e))
+    return tiles
+
+
+@pytest.mark.parametrize("t,k,ne,mode", [(512, 8, 256, "plain"), (512, 8, 256, "keys"), (37, 3, 17, "plain"), (64, 4, 32, "residency"),
+                                         (1, 8, 256, "plain"), (300, 2, 4, "keys"), (0, 8, 16, "plain")])
+def test_device_grouping_equals_host_grouping(gpu, t, k, ne, mode):
+    idx, w = random_routes(t * 131 + k, t, k, ne)
+    keys = None
+    residency = None
+    cell_of = lambda e: e
+    if mode == "keys":
+        order = np.random.default_rng(9).permutation(ne)[: max(1, ne // 2)].astype(np.uint32)
+        keys = HL.expert_sort_keys(order, ne)
+    if mode == "residency":
+        words = np.array([H.residency_word(H.RESIDENT, 100 + e) if e % 3 else H.residency_word(H.LOADING if e % 2 else H.EMPTY, e)
+                          for e in range(ne)], np.uint64)
+        residency = gpu.dev(words)
+        cell_of = lambda e: 100 + e if e % 3 else SENT
+    routes = gpu.GroupedRoutesDevice(t * k, ne)
+    pf = gpu.Prefill(gpu.MoE(64, 64, ne, min(k, 8)))
+    pf.group_pairs(gpu.dev(idx) if t else None, gpu.dev(w) if t else None, t, k, ne, routes,
+                   expert_sort_keys=None if keys is None else gpu.dev(keys), residency=residency)
+    gpu.synchronize()
+    got = routes.download()
+    pairs = HL.make_token_expert_pairs(idx, w, t, k)
+    host = HL.group_token_expert_pairs(pairs, t, k, ne, 16, keys)
+    ref = H.group_token_expert_pairs(H.make_token_expert_pairs(idx, w, t, k), t, k, ne, 16, None if keys is None else keys.tolist())
+    assert got["counts"].tolist() == ref.per_expert_counts == host.per_expert_counts.tolist()
+    assert got["offsets"].tolist() == ref.per_expert_offsets == host.per_expert_offsets.tolist()
+    assert [tuple(r) for r in got["sorted_pairs"].tolist()] == [p.as_tuple() for p in ref.sorted_pairs]
+    assert [tuple(r) for r in got["row_tiles"].tolist()] == expected_row_tiles(ref.groups, cell_of)
+    assert got["row_tile_count"] <= routes.max_row_tiles
+
+
+class PrefillCase:
+    def __init__(self, gpu, L: Layer, t, stride_pad=0, idx=None, moe_kwargs=None, resident=None):
+        self.gpu, self.L, self.t = gpu, L, t
+        self.dl = DeviceLayer(gpu, L, moe_kwargs=moe_kwargs, resident=resident)
+        self.stride = L.d + stride_pad
+        self.x = token_rows(L, t, self.stride)
+        self.hidden = gpu.dev(self.x)
+        self.pf = gpu.Prefill(self.dl.moe)
+        if idx is None:
+            idx, w = random_routes(t + L.ne, t, L.k, L.ne)
+        else:
+            w = np.random.default_rng(1).integers(0x3000, 0x3C00, size=t * L.k).astype(np.uint16)
+        self.idx, self.w = idx, w
+        self.routes = gpu.GroupedRoutesDevice(t * L.k, L.ne)
+        self.d_idx, self.d_w = gpu.dev(idx), gpu.dev(w)
+        self.pf.group_pairs(self.d_idx, self.d_w, t, L.k, L.ne, self.routes, residency=self.dl.pool.table)
+        self.partials = gpu.dev(np.full(t * L.k * L.d, 0xD4D0, np.uint16))  # -77: rows nobody writes keep it
+        self.ws = gpu.empty(self.pf.ffn_workspace_bytes(t, self.routes.max_row_tiles))
+
+    def run(self):
+        self.pf.encode_grouped_expert_gemms(self.dl.pool, self.dl.off, self.routes, self.hidden, self.stride, self.partials,
+                                            self.ws, self.t, self.L.k)
+        self.gpu.synchronize()
+        return self.partials.download(np.uint16, self.t * self.L.k * self.L.d).reshape(self.t, self.L.k, self.L.d)
+
+    def oracle_row(self, tok, rank, act=O.ACT_SILU):
+        L = self.L
+        x = np.ascontiguousarray(self.x[tok * self.stride:tok * self.stride + L.d])
+        return O.prefill_pair_partial(L.blobs[int(self.idx[tok * L.k + rank])], L.oracle_offsets(), x, L.d, L.f, L.bits, L.meta,
+                                      act, L.additive)
+
+    def device_act(self, tok, rank):
+        """The pair's fp16 activation row in the workspace: row tile j keeps rows [64 j, 64 j + 64)."""
+        L = self.L
+        if not hasattr(self, "_tables"):
+            self._tables = self.routes.download()
+            act_off = (self.t * (L.d // 64) * 4 + 255) & ~255
+            rows = self.routes.max_row_tiles * 64
+            self._act = self.ws.download(np.uint16, rows * L.f, offset=act_off).reshape(rows, L.f)
+            self._pos = {(int(r[0]), int(r[2])): i for i, r in enumerate(self._tables["sorted_pairs"])}
+        at = self._pos[(tok, rank)]
+        for j, (cell, start, rows, expert) in enumerate(self._tables["row_tiles"].tolist()):
+            if start <= at < start + rows:
+                return self._act[j * 64 + at - start]
+        raise AssertionError("pair not covered by a row tile")
+
+    def check_pair(self, got, tok, rank, what, act=O.ACT_SILU):
+        """Stage by stage, so that each comparison holds one rounding: the activations against the
+        oracle's, the partial row against the oracle's down projection of the device's own
+        activations; then the whole chain in the reference's relative-error metric."""
+        L = self.L
+        blob, off = L.blobs[int(self.idx[tok * L.k + rank])], L.oracle_offsets()
+        x = np.ascontiguousarray(self.x[tok * self.stride:tok * self.stride + L.d])
+        dev_act = np.ascontiguousarray(self.device_act(tok, rank))
+        assert_ffn_close(dev_act, O.moe_phase1([blob], off, x, L.d, L.f, L.bits, L.meta, act, L.additive), f"{what}: activations")
+        one, zero = np.array([0x3C00], np.uint16), np.zeros(L.d, np.uint16)
+        assert_ffn_close(got[tok, rank], O.moe_phase2([blob], off, dev_act, one, zero, L.d, L.f, L.bits, L.meta, L.additive),
+                         f"{what}: partial row from the device's activations")
+        assert_rel_close(got[tok, rank], self.oracle_row(tok, rank, act), f"{what}: whole chain")
+
+
+FFN_CASES = [
+    # name, d, f, experts, k, tokens, bits, meta, stride pad
+    ("small-int4", 512, 256, 16, 4, 40, 4, S.META_BF16, 0),
+    ("small-int8-f16meta", 512, 256, 16, 4, 40, 8, S.META_F16, 8),
+    ("q-shape-int4-f16meta", 2048, 512, 24, 8, 20, 4, S.META_F16, 0),
+    ("q-shape-int8", 2048, 512, 12, 4, 12, 8, S.META_BF16, 0),
+    ("long-experts-two-tiles", 256, 128, 3, 2, 110, 4, S.META_BF16, 0),
+    ("ragged-k-192x320", 192, 320, 8, 3, 50, 4, S.META_F16, 0),
+    ("kimi-shape-int8", 2304, 1024, 8, 2, 6, 8, S.META_BF16, 0),
+]
+
+
+@pytest.mark.parametrize("case", FFN_CASES, ids=[c[0] for c in FFN_CASES])
+def test_grouped_ffn_against_oracle(gpu, case):
+    name, d, f, ne, k, t, bits, meta, pad = case
+    L = Layer(0x5EED0003, d, f, ne, k, bits=bits, meta=meta)
+    pc = PrefillCase(gpu, L, t, stride_pad=pad)
+    got = pc.run()
+    rng = np.random.default_rng(4)
+    sample = [(int(a), int(b)) for a, b in zip(rng.integers(0, t, 40), rng.integers(0, k, 40))] if t * k > 48 else \
+        [(a, b) for a in range(t) for b in range(k)]
+    for tok, rank in sample:
+        pc.check_pair(got, tok, rank, f"{name} token {tok} rank {rank}")
+    assert not np.any(np.all(got == 0xD4D0, axis=-1)), "a pair's partial row was left unwritten"
+
+
+def test_grouped_ffn_gpt_oss_epilogues(gpu):
+    # additive biases + clamped SwiGLU at the gpt-oss shape (moe.metal:257-288), 45 groups per row
+    d = f = 2880
+    L = Layer(0x5EED0004, d, f, 3, 2, bits=4, additive_biases=True)
+    pc = PrefillCase(gpu, L, 5, moe_kwargs=dict(activation=capi.ACT_CLAMPED_SWIGLU, additive_biases=True))
+    got = pc.run()
+    for tok in range(5):
+        for rank in range(2):
+            pc.check_pair(got, tok, rank, f"gpt-oss token {tok} rank {rank}", O.ACT_CLAMPED_SWIGLU)
+
+
+def test_grouped_ffn_skips_absent_experts(gpu):
+    L = Layer(0x5EED0005, 256, 128, 8, 2, bits=4)
+    pc = PrefillCase(gpu, L, 30, resident=[0, 1, 2, 4, 5, 7])
+    got = pc.run()
+    for tok in range(30):
+        for rank in range(2):
+            e = int(pc.idx[tok * 2 + rank])
+            if e in (3, 6):
+                assert np.all(got[tok, rank] == 0xD4D0)
+            elif tok % 5 == 0:
+                pc.check_pair(got, tok, rank, f"token {tok} rank {rank}")
+            else:
+                assert not np.all(got[tok, rank] == 0xD4D0)
+
+
+def test_one_pair_expert_leaves_other_rows_alone(gpu):
+    # PrefillGroupedRoutedMoETests+Execution.swift:657-763: a single 1-pair expert; the padded
+    # rows of its tile must not leave the staging block
+    L = Layer(0x5EED0006, 512, 512, 8, 1, bits=4)
+    pc = PrefillCase(gpu, L, 1, idx=np.array([5], np.uint32))
+    guard = pc.gpu.dev(np.full(64 * 512, 0xD4D0, np.uint16))
+    got = pc.run()
+    pc.check_pair(got, 0, 0, "single pair")
+    assert np.all(guard.download(np.uint16, 64 * 512) == 0xD4D0)
+
+
+def test_reduce_and_residual_bit_exact(gpu):
+    rng = np.random.default_rng(12)
+    for t, k, d in ((7, 8, 2048), (33, 4, 2880), (1, 1, 64)):
+        partials = S.f32_to_f16_bits(rng.standard_normal(t * k * d).astype(np.float32))
+        weights = S.f32_to_f16_bits(rng.random(t * k).astype(np.float32))
+        pf = gpu.Prefill(gpu.MoE(64, 64, 8, 1))
+        h2 = gpu.empty(2 * t * d)
+        pf.encode_reduce_token_major(gpu.dev(partials), gpu.dev(weights), h2, t, k, d)
+        gpu.synchronize()
+        ref = O.prefill_reduce(partials, weights, t, k, d)
+        assert np.array_equal(h2.download(np.uint16, t * d), ref)
+        hidden = S.f32_to_f16_bits(rng.standard_normal(t * d).astype(np.float32))
+        dh = gpu.dev(hidden)
+        pf.residual_add(dh, h2, t * d)
+        gpu.synchronize()
+        assert np.array_equal(dh.download(np.uint16, t * d), O.residual_add_f16(hidden.copy(), ref))
+
+
+def test_prefill_layer_at_full_size_agrees_with_the_decode_kernels(gpu):
+    """T = 512 tokens, 256 experts, top 8 at the 35B-A3B int4 shape: too large for the CPU oracle,
+    so the whole chain (router -> grouping -> grouped FFN -> reduce) is checked by what does not
+    depend on size: the grouping is a permutation with the host function's tables, and every
+    sampled token's h2 equals the decode kernels' y for that token alone (no shared expert,
+    residual 0), which the decode tests hold to the oracle."""
+    d, f, ne, k, t = 2048, 512, 256, 8, 512
+    L = Layer(0x5EED0003, d, f, ne, k, bits=4, meta=S.META_F16)
+    # Zipf skew through the logit bias operand, over a seeded permutation
+    perm = np.argsort(L.tree.key("zipf.perm").next(ne))
+    bias = np.zeros(ne, np.float32)
+    bias[perm] = -1.1 * np.log(np.arange(ne) + 1.0)
+    L.logit_bias = S.f32_to_bf16_bits(bias)
+    dl = DeviceLayer(gpu, L)
+    x = token_rows(L, t, d)
+    hidden = gpu.dev(x)
+    pf, idx, w, ws = run_router(gpu, dl, L, hidden, t, d)
+    routes = gpu.GroupedRoutesDevice(t * k, ne)
+    pf.group_pairs(idx, w, t, k, ne, routes, residency=dl.pool.table)
+    partials = gpu.dev(np.full(t * k * d, 0xD4D0, np.uint16))
+    work = gpu.empty(pf.ffn_workspace_bytes(t, routes.max_row_tiles))
+    pf.encode_grouped_expert_gemms(dl.pool, dl.off, routes, hidden, d, partials, work, t, k)
+    h2 = gpu.empty(2 * t * d)
+    pf.encode_reduce_token_major(partials, w, h2, t, k, d)
+    gpu.synchronize()
+    h_idx, h_w = idx.download(np.uint32, t * k), w.download(np.uint16, t * k)
+    got = routes.download()
+    host = HL.group_token_expert_pairs(HL.make_token_expert_pairs(h_idx, h_w, t, k), t, k, ne)
+    assert got["counts"].tolist() == host.per_expert_counts.tolist() and int(got["counts"].sum()) == t * k
+    assert got["offsets"].tolist() == host.per_expert_offsets.tolist()
+    assert np.array_equal(got["sorted_pairs"], host.sorted_pairs.view(np.uint32).reshape(-1, 4))
+    out = h2.download(np.uint16, t * d).reshape(t, d)
+    assert not np.any(np.all(partials.download(np.uint16, t * k * d).reshape(t * k, d) == 0xD4D0, axis=-1))
+    zero = gpu.dev(np.zeros(d, np.uint16))
+    for tok in (0, 1, 77, 255, 256, 511):
+        one = gpu.dev(np.ascontiguousarray(x[tok * d:(tok + 1) * d]))
+        dl.moe.encode_router(dl.router_w, None, None, one, dl.eff_scale, dl.expert_scale, dl.logit_bias, dl.out_idx, dl.out_w, ne, d, k)
+        assert np.array_equal(dl.out_idx.download(np.uint32, k), h_idx[tok * k:(tok + 1) * k])
+        cells = np.array([dl.cell_of[int(e)] for e in h_idx[tok * k:(tok + 1) * k]], np.uint32)
+        dl.moe.encode_spec_phase1(dl.pool, gpu.dev(cells), dl.off, one, dl.acts, d, f, k)
+        hid = gpu.dev(np.zeros(d, np.uint16))
+        dl.moe.encode_spec_phase2(dl.pool, gpu.dev(cells), dl.off, dl.acts, dl.out_w, zero, dl.y, hid, d, f, k)
+        gpu.synchronize()
+        # The decode kernel rounds the fp32 sum over the experts once; prefill rounds each of the
+        # eight partial rows to fp16 first (as the reference does), so single elements of a
+        # cancelling sum move by a few fp16 steps of the largest partial: compared in the
+        # reference's relative-error metric.
+        assert_rel_close(out[tok], dl.y.download(np.uint16, d), f"token {tok}: prefill h2 vs decode y", tol=2e-3)
