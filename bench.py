@@ -131,6 +131,88 @@ def cpu_baseline(S, blobs, sample_layers, meta):
                       f"{cores} threads, gcc -O2"}
 
 
+def prefill_main(args, rt, capi, S, meta):
+    """Config 3: one ragged prefill chunk of T tokens through router -> grouping -> grouped expert FFN
+    -> reduce, top-8 of 256 int4 experts with a Zipf skew injected through the router's logit-bias
+    operand. Steps alternate between layers with their own pools so the experts stream from HBM."""
+    T = args.tokens
+    n_layers = min(args.layers, 3)
+    layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta, shared=False)
+    moe = rt.MoE(D, F, NE, K, routed_bits=BITS, router_bits=0, meta=meta)
+    stream = rt.Stream()
+    moe.stream = stream
+    pf = rt.Prefill(moe)
+    tree = S.SeedTree(0x5EED0003)
+    perm = np.argsort(tree.key("zipf.perm").next(NE))
+    bias = np.zeros(NE, np.float32)
+    bias[perm] = -1.1 * np.log(np.arange(NE) + 1.0)
+    d_bias = rt.dev(S.f32_to_bf16_bits(bias))
+    ones_d, ones_e = keep[0], keep[1]
+    hidden = rt.dev(S.activations_f16(tree, "x", T * D))
+    idx, w, logits = rt.empty(4 * T * K), rt.empty(2 * T * K), rt.empty(pf.router_workspace_bytes(T, NE, D))
+    routes = rt.GroupedRoutesDevice(T * K, NE)
+    partials, h2 = rt.empty(2 * T * K * D), rt.empty(2 * T * D)
+    work = rt.empty(pf.ffn_workspace_bytes(T, routes.max_row_tiles))
+
+    def router(lay):
+        pf.encode_block(lay["router"], None, None, hidden, ones_d, ones_e, d_bias, idx, w, logits, T, NE, D, K, D)
+
+    def group(lay):
+        pf.group_pairs(idx, w, T, K, NE, routes, residency=lay["pool"].table)
+
+    def ffn(lay):
+        pf.encode_grouped_expert_gemms(lay["pool"], off, routes, hidden, D, partials, work, T, K)
+
+    def reduce(lay):
+        pf.encode_reduce_token_major(partials, w, h2, T, K, D)
+
+    def step(lay):
+        router(lay); group(lay); ffn(lay); reduce(lay)
+
+    def timed(fn, n):
+        start, stop = rt.Event(), rt.Event()
+        stream.synchronize()
+        start.record(stream)
+        for i in range(n):
+            fn(layers[i % n_layers])
+        stop.record(stream)
+        stop.synchronize()
+        return start.elapsed_ms(stop) / n
+
+    steps, warm = max(1, args.steps // 40), max(1, args.warmup // 40)
+    timed(step, warm)
+    ms = timed(step, steps)
+    parts = {name: timed(fn, max(4, steps // 2)) * 1e3 for name, fn in
+             (("router (2 launches)", router), ("grouping (2 launches)", group), ("grouped FFN (4 launches)", ffn), ("reduce", reduce))}
+    rt.synchronize()
+    counts = routes.counts.download(np.uint32, NE)
+    tiles = int(routes.row_tile_count.download(np.uint32, 1)[0])
+    used = int(np.count_nonzero(counts))
+    m_tiles = int(sum((min(64, c - j) + 31) // 32 for c in counts.tolist() for j in range(0, c, 64)))
+    expert_bytes = used * stride
+    algorithmic = expert_bytes + 2 * T * D * 2 + T * K * 16
+    flops = T * K * 6 * D * F
+    ffn_us = parts["grouped FFN (4 launches)"]
+    out = {
+        "metric": "ragged prefill chunk through the routed experts: tokens/s (ms per chunk in ms_per_step), 35B-A3B int4 shape",
+        "value": round(T / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 x u4 -> f32",
+        "data": "synthetic (seeded SplitMix64: uniform int4 codes, |N(0,0.02)| scales, N(0,1) fp16 activations, Zipf(1.1) expert skew)",
+        "config": {"workload": f"config 3: ragged prefill, {T} tokens, top-8 of 256 int4 experts (hidden 2048, intermediate 512), "
+                               "router + device grouping + grouped FFN + reduce, all slots resident",
+                   "stacked_layers": n_layers, "meta_dtype": args.meta, "experts_with_pairs": used, "row_tiles": tiles,
+                   "mfma_row_tiles_of_32": m_tiles},
+        "kernel_us_per_chunk": {k: round(v, 2) for k, v in parts.items()},
+        "roofline": {"bound": "hbm", "kernel": "k_grouped_ffn<4,0> + k_grouped_ffn<4,1> (gate/up + down of every row tile)",
+                     "achieved": round(expert_bytes / (ffn_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(expert_bytes / (ffn_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "bytes_per_launch": expert_bytes,
+                     "us_per_launch": round(ffn_us, 2), "traffic": None,
+                     "mfma_tflops_on_pair_flops": round(flops / (ffn_us * 1e-6) / 1e12, 2)},
+        "algorithmic_bytes_per_chunk": algorithmic, "pair_flops_per_chunk": flops,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -140,6 +222,9 @@ def main():
     ap.add_argument("--meta", choices=["f16", "bf16"], default="f16")
     ap.add_argument("--cpu-sample", type=int, default=60, help="layer evaluations timed on the CPU (0 = skip)")
     ap.add_argument("--no-shared", action="store_true", help="diagnostic: leave the shared expert out of the layer")
+    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
+                    help="decode: the headline metric (config 2); prefill: the ragged 512-token chunk (config 3)")
+    ap.add_argument("--tokens", type=int, default=512, help="prefill: tokens in the chunk")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path is built and measured on a single MI355X "
@@ -151,6 +236,8 @@ def main():
 
     rt.init(0)
     meta = S.META_F16 if args.meta == "f16" else S.META_BF16
+    if args.workload == "prefill":
+        return prefill_main(args, rt, capi, S, meta)
     n_layers = args.layers
     layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta, shared=not args.no_shared)
     moe = rt.MoE(D, F, NE, K, routed_bits=BITS, router_bits=0, meta=meta)

@@ -239,13 +239,16 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
  * the router for query_count tokens. hidden: fp16[query_count, hidden_stride_elements]
  * (row t at t * stride); out_indices: u32[query_count * top_k]; out_weights:
  * fp16[query_count * top_k], token-major. Every token's logits and selection are
- * bit-identical to shrike_hip_moe_router on that token alone. d_logits_workspace:
- * fp32[query_count * num_experts], caller-owned. */
+ * bit-identical to shrike_hip_moe_router on that token alone. d_workspace is
+ * caller-owned, 16-byte aligned, shrike_hip_prefill_router_workspace_bytes() long;
+ * the fp32 logits [query_count, num_experts] are left at its start. */
+size_t shrike_hip_prefill_router_workspace_bytes(uint32_t query_count, uint32_t num_experts,
+                                                 uint32_t d);
 int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_weights,
                               const void *d_scales, const void *d_biases, const void *d_hidden,
                               const void *d_effective_scale, const void *d_per_expert_scale,
                               const void *d_logit_bias, uint32_t *d_out_indices,
-                              void *d_out_weights, float *d_logits_workspace,
+                              void *d_out_weights, float *d_workspace,
                               uint32_t query_count, uint32_t num_experts, uint32_t d,
                               uint32_t top_k, uint32_t hidden_stride_elements);
 

@@ -181,6 +181,7 @@ SIGNATURES = {
     # prefill operators
     "shrike_hip_prefill_router": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                             _U32, _U32, _U32, _U32, _U32]),
+    "shrike_hip_prefill_router_workspace_bytes": (C.c_size_t, [_U32, _U32, _U32]),
     "shrike_hip_group_max_row_tiles": (_U32, [_U64, _U32]),
     "shrike_hip_group_pairs": (C.c_int, [_VP, _VP, _VP, _U32, _U32, _U32, _VP, _VP, C.POINTER(HipGroupedRoutes)]),
     "shrike_hip_prefill_ffn_workspace_bytes": (C.c_size_t, [_U32, _U32, _U32, _U32]),

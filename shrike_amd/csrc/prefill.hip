@@ -30,6 +30,88 @@ __global__ __launch_bounds__(256) void k_prefill_logits(RouterArgs a, uint32_t q
     }
 }
 
+// The fp16 router's fast path. x * effective_scale is the same for every expert, so it is
+// formed once per token (k_prefill_scale_x, the product router_row forms per row); a wave
+// then keeps its expert's row in registers as fp32 and walks a block of tokens, two at a time.
+// The additions are router_row's, in router_row's order, so the logits are the same bits.
+constexpr uint32_t kFastTokenBlock = 32;
+
+__global__ __launch_bounds__(256) void k_prefill_scale_x(const uint16_t *hidden, const uint16_t *eff, float *xs,
+                                                         uint32_t query_count, uint32_t d, uint32_t stride) {
+    const size_t slot = size_t(blockIdx.x) * 256u + threadIdx.x;  // eight elements each
+    const uint32_t per_row = d / 8u;
+    const uint32_t t = uint32_t(slot / per_row);
+    if (t >= query_count) return;
+    const uint32_t c = uint32_t(slot - size_t(t) * per_row);
+    const uint4 xv = *reinterpret_cast<const uint4 *>(hidden + size_t(t) * stride + size_t(c) * 8u);
+    const uint4 ev = *reinterpret_cast<const uint4 *>(eff + size_t(c) * 8u);
+    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, ew[4] = {ev.x, ev.y, ev.z, ev.w};
+    float o[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {  // moe.metal:357-358 (exact product)
+        o[2 * j] = __fmul_rn(f16_to_f32(uint16_t(xw[j])), bf16_to_f32(uint16_t(ew[j])));
+        o[2 * j + 1] = __fmul_rn(f16_to_f32(uint16_t(xw[j] >> 16)), bf16_to_f32(uint16_t(ew[j] >> 16)));
+    }
+    float4 *dst = reinterpret_cast<float4 *>(xs + size_t(t) * d + size_t(c) * 8u);
+    dst[0] = make_float4(o[0], o[1], o[2], o[3]);
+    dst[1] = make_float4(o[4], o[5], o[6], o[7]);
+}
+
+__global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits,
+                                                            uint32_t query_count, uint32_t num_experts, uint32_t d) {
+    constexpr int MAXI = SHRIKE_MAX_HIDDEN / 8 / 64;  // 16-byte weight chunks a lane can own
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t e = blockIdx.x * 4u + wave;
+    if (e >= num_experts) return;
+    const uint32_t chunks = d / 8u;
+    float w[MAXI][8];
+#pragma unroll
+    for (int i = 0; i < MAXI; ++i) {
+        const uint32_t c = lane + 64u * i;
+        const uint4 v = *reinterpret_cast<const uint4 *>(weights + size_t(e) * d + size_t(c < chunks ? c : 0u) * 8u);
+        const uint32_t ww[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            w[i][2 * j] = f16_to_f32(uint16_t(ww[j]));
+            w[i][2 * j + 1] = f16_to_f32(uint16_t(ww[j] >> 16));
+        }
+    }
+    const uint32_t t0 = blockIdx.y * kFastTokenBlock;
+    const uint32_t t1 = min(t0 + kFastTokenBlock, query_count);
+    for (uint32_t t = t0; t < t1; t += 2u) {
+        const bool two = t + 1u < t1;
+        const float *row[2] = {xs + size_t(t) * d, xs + size_t(two ? t + 1u : t) * d};
+        float acc[2] = {0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < MAXI; ++i) {
+            const uint32_t c = lane + 64u * i;
+            if (c < chunks) {
+                float4 x[2][2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    x[u][0] = reinterpret_cast<const float4 *>(row[u] + size_t(c) * 8u)[0];
+                    x[u][1] = reinterpret_cast<const float4 *>(row[u] + size_t(c) * 8u)[1];
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const float xv[8] = {x[u][0].x, x[u][0].y, x[u][0].z, x[u][0].w, x[u][1].x, x[u][1].y, x[u][1].z, x[u][1].w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[u] = fmaf(w[i][j], xv[j], acc[u]);
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) {
+            acc[0] = __fadd_rn(acc[0], __shfl_xor(acc[0], o));
+            acc[1] = __fadd_rn(acc[1], __shfl_xor(acc[1], o));
+        }
+        if (lane == 0) {
+            logits[size_t(t) * num_experts + e] = acc[0];
+            if (two) logits[size_t(t + 1u) * num_experts + e] = acc[1];
+        }
+    }
+}
+
 // prefill.metal:441-563: one wave selects for one token.
 __global__ __launch_bounds__(256) void k_prefill_select(SelectArgs sel, const float *ws, uint32_t *out_indices,
                                                         uint16_t *out_weights, uint32_t query_count) {
@@ -58,21 +140,32 @@ struct GroupArgs {
     uint32_t *tile_count;
 };
 
-// pass 1: pairs per expert; one wave per expert
-__global__ __launch_bounds__(256) void k_group_count(GroupArgs a) {
-    const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4u + (threadIdx.x >> 6);
-    if (e >= a.num_experts) return;
-    uint32_t n = 0;
-    for (uint32_t i = lane; i < a.pairs; i += 64u) n += a.indices[i] == e ? 1u : 0u;
-    n = wave_sum_u32(n);
-    if (lane == 0) a.counts[e] = n;
+constexpr uint32_t kGroupLdsPairs = 49152;  // pairs whose expert ids (one byte each) fit the LDS copy
+
+__device__ __forceinline__ uint32_t pair_expert(const GroupArgs &a, const uint8_t *ids, bool in_lds, uint32_t i) {
+    return in_lds ? uint32_t(ids[i]) : a.indices[i];
 }
 
-// pass 2: the expert's first position (the pairs of every expert ordered before it), its
-// row tiles, and its pairs written in (token, rank) order. The pairs arrive token-major, so
-// walking them in index order keeps that order within the expert: the permutation equals
-// the reference's sort by (sort key, expert, token, rank) (PrefillMoEGrouping.swift:323-332).
-__global__ __launch_bounds__(256) void k_group_place(GroupArgs a) {
+// One launch, four experts a workgroup (one a wave). Every workgroup builds the whole
+// histogram for itself in LDS (the pairs are a few KB and sit in L2), so no count has to
+// cross workgroups. A wave then knows its expert's first position (the pairs of every
+// expert ordered before it), writes its row tiles, and writes its pairs in index order.
+// The pairs arrive token-major, so index order is (token, rank) order: the permutation
+// equals the reference's sort by (sort key, expert, token, rank)
+// (PrefillMoEGrouping.swift:323-332).
+__global__ __launch_bounds__(256) void k_group(GroupArgs a) {
+    __shared__ uint32_t s_hist[SHRIKE_MAX_ROUTER_EXPERTS];
+    __shared__ uint8_t s_ids[kGroupLdsPairs];
+    const bool in_lds = a.pairs <= kGroupLdsPairs;
+    s_hist[threadIdx.x] = 0u;
+    __syncthreads();
+#pragma unroll 4
+    for (uint32_t i = threadIdx.x; i < a.pairs; i += 256u) {
+        const uint32_t v = a.indices[i];
+        if (v < a.num_experts) atomicAdd(&s_hist[v], 1u);
+        if (in_lds) s_ids[i] = uint8_t(min(v, 255u));
+    }
+    __syncthreads();
     const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (e >= a.num_experts) return;
     const uint64_t key = a.sort_keys ? a.sort_keys[e] : 0u;
@@ -81,7 +174,7 @@ __global__ __launch_bounds__(256) void k_group_place(GroupArgs a) {
     for (uint32_t j = 0; j < SHRIKE_MAX_ROUTER_EXPERTS / 64u; ++j) {
         const uint32_t other = lane + 64u * j;
         if (other >= a.num_experts) continue;
-        const uint32_t c = a.counts[other];
+        const uint32_t c = s_hist[other];
         const uint64_t k2 = a.sort_keys ? a.sort_keys[other] : 0u;
         const bool before = k2 < key || (k2 == key && other < e);
         const uint32_t t = (c + kRowTile - 1u) / kRowTile;
@@ -92,8 +185,9 @@ __global__ __launch_bounds__(256) void k_group_place(GroupArgs a) {
     offset = wave_sum_u32(offset);
     tiles_before = wave_sum_u32(tiles_before);
     tiles_total = wave_sum_u32(tiles_total);
-    const uint32_t count = a.counts[e];
+    const uint32_t count = s_hist[e];
     if (lane == 0) {
+        a.counts[e] = count;
         a.offsets[e] = count ? offset : 0xffffffffu;
         if (e == 0) *a.tile_count = tiles_total;
     }
@@ -114,9 +208,9 @@ __global__ __launch_bounds__(256) void k_group_place(GroupArgs a) {
     if (count == 0) return;
     uint32_t running = 0;
     const uint64_t below = (uint64_t(1) << lane) - 1u;
-    for (uint32_t base = 0; base < a.pairs; base += 64u) {
+    for (uint32_t base = 0; base < a.pairs && running < count; base += 64u) {
         const uint32_t i = base + lane;
-        const bool mine = i < a.pairs && a.indices[i] == e;
+        const bool mine = i < a.pairs && pair_expert(a, s_ids, in_lds, i) == e;
         const uint64_t mask = __ballot(mine);
         if (mine) {
             shrike_token_expert_pair p;
@@ -242,7 +336,8 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
     SHRIKE_REQUIRE(d_weights && d_hidden && d_effective_scale && d_per_expert_scale && d_logit_bias,
                    "prefill router: weights, hidden, effectiveScale, perExpertScale and logitBias must all be bound");
     SHRIKE_REQUIRE(moe->desc.router_weight_bits == 0 || (d_scales && d_biases), "prefill router: affine router needs scales and biases");
-    SHRIKE_REQUIRE(d_out_indices && d_out_weights && d_logits_workspace, "prefill router: outputs and the logits workspace must be bound");
+    SHRIKE_REQUIRE(d_out_indices && d_out_weights && d_logits_workspace, "prefill router: outputs and the workspace must be bound");
+    SHRIKE_REQUIRE(reinterpret_cast<uintptr_t>(d_logits_workspace) % 16u == 0, "prefill router: workspace must be 16-byte aligned");
     RouterArgs a = {};
     a.weights = d_weights;
     a.scales = static_cast<const uint16_t *>(d_scales);
@@ -260,7 +355,17 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
     hipStream_t s = as_stream(stream);
     const dim3 grid((num_experts + 3u) / 4u, (query_count + kRouterTokenBlock - 1u) / kRouterTokenBlock);
     switch (moe->desc.router_weight_bits) {
-        case 0: hipLaunchKernelGGL(k_prefill_logits<0>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;
+        case 0: {
+            float *xs = d_logits_workspace + ((size_t(query_count) * num_experts + 3u) & ~size_t(3));
+            const size_t slots = size_t(query_count) * (d / 8u);
+            hipLaunchKernelGGL(k_prefill_scale_x, dim3(uint32_t((slots + 255u) / 256u)), dim3(256), 0, s, a.hidden, a.effective_scale,
+                               xs, query_count, d, hidden_stride_elements);
+            SHRIKE_HIP(hipGetLastError());
+            hipLaunchKernelGGL(k_prefill_logits_f16, dim3((num_experts + 3u) / 4u, (query_count + kFastTokenBlock - 1u) / kFastTokenBlock),
+                               dim3(256), 0, s, static_cast<const uint16_t *>(d_weights), xs, d_logits_workspace, query_count,
+                               num_experts, d);
+            break;
+        }
         case 8: hipLaunchKernelGGL(k_prefill_logits<8>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;
         default: hipLaunchKernelGGL(k_prefill_logits<4>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;
     }
@@ -269,6 +374,10 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
                        static_cast<uint16_t *>(d_out_weights), query_count);
     SHRIKE_HIP(hipGetLastError());
     return 0;
+}
+
+size_t shrike_hip_prefill_router_workspace_bytes(uint32_t query_count, uint32_t num_experts, uint32_t d) {
+    return (((size_t(query_count) * num_experts + 3u) & ~size_t(3)) + size_t(query_count) * d) * sizeof(float);
 }
 
 uint32_t shrike_hip_group_max_row_tiles(uint64_t pair_count, uint32_t num_experts) {
@@ -300,9 +409,7 @@ int shrike_hip_group_pairs(void *stream, const uint32_t *d_indices, const void *
     a.tile_count = out->row_tile_count;
     hipStream_t s = as_stream(stream);
     const dim3 grid((num_experts + 3u) / 4u);
-    hipLaunchKernelGGL(k_group_count, grid, dim3(256), 0, s, a);
-    SHRIKE_HIP(hipGetLastError());
-    hipLaunchKernelGGL(k_group_place, grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL(k_group, grid, dim3(256), 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     return 0;
 }

@@ -295,6 +295,9 @@ class Prefill:
     def _s(self):
         return self.moe._s()
 
+    def router_workspace_bytes(self, query_count, num_experts, d):
+        return capi.load().shrike_hip_prefill_router_workspace_bytes(query_count, num_experts, d)
+
     def encode_block(self, weights, scales, biases, hidden, effective_scale, per_expert_scale, logit_bias,
                      out_indices, out_weights, logits_workspace, query_count, num_experts, d, top_k,
                      hidden_stride_elements):

@@ -27,7 +27,7 @@ def token_rows(L: Layer, t: int, stride: int, label="prefill.x"):
 def run_router(gpu, dl, L, hidden, t, stride):
     pf = gpu.Prefill(dl.moe)
     idx, w = gpu.empty(4 * t * L.k), gpu.empty(2 * t * L.k)
-    ws = gpu.empty(4 * t * L.ne)
+    ws = gpu.empty(pf.router_workspace_bytes(t, L.ne, L.d))
     pf.encode_block(dl.router_w, dl.router_s, dl.router_b, hidden, dl.eff_scale, dl.expert_scale, dl.logit_bias,
                     idx, w, ws, t, L.ne, L.d, L.k, stride)
     gpu.synchronize()
