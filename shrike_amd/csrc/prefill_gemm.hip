@@ -20,8 +20,9 @@ namespace shrike {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr uint32_t kChunkK = 128;                 // k staged in LDS per step: two groups
+constexpr uint32_t kChunkK = 256;                 // k staged in LDS per step: four groups
 constexpr uint32_t kLdsRow = kChunkK + 8;         // halves per staged row; the pad spreads the banks
+constexpr uint32_t kMaxMT = kRowTile / 32;        // 32-row MFMA tiles per row tile
 constexpr float kTwo24 = 16777216.0f;
 
 struct FfnArgs {
@@ -94,12 +95,6 @@ __device__ __forceinline__ half8 b_step(const BRegs<BITS> &r, int s) {
 // MODE 0: gate and up rows n0..n0+31 of one expert against the gathered token rows, GLU,
 // fp16 activations out. MODE 1: down rows n0..n0+63 against the activations, fp16 partials
 // scattered to (token, rank).
-//
-// A wave owns one 32-row MFMA tile and two 32-column tiles (gate and up of the same columns,
-// or two neighbouring column tiles of down), so every wave of every workgroup carries the
-// same work. A row tile of at most 32 rows gives its workgroup's four waves four column
-// groups; one of 33..64 rows gives them two column groups by two 32-row tiles, and takes
-// twice as many workgroups along y.
 template <int BITS, int MODE>
 __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     __shared__ __align__(16) uint16_t s_a[2][kRowTile][kLdsRow];
@@ -108,45 +103,37 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     const shrike_row_tile tile = a.tiles[tile_index];
     if (tile.cell == kSentinel || tile.rows == 0) return;
 
-    constexpr uint32_t kCols = MODE == 0 ? 32u : 64u;  // output columns a wave owns
     const uint32_t K = MODE == 0 ? a.d : a.f, N = MODE == 0 ? a.f : a.d;
     const uint32_t G = K / kGroup;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t col = lane & 31u, kb = lane >> 5;
-    const uint32_t mt_count = (tile.rows + 31u) / 32u;  // 1 or 2
-    const uint32_t col_groups = 4u / mt_count;
-    if (blockIdx.y * col_groups * kCols >= N) return;  // the whole workgroup lies past the last column
-    const uint32_t mt = wave / col_groups;
-    const uint32_t n0 = (blockIdx.y * col_groups + wave % col_groups) * kCols;
+    const uint32_t mt_count = (tile.rows + 31u) / 32u;
+    const uint32_t n0 = (blockIdx.y * 4u + wave) * (MODE == 0 ? 32u : 64u);
     const bool active = n0 < N;
-    const uint32_t stage_rows = mt_count * 32u;
 
-    // ---- A staging: thread -> (row = tid / 16 + 16 i, 16-byte piece = tid % 16)
-    constexpr uint32_t kPieces = kChunkK / 8u;             // 16-byte pieces per staged row
-    constexpr uint32_t kRowsPerPass = 256u / kPieces;
-    constexpr uint32_t kPasses = kRowTile / kRowsPerPass;
-    const uint32_t piece = threadIdx.x % kPieces, row0 = threadIdx.x / kPieces;
-    const uint16_t *src_row[kPasses];
+    // ---- A staging: thread -> (row = tid / 32 + 8 i, 16-byte piece = tid % 32)
+    const uint32_t piece = threadIdx.x & 31u, row0 = threadIdx.x >> 5;
+    const uint16_t *src_row[kMaxMT * 4];
 #pragma unroll
-    for (uint32_t i = 0; i < kPasses; ++i) {
-        const uint32_t r = min(row0 + kRowsPerPass * i, tile.rows - 1u);  // rows past the tile repeat its last row
+    for (uint32_t i = 0; i < kMaxMT * 4; ++i) {
+        const uint32_t r = min(row0 + 8u * i, tile.rows - 1u);  // rows past the tile repeat its last row
         if (MODE == 0) {
             src_row[i] = a.hidden + size_t(a.pairs[tile.pair_start + r].token) * a.hidden_stride;
         } else {
             src_row[i] = a.act + (size_t(tile_index) * kRowTile + r) * a.f;
         }
     }
-    uint4 stage[kPasses];
+    uint4 stage[kMaxMT * 4];
     auto fetch = [&](uint32_t chunk) {
         const uint32_t k = chunk * kChunkK + piece * 8u;
 #pragma unroll
-        for (uint32_t i = 0; i < kPasses; ++i)
-            if (row0 + kRowsPerPass * i < stage_rows && k < K) stage[i] = *reinterpret_cast<const uint4 *>(src_row[i] + k);
+        for (uint32_t i = 0; i < kMaxMT * 4; ++i)
+            if (i < mt_count * 4u && k < K) stage[i] = *reinterpret_cast<const uint4 *>(src_row[i] + k);
     };
     auto commit = [&](uint32_t buf) {
 #pragma unroll
-        for (uint32_t i = 0; i < kPasses; ++i) {
-            if (row0 + kRowsPerPass * i >= stage_rows) continue;
+        for (uint32_t i = 0; i < kMaxMT * 4; ++i) {
+            if (i >= mt_count * 4u) continue;
             uint4 v = stage[i];
             if (BITS == 4) {  // (0,1,2,3,4,5,6,7) -> (0,4,1,5,2,6,3,7), to meet codes4
                 uint4 p;
@@ -156,7 +143,7 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
                 p.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
                 v = p;
             }
-            *reinterpret_cast<uint4 *>(&s_a[buf][row0 + kRowsPerPass * i][piece * 8u]) = v;
+            *reinterpret_cast<uint4 *>(&s_a[buf][row0 + 8u * i][piece * 8u]) = v;
         }
     };
 
@@ -185,92 +172,79 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
         }
     }
 
-    f32x16 total[2];
+    f32x16 total[2][kMaxMT];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) total[nt][i] = 0.0f;
-
-    // A lane's codes for one group are 16 (4-bit) or 32 (8-bit) bytes of its row, so one
-    // 128-byte line of the row holds a batch of 4 (or 2) groups. The loads of a batch are
-    // issued back to back, one batch ahead of the one being multiplied: the line comes from
-    // L2 once and serves the rest of the batch from L1.
-    constexpr uint32_t kBatch = BITS == 4 ? 4u : 2u;
-    constexpr uint32_t kGroupsPerChunk = kChunkK / kGroup;
-    BRegs<BITS> cur[kBatch][2], nxt[kBatch][2];
-    auto load_batch = [&](uint32_t first_group) {
+        for (uint32_t mt = 0; mt < kMaxMT; ++mt)
 #pragma unroll
-        for (uint32_t j = 0; j < kBatch; ++j) {
-            load_b<BITS>(nxt[j][0], bw[0], bs[0], min(first_group + j, G - 1u), kb);
-            load_b<BITS>(nxt[j][1], bw[1], bs[1], min(first_group + j, G - 1u), kb);
-        }
-    };
-    if (active) load_batch(0);
+            for (int i = 0; i < 16; ++i) total[nt][mt][i] = 0.0f;
+
+    BRegs<BITS> cur[2], nxt[2];
+    if (active) {
+        load_b<BITS>(cur[0], bw[0], bs[0], 0, kb);
+        load_b<BITS>(cur[1], bw[1], bs[1], 0, kb);
+    }
     const uint32_t chunks = (K + kChunkK - 1u) / kChunkK;
     fetch(0);
     commit(0);
     __syncthreads();
-    // two chunks (four groups) an iteration, so that batch slots and LDS buffers are compile-time choices
-    for (uint32_t c2 = 0; c2 < chunks; c2 += 2u) {
+    for (uint32_t c = 0; c < chunks; ++c) {
+        const uint32_t buf = c & 1u;
+        if (c + 1u < chunks) fetch(c + 1u);
+        const uint32_t groups_here = min(4u, G - 4u * c);
+        if (active) {
+            for (uint32_t gi = 0; gi < groups_here; ++gi) {
+                const uint32_t g = 4u * c + gi;
+                const uint32_t gn = min(g + 1u, G - 1u);
+                load_b<BITS>(nxt[0], bw[0], bs[0], gn, kb);
+                load_b<BITS>(nxt[1], bw[1], bs[1], gn, kb);
+                half8 af[kMaxMT][4];
 #pragma unroll
-        for (uint32_t half = 0; half < 2u; ++half) {
-            const uint32_t c = c2 + half;
-            if (c < chunks) {  // uniform over the workgroup
-                if (c + 1u < chunks) fetch(c + 1u);
-                const uint32_t groups_here = min(kGroupsPerChunk, G - kGroupsPerChunk * c);
-                if (active) {
+                for (uint32_t mt = 0; mt < kMaxMT; ++mt)
 #pragma unroll
-                    for (uint32_t gi = 0; gi < kGroupsPerChunk; ++gi) {
-                        if (gi < groups_here) {
-                            const uint32_t g = kGroupsPerChunk * c + gi;
-                            constexpr uint32_t kPerIter = 2u * kGroupsPerChunk;
-                            const uint32_t q = (half * kGroupsPerChunk + gi) % kBatch;  // compile-time after unrolling
-                            if (q == 0u) {
+                    for (int s = 0; s < 4; ++s)
+                        if (mt < mt_count)
+                            af[mt][s] = *reinterpret_cast<const half8 *>(&s_a[buf][mt * 32u + col][gi * 64u + kb * 32u + s * 8u]);
 #pragma unroll
-                                for (uint32_t j = 0; j < kBatch; ++j) {
-                                    cur[j][0] = nxt[j][0];
-                                    cur[j][1] = nxt[j][1];
-                                }
-                                load_batch(g + kBatch);
-                            }
-                            static_assert(kPerIter % kBatch == 0, "a batch must not straddle loop iterations");
-                            half8 af[4];
+                for (int nt = 0; nt < 2; ++nt) {
+                    half8 bf[4];
 #pragma unroll
-                            for (int s = 0; s < 4; ++s)
-                                af[s] = *reinterpret_cast<const half8 *>(&s_a[half][mt * 32u + col][gi * 64u + kb * 32u + s * 8u]);
-                            f32x16 p[2];
+                    for (int s = 0; s < 4; ++s) bf[s] = b_step<BITS>(cur[nt], s);
+                    const float sc = meta_f32(cur[nt].scale, a.meta) * kTwo24;
 #pragma unroll
-                            for (int nt = 0; nt < 2; ++nt) {
-                                p[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0], b_step<BITS>(cur[q][nt], 0), f32x16{0}, 0, 0, 0);
+                    for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+                        if (mt < mt_count) {
+                            f32x16 p = {0};
 #pragma unroll
-                                for (int s = 1; s < 4; ++s)
-                                    p[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[s], b_step<BITS>(cur[q][nt], s), p[nt], 0, 0, 0);
-                            }
+                            for (int s = 0; s < 4; ++s) p = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt][s], bf[s], p, 0, 0, 0);
 #pragma unroll
-                            for (int nt = 0; nt < 2; ++nt) {
-                                const float sc = meta_f32(cur[q][nt].scale, a.meta) * kTwo24;
-#pragma unroll
-                                for (int i = 0; i < 16; ++i) total[nt][i] = fmaf(sc, p[nt][i], total[nt][i]);
-                            }
+                            for (int i = 0; i < 16; ++i) total[nt][mt][i] = fmaf(sc, p[i], total[nt][mt][i]);
                         }
                     }
                 }
-                if (c + 1u < chunks) commit(half ^ 1u);
-                __syncthreads();
+                cur[0] = nxt[0];
+                cur[1] = nxt[1];
             }
         }
+        if (c + 1u < chunks) commit(buf ^ 1u);
+        __syncthreads();
     }
     if (!active) return;
 
     // ---- bias term: (group sums of the rows) x (group biases), sixteen k' = eight groups a step
     {
         const uint32_t *sums = MODE == 0 ? a.hidden_sums : a.act_sums;
-        const uint32_t r = min(mt * 32u + col, tile.rows - 1u);
-        const uint32_t *sum_row = MODE == 0 ? sums + size_t(a.pairs[tile.pair_start + r].token) * G
-                                            : sums + (size_t(tile_index) * kRowTile + r) * G;
+        const uint32_t *sum_row[kMaxMT];
+#pragma unroll
+        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+            const uint32_t r = min(mt * 32u + col, tile.rows - 1u);
+            sum_row[mt] = MODE == 0 ? sums + size_t(a.pairs[tile.pair_start + r].token) * G
+                                    : sums + (size_t(tile_index) * kRowTile + r) * G;
+        }
         for (uint32_t g0 = 0; g0 < G; g0 += 8u) {
             const uint32_t gl = g0 + 4u * kb;  // this lane's four groups
-            Frag bfr[2], afr;
+            Frag bfr[2], afr[kMaxMT];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const bool on = gl + j < G;
@@ -280,10 +254,14 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
                     if (a.meta == SHRIKE_META_BF16) bits = f32_to_f16(bf16_to_f32(bits));
                     bfr[nt].u[j] = uint32_t(bits) * 0x00010001u;  // against (hi, lo)
                 }
-                afr.u[j] = on ? sum_row[gl + j] : 0u;
+#pragma unroll
+                for (uint32_t mt = 0; mt < kMaxMT; ++mt) afr[mt].u[j] = (on && mt < mt_count) ? sum_row[mt][gl + j] : 0u;
             }
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) total[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr.h, bfr[nt].h, total[nt], 0, 0, 0);
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (uint32_t mt = 0; mt < kMaxMT; ++mt)
+                    if (mt < mt_count) total[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[mt].h, bfr[nt].h, total[nt][mt], 0, 0, 0);
         }
     }
 
@@ -296,11 +274,14 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
             uab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.up_ab_off)[n]);
         }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
-            if (m < tile.rows) {
-                const float act = glu_rt(total[0][i] + gab, total[1][i] + uab, a.act_kind);
-                a.act[(size_t(tile_index) * kRowTile + m) * a.f + n] = f32_to_f16(act);
+        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
+                if (mt < mt_count && m < tile.rows) {
+                    const float act = glu_rt(total[0][mt][i] + gab, total[1][mt][i] + uab, a.act_kind);
+                    a.act[(size_t(tile_index) * kRowTile + m) * a.f + n] = f32_to_f16(act);
+                }
             }
         }
     } else {
@@ -310,13 +291,16 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
             dab[1] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n + 32u]);
         }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
-            if (m < tile.rows) {
-                const shrike_token_expert_pair p = a.pairs[tile.pair_start + m];
-                uint16_t *dst = a.partials + (size_t(p.token) * a.top_k + p.rank) * a.d + n;
-                dst[0] = f32_to_f16(total[0][i] + dab[0]);
-                dst[32] = f32_to_f16(total[1][i] + dab[1]);
+        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
+                if (mt < mt_count && m < tile.rows) {
+                    const shrike_token_expert_pair p = a.pairs[tile.pair_start + m];
+                    uint16_t *dst = a.partials + (size_t(p.token) * a.top_k + p.rank) * a.d + n;
+                    dst[0] = f32_to_f16(total[0][mt][i] + dab[0]);
+                    dst[32] = f32_to_f16(total[1][mt][i] + dab[1]);
+                }
             }
         }
     }
@@ -328,10 +312,10 @@ int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uin
 template <int BITS>
 static int launch_ffn(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
     const dim3 block(256);
-    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0>), dim3(max_tiles, (a.f + 63u) / 64u), block, 0, s, a);
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0>), dim3(max_tiles, (a.f + 127u) / 128u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     if (int rc = launch_row_group_sums(a.act, a.f, max_tiles * kRowTile, a.f, const_cast<uint32_t *>(a.act_sums), a.tile_count, s)) return rc;
-    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1>), dim3(max_tiles, (a.d + 127u) / 128u), block, 0, s, a);
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1>), dim3(max_tiles, (a.d + 255u) / 256u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     return 0;
 }
