@@ -31,6 +31,10 @@ if ROOT not in sys.path:
 
 D, F, NE, K, FS, BITS = 2048, 512, 256, 8, 512, 4
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes of one routed gate/up launch read from the FETCH_SIZE and WRITE_SIZE counters (two
+# rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for the 453 MB
+# pool copies): 9,589,555 fetched + 8,192 written. profiles/decode_phase1_q35b_int4_hbm_traffic.txt
+PHASE1_TRAFFIC_BYTES = 9_597_747
 
 
 def build_layers(rt, capi, S, n_layers, meta, shared=True):
@@ -314,10 +318,10 @@ def main():
         "hbm_peak_frac_on_expert_bytes": round(value / HBM_PEAK_GBPS, 4),
         "expert_bytes_per_step": expert_bytes, "total_bytes_per_step": total_bytes,
         "kernel_us_per_layer": {k: round(v, 3) for k, v in parts.items()},
-        "roofline": {"bound": "hbm", "kernel": "k_phase1<4,1,2> (routed gate/up matvec + SiLU-multiply)",
+        "roofline": {"bound": "hbm", "kernel": "k_phase1<4,1,4,false,0> (routed gate/up matvec + SiLU-multiply)",
                      "achieved": round(p1_bytes / (p1_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(p1_bytes / (p1_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-                     "bytes_per_launch": p1_bytes, "us_per_launch": round(p1_us, 3), "traffic": None},
+                     "bytes_per_launch": p1_bytes, "us_per_launch": round(p1_us, 3), "traffic": PHASE1_TRAFFIC_BYTES},
         "setup_seconds": round(gen_s, 1),
     }
     if args.cpu_sample > 0:
