@@ -307,3 +307,19 @@ def test_prefill_reduce_and_residual():  # PrefillMoETests.swift:8-64
     want = (f16(hidden) + f16(h2)).astype(np.float16)
     got = O.residual_add_f16(hidden.copy(), h2)
     assert np.array_equal(got.view(np.float16), want)
+
+
+def test_int4_gemv_against_committed_reference_vectors():
+    """tests/golden/ref_int4_gemv.json holds what the reference's C kernel returned for these seeded
+    inputs (written by tests/golden/make_ref_gemv_vectors.py): the check that travels without the
+    reference checkout."""
+    import json
+    import zlib
+    from tests.golden.make_ref_gemv_vectors import inputs
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_int4_gemv.json")
+    for case in json.load(open(path))["cases"]:
+        rows, n = case["rows"], case["n"]
+        w, s, b, x = inputs(rows, n)
+        y = O.int4_affine_gemv(w, s, b, x, rows, n, S.META_BF16).view(np.uint32)
+        assert [int(v) for v in y[:16]] == case["head"], (rows, n)
+        assert zlib.crc32(y.tobytes()) == case["crc32"], (rows, n)
