@@ -1,0 +1,376 @@
+// C++ host side above the C ABI: the reference's operator classes with their method names and
+// argument order (the reference's host is Swift; this is the same surface for a C++ host).
+// Header only; every method forwards to one C entry point and throws shrike::Error with the
+// library's message where the reference throws (runtime conditions) or traps (preconditions).
+//
+//   reference class                                   here
+//   MoE (Kernels/MoE/MoE.swift)                       shrike::MoE
+//   SharedExpertRuntime (Kernels/MoE/SharedExpert*)   shrike::MoE::encodeSharedExpert
+//   ExpertCellArena + residency table                 shrike::ExpertPool
+//   PreadExpertStreamer's cache planning              shrike::SlotCache
+//   PrefillRouter / PrefillMoEGrouping /              shrike::PrefillRouter, shrike::PrefillMoEGrouping,
+//   PrefillGroupedRoutedMoE / PrefillMoE              shrike::PrefillGroupedRoutedMoE, shrike::PrefillMoE
+//   RuntimeConfiguration (budget -> slots)            shrike::RuntimeConfiguration
+#pragma once
+
+#include <cerrno>
+#include <cstdint>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "shrike_hip.h"
+#include "shrike_host.h"
+
+namespace shrike {
+
+struct Error : std::runtime_error {
+    int code;
+    Error(int c, const std::string &what) : std::runtime_error(what), code(c) {}
+};
+inline void check(int rc) {
+    if (rc != 0) throw Error(rc, shrike_hip_last_error());
+}
+
+using Stream = void *;  // a hipStream_t; nullptr = the default stream
+
+// RuntimeConfiguration.parseBudgetBytes / expertCacheSlots (RuntimeConfiguration.swift:111-149)
+struct RuntimeConfiguration {
+    static constexpr int64_t defaultExpertCacheBudgetBytes = int64_t(8) << 30;
+    static std::optional<int64_t> parseBudgetBytes(const std::string &text) {
+        const int64_t v = shrike_parse_budget_bytes(text.c_str());
+        return v < 0 ? std::nullopt : std::optional<int64_t>(v);
+    }
+    static int expertCacheSlots(uint64_t expertStrideBytes, int layers, int64_t budgetBytes = defaultExpertCacheBudgetBytes) {
+        return shrike_expert_cache_slots(expertStrideBytes, layers, budgetBytes);
+    }
+};
+
+// MoEExpertOffsets / CPUExpertFFN.Offsets (MoE.swift:4-39, CPUExpertFFN.swift:34-61)
+struct ExpertOffsets : shrike_expert_offsets {
+    uint64_t strideBytes = 0;
+    ExpertOffsets(uint32_t d, uint32_t f, uint32_t bits = 4, bool additiveBiases = false) {
+        strideBytes = shrike_expert_offsets_make(d, f, bits, additiveBiases, this);
+        if (!strideBytes) throw Error(EINVAL, "D and F must be positive multiples of 64, bits 4 or 8");
+    }
+};
+
+// ExpertCellArena (ExpertCellArena.swift:16-133) with the streamer's residency table
+class ExpertPool {
+public:
+    ExpertPool(uint32_t cellCount, uint64_t expertStride, uint32_t expertsPerLayer, uint64_t chunkBytes = 0) {
+        int err = 0;
+        h_ = shrike_hip_pool_create(cellCount, expertStride, expertsPerLayer, chunkBytes, &err);
+        if (!h_) throw Error(err, shrike_hip_last_error());
+    }
+    ~ExpertPool() { shrike_hip_pool_destroy(h_); }
+    ExpertPool(const ExpertPool &) = delete;
+    ExpertPool &operator=(const ExpertPool &) = delete;
+    uint64_t stride() const { return shrike_hip_pool_slot_stride(h_); }
+    uint32_t cellCount() const { return shrike_hip_pool_cell_count(h_); }
+    void *pointer(uint32_t cell) const { return shrike_hip_pool_cell_ptr(h_, cell); }
+    const shrike_pool_bases *bases() const { return shrike_hip_pool_bases(h_); }
+    const uint64_t *residencyTable() const { return static_cast<const uint64_t *>(shrike_hip_pool_residency_table(h_)); }
+    void upload(uint32_t cell, const void *hostBlob, uint64_t bytes, Stream s) { check(shrike_hip_pool_upload_async(h_, cell, hostBlob, bytes, s)); }
+    void publish(uint32_t expert, uint32_t cell, uint32_t state, Stream s) { check(shrike_hip_pool_table_publish(h_, expert, cell, state, s)); }
+    uint64_t residencyEntry(uint32_t expert) const { return shrike_hip_pool_table_entry(h_, expert); }
+    shrike_hip_pool *handle() const { return h_; }
+
+private:
+    shrike_hip_pool *h_;
+};
+
+// ExpertCachePlan (PreadExpertStreamer.swift:17-38)
+struct ExpertCachePlan {
+    std::vector<int32_t> experts, assignedSlots;
+    std::vector<uint64_t> assignedGenerations;
+    std::vector<uint32_t> misses;
+    uint32_t hits = 0;
+    int32_t layer = 0;
+    shrike_expert_cache_plan raw() {
+        return {uint32_t(experts.size()), layer, experts.data(), assignedSlots.data(), assignedGenerations.data(),
+                misses.data(), uint32_t(misses.size()), hits};
+    }
+};
+
+// The cache planning of PreadExpertStreamer (PreadExpertStreamer.swift:405-543, :676-767)
+class SlotCache {
+public:
+    SlotCache(uint32_t slotCount, uint32_t expertsPerLayer, uint32_t firstCell = 0, std::optional<double> slruProtectedShare = std::nullopt) {
+        int err = 0;
+        h_ = shrike_slot_cache_create(slotCount, expertsPerLayer, firstCell, slruProtectedShare ? SHRIKE_EVICT_SLRU : SHRIKE_EVICT_AGING_LFU,
+                                      slruProtectedShare.value_or(0.0), &err);
+        if (!h_) throw Error(err, shrike_hip_last_error());
+    }
+    ~SlotCache() { shrike_slot_cache_destroy(h_); }
+    SlotCache(const SlotCache &) = delete;
+    SlotCache &operator=(const SlotCache &) = delete;
+
+    // planExpertsCachedIfPossible: nullopt when the experts cannot be placed
+    std::optional<ExpertCachePlan> planExpertsCachedIfPossible(const std::vector<int32_t> &experts, int32_t layer = 0,
+                                                               const std::vector<int32_t> &avoidingSlots = {},
+                                                               const std::vector<uint8_t> *protectedExperts = nullptr,
+                                                               int64_t missesCounted = -1) {
+        ExpertCachePlan p;
+        const size_t n = experts.size();
+        p.experts.resize(n);
+        p.assignedSlots.resize(n);
+        p.assignedGenerations.resize(n);
+        p.misses.resize(n);
+        shrike_expert_cache_plan raw = p.raw();
+        const int rc = shrike_slot_cache_plan(h_, experts.data(), uint32_t(n), layer, avoidingSlots.data(), uint32_t(avoidingSlots.size()),
+                                              protectedExperts ? protectedExperts->data() : nullptr,
+                                              protectedExperts ? uint32_t(protectedExperts->size()) : 0u, missesCounted, &raw);
+        if (rc == ENOSPC) return std::nullopt;
+        check(rc);
+        p.misses.resize(raw.miss_count);
+        p.hits = raw.hits;
+        p.layer = raw.layer;
+        return p;
+    }
+    // planExpertsCached: throws ModelError.expertCacheUnplaceable's counterpart
+    ExpertCachePlan planExpertsCached(const std::vector<int32_t> &experts, int32_t layer = 0, const std::vector<int32_t> &avoidingSlots = {},
+                                      const std::vector<uint8_t> *protectedExperts = nullptr) {
+        auto p = planExpertsCachedIfPossible(experts, layer, avoidingSlots, protectedExperts);
+        if (!p) throw Error(ENOSPC, shrike_hip_last_error());
+        return *p;
+    }
+    void markPlanMissesResident(ExpertCachePlan &plan, uint64_t elapsedNanos = 0, uint64_t fetchNanos = 0) {
+        shrike_expert_cache_plan raw = plan.raw();
+        check(shrike_slot_cache_complete(h_, &raw, elapsedNanos, fetchNanos));
+    }
+    void abandonExpertCachePlan(ExpertCachePlan &plan) {
+        shrike_expert_cache_plan raw = plan.raw();
+        shrike_slot_cache_abandon(h_, &raw);
+    }
+    void pin(ExpertCachePlan &plan) {
+        shrike_expert_cache_plan raw = plan.raw();
+        check(shrike_slot_cache_pin(h_, &raw));
+    }
+    void unpin(const ExpertCachePlan &plan) {
+        shrike_slot_cache_unpin(h_, plan.assignedSlots.data(), plan.assignedGenerations.data(), uint32_t(plan.assignedSlots.size()));
+    }
+    shrike_streaming_statistics statistics(uint64_t expertStrideBytes = 0) {
+        shrike_streaming_statistics s{};
+        shrike_slot_cache_statistics(h_, expertStrideBytes, &s);
+        return s;
+    }
+    std::vector<int32_t> residentExperts(size_t capacity = 4096) {
+        std::vector<int32_t> out(capacity);
+        out.resize(shrike_slot_cache_resident_experts(h_, out.data(), capacity));
+        return out;
+    }
+    uint64_t residencyEntry(uint32_t expert) { return shrike_slot_cache_entry(h_, expert); }
+    // mirrors every changed residency word into the pool's device table, in order, on `s`
+    void publishTo(ExpertPool &pool, Stream s, size_t expertsPerLayer) {
+        std::vector<uint32_t> ids(expertsPerLayer);
+        std::vector<uint64_t> words(expertsPerLayer);
+        const size_t n = shrike_slot_cache_drain_publications(h_, ids.data(), words.data(), ids.size());
+        for (size_t i = 0; i < n; ++i) pool.publish(ids[i], uint32_t(words[i]), uint32_t(words[i] >> 32), s);
+    }
+
+private:
+    shrike_slot_cache *h_;
+};
+
+// MoE (MoE.swift:41-216): enqueue-only operators on a stream
+class MoE {
+public:
+    explicit MoE(const shrike_moe_desc &desc) {
+        int err = 0;
+        h_ = shrike_hip_moe_create(&desc, &err);
+        if (!h_) throw Error(err, shrike_hip_last_error());
+    }
+    ~MoE() { shrike_hip_moe_destroy(h_); }
+    MoE(const MoE &) = delete;
+    MoE &operator=(const MoE &) = delete;
+    shrike_hip_moe *handle() const { return h_; }
+
+    void encodeRouter(Stream s, const void *weights, const void *scales, const void *biases, const void *hidden,
+                      const void *effectiveScale, const void *perExpertScale, const void *logitBias, uint32_t *outIndices,
+                      void *outWeights, uint32_t numExperts, uint32_t d, uint32_t topK) {  // MoE.swift:249-261
+        check(shrike_hip_moe_router(h_, s, weights, scales, biases, hidden, effectiveScale, perExpertScale, logitBias, outIndices,
+                                    outWeights, numExperts, d, topK));
+    }
+    void encodeResidencyClassification(Stream s, const uint32_t *topKIndices, const uint64_t *residency, uint32_t *hitCount,
+                                       uint32_t *hitPositions, uint32_t *missCount, uint32_t *missPositions, uint32_t *missExperts,
+                                       uint32_t *resolvedSlots, uint32_t topK, uint32_t numExperts, const uint32_t fullGrids[12],
+                                       uint32_t *specArgs, uint32_t *hostReadback = nullptr, uint32_t readbackTag = 0,
+                                       const void *topKWeights = nullptr, const uint32_t *predicted = nullptr) {  // MoE.swift:552-566
+        check(shrike_hip_moe_classify(h_, s, topKIndices, residency, hitCount, hitPositions, missCount, missPositions, missExperts,
+                                      resolvedSlots, topK, numExperts, fullGrids, specArgs, hostReadback, readbackTag, topKWeights,
+                                      predicted));
+    }
+    void encodeSpecPhase1U16Load(Stream s, const ExpertPool &pool, const uint32_t *resolvedSlots, const shrike_expert_offsets &offsets,
+                                 const void *x, void *acts, uint32_t d, uint32_t f, uint32_t topK, const uint32_t *indirect = nullptr,
+                                 const uint32_t *ioStatus = nullptr) {  // MoE.swift:906-923
+        check(shrike_hip_moe_phase1_pool(h_, s, pool.bases(), pool.stride(), resolvedSlots, &offsets, x, acts, d, f, topK, indirect, ioStatus));
+    }
+    void encodeSpecPhase2Reduce(Stream s, const ExpertPool &pool, const uint32_t *resolvedSlots, const uint32_t *fallbackCells,
+                                const shrike_expert_offsets &offsets, const void *acts, const void *routingWeights, const void *residual,
+                                void *y, void *hidden, uint32_t d, uint32_t f, uint32_t topK, const uint32_t *indirect = nullptr,
+                                const uint32_t *ioStatus = nullptr) {  // MoE.swift:992-1014
+        check(shrike_hip_moe_phase2_pool(h_, s, pool.bases(), pool.stride(), resolvedSlots, fallbackCells, &offsets, acts, routingWeights,
+                                         residual, y, hidden, d, f, topK, indirect, ioStatus));
+    }
+    void encodeSharedExpert(Stream s, const shrike_projection &gate, const shrike_projection &up, const shrike_projection &down,
+                            uint32_t bits, const void *x, void *scratch, void *h1, const void *scalarGate, uint32_t d, uint32_t fShared) {
+        check(shrike_hip_shared_expert(h_, s, &gate, &up, &down, bits, x, scratch, h1, scalarGate, d, fShared));
+    }
+    void encodeDecodeLayer(Stream s, const shrike_decode_layer_args &args) { check(shrike_hip_moe_decode_layer(h_, s, &args)); }
+
+private:
+    shrike_hip_moe *h_;
+};
+
+// PrefillRouter (PrefillRouter.swift:41-152)
+struct PrefillRouter {
+    static constexpr int tokenBlock = 12;
+    static size_t workspaceBytes(uint32_t queryCount, uint32_t numExperts, uint32_t d) {
+        return shrike_hip_prefill_router_workspace_bytes(queryCount, numExperts, d);
+    }
+    static void encodeBlock(MoE &moe, Stream s, const void *weights, const void *scales, const void *biases, const void *hidden,
+                            const void *effectiveScale, const void *perExpertScale, const void *logitBias, uint32_t *outIndices,
+                            void *outWeights, float *workspace, uint32_t queryCount, uint32_t numExperts, uint32_t d, uint32_t topK,
+                            uint32_t hiddenStrideElements) {
+        check(shrike_hip_prefill_router(moe.handle(), s, weights, scales, biases, hidden, effectiveScale, perExpertScale, logitBias,
+                                        outIndices, outWeights, workspace, queryCount, numExperts, d, topK, hiddenStrideElements));
+    }
+    static std::vector<shrike_token_expert_pair> makeTokenExpertPairs(const std::vector<uint32_t> &indices, const std::vector<uint16_t> &weights,
+                                                                      uint32_t queryCount, uint32_t topK) {
+        if (indices.size() != size_t(queryCount) * topK || weights.size() != indices.size()) throw Error(EINVAL, "indices count mismatch");
+        std::vector<shrike_token_expert_pair> pairs(indices.size());
+        check(shrike_make_token_expert_pairs(indices.data(), weights.data(), queryCount, topK, pairs.data()));
+        return pairs;
+    }
+};
+
+// PrefillMoEGroupedRoutes and PrefillMoEGrouping.groupTokenExpertPairs (PrefillMoEGrouping.swift:32-50, :269-370)
+struct PrefillMoEGroupedRoutes {
+    std::vector<shrike_token_expert_pair> sortedPairs;
+    std::vector<uint32_t> perExpertOffsets, perExpertCounts;
+    std::vector<shrike_moe_group> groups;
+    std::vector<shrike_moe_tile> tiles;
+    int64_t queryCount = 0;
+    uint32_t maxPairsPerExpert = 0, maxPairsPerTile = 0, maxLiveExpertsPerTile = 0;
+};
+struct GroupingError : Error {
+    int64_t values[2];
+    GroupingError(int code, const int64_t v[2]) : Error(code, shrike_hip_last_error()) { values[0] = v[0]; values[1] = v[1]; }
+};
+struct PrefillMoEGrouping {
+    static PrefillMoEGroupedRoutes groupTokenExpertPairs(const std::vector<shrike_token_expert_pair> &pairs, int64_t queryCount, int64_t topK,
+                                                         int64_t numExperts, int64_t tileExpertCount = 16,
+                                                         const std::vector<uint64_t> *expertSortKeys = nullptr) {
+        PrefillMoEGroupedRoutes r;
+        const size_t e = numExperts > 0 ? size_t(numExperts) : 1, cap = std::max<size_t>(1, std::min(e, pairs.size()));
+        r.sortedPairs.resize(std::max<size_t>(1, pairs.size()));
+        r.perExpertOffsets.resize(e);
+        r.perExpertCounts.resize(e);
+        r.groups.resize(cap);
+        r.tiles.resize(cap);
+        shrike_grouped_routes out{r.sortedPairs.data(), r.perExpertOffsets.data(), r.perExpertCounts.data(), r.groups.data(), r.tiles.data()};
+        const int rc = shrike_group_pairs(pairs.data(), pairs.size(), queryCount, topK, numExperts, tileExpertCount,
+                                          expertSortKeys ? expertSortKeys->data() : nullptr, expertSortKeys ? expertSortKeys->size() : 0, &out);
+        if (rc != 0) throw GroupingError(rc, out.error_value);
+        r.sortedPairs.resize(pairs.size());
+        r.perExpertOffsets.resize(size_t(numExperts));
+        r.perExpertCounts.resize(size_t(numExperts));
+        r.groups.resize(out.group_count);
+        r.tiles.resize(out.tile_count);
+        r.queryCount = queryCount;
+        r.maxPairsPerExpert = out.max_pairs_per_expert;
+        r.maxPairsPerTile = out.max_pairs_per_tile;
+        r.maxLiveExpertsPerTile = out.max_live_experts_per_tile;
+        return r;
+    }
+    // the same permutation on the device, from the router's token-major output
+    static void encodeGroupPairs(Stream s, const uint32_t *indices, const void *weights, uint32_t queryCount, uint32_t topK, uint32_t numExperts,
+                                 const uint64_t *expertSortKeys, const uint64_t *residency, const shrike_hip_grouped_routes &out) {
+        check(shrike_hip_group_pairs(s, indices, weights, queryCount, topK, numExperts, expertSortKeys, residency, &out));
+    }
+};
+
+// PrefillSweepOrder (PrefillMoEGrouping.swift:91-266)
+struct PrefillSweepOrder {
+    static std::vector<uint32_t> residentFirstBalanced(const std::vector<uint32_t> &experts, const std::vector<int64_t> &rows,
+                                                       const std::vector<int64_t> &lastRow, const std::vector<uint8_t> &resident, int64_t slots,
+                                                       int64_t tileWidth) {
+        std::vector<uint32_t> order(std::max<size_t>(1, experts.size()));
+        size_t n = 0;
+        check(shrike_sweep_order_resident_first_balanced(experts.data(), rows.data(), lastRow.data(), experts.size(), resident.data(),
+                                                         resident.size(), slots, tileWidth, order.data(), &n));
+        order.resize(n);
+        return order;
+    }
+    static std::vector<uint64_t> expertSortKeys(const std::vector<uint32_t> &order, size_t numExperts) {
+        std::vector<uint64_t> keys(std::max<size_t>(1, numExperts));
+        shrike_expert_sort_keys(order.data(), order.size(), numExperts, keys.data());
+        keys.resize(numExperts);
+        return keys;
+    }
+};
+
+// PrefillGroupedRoutedMoE (PrefillGroupedRoutedMoE.swift:104-284, :925-939)
+struct PrefillRoutedExpertWave {
+    std::vector<shrike_routed_expert_block> blocks;
+    int paddedRows = 0, tailRows = 0;
+};
+struct PrefillGroupedRoutedMoE {
+    static constexpr int groupedRowTile = 64, groupedTailRowTile = 32;
+    static std::vector<PrefillRoutedExpertWave> planExpertWaves(const std::vector<shrike_expert_pair_range> &ranges,
+                                                                const std::vector<uint32_t> &boundExperts, int64_t stagingRows,
+                                                                int64_t rowTile = groupedRowTile, int64_t tailTile = 0) {
+        std::vector<shrike_routed_expert_block> blocks(64);
+        std::vector<shrike_routed_expert_wave> waves(16);
+        size_t nb = 0, nw = 0;
+        for (;;) {
+            const int rc = shrike_plan_expert_waves(ranges.data(), ranges.size(), boundExperts.data(), boundExperts.size(), stagingRows, rowTile,
+                                                    tailTile, blocks.data(), blocks.size(), &nb, waves.data(), waves.size(), &nw);
+            if (rc == ENOSPC) {
+                blocks.resize(std::max(blocks.size(), nb));
+                waves.resize(std::max(waves.size(), nw));
+                continue;
+            }
+            check(rc);
+            break;
+        }
+        std::vector<PrefillRoutedExpertWave> out(nw);
+        for (size_t i = 0; i < nw; ++i) {
+            out[i].blocks.assign(blocks.begin() + waves[i].block_start, blocks.begin() + waves[i].block_start + waves[i].block_count);
+            out[i].paddedRows = int(waves[i].padded_rows);
+            out[i].tailRows = int(waves[i].tail_rows);
+        }
+        return out;
+    }
+    static std::vector<uint32_t> rowTileTable(const PrefillRoutedExpertWave &wave, uint32_t rowTile = groupedRowTile) {
+        std::vector<uint32_t> table(std::max<size_t>(1, size_t(wave.paddedRows) / rowTile));
+        check(shrike_row_tile_table(wave.blocks.data(), wave.blocks.size(), uint32_t(wave.paddedRows), rowTile, table.data()));
+        table.resize(size_t(wave.paddedRows) / rowTile);
+        return table;
+    }
+    static size_t workspaceBytes(uint32_t queryCount, uint32_t maxRowTiles, uint32_t d, uint32_t f) {
+        return shrike_hip_prefill_ffn_workspace_bytes(queryCount, maxRowTiles, d, f);
+    }
+    static void encodeGroupedExpertGEMMs(MoE &moe, Stream s, const ExpertPool &pool, const shrike_expert_offsets &offsets,
+                                         const shrike_hip_grouped_routes &routes, uint32_t maxRowTiles, const void *hidden,
+                                         uint32_t hiddenStrideElements, void *routePartials, void *workspace, size_t workspaceSize,
+                                         uint32_t queryCount, uint32_t d, uint32_t f, uint32_t topK) {
+        check(shrike_hip_prefill_grouped_ffn(moe.handle(), s, pool.bases(), pool.stride(), &offsets, &routes, maxRowTiles, hidden,
+                                             hiddenStrideElements, routePartials, workspace, workspaceSize, queryCount, d, f, topK));
+    }
+};
+
+// PrefillMoE (PrefillMoE.swift:11-40)
+struct PrefillMoE {
+    static void encodeReduceTokenMajor(Stream s, const void *routePartials, const void *routeWeights, void *h2, uint32_t queryCount,
+                                       uint32_t topK, uint32_t d) {
+        check(shrike_hip_prefill_reduce(s, routePartials, routeWeights, h2, queryCount, topK, d));
+    }
+    static void encodeResidualAdd(Stream s, void *hidden, const void *delta, uint64_t count) {
+        check(shrike_hip_residual_add_f16(s, hidden, delta, count));
+    }
+};
+
+}  // namespace shrike

@@ -1,0 +1,140 @@
+// The reference's host-side unit tests, written against include/shrike.hpp the way the
+// reference writes them against its Swift classes. No GPU call is made: budget ladder,
+// grouping, sweep order, wave planner and slot cache run on the host. Exit code 0 = all passed.
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <optional>
+
+#include "shrike.hpp"
+
+using namespace shrike;
+
+static int failures = 0;
+#define EXPECT(cond)                                                      \
+    do {                                                                  \
+        if (!(cond)) {                                                    \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+            ++failures;                                                   \
+        }                                                                 \
+    } while (0)
+
+static shrike_token_expert_pair pair(uint32_t token, uint32_t expert, uint32_t rank, uint32_t bits) { return {token, expert, rank, bits}; }
+
+// ExpertCacheBudgetTests.swift:20-29, :85-89, :117-153
+static void budget() {
+    EXPECT(RuntimeConfiguration::expertCacheSlots(1769472, 40) == 128);
+    EXPECT(RuntimeConfiguration::expertCacheSlots(3342336, 40) == 64);
+    EXPECT(RuntimeConfiguration::expertCacheSlots(1769472, 40, 11324620800LL) == 160);
+    EXPECT(RuntimeConfiguration::parseBudgetBytes("8G") == int64_t(8) << 30);
+    EXPECT(RuntimeConfiguration::parseBudgetBytes(" 4G ") == int64_t(4) << 30);
+    EXPECT(RuntimeConfiguration::parseBudgetBytes("1.5G") == int64_t(1.5 * double(1 << 30)));
+    for (const char *bad : {"", " ", "bogus", "G", "-2G", "0", "0G", "abcG", "2X", "2GG"}) EXPECT(!RuntimeConfiguration::parseBudgetBytes(bad));
+    EXPECT(ExpertOffsets(2048, 512).strideBytes == 1769472);  // CPUExpertFFNTests.swift:56-67
+}
+
+// PrefillMoEGroupingTests.swift:5-53, :117-173
+static void grouping() {
+    std::vector<shrike_token_expert_pair> pairs = {
+        pair(0, 3, 0, 10), pair(0, 1, 1, 11), pair(0, 4, 2, 12), pair(1, 1, 0, 13), pair(1, 3, 1, 14), pair(1, 2, 2, 15),
+        pair(2, 4, 0, 16), pair(2, 3, 1, 17), pair(2, 1, 2, 18), pair(3, 5, 0, 19), pair(3, 1, 1, 20), pair(3, 4, 2, 21)};
+    std::reverse(pairs.begin(), pairs.end());
+    auto g = PrefillMoEGrouping::groupTokenExpertPairs(pairs, 4, 3, 6, 2);
+    const uint32_t experts[12] = {1, 1, 1, 1, 2, 3, 3, 3, 4, 4, 4, 5};
+    for (int i = 0; i < 12; ++i) EXPECT(g.sortedPairs[i].expert == experts[i]);
+    EXPECT((g.perExpertOffsets == std::vector<uint32_t>{UINT32_MAX, 0, 4, 5, 8, 11}));
+    EXPECT((g.perExpertCounts == std::vector<uint32_t>{0, 4, 1, 3, 3, 1}));
+    EXPECT(g.groups.size() == 5 && g.tiles.size() == 3);
+    EXPECT(g.tiles[1].group_start == 2 && g.tiles[1].group_count == 2 && g.tiles[1].pair_start == 5 && g.tiles[1].pair_count == 6);
+    EXPECT(g.maxPairsPerExpert == 4 && g.maxPairsPerTile == 6 && g.maxLiveExpertsPerTile == 2);
+    try {
+        PrefillMoEGrouping::groupTokenExpertPairs({pair(0, 0, 0, 1), pair(0, 1, 0, 2)}, 1, 2, 2, 1);
+        EXPECT(false);
+    } catch (const GroupingError &e) {
+        EXPECT(e.code == SHRIKE_GROUPING_DUPLICATE_TOKEN_RANK && e.values[0] == 0 && e.values[1] == 0);
+    }
+    try {
+        PrefillMoEGrouping::groupTokenExpertPairs({pair(0, 0, 0, 1)}, 1, 1, 1, 17);
+        EXPECT(false);
+    } catch (const GroupingError &e) {
+        EXPECT(e.code == SHRIKE_GROUPING_INVALID_TILE_EXPERT_COUNT && e.values[0] == 17);
+    }
+}
+
+// PrefillMoEGroupingTests.swift:270-289, :205-246
+static void sweepOrder() {
+    std::vector<uint32_t> experts;
+    std::vector<int64_t> rows, last;
+    for (uint32_t id = 1; id <= 9; ++id) { experts.push_back(id); rows.push_back(1); last.push_back(9 + id); }
+    for (uint32_t id = 100; id <= 102; ++id) { experts.push_back(id); rows.push_back(1); last.push_back(id - 100); }
+    std::vector<uint8_t> resident(103, 0);
+    for (int id = 1; id <= 9; ++id) resident[id] = 1;
+    auto order = PrefillSweepOrder::residentFirstBalanced(experts, rows, last, resident, 20, 8);
+    EXPECT((order == std::vector<uint32_t>{1, 2, 3, 4, 5, 6, 7, 8, 100, 101, 102, 9}));
+    auto keys = PrefillSweepOrder::expertSortKeys({3, 8, 5}, 9);
+    EXPECT(keys[3] == 0 && keys[8] == 1 && keys[5] == 2 && keys[0] == 3 && keys[7] == 3);
+}
+
+// PrefillGroupedRoutedMoETests+Execution.swift:382-432, :535-577
+static void wavePlanner() {
+    const std::vector<shrike_expert_pair_range> ranges = {{0, 0, 40}, {1, 40, 32}, {2, 72, 5}, {3, 77, 3}};
+    auto one = PrefillGroupedRoutedMoE::planExpertWaves(ranges, {0, 1, 2, 3}, 512);
+    EXPECT(one.size() == 1 && one[0].paddedRows == 256 && one[0].blocks.size() == 4);
+    EXPECT(one[0].blocks[2].slot == 2 && one[0].blocks[2].pair_start == 72 && one[0].blocks[2].rows == 5 && one[0].blocks[2].staging_row == 128);
+    EXPECT((PrefillGroupedRoutedMoE::rowTileTable(one[0]) == std::vector<uint32_t>{0, 1, 2, 3}));
+    auto tailed = PrefillGroupedRoutedMoE::planExpertWaves(ranges, {0, 1, 2, 3}, 512, 64, 32);
+    EXPECT(tailed.size() == 1 && tailed[0].paddedRows == 160 && tailed[0].tailRows == 96);
+    auto longExpert = PrefillGroupedRoutedMoE::planExpertWaves({{2, 0, 600}}, {0, 1, 2, 3}, 512);
+    EXPECT(longExpert.size() == 2 && longExpert[1].blocks[0].pair_start == 512 && longExpert[1].blocks[0].rows == 88 && longExpert[1].paddedRows == 128);
+    try {
+        PrefillGroupedRoutedMoE::planExpertWaves(ranges, {0, 1, 2, 3}, 96);
+        EXPECT(false);
+    } catch (const Error &e) {
+        EXPECT(e.code == EINVAL);
+    }
+}
+
+// PreadExpertStreamerTests+CachePlanning.swift:130-154, :225-270, :320-341
+static void slotCache() {
+    {
+        SlotCache c(4, 8);
+        auto warm = c.planExpertsCached({0, 1});
+        c.markPlanMissesResident(warm);
+        auto plan = c.planExpertsCached({0, 2}, 0, {0, 1});
+        EXPECT((plan.assignedSlots == std::vector<int32_t>{0, 2}) && plan.hits == 1 && (plan.misses == std::vector<uint32_t>{1}));
+    }
+    {
+        SlotCache c(2, 8);
+        for (auto experts : {std::vector<int32_t>{0, 1}, {0, 2}, {0, 1}}) {
+            auto p = c.planExpertsCached(experts);
+            c.markPlanMissesResident(p);
+        }
+        auto s = c.statistics(1000);
+        EXPECT(s.plans == 3 && s.requested_experts == 6 && s.hits == 2 && s.misses == 4 && s.evictions == 2 && s.reloads == 1);
+        EXPECT(s.read_operations == 4 && s.bytes_read == 4000 && s.load_batches == 3 && s.loading_slots == 0);
+    }
+    {
+        SlotCache c(2, 8);
+        auto warm = c.planExpertsCached({0, 1});
+        c.markPlanMissesResident(warm);
+        auto resident = c.planExpertsCached({0, 1});
+        c.pin(resident);
+        EXPECT(c.statistics().pinned_slots == 2 && !c.planExpertsCachedIfPossible({2}));
+        c.unpin(resident);
+        auto dropped = c.planExpertsCached({2, 3});
+        EXPECT(dropped.misses.size() == 2 && c.statistics().loading_slots == 2 && !c.planExpertsCachedIfPossible({0}));
+        c.abandonExpertCachePlan(dropped);
+        EXPECT(c.statistics().loading_slots == 0);
+        EXPECT((c.residencyEntry(2) >> 32) == SHRIKE_RESIDENCY_EMPTY);
+    }
+}
+
+int main() {
+    budget();
+    grouping();
+    sweepOrder();
+    wavePlanner();
+    slotCache();
+    std::printf(failures ? "%d checks failed\n" : "all host checks passed\n", failures);
+    return failures ? 1 : 0;
+}
