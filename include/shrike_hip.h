@@ -28,6 +28,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "shrike_host.h"
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -116,6 +118,17 @@ int shrike_hip_pool_upload_async(shrike_hip_pool *pool, uint32_t cell, const voi
 int shrike_hip_pool_table_publish(shrike_hip_pool *pool, uint32_t expert, uint32_t cell,
                                   uint32_t state, void *stream);
 uint64_t shrike_hip_pool_table_entry(const shrike_hip_pool *pool, uint32_t expert);
+
+/* PreadExpertStreamer.executeExpertCachePlan (PreadExpertStreamer.swift:545-574) with the
+ * file reads replaced by host-to-device copies: for every miss of `plan` (made by
+ * shrike_slot_cache_plan on a cache whose cells are this pool's), expert e is copied from
+ * host_store + e * store_expert_stride (pinned memory for an asynchronous copy) into its
+ * reserved cell on `stream`; the misses become resident in the cache and every residency
+ * word that changed is stored to the device table on the same stream, behind the copies.
+ * The caller orders `stream` against the kernels that still read an evicted cell. */
+int shrike_hip_pool_execute_plan(shrike_hip_pool *pool, shrike_slot_cache *cache,
+                                 const shrike_expert_cache_plan *plan, const void *host_store, uint64_t store_expert_stride,
+                                 uint64_t expert_bytes, void *stream, uint64_t elapsed_nanos);
 
 /* ------------------------------------------------------------ MoE operators */
 
@@ -302,6 +315,20 @@ int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shri
                                    const void *d_hidden, uint32_t hidden_stride_elements,
                                    void *d_route_partials, void *d_workspace, size_t workspace_bytes,
                                    uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k);
+
+/* The shared expert for query_count tokens (RealForwardRunner.swift:4620-4647: the dense
+ * int4/int8 QMMs of MPPPrefillInt4QMM + silu_mul_fp16) on the grouped kernel: h1[t, :] =
+ * half(down . half(glu(half(gate . x_t), half(up . x_t)))), optionally * sigmoid(scalar_gate[0])
+ * — the roundings of shrike_hip_shared_expert, token by token. h1: fp16[query_count, d]. */
+size_t shrike_hip_prefill_shared_expert_workspace_bytes(uint32_t query_count, uint32_t d,
+                                                        uint32_t f_shared);
+int shrike_hip_prefill_shared_expert(shrike_hip_moe *moe, void *stream, const shrike_projection *gate,
+                                     const shrike_projection *up, const shrike_projection *down,
+                                     uint32_t bits, const void *d_hidden,
+                                     uint32_t hidden_stride_elements, void *d_h1,
+                                     const void *d_scalar_gate, void *d_workspace,
+                                     size_t workspace_bytes, uint32_t query_count, uint32_t d,
+                                     uint32_t f_shared);
 
 /* PrefillMoE.encodeReduceTokenMajor, sources/Shrike/Kernels/Prefill/MoE/PrefillMoE.swift:11-40
  * (prefill_moe_reduce_token_major, prefill.metal:624-645): h2[t, :] =

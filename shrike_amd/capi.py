@@ -178,6 +178,7 @@ SIGNATURES = {
     "shrike_hip_graph_end_capture": (_VP, [_VP]),
     "shrike_hip_graph_launch": (C.c_int, [_VP, _VP]),
     "shrike_hip_graph_destroy": (C.c_int, [_VP]),
+    "shrike_hip_pool_execute_plan": (C.c_int, [_VP, _VP, C.POINTER(ExpertCachePlan), _VP, _U64, _U64, _VP, _U64]),
     # prefill operators
     "shrike_hip_prefill_router": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                             _U32, _U32, _U32, _U32, _U32]),
@@ -188,6 +189,9 @@ SIGNATURES = {
     "shrike_hip_prefill_grouped_ffn": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, C.POINTER(ExpertOffsets),
                                                  C.POINTER(HipGroupedRoutes), _U32, _VP, _U32, _VP, _VP, C.c_size_t,
                                                  _U32, _U32, _U32, _U32]),
+    "shrike_hip_prefill_shared_expert_workspace_bytes": (C.c_size_t, [_U32, _U32, _U32]),
+    "shrike_hip_prefill_shared_expert": (C.c_int, [_VP, _VP, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection),
+                                                   _U32, _VP, _U32, _VP, _VP, _VP, C.c_size_t, _U32, _U32, _U32]),
     "shrike_hip_prefill_reduce": (C.c_int, [_VP, _VP, _VP, _VP, _U32, _U32, _U32]),
     "shrike_hip_residual_add_f16": (C.c_int, [_VP, _VP, _VP, _U64]),
     # include/shrike_host.h

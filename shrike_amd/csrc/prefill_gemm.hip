@@ -39,6 +39,13 @@ struct FfnArgs {
     const uint32_t *act_sums;     // (hi, lo)[tiles * 64, f / 64]
     uint16_t *partials;           // fp16[T * top_k, d]
     uint32_t d, f, top_k, meta, act_kind, ebias;
+    // dense mode (one resident FFN over all rows, the shared expert): the three projections as
+    // separate tensors, rows in token order, output row = token
+    const uint8_t *dense_w[3];
+    const uint16_t *dense_s[3], *dense_b[3];
+    uint32_t dense_rows;
+    uint32_t round_gate_up;        // gate and up pass through fp16 before the GLU (dequant_int4.metal:206-287)
+    const uint16_t *scalar_gate;   // fp16[1] or null: output * sigmoid(gate) (dequant_int4.metal:322-329)
 };
 
 union Frag {
@@ -95,13 +102,22 @@ __device__ __forceinline__ half8 b_step(const BRegs<BITS> &r, int s) {
 // MODE 0: gate and up rows n0..n0+31 of one expert against the gathered token rows, GLU,
 // fp16 activations out. MODE 1: down rows n0..n0+63 against the activations, fp16 partials
 // scattered to (token, rank).
-template <int BITS, int MODE>
+template <int BITS, int MODE, bool DENSE>
 __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     __shared__ __align__(16) uint16_t s_a[2][kRowTile][kLdsRow];
     const uint32_t tile_index = blockIdx.x;
-    if (tile_index >= *a.tile_count) return;
-    const shrike_row_tile tile = a.tiles[tile_index];
-    if (tile.cell == kSentinel || tile.rows == 0) return;
+    shrike_row_tile tile;
+    if (DENSE) {
+        if (tile_index * kRowTile >= a.dense_rows) return;
+        tile.cell = 0;
+        tile.pair_start = tile_index * kRowTile;
+        tile.rows = min(kRowTile, a.dense_rows - tile.pair_start);
+        tile.expert = 0;
+    } else {
+        if (tile_index >= *a.tile_count) return;
+        tile = a.tiles[tile_index];
+        if (tile.cell == kSentinel || tile.rows == 0) return;
+    }
 
     const uint32_t K = MODE == 0 ? a.d : a.f, N = MODE == 0 ? a.f : a.d;
     const uint32_t G = K / kGroup;
@@ -118,7 +134,8 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     for (uint32_t i = 0; i < kMaxMT * 4; ++i) {
         const uint32_t r = min(row0 + 8u * i, tile.rows - 1u);  // rows past the tile repeat its last row
         if (MODE == 0) {
-            src_row[i] = a.hidden + size_t(a.pairs[tile.pair_start + r].token) * a.hidden_stride;
+            const uint32_t token = DENSE ? tile.pair_start + r : a.pairs[tile.pair_start + r].token;
+            src_row[i] = a.hidden + size_t(token) * a.hidden_stride;
         } else {
             src_row[i] = a.act + (size_t(tile_index) * kRowTile + r) * a.f;
         }
@@ -148,13 +165,22 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     };
 
     // ---- B rows of this lane
-    const uint8_t *base = cell_base(a.pool, tile.cell, a.stride);
+    const uint8_t *base = DENSE ? nullptr : cell_base(a.pool, tile.cell, a.stride);
     const uint32_t row_bytes = K * BITS / 8u;
     const uint8_t *bw[2];
     const uint16_t *bs[2], *bb[2];
     {
         const uint32_t n = active ? n0 + col : 0u;
-        if (MODE == 0) {
+        if (DENSE) {
+            const int first = MODE == 0 ? 0 : 2, second = MODE == 0 ? 1 : 2;
+            const uint32_t n1 = MODE == 0 ? n : n + 32u;
+            bw[0] = a.dense_w[first] + size_t(n) * row_bytes;
+            bw[1] = a.dense_w[second] + size_t(n1) * row_bytes;
+            bs[0] = a.dense_s[first] + size_t(n) * G;
+            bs[1] = a.dense_s[second] + size_t(n1) * G;
+            bb[0] = a.dense_b[first] + size_t(n) * G;
+            bb[1] = a.dense_b[second] + size_t(n1) * G;
+        } else if (MODE == 0) {
             bw[0] = base + a.off.gate_w_off + size_t(n) * row_bytes;
             bw[1] = base + a.off.up_w_off + size_t(n) * row_bytes;
             bs[0] = reinterpret_cast<const uint16_t *>(base + a.off.gate_s_off) + size_t(n) * G;
@@ -239,8 +265,8 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
 #pragma unroll
         for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
             const uint32_t r = min(mt * 32u + col, tile.rows - 1u);
-            sum_row[mt] = MODE == 0 ? sums + size_t(a.pairs[tile.pair_start + r].token) * G
-                                    : sums + (size_t(tile_index) * kRowTile + r) * G;
+            const uint32_t token = (MODE != 0) ? 0u : DENSE ? tile.pair_start + r : a.pairs[tile.pair_start + r].token;
+            sum_row[mt] = MODE == 0 ? sums + size_t(token) * G : sums + (size_t(tile_index) * kRowTile + r) * G;
         }
         for (uint32_t g0 = 0; g0 < G; g0 += 8u) {
             const uint32_t gl = g0 + 4u * kb;  // this lane's four groups
@@ -269,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     const uint32_t n = n0 + col;
     if (MODE == 0) {
         float gab = 0.0f, uab = 0.0f;
-        if (a.ebias) {  // moe.metal:261-269
+        if (!DENSE && a.ebias) {  // moe.metal:261-269
             gab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.gate_ab_off)[n]);
             uab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.up_ab_off)[n]);
         }
@@ -279,14 +305,21 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
             for (int i = 0; i < 16; ++i) {
                 const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
                 if (mt < mt_count && m < tile.rows) {
-                    const float act = glu_rt(total[0][mt][i] + gab, total[1][mt][i] + uab, a.act_kind);
+                    float g = total[0][mt][i] + gab, u = total[1][mt][i] + uab;
+                    if (DENSE && a.round_gate_up) {
+                        g = f16_to_f32(f32_to_f16(g));
+                        u = f16_to_f32(f32_to_f16(u));
+                    }
+                    const float act = glu_rt(g, u, a.act_kind);
                     a.act[(size_t(tile_index) * kRowTile + m) * a.f + n] = f32_to_f16(act);
                 }
             }
         }
     } else {
         float dab[2] = {0.0f, 0.0f};
-        if (a.ebias) {
+        float gate_mul = 0.0f;
+        if (DENSE && a.scalar_gate) gate_mul = 1.0f + expf(-f16_to_f32(a.scalar_gate[0]));
+        if (!DENSE && a.ebias) {
             dab[0] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n]);
             dab[1] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n + 32u]);
         }
@@ -296,10 +329,20 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
             for (int i = 0; i < 16; ++i) {
                 const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
                 if (mt < mt_count && m < tile.rows) {
-                    const shrike_token_expert_pair p = a.pairs[tile.pair_start + m];
-                    uint16_t *dst = a.partials + (size_t(p.token) * a.top_k + p.rank) * a.d + n;
-                    dst[0] = f32_to_f16(total[0][mt][i] + dab[0]);
-                    dst[32] = f32_to_f16(total[1][mt][i] + dab[1]);
+                    uint16_t *dst;
+                    if (DENSE) {
+                        dst = a.partials + size_t(tile.pair_start + m) * a.d + n;
+                    } else {
+                        const shrike_token_expert_pair p = a.pairs[tile.pair_start + m];
+                        dst = a.partials + (size_t(p.token) * a.top_k + p.rank) * a.d + n;
+                    }
+                    uint16_t y0 = f32_to_f16(total[0][mt][i] + dab[0]), y1 = f32_to_f16(total[1][mt][i] + dab[1]);
+                    if (DENSE && a.scalar_gate) {
+                        y0 = f32_to_f16(f16_to_f32(y0) / gate_mul);
+                        y1 = f32_to_f16(f16_to_f32(y1) / gate_mul);
+                    }
+                    dst[0] = y0;
+                    dst[32] = y1;
                 }
             }
         }
@@ -309,13 +352,13 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
 int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uint32_t n, uint32_t *out,
                           const uint32_t *row_limit_tiles, hipStream_t s);
 
-template <int BITS>
+template <int BITS, bool DENSE>
 static int launch_ffn(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
     const dim3 block(256);
-    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0>), dim3(max_tiles, (a.f + 127u) / 128u), block, 0, s, a);
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0, DENSE>), dim3(max_tiles, (a.f + 127u) / 128u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     if (int rc = launch_row_group_sums(a.act, a.f, max_tiles * kRowTile, a.f, const_cast<uint32_t *>(a.act_sums), a.tile_count, s)) return rc;
-    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1>), dim3(max_tiles, (a.d + 255u) / 256u), block, 0, s, a);
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1, DENSE>), dim3(max_tiles, (a.d + 255u) / 256u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     return 0;
 }
@@ -381,7 +424,50 @@ int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shri
     a.ebias = moe->desc.expert_additive_biases;
     hipStream_t s = as_stream(stream);
     if (int rc = launch_row_group_sums(a.hidden, hidden_stride_elements, query_count, d, const_cast<uint32_t *>(a.hidden_sums), nullptr, s)) return rc;
-    return moe->desc.routed_weight_bits == 8 ? launch_ffn<8>(a, max_row_tiles, s) : launch_ffn<4>(a, max_row_tiles, s);
+    return moe->desc.routed_weight_bits == 8 ? launch_ffn<8, false>(a, max_row_tiles, s) : launch_ffn<4, false>(a, max_row_tiles, s);
+}
+
+size_t shrike_hip_prefill_shared_expert_workspace_bytes(uint32_t query_count, uint32_t d, uint32_t f_shared) {
+    return workspace_layout(query_count, (query_count + kRowTile - 1u) / kRowTile, d, f_shared).total;
+}
+
+int shrike_hip_prefill_shared_expert(shrike_hip_moe *moe, void *stream, const shrike_projection *gate,
+                                     const shrike_projection *up, const shrike_projection *down, uint32_t bits,
+                                     const void *d_hidden, uint32_t hidden_stride_elements, void *d_h1, const void *d_scalar_gate,
+                                     void *d_workspace, size_t workspace_bytes, uint32_t query_count, uint32_t d,
+                                     uint32_t f_shared) {
+    SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
+    if (int rc = check_shared(gate, up, down, bits, d, f_shared)) return rc;
+    SHRIKE_REQUIRE(hidden_stride_elements >= d && hidden_stride_elements % 8u == 0, "hidden stride is too small or leaves rows unaligned");
+    SHRIKE_REQUIRE(d_hidden && d_h1 && d_workspace, "shared expert: NULL buffer");
+    SHRIKE_REQUIRE(reinterpret_cast<uintptr_t>(d_workspace) % 256u == 0, "shared expert: workspace must be 256-byte aligned");
+    if (query_count == 0) return 0;
+    const uint32_t tiles = (query_count + kRowTile - 1u) / kRowTile;
+    const Workspace w = workspace_layout(query_count, tiles, d, f_shared);
+    SHRIKE_REQUIRE(workspace_bytes >= w.total, "shared expert: workspace of %zu bytes, %zu needed", workspace_bytes, w.total);
+    uint8_t *ws = static_cast<uint8_t *>(d_workspace);
+    FfnArgs a = {};
+    a.hidden = static_cast<const uint16_t *>(d_hidden);
+    a.hidden_stride = hidden_stride_elements;
+    a.hidden_sums = reinterpret_cast<uint32_t *>(ws + w.hidden_sums);
+    a.act = reinterpret_cast<uint16_t *>(ws + w.act);
+    a.act_sums = reinterpret_cast<uint32_t *>(ws + w.act_sums);
+    a.partials = static_cast<uint16_t *>(d_h1);
+    a.d = d; a.f = f_shared; a.top_k = 1;
+    a.meta = moe->desc.meta_dtype;
+    a.act_kind = moe->desc.activation;
+    const shrike_projection *proj[3] = {gate, up, down};
+    for (int i = 0; i < 3; ++i) {
+        a.dense_w[i] = static_cast<const uint8_t *>(proj[i]->weights);
+        a.dense_s[i] = static_cast<const uint16_t *>(proj[i]->scales);
+        a.dense_b[i] = static_cast<const uint16_t *>(proj[i]->biases);
+    }
+    a.dense_rows = query_count;
+    a.round_gate_up = 1;
+    a.scalar_gate = static_cast<const uint16_t *>(d_scalar_gate);
+    hipStream_t s = as_stream(stream);
+    if (int rc = launch_row_group_sums(a.hidden, hidden_stride_elements, query_count, d, const_cast<uint32_t *>(a.hidden_sums), nullptr, s)) return rc;
+    return bits == 8 ? launch_ffn<8, true>(a, tiles, s) : launch_ffn<4, true>(a, tiles, s);
 }
 
 }  // extern "C"

@@ -1,6 +1,8 @@
 // Handles, the HBM slot pool and the small pure functions of the C ABI.
 #include "host_common.h"
 
+#include "../../include/shrike_host.h"
+
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -26,6 +28,17 @@ int hip_failed(hipError_t err, const char *what) {
 }
 
 __global__ void k_store_u64(uint64_t *dst, uint64_t value) { *dst = value; }
+
+// up to 32 residency words in one launch, in order (a later entry for the same expert wins)
+struct StoreBatch {
+    uint32_t count;
+    uint32_t expert[32];
+    uint64_t word[32];
+};
+__global__ void k_store_batch(uint64_t *table, StoreBatch b) {
+    if (threadIdx.x != 0) return;
+    for (uint32_t i = 0; i < b.count; ++i) table[b.expert[i]] = b.word[i];
+}
 
 }  // namespace shrike
 
@@ -234,6 +247,49 @@ int shrike_hip_pool_table_publish(shrike_hip_pool *pool, uint32_t expert, uint32
     pool->shadow[expert] = word;
     hipLaunchKernelGGL(k_store_u64, dim3(1), dim3(1), 0, as_stream(stream), pool->d_table + expert, word);
     SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int shrike_hip_pool_execute_plan(shrike_hip_pool *pool, shrike_slot_cache *cache, const shrike_expert_cache_plan *plan,
+                                 const void *host_store, uint64_t store_expert_stride, uint64_t expert_bytes, void *stream,
+                                 uint64_t elapsed_nanos) {
+    SHRIKE_REQUIRE(pool && cache && plan, "execute plan: NULL argument");
+    SHRIKE_REQUIRE(plan->miss_count == 0 || host_store, "execute plan: the plan has misses and no host store to read them from");
+    SHRIKE_REQUIRE(expert_bytes <= pool->stride && expert_bytes <= store_expert_stride, "execute plan: expert bytes exceed a cell or the store's stride");
+    // the reads (PreadExpertStreamer.swift:610-621): one host-to-device copy per miss into the cell the plan reserved
+    for (uint32_t m = 0; m < plan->miss_count; ++m) {
+        const uint32_t i = plan->misses[m];
+        const int32_t expert = plan->experts[i];
+        SHRIKE_REQUIRE(expert >= 0 && uint32_t(expert) < pool->num_experts, "execute plan: expert %d out of range", expert);
+        const uint64_t word = shrike_slot_cache_entry(cache, uint32_t(expert));
+        SHRIKE_REQUIRE(uint32_t(word >> 32) == SHRIKE_RESIDENCY_LOADING, "execute plan: expert %d is not loading (stale plan)", expert);
+        const uint32_t cell = uint32_t(word);
+        SHRIKE_REQUIRE(cell < pool->cells, "execute plan: cell %u out of range", cell);
+        SHRIKE_HIP(hipMemcpyAsync(shrike_hip_pool_cell_ptr(pool, cell), static_cast<const uint8_t *>(host_store) + uint64_t(expert) * store_expert_stride,
+                                  expert_bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    }
+    // markPlanMissesResident, then every residency word that changed since the last drain goes to
+    // the device table behind the copies on the same stream
+    if (int rc = shrike_slot_cache_complete(cache, plan, elapsed_nanos, elapsed_nanos)) return rc;
+    uint32_t experts[32];
+    uint64_t words[32];
+    for (;;) {
+        const size_t n = shrike_slot_cache_drain_publications(cache, experts, words, 32);
+        if (n == 0) break;
+        StoreBatch b;
+        b.count = 0;
+        for (size_t i = 0; i < n; ++i) {
+            if (experts[i] >= pool->num_experts) continue;
+            pool->shadow[experts[i]] = words[i];
+            b.expert[b.count] = experts[i];
+            b.word[b.count] = words[i];
+            ++b.count;
+        }
+        if (b.count) {
+            hipLaunchKernelGGL(k_store_batch, dim3(1), dim3(64), 0, as_stream(stream), pool->d_table, b);
+            SHRIKE_HIP(hipGetLastError());
+        }
+    }
     return 0;
 }
 

@@ -87,7 +87,31 @@ def empty(nbytes: int) -> DeviceBuffer:
 def ptr(b) -> int | None:
     if b is None:
         return None
-    return b.ptr if isinstance(b, DeviceBuffer) else int(b)
+    return b.ptr if isinstance(b, (DeviceBuffer, PinnedBuffer)) else int(b)
+
+
+class PinnedBuffer:
+    """Page-locked host memory from the library (hipHostMalloc), viewed as a numpy array."""
+
+    def __init__(self, nbytes: int):
+        init()
+        self.nbytes = int(nbytes)
+        self.ptr = capi.load().shrike_hip_host_alloc(self.nbytes)
+        if not self.ptr:
+            raise ShrikeError(f"shrike_hip_host_alloc({nbytes}) failed: {capi.last_error()}")
+        self.array = np.ctypeslib.as_array((C.c_uint8 * self.nbytes).from_address(self.ptr))
+
+    def free(self):
+        if self.ptr:
+            self.array = None
+            capi.load().shrike_hip_host_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
 
 
 class Stream:
@@ -99,6 +123,9 @@ class Stream:
 
     def synchronize(self):
         check(capi.load().shrike_hip_stream_synchronize(self.handle), "stream_synchronize")
+
+    def wait_event(self, event: "Event"):
+        check(capi.load().shrike_hip_stream_wait_event(self.handle, event.handle), "stream_wait_event")
 
     def close(self):
         if self.handle:
@@ -168,6 +195,16 @@ class ExpertPool:
 
     def entry(self, expert: int) -> int:
         return capi.load().shrike_hip_pool_table_entry(self.handle, expert)
+
+    def execute_plan(self, cache, plan, host_store, store_expert_stride: int, expert_bytes: int,
+                     stream: Stream | None = None, elapsed_nanos: int = 0) -> None:
+        """executeExpertCachePlan: copy the plan's misses from the pinned host store into their cells,
+        mark them resident and store the changed residency words, all on `stream`. `cache` is a
+        shrike_amd.host.SlotCache, `plan` its CachePlan."""
+        check(capi.load().shrike_hip_pool_execute_plan(self.handle, cache._h, C.byref(plan.c), ptr(host_store),
+                                                       store_expert_stride, expert_bytes,
+                                                       stream.handle if stream else None, elapsed_nanos),
+              "shrike_hip_pool_execute_plan")
 
     def close(self) -> None:
         if self.handle:
@@ -325,6 +362,19 @@ class Prefill:
             ptr(route_partials), ptr(workspace), workspace.nbytes, query_count, self.moe.desc.d, self.moe.desc.f, top_k),
             "shrike_hip_prefill_grouped_ffn")
 
+    def encode_shared_expert(self, gate, up, down, bits, hidden, hidden_stride_elements, h1, query_count, f_shared,
+                             workspace: DeviceBuffer | None = None, scalar_gate=None):
+        """The shared expert for every token of the chunk; returns the workspace it used."""
+        need = capi.load().shrike_hip_prefill_shared_expert_workspace_bytes(query_count, self.moe.desc.d, f_shared)
+        if workspace is None or workspace.nbytes < need:
+            workspace = empty(need)
+        g, u, dn = (Projection(ptr(t[0]), ptr(t[1]), ptr(t[2])) for t in (gate, up, down))
+        check(capi.load().shrike_hip_prefill_shared_expert(
+            self.moe.handle, self._s(), C.byref(g), C.byref(u), C.byref(dn), bits, ptr(hidden), hidden_stride_elements,
+            ptr(h1), ptr(scalar_gate), ptr(workspace), workspace.nbytes, query_count, self.moe.desc.d, f_shared),
+            "shrike_hip_prefill_shared_expert")
+        return workspace
+
     def encode_reduce_token_major(self, route_partials, route_weights, h2, query_count, top_k, d):
         check(capi.load().shrike_hip_prefill_reduce(self._s(), ptr(route_partials), ptr(route_weights), ptr(h2),
                                                     query_count, top_k, d), "shrike_hip_prefill_reduce")
@@ -332,3 +382,78 @@ class Prefill:
     def residual_add(self, hidden, delta, count):
         check(capi.load().shrike_hip_residual_add_f16(self._s(), ptr(hidden), ptr(delta), count),
               "shrike_hip_residual_add_f16")
+
+
+class BatchedDecodeLayer:
+    """One MoE layer for a batch of tokens whose experts stream through a slot pool smaller than
+    the expert set: the runner's loop around the operators (RealForwardRunner.swift:4552-4686 with
+    the tile sequencing of PrefillRoutedTileSequencer). Router for all tokens, then passes: a
+    pass plans as many of the still-unserved experts as the pool can take (shrike_amd.host.SlotCache),
+    copies the misses from the pinned host store on the upload stream, and runs the grouped FFN
+    for exactly that pass's experts; the token-major reduce and the shared expert close the layer.
+    Everything numeric happens in libshrikehip; this class only sequences calls."""
+
+    def __init__(self, moe: MoE, pool: ExpertPool, cache, offsets, host_store: PinnedBuffer, store_stride: int,
+                 expert_bytes: int, max_tokens: int):
+        d, f, ne, k = moe.desc.d, moe.desc.f, moe.desc.num_experts, moe.desc.top_k
+        self.moe, self.pool, self.cache, self.off = moe, pool, cache, offsets
+        self.store, self.store_stride, self.expert_bytes = host_store, store_stride, expert_bytes
+        self.pf = Prefill(moe)
+        self.upload_stream = Stream()
+        self.t_max = max_tokens
+        self.idx, self.w = empty(4 * max_tokens * k), empty(2 * max_tokens * k)
+        self.router_ws = empty(self.pf.router_workspace_bytes(max_tokens, ne, d))
+        self.routes = GroupedRoutesDevice(max_tokens * k, ne)
+        self.partials = empty(2 * max_tokens * k * d)
+        self.ffn_ws = empty(self.pf.ffn_workspace_bytes(max_tokens, self.routes.max_row_tiles))
+        self.h2 = empty(2 * max_tokens * d)
+        self.pass_table = empty(8 * ne)
+        self.passes = 0
+
+    def run(self, router, hidden, t: int, stride: int):
+        """router: dict(weights, scales, biases, eff_scale, expert_scale, bias) of device buffers.
+        Returns the device buffer h2[t, d]; self.idx / self.w hold the routes."""
+        m, pf = self.moe, self.pf
+        d, ne, k = m.desc.d, m.desc.num_experts, m.desc.top_k
+        compute = m.stream
+        pf.encode_block(router["weights"], router.get("scales"), router.get("biases"), hidden, router["eff_scale"],
+                        router["expert_scale"], router["bias"], self.idx, self.w, self.router_ws, t, ne, d, k, stride)
+        (compute.synchronize() if compute else synchronize())
+        ids = self.idx.download(np.uint32, t * k)  # the router's host readback
+        # experts the pool already holds go first (PrefillSweepOrder.residentFirstBalanced), so a
+        # step does not evict what it is about to use
+        from . import host as _host
+        rows, last = {}, {}
+        for i, e in enumerate(ids.tolist()):
+            rows[e] = rows.get(e, 0) + 1
+            last[e] = i // k
+        resident = np.zeros(ne, np.uint8)
+        resident[self.cache.resident_experts()] = 1
+        todo = _host.resident_first_balanced(rows, last, resident, self.cache.slot_count, min(16, self.cache.slot_count))
+        uploaded, served = Event(), Event()
+        self.passes = 0
+        while todo:
+            batch = todo[: self.cache.slot_count]
+            plan = self.cache.plan(batch)
+            if plan is None:
+                raise ShrikeError(capi.last_error())
+            if self.passes:
+                self.upload_stream.wait_event(served)  # the cells about to be overwritten were still being read
+            self.pool.execute_plan(self.cache, plan, self.store, self.store_stride, self.expert_bytes, self.upload_stream)
+            # this pass's residency view: only its experts count as resident for the grouping
+            table = np.full(ne, (capi.EMPTY << 32) | SENTINEL, np.uint64)
+            for e in batch:
+                table[e] = self.cache.entry(e)
+            self.upload_stream.synchronize()  # the copy of `table` below reuses pageable memory
+            self.pass_table.upload(table)
+            uploaded.record(self.upload_stream)
+            if compute:
+                compute.wait_event(uploaded)
+            pf.group_pairs(self.idx, self.w, t, k, ne, self.routes, residency=self.pass_table)
+            pf.encode_grouped_expert_gemms(self.pool, self.off, self.routes, hidden, stride, self.partials, self.ffn_ws, t, k)
+            served.record(compute)
+            (compute.synchronize() if compute else synchronize())
+            todo = todo[len(batch):]
+            self.passes += 1
+        pf.encode_reduce_token_major(self.partials, self.w, self.h2, t, k, d)
+        return self.h2

@@ -298,3 +298,76 @@ def test_prefill_layer_at_full_size_agrees_with_the_decode_kernels(gpu):
         # cancelling sum move by a few fp16 steps of the largest partial: compared in the
         # reference's relative-error metric.
         assert_rel_close(out[tok], dl.y.download(np.uint16, d), f"token {tok}: prefill h2 vs decode y", tol=2e-3)
+
+
+@pytest.mark.parametrize("d,fs,bits,t,gated", [(2048, 512, 4, 20, False), (2304, 1024, 8, 16, True), (192, 320, 4, 70, False), (128, 64, 8, 1, True)])
+def test_shared_expert_for_a_token_block(gpu, d, fs, bits, t, gated):
+    L = Layer(0x5EED0007, d, 64, 4, 2, bits=bits, shared_f=fs, shared_bits=bits)
+    dl = DeviceLayer(gpu, L, resident=[])
+    pf = gpu.Prefill(dl.moe)
+    x = token_rows(L, t, d + 8)
+    h1 = gpu.dev(np.full(t * d, 0xD4D0, np.uint16))
+    gate_bits = S.f32_to_f16_bits(np.array([0.37], np.float32)) if gated else None
+    pf.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, gpu.dev(x), d + 8, h1, t, fs,
+                            scalar_gate=gpu.dev(gate_bits) if gated else None)
+    gpu.synchronize()
+    got = h1.download(np.uint16, t * d).reshape(t, d)
+    for tok in range(t):
+        xt = np.ascontiguousarray(x[tok * (d + 8):tok * (d + 8) + d])
+        ref = O.shared_expert(L.shared["gate"], L.shared["up"], L.shared["down"], xt, d, fs, bits=bits, meta=L.meta,
+                              scalar_gate_f16=gate_bits)
+        # gate/up -> fp16 -> act -> fp16 -> down -> fp16 (-> gate -> fp16): whole chain, the reference's metric
+        assert_rel_close(got[tok], ref, f"token {tok}", tol=2e-3 if gated else 1e-3)
+        # and equal to the single-token operator on the same token
+        if tok in (0, t - 1):
+            one = gpu.empty(2 * d)
+            dl.moe.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, gpu.dev(xt), dl.shared_scratch,
+                                        one, d, fs, scalar_gate=gpu.dev(gate_bits) if gated else None)
+            gpu.synchronize()
+            assert_rel_close(got[tok], one.download(np.uint16, d), f"token {tok} vs the decode operator", tol=2e-3 if gated else 1e-3)
+
+
+@pytest.mark.parametrize("bits,slots,slru", [(8, 16, None), (4, 8, 0.5)])
+def test_batched_decode_through_a_pool_smaller_than_the_expert_set(gpu, bits, slots, slru):
+    """Config 5 in small: 12 sequences, top-4 of 48 experts, a pool of 16 (or 8) cells; the experts
+    stream from pinned host memory in passes. Routes are bit-exact, every partial row matches the
+    oracle stage by stage, the statistics count what happened, and a second step hits the cache."""
+    d, f, ne, k, t = 256, 128, 48, 4, 12
+    L = Layer(0x5EED0005, d, f, ne, k, bits=bits)
+    dl = DeviceLayer(gpu, L, cells=slots, resident=[])
+    dl.moe.stream = gpu.Stream()
+    cache = HL.SlotCache(slots, ne, slru_share=slru)
+    store = gpu.PinnedBuffer(ne * L.stride)
+    for e in range(ne):
+        store.array[e * L.stride:(e + 1) * L.stride] = L.blobs[e]
+    layer = gpu.BatchedDecodeLayer(dl.moe, dl.pool, cache, dl.off, store, L.stride, L.stride, t)
+    x = token_rows(L, t, d)
+    hidden = gpu.dev(x)
+    router = dict(weights=dl.router_w, eff_scale=dl.eff_scale, expert_scale=dl.expert_scale, bias=dl.logit_bias)
+    h2 = layer.run(router, hidden, t, d)
+    dl.moe.stream.synchronize()
+    ref_idx, ref_w, _ = O.prefill_router(L.router_dict(), x, t, d, k)
+    idx, w = layer.idx.download(np.uint32, t * k), layer.w.download(np.uint16, t * k)
+    assert np.array_equal(idx, ref_idx)
+    used = len(set(idx.tolist()))
+    assert layer.passes == -(-used // slots) and layer.passes >= 2
+    partials = layer.partials.download(np.uint16, t * k * d).reshape(t, k, d)
+    off = L.oracle_offsets()
+    for tok in range(t):
+        xt = np.ascontiguousarray(x[tok * d:(tok + 1) * d])
+        for rank in range(k):
+            ref = O.prefill_pair_partial(L.blobs[int(idx[tok * k + rank])], off, xt, d, f, bits, L.meta)
+            assert_rel_close(partials[tok, rank], ref, f"token {tok} rank {rank}")
+    assert np.array_equal(h2.download(np.uint16, t * d), O.prefill_reduce(partials.reshape(-1), w, t, k, d))
+    st = cache.statistics(L.stride)
+    assert (st.plans, st.requested_experts, st.misses, st.hits) == (layer.passes, used, used, 0)
+    assert st.bytes_read == used * L.stride and st.loading_slots == 0 and st.resident_slots == min(slots, used)
+    # every device residency word equals the cache's own
+    assert [dl.pool.entry(e) for e in range(ne)] == [cache.entry(e) for e in range(ne)]
+    # a second step over the same tokens: the experts of the last pass are still resident
+    before = cache.statistics().hits
+    layer.run(router, hidden, t, d)
+    dl.moe.stream.synchronize()
+    assert cache.statistics().hits > before
+    again = layer.partials.download(np.uint16, t * k * d)
+    assert np.array_equal(again, partials.reshape(-1))  # same bytes whatever cell an expert landed in
