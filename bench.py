@@ -217,6 +217,136 @@ def prefill_main(args, rt, capi, S, meta):
     print(json.dumps(out))
 
 
+def gptoss_main(args, rt, capi, S, meta):
+    """Config 4: a batch of 4 independent tokens through 24 stacked gpt-oss-20B-shape layers (hidden 2880,
+    32 experts of intermediate 2880, top-4, int4 or int8 codes): router -> grouping -> grouped FFN -> reduce
+    per layer, every layer with its own pool."""
+    d = f = 2880
+    ne, k, t, bits, n_layers = 32, 4, 4, args.bits, min(args.layers, 24)
+    tree = S.SeedTree(0x5EED0004)
+    off, stride = rt.expert_offsets(d, f, bits)
+    blobs = [S.expert_blob(tree, f"layer.0.expert.{e}", d, f, bits, meta) for e in range(ne)]
+    pools, routers = [], []
+    for l in range(n_layers):
+        pool = rt.ExpertPool(ne, stride, ne)
+        if l == 0:
+            for e in range(ne):
+                capi.check(capi.load().shrike_hip_memcpy_h2d(pool.cell_ptr(e), blobs[e].ctypes.data, blobs[e].nbytes), "h2d")
+        else:
+            capi.check(capi.load().shrike_hip_memcpy_d2d(pool.cell_ptr(0), pools[0].cell_ptr(0), ne * pool.stride), "d2d")
+        for e in range(ne):
+            pool.publish(e, e, capi.RESIDENT)
+        pools.append(pool)
+        routers.append(rt.dev(S.router_f16(tree, f"layer.{l}.router.w", ne, d)))
+    moe = rt.MoE(d, f, ne, k, routed_bits=bits, router_bits=0, meta=meta)
+    stream = rt.Stream()
+    moe.stream = stream
+    pf = rt.Prefill(moe)
+    ones_d, ones_e = rt.dev(S.f32_to_bf16_bits(np.ones(d, np.float32))), rt.dev(S.f32_to_bf16_bits(np.ones(ne, np.float32)))
+    zeros_e = rt.dev(np.zeros(ne, np.uint16))
+    hidden = rt.dev(S.activations_f16(tree, "x", t * d))
+    idx, w, rws = rt.empty(4 * t * k), rt.empty(2 * t * k), rt.empty(pf.router_workspace_bytes(t, ne, d))
+    routes = rt.GroupedRoutesDevice(t * k, ne)
+    partials, h2 = rt.empty(2 * t * k * d), rt.empty(2 * t * d)
+    work = rt.empty(pf.ffn_workspace_bytes(t, routes.max_row_tiles))
+
+    resolved, acts, y = rt.empty(4 * t * k), rt.empty(2 * t * k * f), rt.empty(2 * t * d)
+    grouped = os.environ.get("SHRIKE_BENCH_GROUPED") == "1"  # diagnostic: the prefill operators instead of the decode ones
+
+    def all_layers():
+        for l in range(n_layers):
+            pf.encode_block(routers[l], None, None, hidden, ones_d, ones_e, zeros_e, idx, w, rws, t, ne, d, k, d)
+            if grouped:
+                pf.group_pairs(idx, w, t, k, ne, routes, residency=pools[l].table)
+                pf.encode_grouped_expert_gemms(pools[l], off, routes, hidden, d, partials, work, t, k)
+                pf.encode_reduce_token_major(partials, w, h2, t, k, d)
+            else:
+                moe.encode_resolve_batch(idx, pools[l].table, resolved, t * k, ne)
+                moe.encode_phase1_batch(pools[l], resolved, off, hidden, d, acts, d, f, k, t)
+                moe.encode_phase2_batch(pools[l], resolved, off, acts, w, None, y, None, d, f, k, t)
+
+    all_layers()
+    stream.synchronize()
+    used = sum(len(set(idx.download(np.uint32, t * k).tolist())) for _ in range(1))  # last layer's distinct experts
+    graph = capture(rt, capi, stream, all_layers)
+    reps = max(2, args.steps // 200)
+    time_graph(rt, capi, stream, graph, max(1, args.warmup // 200))
+    ms = time_graph(rt, capi, stream, graph, reps) / reps
+    # distinct experts differ per layer (own router); count them from one eager pass per layer
+    distinct = []
+    for l in range(n_layers):
+        pf.encode_block(routers[l], None, None, hidden, ones_d, ones_e, zeros_e, idx, w, rws, t, ne, d, k, d)
+        stream.synchronize()
+        distinct.append(len(set(idx.download(np.uint32, t * k).tolist())))
+    expert_bytes = sum(distinct) * stride
+    print(json.dumps({
+        "metric": "gpt-oss-20B-shape MoE layers, 4 tokens: us per layer (ms per 24-layer stack in ms_per_step)",
+        "value": round(expert_bytes / (ms * 1e-3) / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": reps, "warmup": max(1, args.warmup // 200),
+        "ms_per_step": round(ms, 5), "us_per_layer": round(ms * 1e3 / n_layers, 2), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 x u%d -> f32" % bits, "data": "synthetic (seeded SplitMix64)",
+        "config": {"workload": f"config 4: {t} tokens, top-{k} of {ne} int{bits} experts, hidden {d}, intermediate {f}, {n_layers} stacked layers "
+                               "in one HIP graph, all slots resident", "operators": "grouped (prefill)" if grouped else "batched decode",
+                   "distinct_experts_per_layer": distinct, "expert_bytes_per_stack": expert_bytes,
+                   "pair_bytes_per_stack": n_layers * t * k * stride, "meta_dtype": args.meta},
+        "GBps_on_pair_bytes": round(n_layers * t * k * stride / (ms * 1e-3) / 1e9, 2),
+        "hbm_peak_frac_on_expert_bytes": round(expert_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}))
+
+
+def kimi_main(args, rt, capi, S, meta):
+    """Config 5: 16 sequences, one token each, Kimi-Linear-48B shape (hidden 2304, 256 int8 experts of
+    intermediate 1024, top-8, shared expert 1024); the pool holds 64 of the 256 experts and misses are copied
+    from pinned host memory on a side stream. Reports the miss rate, the wall time per step and the host->device rate."""
+    from shrike_amd import host as HL
+    d, f, ne, k, t, bits, slots = 2304, 1024, 256, 8, 16, 8, 64
+    tree = S.SeedTree(0x5EED0005)
+    off, stride = rt.expert_offsets(d, f, bits)
+    store = rt.PinnedBuffer(ne * stride)
+    for e in range(ne):
+        store.array[e * stride:(e + 1) * stride] = S.expert_blob(tree, f"layer.0.expert.{e}", d, f, bits, meta)
+    pool = rt.ExpertPool(slots, stride, ne)
+    cache = HL.SlotCache(slots, ne)
+    moe = rt.MoE(d, f, ne, k, routed_bits=bits, router_bits=0, meta=meta)
+    moe.stream = rt.Stream()
+    layer = rt.BatchedDecodeLayer(moe, pool, cache, off, store, stride, stride, t)
+    router = dict(weights=rt.dev(S.router_f16(tree, "router.w", ne, d)), eff_scale=rt.dev(S.f32_to_bf16_bits(np.ones(d, np.float32))),
+                  expert_scale=rt.dev(S.f32_to_bf16_bits(np.ones(ne, np.float32))), bias=rt.dev(np.zeros(ne, np.uint16)))
+    shared = {n: tuple(rt.dev(a) for a in S.affine_matrix(tree.key(f"shared.{n}"), r, c, bits, meta))
+              for n, r, c in (("gate", f, d), ("up", f, d), ("down", d, f))}
+    h1 = rt.empty(2 * t * d)
+    batches = [rt.dev(S.activations_f16(tree, f"x.{i}", t * d)) for i in range(8)]
+    steps, warm = max(8, args.steps // 100), 8
+    sws = None
+
+    def step(i):
+        nonlocal sws
+        x = batches[i % len(batches)]
+        layer.run(router, x, t, d)
+        sws = layer.pf.encode_shared_expert(shared["gate"], shared["up"], shared["down"], bits, x, d, h1, t, f, workspace=sws)
+        layer.pf.residual_add(layer.h2, h1, t * d)
+        moe.stream.synchronize()
+
+    for i in range(warm):
+        step(i)
+    base = cache.statistics(stride)
+    base = (base.requested_experts, base.misses, base.bytes_read, base.plans)
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(warm + i)
+    dt = time.perf_counter() - t0
+    st = cache.statistics(stride)
+    req, miss, read, plans = st.requested_experts - base[0], st.misses - base[1], st.bytes_read - base[2], st.plans - base[3]
+    print(json.dumps({
+        "metric": "Kimi-Linear-48B-shape MoE decode, 16 sequences through a 64-of-256 slot pool: ms per step (wall clock, misses included)",
+        "value": round(t / (dt / steps), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 x u8 -> f32", "data": "synthetic (seeded SplitMix64), 8 token batches in rotation",
+        "config": {"workload": f"config 5: {t} sequences, top-{k} of {ne} int8 experts, hidden {d}, intermediate {f}, shared expert {f}, "
+                               f"pool of {slots} cells, misses from pinned host memory on a side stream",
+                   "passes_per_step": round(plans / steps, 2)},
+        "miss_rate": round(miss / max(1, req), 4), "experts_requested_per_step": round(req / steps, 1),
+        "host_to_device_GBps": round(read / dt / 1e9, 2), "bytes_copied_per_step": int(read / steps)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -226,8 +356,11 @@ def main():
     ap.add_argument("--meta", choices=["f16", "bf16"], default="f16")
     ap.add_argument("--cpu-sample", type=int, default=60, help="layer evaluations timed on the CPU (0 = skip)")
     ap.add_argument("--no-shared", action="store_true", help="diagnostic: leave the shared expert out of the layer")
-    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
-                    help="decode: the headline metric (config 2); prefill: the ragged 512-token chunk (config 3)")
+    ap.add_argument("--workload", choices=["decode", "prefill", "gptoss", "kimi"], default="decode",
+                    help="decode: the headline metric (config 2); prefill: the ragged 512-token chunk (config 3); "
+                         "gptoss: 4 tokens through 24 gpt-oss-shape layers (config 4); kimi: 16 sequences through a "
+                         "64-cell pool fed from pinned host memory (config 5)")
+    ap.add_argument("--bits", type=int, choices=[4, 8], default=4, help="gptoss: code width")
     ap.add_argument("--tokens", type=int, default=512, help="prefill: tokens in the chunk")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -242,6 +375,10 @@ def main():
     meta = S.META_F16 if args.meta == "f16" else S.META_BF16
     if args.workload == "prefill":
         return prefill_main(args, rt, capi, S, meta)
+    if args.workload == "gptoss":
+        return gptoss_main(args, rt, capi, S, meta)
+    if args.workload == "kimi":
+        return kimi_main(args, rt, capi, S, meta)
     n_layers = args.layers
     layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta, shared=not args.no_shared)
     moe = rt.MoE(D, F, NE, K, routed_bits=BITS, router_bits=0, meta=meta)

@@ -202,6 +202,28 @@ int shrike_hip_moe_phase2_pool(shrike_hip_moe *moe, void *stream, const shrike_p
                                uint32_t top_k, const uint32_t *d_indirect,
                                const uint32_t *d_io_status);
 
+/* The same operators for a batch of independent decode tokens (several sequences, one token
+ * each; RealForwardRunner's batched decode encodes the per-token kernels back to back, here
+ * grid.y walks the tokens). resolve: moe.metal:121-151 per position, resolved[t*top_k + p] =
+ * cell or SHRIKE_SLOT_SENTINEL, misses added to *d_miss_count when given. phase 1: x is
+ * fp16[tokens, x_stride_elements], acts fp16[tokens, top_k, f]. phase 2: routing weights
+ * fp16[tokens, top_k]; residual (may be NULL = 0), y and hidden (may be NULL) are
+ * fp16[tokens, d]. Per token the results are those of the single-token calls, bit for bit. */
+int shrike_hip_moe_resolve_batch(void *stream, const uint32_t *d_topk_indices,
+                                 const uint64_t *d_residency, uint32_t *d_resolved_slots,
+                                 uint32_t count, uint32_t num_experts, uint32_t *d_miss_count);
+int shrike_hip_moe_phase1_batch(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                uint64_t pool_slot_stride, const uint32_t *d_resolved_slots,
+                                const shrike_expert_offsets *offsets, const void *d_x,
+                                uint32_t x_stride_elements, void *d_acts, uint32_t d, uint32_t f,
+                                uint32_t top_k, uint32_t tokens);
+int shrike_hip_moe_phase2_batch(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                uint64_t pool_slot_stride, const uint32_t *d_resolved_slots,
+                                const shrike_expert_offsets *offsets, const void *d_acts,
+                                const void *d_routing_weights, const void *d_residual, void *d_y,
+                                void *d_hidden, uint32_t d, uint32_t f, uint32_t top_k,
+                                uint32_t tokens);
+
 /* SharedExpertInt4.encodeGateUp + encodeFusedDown / SharedExpertInt8
  * (sources/Shrike/Kernels/MoE/SharedExpertInt4.swift:91-164, :251-342;
  * dequant_int4.metal:206-331, dequant_int8.metal:109-164): h1 = half(down .

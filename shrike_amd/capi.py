@@ -179,6 +179,11 @@ SIGNATURES = {
     "shrike_hip_graph_launch": (C.c_int, [_VP, _VP]),
     "shrike_hip_graph_destroy": (C.c_int, [_VP]),
     "shrike_hip_pool_execute_plan": (C.c_int, [_VP, _VP, C.POINTER(ExpertCachePlan), _VP, _U64, _U64, _VP, _U64]),
+    "shrike_hip_moe_resolve_batch": (C.c_int, [_VP, _VP, _VP, _VP, _U32, _U32, _VP]),
+    "shrike_hip_moe_phase1_batch": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, _VP, C.POINTER(ExpertOffsets), _VP, _U32, _VP,
+                                              _U32, _U32, _U32, _U32]),
+    "shrike_hip_moe_phase2_batch": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, _VP, C.POINTER(ExpertOffsets), _VP, _VP, _VP, _VP,
+                                              _VP, _U32, _U32, _U32, _U32]),
     # prefill operators
     "shrike_hip_prefill_router": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                             _U32, _U32, _U32, _U32, _U32]),

@@ -26,6 +26,7 @@ struct Phase1Args {
     uint16_t *acts;
     uint32_t d, f, top_k, meta, act, ebias;
     const uint32_t *indirect, *io_status;
+    uint32_t tokens, x_stride;  // tokens > 1: grid.y walks tokens; x rows x_stride elements apart
     // fused layer only: route from the logits of the previous launch (sel.logits != nullptr),
     // and run the shared expert's down projection in workgroups past `routed_blocks`
     SelectArgs sel;
@@ -43,6 +44,7 @@ struct Phase2Args {
     uint16_t *y, *hidden;
     uint32_t d, f, top_k, meta, ebias;
     const uint32_t *indirect, *io_status;
+    uint32_t tokens;  // tokens > 1: grid.y walks tokens; residual, y and hidden rows are d apart
 };
 
 int launch_router(const RouterArgs &a, uint32_t router_bits, hipStream_t s);

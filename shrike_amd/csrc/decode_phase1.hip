@@ -23,6 +23,12 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     }
     if (a.indirect && a.indirect[0] == 0u) return;
     if (!io_ready(a.io_status)) return;
+    // a batch of tokens: grid.y is this workgroup's token (the argument block itself stays untouched:
+    // writing to it would move it to private memory)
+    const size_t tok = ROUTE ? 0u : blockIdx.y;
+    const uint16_t *x_tok = a.x + tok * a.x_stride;
+    const uint32_t *resolved_tok = a.resolved + tok * a.top_k;
+    uint16_t *acts_tok = a.acts + tok * a.top_k * a.f;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t cpr = a.d * BITS / 128u, groups = a.d / kGroup, row_bytes = cpr * 16u;
     const uint32_t pair0 = (blockIdx.x * 4u + wave) * RP;
@@ -31,7 +37,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     const uint32_t f0 = pair0 - k * a.f;
 
     SliceRegs<BITS, NCH> xr;
-    load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(a.x), cpr, lane, true);
+    load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
 
     uint32_t cell = kSentinel;
     if (ROUTE) {
@@ -44,7 +50,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
         __syncthreads();
         if (in_range) cell = s_cell[k];
     } else if (in_range) {
-        cell = a.resolved[k];
+        cell = resolved_tok[k];
     }
     if (cell == kSentinel) return;  // moe.metal:986, and waves past the last row
     const uint8_t *base = cell_base(a.pool, cell, a.stride);
@@ -79,7 +85,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
         u = lane == uint32_t(p) ? res[RP + p] : u;
     }
     const uint16_t act = f32_to_f16(glu_rt(g + gab, u + uab, a.act));
-    if (lane < uint32_t(RP)) a.acts[size_t(k) * a.f + f0 + lane] = act;
+    if (lane < uint32_t(RP)) acts_tok[size_t(k) * a.f + f0 + lane] = act;
 }
 
 uint32_t phase1_blocks(uint32_t top_k, uint32_t f) {
@@ -107,7 +113,7 @@ int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t sha
                        "phase1: the shared down rows ride along only in the routed launch and with one chunk column per lane");
         extra = gemv_blocks(a.shared_down.rows, a.shared_down.n, shared_down_bits);
     }
-    const dim3 grid(a.routed_blocks + extra);
+    const dim3 grid(a.routed_blocks + extra, a.tokens ? a.tokens : 1u);
     if (bits == 4) {
         if (!routing) launch_phase1_nch<4, false, 0>(a, grid, s);
         else if (shared_down_bits == 0) launch_phase1_nch<4, true, 0>(a, grid, s);
@@ -162,6 +168,29 @@ int shrike_hip_moe_phase1_pool(shrike_hip_moe *moe, void *stream, const shrike_p
     a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.act = moe->desc.activation;
     a.ebias = moe->desc.expert_additive_biases;
     a.indirect = d_indirect; a.io_status = moe->desc.event_gated_io ? d_io_status : nullptr;
+    a.routed_blocks = phase1_blocks(top_k, f);
+    return launch_phase1(a, bits, false, 0, as_stream(stream));
+}
+
+int shrike_hip_moe_phase1_batch(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                uint64_t pool_slot_stride, const uint32_t *d_resolved_slots,
+                                const shrike_expert_offsets *offsets, const void *d_x, uint32_t x_stride_elements,
+                                void *d_acts, uint32_t d, uint32_t f, uint32_t top_k, uint32_t tokens) {
+    SHRIKE_REQUIRE(moe != nullptr && pool != nullptr, "moe handle or pool is NULL");
+    SHRIKE_REQUIRE(top_k >= 1 && top_k <= SHRIKE_MAX_TOP_K, "phase1: topK=%u not in 1...8", top_k);
+    SHRIKE_REQUIRE(tokens >= 1 && tokens <= 65535u, "phase1: %u tokens not in 1...65535", tokens);
+    SHRIKE_REQUIRE(x_stride_elements >= d && x_stride_elements % 8u == 0, "phase1: x stride is too small or leaves rows unaligned");
+    const uint32_t bits = moe->desc.routed_weight_bits;
+    if (int rc = check_offsets(offsets, d, f, bits)) return rc;
+    SHRIKE_REQUIRE(d_resolved_slots && d_x && d_acts, "phase1: resolvedSlots, x and acts must be bound");
+    SHRIKE_REQUIRE(pool_slot_stride % 16u == 0, "phase1: pool slot stride must be a multiple of 16");
+    Phase1Args a = {};
+    fill_pool(a.pool, pool);
+    a.stride = pool_slot_stride; a.resolved = d_resolved_slots; a.off = *offsets;
+    a.x = static_cast<const uint16_t *>(d_x); a.acts = static_cast<uint16_t *>(d_acts);
+    a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.act = moe->desc.activation;
+    a.ebias = moe->desc.expert_additive_biases;
+    a.tokens = tokens; a.x_stride = x_stride_elements;
     a.routed_blocks = phase1_blocks(top_k, f);
     return launch_phase1(a, bits, false, 0, as_stream(stream));
 }

@@ -22,17 +22,26 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     typedef Chunk<BITS> C;
     __shared__ float partial[SHRIKE_MAX_TOP_K][kPhase2Rows];
     if (a.indirect && a.indirect[0] == 0u) return;
+    // a batch of tokens: grid.y is this workgroup's token (the argument block itself stays untouched)
+    const size_t tok = blockIdx.y;
+    const uint16_t *acts_tok = a.acts + tok * a.top_k * a.f;
+    const uint32_t *resolved_tok = a.resolved + tok * a.top_k;
+    const uint32_t *fallback_tok = a.fallback ? a.fallback + tok * a.top_k : nullptr;
+    const uint16_t *routing_tok = a.routing_w + tok * a.top_k;
+    const uint16_t *residual_tok = a.residual ? a.residual + tok * a.d : nullptr;
+    uint16_t *y_tok = a.y + tok * a.d;
+    uint16_t *hidden_tok = a.hidden ? a.hidden + tok * a.d : nullptr;
     const uint32_t lane = threadIdx.x & 63u, k = threadIdx.x >> 6;
     const uint32_t d0 = blockIdx.x * kPhase2Rows;
     // the epilogue's operands do not depend on anything computed here: fetch them first
     const bool finisher = threadIdx.x < kPhase2Rows && d0 + threadIdx.x < a.d;
     uint16_t res_bits = 0, hid_bits = 0;
     if (finisher) {
-        if (a.residual) res_bits = a.residual[d0 + threadIdx.x];
-        if (a.hidden) hid_bits = a.hidden[d0 + threadIdx.x];
+        if (residual_tok) res_bits = residual_tok[d0 + threadIdx.x];
+        if (hidden_tok) hid_bits = hidden_tok[d0 + threadIdx.x];
     }
     if (!io_ready(a.io_status)) {  // moe.metal:1032-1035
-        if (finisher) phase2_finish(a.y, a.hidden, d0 + threadIdx.x, res_bits, hid_bits);
+        if (finisher) phase2_finish(y_tok, hidden_tok, d0 + threadIdx.x, res_bits, hid_bits);
         return;
     }
     const uint32_t cpr = a.f * BITS / 128u, groups = a.f / kGroup, row_bytes = cpr * 16u;
@@ -43,10 +52,10 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     const bool lane_on = sub < rpl;
 
     SliceRegs<BITS, NCH> xr;
-    load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(a.acts + size_t(k) * a.f), cpr, col, lane_on);
-    uint32_t cell = a.resolved[k];
-    const float wk = f16_to_f32(a.routing_w[k]);
-    if (cell == kSentinel && a.fallback) cell = a.fallback[k];  // moe.metal:1037-1038
+    load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(acts_tok + size_t(k) * a.f), cpr, col, lane_on);
+    uint32_t cell = resolved_tok[k];
+    const float wk = f16_to_f32(routing_tok[k]);
+    if (cell == kSentinel && fallback_tok) cell = fallback_tok[k];  // moe.metal:1037-1038
     const bool live = cell != kSentinel;
     const uint8_t *base = cell_base(a.pool, live ? cell : 0u, a.stride);
     const uint16_t *s_all = reinterpret_cast<const uint16_t *>(base + a.off.down_s_off);
@@ -84,9 +93,9 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     }
     __syncthreads();
     if (finisher) {
-        float acc = a.residual ? f16_to_f32(res_bits) : 0.0f;
+        float acc = residual_tok ? f16_to_f32(res_bits) : 0.0f;
         for (uint32_t i = 0; i < a.top_k; ++i) acc += partial[i][threadIdx.x];
-        phase2_finish(a.y, a.hidden, d0 + threadIdx.x, f32_to_f16(acc), hid_bits);
+        phase2_finish(y_tok, hidden_tok, d0 + threadIdx.x, f32_to_f16(acc), hid_bits);
     }
 }
 
@@ -105,7 +114,7 @@ static void launch_phase2_batch(const Phase2Args &a, dim3 grid, dim3 block, hipS
 
 template <int BITS>
 static void launch_phase2_bits(const Phase2Args &a, hipStream_t s) {
-    const dim3 grid((a.d + kPhase2Rows - 1) / kPhase2Rows), block(64 * a.top_k);
+    const dim3 grid((a.d + kPhase2Rows - 1) / kPhase2Rows, a.tokens ? a.tokens : 1u), block(64 * a.top_k);
     switch (nch_for(a.f, BITS)) {
         case 1: launch_phase2_batch<BITS, 1>(a, grid, block, s); break;
         case 2: launch_phase2_batch<BITS, 2>(a, grid, block, s); break;
@@ -197,6 +206,57 @@ int shrike_hip_moe_phase2_pool(shrike_hip_moe *moe, void *stream, const shrike_p
     a.y = static_cast<uint16_t *>(d_y); a.hidden = static_cast<uint16_t *>(d_hidden);
     a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.ebias = moe->desc.expert_additive_biases;
     a.indirect = d_indirect; a.io_status = moe->desc.event_gated_io ? d_io_status : nullptr;
+    return launch_phase2(a, bits, as_stream(stream));
+}
+
+// moe.metal:121-151 for a batch: position p of token t resolves to its expert's cell or the sentinel
+__global__ __launch_bounds__(256) void k_resolve_batch(const uint32_t *indices, const uint64_t *residency, uint32_t *resolved,
+                                                       uint32_t count, uint32_t num_experts, uint32_t *miss_count) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    bool miss = false;
+    if (i < count) {
+        const uint64_t word = residency[min(indices[i], num_experts - 1u)];
+        const bool hit = uint32_t(word >> 32) == SHRIKE_RESIDENCY_RESIDENT && uint32_t(word) != kSentinel;
+        resolved[i] = hit ? uint32_t(word) : kSentinel;
+        miss = !hit;
+    }
+    if (miss_count) {
+        const uint32_t n = __popcll(__ballot(miss));
+        if ((threadIdx.x & 63u) == 0u && n) atomicAdd(miss_count, n);
+    }
+}
+
+int shrike_hip_moe_resolve_batch(void *stream, const uint32_t *d_topk_indices, const uint64_t *d_residency,
+                                 uint32_t *d_resolved_slots, uint32_t count, uint32_t num_experts, uint32_t *d_miss_count) {
+    SHRIKE_REQUIRE(d_topk_indices && d_residency && d_resolved_slots, "resolve: indices, residency and resolvedSlots must be bound");
+    SHRIKE_REQUIRE(num_experts >= 1, "resolve: numExperts must be positive");
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(k_resolve_batch, dim3((count + 255u) / 256u), dim3(256), 0, as_stream(stream), d_topk_indices, d_residency,
+                       d_resolved_slots, count, num_experts, d_miss_count);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int shrike_hip_moe_phase2_batch(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                uint64_t pool_slot_stride, const uint32_t *d_resolved_slots,
+                                const shrike_expert_offsets *offsets, const void *d_acts, const void *d_routing_weights,
+                                const void *d_residual, void *d_y, void *d_hidden, uint32_t d, uint32_t f, uint32_t top_k,
+                                uint32_t tokens) {
+    SHRIKE_REQUIRE(moe != nullptr && pool != nullptr, "moe handle or pool is NULL");
+    SHRIKE_REQUIRE(top_k >= 1 && top_k <= SHRIKE_MAX_TOP_K, "phase2: topK=%u not in 1...8", top_k);
+    SHRIKE_REQUIRE(tokens >= 1 && tokens <= 65535u, "phase2: %u tokens not in 1...65535", tokens);
+    const uint32_t bits = moe->desc.routed_weight_bits;
+    if (int rc = check_offsets(offsets, d, f, bits)) return rc;
+    SHRIKE_REQUIRE(d_resolved_slots && d_acts && d_routing_weights && d_y, "phase2: resolvedSlots, acts, routingWeights and y must be bound");
+    SHRIKE_REQUIRE(pool_slot_stride % 16u == 0, "phase2: pool slot stride must be a multiple of 16");
+    Phase2Args a = {};
+    fill_pool(a.pool, pool);
+    a.stride = pool_slot_stride; a.resolved = d_resolved_slots; a.off = *offsets;
+    a.acts = static_cast<const uint16_t *>(d_acts); a.routing_w = static_cast<const uint16_t *>(d_routing_weights);
+    a.residual = static_cast<const uint16_t *>(d_residual);
+    a.y = static_cast<uint16_t *>(d_y); a.hidden = static_cast<uint16_t *>(d_hidden);
+    a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.ebias = moe->desc.expert_additive_biases;
+    a.tokens = tokens;
     return launch_phase2(a, bits, as_stream(stream));
 }
 

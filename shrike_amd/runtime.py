@@ -286,6 +286,21 @@ class MoE:
             C.byref(offsets), ptr(acts), ptr(routing_weights), ptr(residual), ptr(y), ptr(hidden),
             d, f, top_k, ptr(indirect), ptr(io_status)), "shrike_hip_moe_phase2_pool")
 
+    def encode_resolve_batch(self, topk, residency, resolved_slots, count, num_experts, miss_count=None):
+        check(capi.load().shrike_hip_moe_resolve_batch(self._s(), ptr(topk), ptr(residency), ptr(resolved_slots), count,
+                                                       num_experts, ptr(miss_count)), "shrike_hip_moe_resolve_batch")
+
+    def encode_phase1_batch(self, pool: ExpertPool, resolved_slots, offsets, x, x_stride, acts, d, f, top_k, tokens):
+        check(capi.load().shrike_hip_moe_phase1_batch(self.handle, self._s(), pool.bases, pool.stride, ptr(resolved_slots),
+                                                      C.byref(offsets), ptr(x), x_stride, ptr(acts), d, f, top_k, tokens),
+              "shrike_hip_moe_phase1_batch")
+
+    def encode_phase2_batch(self, pool: ExpertPool, resolved_slots, offsets, acts, routing_weights, residual, y, hidden,
+                            d, f, top_k, tokens):
+        check(capi.load().shrike_hip_moe_phase2_batch(self.handle, self._s(), pool.bases, pool.stride, ptr(resolved_slots),
+                                                      C.byref(offsets), ptr(acts), ptr(routing_weights), ptr(residual), ptr(y),
+                                                      ptr(hidden), d, f, top_k, tokens), "shrike_hip_moe_phase2_batch")
+
     def encode_shared_expert(self, gate, up, down, bits, x, scratch, h1, d, f_shared, scalar_gate=None):
         def proj(t):
             return Projection(ptr(t[0]), ptr(t[1]), ptr(t[2]))

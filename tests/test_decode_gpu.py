@@ -453,3 +453,59 @@ def test_argument_errors_are_reported_not_trapped(gpu):
         gpu.MoE(128, 64, 16, 9)
     with pytest.raises(capi.ShrikeError):
         gpu.ExpertPool(0, 4096, 4)
+
+
+@pytest.mark.parametrize("d,f,ne,k,t,bits", [(2880, 2880, 6, 4, 4, 4), (2880, 2880, 5, 4, 3, 8), (2304, 1024, 24, 8, 16, 8), (512, 256, 16, 4, 7, 4)])
+def test_batched_decode_operators_equal_the_single_token_ones(gpu, d, f, ne, k, t, bits):
+    """A batch of independent decode tokens (config 4: 4 tokens; config 5: 16 sequences): resolve,
+    phase 1 and phase 2 with the token dimension on the grid give, per token, the bytes of the
+    single-token operators, which the tests above hold to the oracle; routes come from the
+    block router and are checked against the oracle bit for bit."""
+    L = Layer(0x5EED0004, d, f, ne, k, bits=bits)
+    resident = [e for e in range(ne) if e % 5 != 3]  # some experts miss
+    dl = DeviceLayer(gpu, L, resident=resident)
+    stride = d + 16
+    x = S.activations_f16(L.tree, "batch.x", t * stride)
+    hidden0 = S.activations_f16(L.tree, "batch.hidden", t * d)
+    dx = gpu.dev(x)
+    pf = gpu.Prefill(dl.moe)
+    idx, w = gpu.empty(4 * t * k), gpu.empty(2 * t * k)
+    pf.encode_block(dl.router_w, dl.router_s, dl.router_b, dx, dl.eff_scale, dl.expert_scale, dl.logit_bias, idx, w,
+                    gpu.empty(pf.router_workspace_bytes(t, ne, d)), t, ne, d, k, stride)
+    resolved, misses = gpu.empty(4 * t * k), gpu.empty(4)
+    dl.moe.encode_resolve_batch(idx, dl.pool.table, resolved, t * k, ne, misses)
+    acts = gpu.empty(2 * t * k * f)
+    dl.moe.encode_phase1_batch(dl.pool, resolved, dl.off, dx, stride, acts, d, f, k, t)
+    residual = gpu.dev(S.activations_f16(L.tree, "batch.residual", t * d))
+    y, hid = gpu.empty(2 * t * d), gpu.dev(hidden0)
+    dl.moe.encode_phase2_batch(dl.pool, resolved, dl.off, acts, w, residual, y, hid, d, f, k, t)
+    gpu.synchronize()
+    h_idx, h_w = idx.download(np.uint32, t * k), w.download(np.uint16, t * k)
+    ref_idx, _, _ = O.prefill_router(L.router_dict(), x, t, d, k, stride=stride)
+    assert np.array_equal(h_idx, ref_idx)
+    h_res = resolved.download(np.uint32, t * k)
+    want = [dl.cell_of.get(int(e), SENT) for e in h_idx]
+    assert h_res.tolist() == want
+    assert int(misses.download(np.uint32, 1)[0]) == sum(1 for c in want if c == SENT)
+    all_acts, all_y, all_hid = acts.download(np.uint16, t * k * f), y.download(np.uint16, t * d), hid.download(np.uint16, t * d)
+    res_host = residual.download(np.uint16, t * d)
+    for tok in range(t):
+        one_x = gpu.dev(np.ascontiguousarray(x[tok * stride:tok * stride + d]))
+        one_res = gpu.dev(h_res[tok * k:(tok + 1) * k].copy())
+        dl.moe.encode_spec_phase1(dl.pool, one_res, dl.off, one_x, dl.acts, d, f, k)
+        one_hid = gpu.dev(hidden0[tok * d:(tok + 1) * d].copy())
+        dl.moe.encode_spec_phase2(dl.pool, one_res, dl.off, dl.acts, gpu.dev(h_w[tok * k:(tok + 1) * k].copy()),
+                                  gpu.dev(res_host[tok * d:(tok + 1) * d].copy()), dl.y, one_hid, d, f, k)
+        gpu.synchronize()
+        live = np.repeat(np.array(want[tok * k:(tok + 1) * k]) != SENT, f)
+        assert np.array_equal(all_acts[tok * k * f:(tok + 1) * k * f][live], dl.acts.download(np.uint16, k * f)[live])
+        assert np.array_equal(all_y[tok * d:(tok + 1) * d], dl.y.download(np.uint16, d))
+        assert np.array_equal(all_hid[tok * d:(tok + 1) * d], one_hid.download(np.uint16, d))
+    # and against the oracle for the first token
+    blobs = [None if c == SENT else dl.pool_blobs()[c] for c in want[:k]]
+    off = L.oracle_offsets()
+    ref_acts = O.moe_phase1(blobs, off, np.ascontiguousarray(x[:d]), d, f, bits, L.meta)
+    live0 = np.repeat(np.array(want[:k]) != SENT, f)
+    assert_ffn_close(all_acts[:k * f][live0], ref_acts[live0], "token 0 activations")
+    ref_y = O.moe_phase2(blobs, off, np.ascontiguousarray(all_acts[:k * f]), h_w[:k].copy(), res_host[:d].copy(), d, f, bits, L.meta)
+    assert_ffn_close(all_y[:d], ref_y, "token 0 y from the device's activations")
