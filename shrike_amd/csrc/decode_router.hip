@@ -12,23 +12,21 @@ __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
     __shared__ uint32_t s_last;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t e = blockIdx.x * 4u + wave;
-    if (e < a.sel.num_experts) {
-        router_row<RK>(a, e, lane);
-        if (lane == 0) __threadfence();
-    }
-    if (!a.lists.out_indices) return;  // logits only
+    const bool select_too = a.lists.out_indices != nullptr;
+    if (e < a.sel.num_experts) router_row<RK>(a, e, lane, select_too);
+    if (!select_too) return;  // logits only
+    // The logits went out as write-through stores: once they are complete, the workgroup
+    // counts itself in; the last to arrive reads all logits back past the caches.
+    wait_stores();
     __syncthreads();
-    if (threadIdx.x == 0) {
-        __threadfence();
-        s_last = atomicAdd(a.counter, 1u) == gridDim.x - 1u ? 1u : 0u;
-    }
+    if (threadIdx.x == 0)
+        s_last = __hip_atomic_fetch_add(a.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1u ? 1u : 0u;
     __syncthreads();
     if (!s_last || wave != 0) return;
-    __threadfence();
     __shared__ RouteScratch s_route;
     uint32_t cell;
     route_wave<true>(a.sel, a.lists, lane, true, cell, s_route);
-    if (lane == 0) *a.counter = 0u;
+    if (lane == 0) __hip_atomic_store(a.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The head of the fused layer: the router's logit rows and, beside them in the same grid,

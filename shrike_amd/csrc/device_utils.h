@@ -56,6 +56,11 @@ __device__ __forceinline__ float wave_sum(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Every store this wave has issued is complete; for a write-through (device-scope atomic)
+// store that means visible device-wide. Cheaper than a device-scope release fence, which
+// also writes back the whole second-level cache of this group of compute units.
+__device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // Wave-wide float max / unsigned min, broadcast to every lane. Rows a step does not
 // write keep their own value (old = self), so the partial results stay valid operands.
 template <int CTRL, int ROW_MASK = 0xf>

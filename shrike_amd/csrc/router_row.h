@@ -11,7 +11,7 @@ namespace shrike {
 // fixed so that the fp32 logits are reproducible bit for bit (lane l takes chunks
 // l, l+64, ...).
 template <int RK>
-__device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint32_t lane) {
+__device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint32_t lane, bool publish = false) {
     constexpr int E = RK == 0 ? 8 : RK == 8 ? 16 : 32;  // elements per 16-byte weight chunk
     constexpr int PIECES = E / 8;
     constexpr int MAXI = RK == 0 ? 8 : 4;
@@ -75,7 +75,12 @@ __device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint
     }
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, o));
-    if (lane == 0) a.logits_out[e] = acc;
+    // publish: the logit is for another workgroup of the same launch and is written through to
+    // device-coherent memory
+    if (lane == 0) {
+        if (publish) __hip_atomic_store(a.logits_out + e, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else a.logits_out[e] = acc;
+    }
 }
 
 }  // namespace shrike
