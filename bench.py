@@ -418,6 +418,23 @@ def main():
             moe.encode_spec_phase1(lay["pool"], lay["res"], off, lay["x"], lay["acts"], D, F, K)
             moe.encode_spec_phase2(lay["pool"], lay["res"], off, lay["acts"], lay["w"], lay["h1"], lay["y"], None, D, F, K)
 
+    # the floors phase 1 is bounded by on this part: a launch with nothing to do, and a kernel that only
+    # reads the bytes phase 1 reads (gate + up sub-tensors of the same eight cells) with no arithmetic
+    sink = rt.empty(4)
+    p1_blocks = K * F // 4 // 4
+    p1_bytes_per_cell = 2 * (F * D // 2 + 2 * F * (D // 64) * 2)
+
+    def empty_only():
+        for lay in layers:
+            capi.check(capi.load().shrike_hip_probe_empty_launch(stream.handle, p1_blocks, sink.ptr), "probe_empty_launch")
+
+    def read_only():
+        for lay in layers:
+            capi.check(capi.load().shrike_hip_probe_read(stream.handle, lay["pool"].bases, lay["pool"].stride, lay["res"].ptr,
+                                                         K, off.gate_w_off, p1_bytes_per_cell, sink.ptr), "probe_read")
+
+    g_empty = capture(rt, capi, stream, empty_only)
+    g_read = capture(rt, capi, stream, read_only)
     g_p12 = capture(rt, capi, stream, phase12)
     g_p1 = capture(rt, capi, stream, phase1_only)
     g_p2 = capture(rt, capi, stream, phase2_only)
@@ -433,7 +450,8 @@ def main():
     reps = max(1, steps // n_layers // 2)
     parts = {}
     for name, g, launches_per_layer in (("phase1+phase2 alternating", g_p12, 2), ("phase1", g_p1, 1), ("phase2", g_p2, 1), ("router_select_classify", g_rt, 1),
-                                        ("shared_expert(2 launches)", g_sh, 1)):
+                                        ("shared_expert(2 launches)", g_sh, 1), ("empty launch of phase 1's grid", g_empty, 1),
+                                        ("read-only kernel over phase 1's bytes", g_read, 1)):
         time_graph(rt, capi, stream, g, 2)
         parts[name] = time_graph(rt, capi, stream, g, reps) / (reps * n_layers) * 1e3  # us per layer
 
@@ -458,7 +476,9 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "k_phase1<4,1,4,false,0> (routed gate/up matvec + SiLU-multiply)",
                      "achieved": round(p1_bytes / (p1_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(p1_bytes / (p1_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-                     "bytes_per_launch": p1_bytes, "us_per_launch": round(p1_us, 3), "traffic": PHASE1_TRAFFIC_BYTES},
+                     "bytes_per_launch": p1_bytes, "us_per_launch": round(p1_us, 3), "traffic": PHASE1_TRAFFIC_BYTES,
+                     "floors_us": {"empty_launch": round(parts["empty launch of phase 1's grid"], 3),
+                                   "read_only_same_bytes": round(parts["read-only kernel over phase 1's bytes"], 3)}},
         "setup_seconds": round(gen_s, 1),
     }
     if args.cpu_sample > 0:

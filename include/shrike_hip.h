@@ -267,6 +267,16 @@ typedef struct {
 int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
                                 const shrike_decode_layer_args *args);
 
+/* ------------------------------------------------------- measurement aids
+ * No counterpart in the reference. An empty launch of `workgroups` x 256 threads, and a
+ * kernel that only reads bytes [byte_offset, byte_offset + bytes_per_cell) of each pool cell
+ * in d_cells (u32[cell_count], as resolvedSlots holds them): the two floors a decode kernel
+ * on the same cells is measured against. d_sink: u32[1], never written in practice. */
+int shrike_hip_probe_empty_launch(void *stream, uint32_t workgroups, uint32_t *d_sink);
+int shrike_hip_probe_read(void *stream, const shrike_pool_bases *pool, uint64_t pool_slot_stride,
+                          const uint32_t *d_cells, uint32_t cell_count, uint64_t byte_offset,
+                          uint64_t bytes_per_cell, uint32_t *d_sink);
+
 /* ------------------------------------------------------- prefill operators */
 
 /* PrefillRouter.encodeBlock, sources/Shrike/Kernels/Prefill/MoE/PrefillRouter.swift:75-152

@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     const uint16_t *x_tok = a.x + tok * a.x_stride;
     const uint32_t *resolved_tok = a.resolved + tok * a.top_k;
     uint16_t *acts_tok = a.acts + tok * a.top_k * a.f;
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t cpr = a.d * BITS / 128u, groups = a.d / kGroup, row_bytes = cpr * 16u;
     const uint32_t pair0 = (blockIdx.x * 4u + wave) * RP;
     const bool in_range = pair0 < a.top_k * a.f;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
         cell = resolved_tok[k];
     }
     if (cell == kSentinel) return;  // moe.metal:986, and waves past the last row
-    const uint8_t *base = cell_base(a.pool, cell, a.stride);
+    const uint8_t *base = cell_base_uniform(a.pool, cell, a.stride);
 
     RowRegs<BITS, NCH> rows[2 * RP];
 #pragma unroll

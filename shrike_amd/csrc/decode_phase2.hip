@@ -31,7 +31,7 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     const uint16_t *residual_tok = a.residual ? a.residual + tok * a.d : nullptr;
     uint16_t *y_tok = a.y + tok * a.d;
     uint16_t *hidden_tok = a.hidden ? a.hidden + tok * a.d : nullptr;
-    const uint32_t lane = threadIdx.x & 63u, k = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63u, k = wave_index();
     const uint32_t d0 = blockIdx.x * kPhase2Rows;
     // the epilogue's operands do not depend on anything computed here: fetch them first
     const bool finisher = threadIdx.x < kPhase2Rows && d0 + threadIdx.x < a.d;
@@ -57,7 +57,7 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     const float wk = f16_to_f32(routing_tok[k]);
     if (cell == kSentinel && fallback_tok) cell = fallback_tok[k];  // moe.metal:1037-1038
     const bool live = cell != kSentinel;
-    const uint8_t *base = cell_base(a.pool, live ? cell : 0u, a.stride);
+    const uint8_t *base = cell_base_uniform(a.pool, live ? cell : 0u, a.stride);
     const uint16_t *s_all = reinterpret_cast<const uint16_t *>(base + a.off.down_s_off);
     const uint16_t *b_all = reinterpret_cast<const uint16_t *>(base + a.off.down_b_off);
 

@@ -10,7 +10,7 @@ namespace shrike {
 template <int RK>
 __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
     __shared__ uint32_t s_last;
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t e = blockIdx.x * 4u + wave;
     const bool select_too = a.lists.out_indices != nullptr;
     if (e < a.sel.num_experts) router_row<RK>(a, e, lane, select_too);
@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
 template <int RK, int BITS, int NCH>
 __global__ __launch_bounds__(256) void k_head(RouterArgs r, GemvArgs g, uint32_t router_blocks) {
     if (blockIdx.x < router_blocks) {
-        const uint32_t e = blockIdx.x * 4u + (threadIdx.x >> 6);
+        const uint32_t e = blockIdx.x * 4u + wave_index();
         if (e < r.sel.num_experts) router_row<RK>(r, e, threadIdx.x & 63u);
     } else {
         gemv_job<BITS, NCH>(g, blockIdx.x - router_blocks);

@@ -56,6 +56,10 @@ __device__ __forceinline__ float wave_sum(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// The wave's index in its workgroup, as a scalar: what is derived from it (rows, routed
+// position, the cell and its base) then lives in scalar registers and scalar loads.
+__device__ __forceinline__ uint32_t wave_index() { return uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6))); }
+
 // Every store this wave has issued is complete; for a write-through (device-scope atomic)
 // store that means visible device-wide. Cheaper than a device-scope release fence, which
 // also writes back the whole second-level cache of this group of compute units.

@@ -1,0 +1,67 @@
+// Measurement aids, not operators: an empty launch and a kernel that only reads a byte range
+// of each listed pool cell. Timed beside a real kernel on the same cells they give the two
+// floors that bound it on this part: what a launch costs with nothing to do, and what
+// moving the same bytes costs with no arithmetic and no dependent loads behind it.
+#include "gemv_common.h"
+
+namespace shrike {
+
+__global__ __launch_bounds__(256) void k_probe_empty(uint32_t *sink) {
+    if (sink == nullptr && threadIdx.x == 0xffffffffu) *sink = 0u;  // never true; keeps the argument live
+}
+
+// A wave reads kProbeLoads x 1 KiB (16 bytes a lane) of one cell's range.
+constexpr uint32_t kProbeLoads = 4;
+
+__global__ __launch_bounds__(256) void k_probe_read(PoolArg pool, uint64_t stride, const uint32_t *cells, uint32_t cell_count,
+                                                    uint64_t byte_offset, uint32_t waves_per_cell, uint32_t loads_per_cell, uint32_t *sink) {
+    const uint32_t lane = threadIdx.x & 63u, wave = blockIdx.x * 4u + wave_index();
+    const uint32_t which = wave / waves_per_cell, part = wave % waves_per_cell;
+    if (which >= cell_count) return;
+    const uint4 *base = reinterpret_cast<const uint4 *>(cell_base_uniform(pool, cells[which], stride) + byte_offset);
+    uint4 v[kProbeLoads];
+#pragma unroll
+    for (uint32_t i = 0; i < kProbeLoads; ++i) {
+        const uint32_t load = part * kProbeLoads + i;
+        v[i] = load < loads_per_cell ? base[size_t(load) * 64u + lane] : zero4();
+    }
+    uint32_t acc = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < kProbeLoads; ++i) acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    // the loads must not be optimised away; uniform int4 codes never fold to this word in practice,
+    // and nothing reads the sink
+    if (acc == 0x9E3779B9u) sink[0] = wave;
+}
+
+}  // namespace shrike
+
+using namespace shrike;
+
+extern "C" {
+
+int shrike_hip_probe_empty_launch(void *stream, uint32_t workgroups, uint32_t *d_sink) {
+    SHRIKE_REQUIRE(workgroups >= 1 && d_sink != nullptr, "probe: workgroups must be positive and the sink bound");
+    hipLaunchKernelGGL(k_probe_empty, dim3(workgroups), dim3(256), 0, as_stream(stream), d_sink);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int shrike_hip_probe_read(void *stream, const shrike_pool_bases *pool, uint64_t pool_slot_stride, const uint32_t *d_cells,
+                          uint32_t cell_count, uint64_t byte_offset, uint64_t bytes_per_cell, uint32_t *d_sink) {
+    SHRIKE_REQUIRE(pool != nullptr && d_cells != nullptr && d_sink != nullptr, "probe: pool, cells and sink must be bound");
+    SHRIKE_REQUIRE(cell_count >= 1 && bytes_per_cell >= 1024u, "probe: nothing to read");
+    SHRIKE_REQUIRE(byte_offset % 16u == 0 && bytes_per_cell % 1024u == 0 && pool_slot_stride % 16u == 0,
+                   "probe: the range must be 16-byte aligned and a multiple of 1 KiB long");
+    SHRIKE_REQUIRE(byte_offset + bytes_per_cell <= pool_slot_stride, "probe: the range leaves the cell");
+    PoolArg p;
+    fill_pool(p, pool);
+    const uint32_t loads = uint32_t(bytes_per_cell / 1024u);
+    const uint32_t waves_per_cell = (loads + kProbeLoads - 1) / kProbeLoads;
+    const uint32_t waves = waves_per_cell * cell_count;
+    hipLaunchKernelGGL(k_probe_read, dim3((waves + 3) / 4), dim3(256), 0, as_stream(stream), p, pool_slot_stride, d_cells,
+                       cell_count, byte_offset, waves_per_cell, loads, d_sink);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // extern "C"

@@ -23,6 +23,12 @@ struct PoolArg {
 __device__ __forceinline__ const uint8_t *cell_base(const PoolArg &pool, uint32_t cell, uint64_t stride) {
     return pool.base[cell / pool.cells_per_chunk] + uint64_t(cell % pool.cells_per_chunk) * stride;
 }
+// The same for a cell every lane of the wave agrees on: the division and the look-up of the
+// chunk's base run on the scalar unit (a per-lane index into the argument block would be
+// one more dependent memory load ahead of the rows).
+__device__ __forceinline__ const uint8_t *cell_base_uniform(const PoolArg &pool, uint32_t cell, uint64_t stride) {
+    return cell_base(pool, uint32_t(__builtin_amdgcn_readfirstlane(int(cell))), stride);
+}
 
 __device__ __forceinline__ float meta_f32(uint16_t b, uint32_t meta) {
     return meta == SHRIKE_META_F16 ? f16_to_f32(b) : bf16_to_f32(b);
@@ -64,26 +70,28 @@ template <> struct Chunk<8> {
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0u, 0u, 0u, 0u); }
 
 // Raw 16-byte pieces of the lane's activation slices for column chunks col + 64*i.
+// `off` has bit i set when slice i is not this lane's to use: the load then went to a valid
+// stand-in address and unpack_slices zeroes the slice. (Zeroing right behind the load would
+// make the wave wait for that load there and then, one load at a time.)
 template <int BITS, int NCH>
 struct SliceRegs {
     uint4 v[NCH][Chunk<BITS>::PIECES];
+    uint32_t off;
 };
 
 template <int BITS, int NCH>
 __device__ __forceinline__ void load_slice_regs(SliceRegs<BITS, NCH> &r, const uint4 *vec, uint32_t cpr,
                                                 uint32_t col, bool lane_on) {
     typedef Chunk<BITS> C;
+    r.off = 0u;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
         const uint32_t c = col + 64u * i;
         const bool on = lane_on && c < cpr;
         const uint32_t cc = on ? c : 0u;
+        r.off |= on ? 0u : 1u << i;
 #pragma unroll
-        for (int j = 0; j < C::PIECES; ++j) {
-            uint4 v = vec[cc * C::PIECES + j];
-            if (!on) v = zero4();
-            r.v[i][j] = v;
-        }
+        for (int j = 0; j < C::PIECES; ++j) r.v[i][j] = vec[cc * C::PIECES + j];
     }
 }
 
@@ -97,8 +105,9 @@ __device__ __forceinline__ void unpack_slices(const SliceRegs<BITS, NCH> &r, typ
         float s = 0.0f;
 #pragma unroll
         for (int j = 0; j < C::PIECES; ++j) {
-            C::fill(x[i], j, r.v[i][j]);
-            s += sum_x8(r.v[i][j]);
+            const uint4 v = (r.off >> i) & 1u ? zero4() : r.v[i][j];
+            C::fill(x[i], j, v);
+            s += sum_x8(v);
         }
         xs[i] = s;
     }
@@ -112,7 +121,9 @@ __device__ __forceinline__ void load_slices(const uint4 *vec, uint32_t cpr, uint
     unpack_slices<BITS, NCH>(r, x, xs);
 }
 
-// One row's codes and metadata for the lane's column chunks.
+// One row's codes and metadata for the lane's column chunks. A chunk that is not this lane's
+// is loaded from a valid stand-in address (chunk 0 of the same row) and left as it is: the
+// lane's activation slice for it is zero, and so is its term (the row's data being finite).
 template <int BITS, int NCH>
 struct RowRegs {
     uint4 w[NCH];
@@ -129,10 +140,9 @@ __device__ __forceinline__ void load_row(RowRegs<BITS, NCH> &r, const uint8_t *w
         const bool on = lane_on && c < cpr;
         const uint32_t cc = on ? c : 0u;
         const uint32_t g = cc * C::E / kGroup;
-        uint4 w = *reinterpret_cast<const uint4 *>(w_row + 16u * cc);
-        uint16_t s = s_row[g], b = b_row[g];
-        if (!on) { w = zero4(); s = 0; b = 0; }
-        r.w[i] = w; r.s[i] = s; r.b[i] = b;
+        r.w[i] = *reinterpret_cast<const uint4 *>(w_row + 16u * cc);
+        r.s[i] = s_row[g];
+        r.b[i] = b_row[g];
     }
 }
 
@@ -170,7 +180,7 @@ constexpr uint32_t kGemvRowsPerWave = 4;
 template <int BITS, int NCH>
 __device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block) {
     typedef Chunk<BITS> C;
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t cpr = a.n * BITS / 128u, groups = a.n / kGroup, row_bytes = cpr * 16u;
     const bool packed = cpr < 64u && (64u % cpr) == 0u;
     const uint32_t rpl = packed ? 64u / cpr : 1u;

@@ -441,6 +441,27 @@ def test_multi_chunk_pool_addressing(gpu):
     assert np.array_equal(outs[0], outs[1])
 
 
+def test_measurement_probes_run_and_check_their_arguments(gpu):
+    """The empty launch and the read-only kernel that bench.py times beside phase 1."""
+    L = Layer(33, 256, 128, 12, 4)
+    dl = DeviceLayer(gpu, L)
+    lib = capi.load()
+    sink = gpu.empty(4).fill(0)
+    cells = gpu.empty(4 * 4)
+    cells.upload(np.array([dl.cell_of[e] for e in (0, 5, 7, 11)], np.uint32))
+    nbytes = (dl.off.down_w_off - dl.off.gate_w_off) // 1024 * 1024
+    capi.check(lib.shrike_hip_probe_empty_launch(None, 64, sink.ptr), "probe_empty_launch")
+    capi.check(lib.shrike_hip_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, dl.off.gate_w_off, nbytes,
+                                         sink.ptr), "probe_read")
+    gpu.synchronize()
+    assert sink.download(np.uint32, 1)[0] == 0
+    assert lib.shrike_hip_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 0, dl.pool.stride + 1024,
+                                     sink.ptr) != 0
+    assert "leaves the cell" in capi.last_error()
+    assert lib.shrike_hip_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 8, 1024, sink.ptr) != 0
+    assert lib.shrike_hip_probe_empty_launch(None, 0, sink.ptr) != 0
+
+
 def test_argument_errors_are_reported_not_trapped(gpu):
     moe = gpu.MoE(128, 64, 16, 8)
     with pytest.raises(capi.ShrikeError, match="topK"):
