@@ -11,6 +11,8 @@
 //   PrefillRouter / PrefillMoEGrouping /              shrike::PrefillRouter, shrike::PrefillMoEGrouping,
 //   PrefillGroupedRoutedMoE / PrefillMoE              shrike::PrefillGroupedRoutedMoE, shrike::PrefillMoE
 //   RuntimeConfiguration (budget -> slots)            shrike::RuntimeConfiguration
+//   ParallelExpertReader (Infrastructure/Streaming)   shrike::ParallelExpertReader
+//   PackedExpertsLayout(Reader) (Infrastructure/ModelIO) shrike::PackedExpertsLayout
 #pragma once
 
 #include <cerrno>
@@ -74,11 +76,100 @@ public:
     const uint64_t *residencyTable() const { return static_cast<const uint64_t *>(shrike_hip_pool_residency_table(h_)); }
     void upload(uint32_t cell, const void *hostBlob, uint64_t bytes, Stream s) { check(shrike_hip_pool_upload_async(h_, cell, hostBlob, bytes, s)); }
     void publish(uint32_t expert, uint32_t cell, uint32_t state, Stream s) { check(shrike_hip_pool_table_publish(h_, expert, cell, state, s)); }
+    // blobs at fileOffsets of the reader's layer file -> cells, through pinned staging memory
+    void fetchExperts(shrike_expert_reader *reader, const std::vector<uint64_t> &fileOffsets, const std::vector<uint32_t> &cells,
+                      uint64_t blobBytes, void *pinnedStaging, uint64_t stagingBytes, Stream s) {
+        if (fileOffsets.size() != cells.size()) throw Error(EINVAL, "one cell per file offset");
+        check(shrike_hip_pool_fetch_experts(h_, s, reader, fileOffsets.data(), cells.data(), uint32_t(cells.size()), blobBytes,
+                                            pinnedStaging, stagingBytes));
+    }
     uint64_t residencyEntry(uint32_t expert) const { return shrike_hip_pool_table_entry(h_, expert); }
     shrike_hip_pool *handle() const { return h_; }
 
 private:
     shrike_hip_pool *h_;
+};
+
+// ParallelExpertReader (sources/Shrike/Infrastructure/Streaming/ParallelExpertReader.swift) over the
+// reference's own C reader interface
+class ParallelExpertReader {
+public:
+    struct Failure : Error {
+        using Error::Error;
+    };
+    ParallelExpertReader(const std::string &path, size_t expertStride, int threads = 4, int batchDepth = 1, bool bypassCache = false) {
+        int err = 0;
+        h_ = shrike_expert_reader_create(path.c_str(), expertStride, threads, batchDepth, bypassCache, &err);
+        if (!h_) throw Failure(err, "cannot open " + path);
+    }
+    ~ParallelExpertReader() { shrike_expert_reader_destroy(h_); }
+    ParallelExpertReader(const ParallelExpertReader &) = delete;
+    ParallelExpertReader &operator=(const ParallelExpertReader &) = delete;
+    int threadCount() const { return shrike_expert_reader_threads(h_); }
+    int batchDepth() const { return shrike_expert_reader_batch_depth(h_); }
+    void fetch(const std::vector<uint32_t> &experts, const std::vector<void *> &into) {
+        if (experts.size() != into.size()) throw Failure(EINVAL, "one destination per expert");
+        if (int rc = shrike_expert_reader_fetch(h_, experts.data(), into.data(), experts.size())) throw Failure(rc, "expert read failed");
+    }
+    void fetch(const std::vector<uint64_t> &offsets, const std::vector<void *> &into) {
+        if (offsets.size() != into.size()) throw Failure(EINVAL, "one destination per offset");
+        if (int rc = shrike_expert_reader_fetch_offsets(h_, offsets.data(), into.data(), offsets.size())) throw Failure(rc, "expert read failed");
+    }
+    shrike_expert_reader *handle() const { return h_; }
+
+private:
+    shrike_expert_reader *h_;
+};
+
+// PackedExpertsLayout + PackedExpertsLayoutReader (PackedExpertsLayout.swift:34-129) and
+// Model.routedExpertOffsets (ModelExpertIO.swift:69-94)
+class PackedExpertsLayout {
+public:
+    static PackedExpertsLayout load(const std::string &modelDirectory, uint64_t maxBytes = 0) {
+        int err = 0;
+        shrike_packed_layout *h = shrike_packed_layout_load(modelDirectory.c_str(), maxBytes, &err);
+        if (!h) throw Error(err, shrike_host_last_error());
+        return PackedExpertsLayout(h);
+    }
+    static PackedExpertsLayout decode(const std::string &json) {
+        int err = 0;
+        shrike_packed_layout *h = shrike_packed_layout_decode(json.data(), json.size(), &err);
+        if (!h) throw Error(err, shrike_host_last_error());
+        return PackedExpertsLayout(h);
+    }
+    PackedExpertsLayout(PackedExpertsLayout &&o) noexcept : h_(o.h_) { o.h_ = nullptr; }
+    PackedExpertsLayout(const PackedExpertsLayout &) = delete;
+    PackedExpertsLayout &operator=(const PackedExpertsLayout &) = delete;
+    ~PackedExpertsLayout() { shrike_packed_layout_destroy(h_); }
+    uint64_t expertStride() const { return shrike_packed_layout_expert_stride(h_); }
+    int numLayers() const { return shrike_packed_layout_num_layers(h_); }
+    int expertsPerLayer() const { return shrike_packed_layout_experts_per_layer(h_); }
+    std::string file(int layer) const {
+        const char *name = nullptr;
+        check(shrike_packed_layout_layer(h_, layer, nullptr, &name, nullptr));
+        return name;
+    }
+    shrike_packed_expert expert(int layer, int expert) const {
+        shrike_packed_expert out;
+        check(shrike_packed_layout_expert(h_, layer, expert, &out));
+        return out;
+    }
+    std::optional<shrike_packed_tensor> subTensor(int layer, int expert, const std::string &role) const {
+        shrike_packed_tensor out;
+        const int rc = shrike_packed_layout_tensor(h_, layer, expert, role.c_str(), &out);
+        if (rc == ENOENT) return std::nullopt;
+        check(rc);
+        return out;
+    }
+    shrike_expert_offsets routedExpertOffsets(int layer, bool expertsHaveAdditiveBiases = false) const {
+        shrike_expert_offsets out;
+        check(shrike_packed_layout_expert_offsets(h_, layer, expertsHaveAdditiveBiases, &out));
+        return out;
+    }
+
+private:
+    explicit PackedExpertsLayout(shrike_packed_layout *h) : h_(h) {}
+    shrike_packed_layout *h_;
 };
 
 // ExpertCachePlan (PreadExpertStreamer.swift:17-38)

@@ -52,13 +52,7 @@ int shrike_hip_init(int device);
 
 /* ---------------------------------------------------------------- layouts */
 
-/* MoEExpertOffsets, sources/Shrike/Kernels/MoE/MoE.swift:4-39 (field for field). */
-typedef struct {
-    uint32_t gate_w_off, gate_s_off, gate_b_off;
-    uint32_t up_w_off, up_s_off, up_b_off;
-    uint32_t down_w_off, down_s_off, down_b_off;
-    uint32_t gate_ab_off, up_ab_off, down_ab_off;
-} shrike_expert_offsets;
+/* shrike_expert_offsets (MoEExpertOffsets) is declared in shrike_host.h. */
 
 /* CPUExpertFFN.Offsets(d:f:), sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:34-61,
  * for 4- or 8-bit codes; additive biases (gpt-oss) are appended when asked for.
@@ -129,6 +123,18 @@ uint64_t shrike_hip_pool_table_entry(const shrike_hip_pool *pool, uint32_t exper
 int shrike_hip_pool_execute_plan(shrike_hip_pool *pool, shrike_slot_cache *cache,
                                  const shrike_expert_cache_plan *plan, const void *host_store, uint64_t store_expert_stride,
                                  uint64_t expert_bytes, void *stream, uint64_t elapsed_nanos);
+
+/* The streamer's read into the slots (PreadExpertStreamer.swift:577-628) for a pool in HBM:
+ * `count` blobs of blob_bytes at file_offsets[i] of the reader's layer file (blob_bytes is the
+ * stride the reader was created with) are read through the parallel reader into the pinned
+ * staging buffer and copied from there into cells[i] on `stream`. The staging buffer is used
+ * as two halves, so the reads of one batch run beside the copies of the one before; it must
+ * hold at least two blobs. Blocks until the last copy has finished; returns the reader's errno
+ * on a failed read (cells already written are then undefined, as the reference's are). */
+int shrike_hip_pool_fetch_experts(shrike_hip_pool *pool, void *stream, shrike_expert_reader *reader,
+                                  const uint64_t *file_offsets, const uint32_t *cells, uint32_t count,
+                                  uint64_t blob_bytes, void *pinned_staging, uint64_t staging_bytes);
+
 
 /* ------------------------------------------------------------ MoE operators */
 

@@ -210,6 +210,113 @@ uint64_t shrike_slot_cache_entry(shrike_slot_cache *cache, uint32_t expert);
 size_t shrike_slot_cache_drain_publications(shrike_slot_cache *cache, uint32_t *experts,
                                             uint64_t *words, size_t capacity);
 
+/* MoEExpertOffsets, sources/Shrike/Kernels/MoE/MoE.swift:4-39 (field for field). */
+typedef struct {
+    uint32_t gate_w_off, gate_s_off, gate_b_off;
+    uint32_t up_w_off, up_s_off, up_b_off;
+    uint32_t down_w_off, down_s_off, down_b_off;
+    uint32_t gate_ab_off, up_ab_off, down_ab_off;
+} shrike_expert_offsets;
+
+/* ------------------------------------------------------- parallel expert reader */
+
+/* The reference's reader interface, name for name
+ * (sources/ShrikeKernelsC/include/shrike_expert_io.h:20-129; implementation
+ * sources/ShrikeKernelsC/expert_io.c), for Linux: `threads` workers with a descriptor each
+ * serve up to `batch_depth` published batches, oldest first; reads are plain pread, no
+ * shared offset, no mmap. bypass_cache opens the descriptors with O_DIRECT (the reference
+ * sets F_NOCACHE, expert_io.c:216-229) and, like the reference, fails the reader when the
+ * file system refuses rather than read through the page cache; with it, destinations,
+ * offsets and the stride must meet the device's direct-I/O alignment (the format's 16 KiB
+ * does). create returns NULL and the cause in *out_errno; fetch returns 0 or the first
+ * errno any worker saw (EIO for a blob that runs past the end of the file). */
+typedef struct shrike_expert_reader shrike_expert_reader;
+#define SHRIKE_IO_MAX_THREADS 16
+#define SHRIKE_IO_MAX_BATCHES 2
+shrike_expert_reader *shrike_expert_reader_create(const char *path, size_t expert_stride, int threads,
+                                                  int batch_depth, int bypass_cache, int *out_errno);
+/* no other thread may be inside a fetch when this runs (shrike_expert_io.h:58-60) */
+void shrike_expert_reader_destroy(shrike_expert_reader *reader);
+/* expert_ids[i] * expert_stride -> destinations[i], each expert_stride bytes; blocks until all landed */
+int shrike_expert_reader_fetch(shrike_expert_reader *reader, const uint32_t *expert_ids,
+                               void *const *destinations, size_t count);
+/* the same with absolute byte offsets (shrike_expert_io.h:74-82) */
+int shrike_expert_reader_fetch_offsets(shrike_expert_reader *reader, const uint64_t *offsets,
+                                       void *const *destinations, size_t count);
+int shrike_expert_reader_threads(const shrike_expert_reader *reader);
+int shrike_expert_reader_batch_depth(const shrike_expert_reader *reader);
+
+/* The claim, free-slot and cancel rules as pure functions (shrike_expert_io.h:90-129). */
+typedef struct {
+    int active;          /* published, not yet reaped by its submitter */
+    uint64_t sequence;   /* publication order, lower is older */
+    size_t next_index;   /* next unclaimed read */
+    size_t count;        /* reads in the batch */
+} shrike_expert_batch_slot;
+int shrike_expert_reader_claim_slot(const shrike_expert_batch_slot *slots, int slot_count);
+int shrike_expert_reader_free_slot(const shrike_expert_batch_slot *slots, int slot_count);
+typedef struct {
+    size_t count, next_index, outstanding;
+    int first_errno;
+} shrike_expert_batch_cancel_state;
+void shrike_expert_reader_cancel_slot(shrike_expert_batch_cancel_state *slot);
+
+/* ------------------------------------------------------- packed experts layout */
+
+/* packed_experts/layout.json of a .gturbo model directory: the wire form
+ * (sources/ShrikeFormat/GTurboPackedExpertsLayoutV1.swift:3-62), its structural validator
+ * (:75-164), the manifest cross-check (:166-199) and the runtime view sorted by layer and by
+ * logical expert id (sources/Shrike/Infrastructure/ModelIO/PackedExpertsLayout.swift:4-129).
+ * decode: JSON text -> validated layout, NULL + EINVAL with the reference's field/reason in
+ * shrike_host_last_error() otherwise. load: <model_dir>/packed_experts/layout.json; ENOENT
+ * when missing, EFBIG when the file exceeds max_bytes ("exceeds metadata cap",
+ * GTurboModelDirectory.swift:70-75; 0 = the format's 32 MiB). */
+typedef struct shrike_packed_layout shrike_packed_layout;
+#define SHRIKE_LAYOUT_ALIGNMENT_BYTES 16384u            /* GTurboFormatV1.alignmentBytes */
+#define SHRIKE_LAYOUT_MAX_BYTES (32u * 1024u * 1024u)   /* GTurboFormatV1.residentIndexMaxBytes */
+shrike_packed_layout *shrike_packed_layout_decode(const char *json, size_t bytes, int *out_errno);
+shrike_packed_layout *shrike_packed_layout_load(const char *model_dir, uint64_t max_bytes, int *out_errno);
+void shrike_packed_layout_destroy(shrike_packed_layout *layout);
+const char *shrike_host_last_error(void);   /* of the calling thread; same text as shrike_hip_last_error */
+
+uint64_t shrike_packed_layout_expert_stride(const shrike_packed_layout *layout);
+int shrike_packed_layout_num_layers(const shrike_packed_layout *layout);
+int shrike_packed_layout_experts_per_layer(const shrike_packed_layout *layout);
+/* Layer `index` in ascending layer order: its id, file basename and expert count (0 for a
+ * dense layer, which has no file). EINVAL past the end. */
+int shrike_packed_layout_layer(const shrike_packed_layout *layout, int index, int *layer_id,
+                               const char **file, int *expert_count);
+/* PackedExpertsLayout.expert(layer:expert:) (PackedExpertsLayout.swift:53-65): position
+ * `expert` in the layer's list sorted by logical id. ERANGE with the reference's wording
+ * when either index is out of range. */
+typedef struct {
+    int32_t expert, physical_rank;
+    uint64_t offset, size;      /* of the blob inside the layer file */
+    uint32_t tensor_count;
+} shrike_packed_expert;
+int shrike_packed_layout_expert(const shrike_packed_layout *layout, int layer, int expert,
+                                shrike_packed_expert *out);
+/* A sub-tensor by role name ("gate", "gate_scales", ...). ENOENT when the blob has none. */
+typedef struct {
+    uint64_t offset, size;      /* relative to the blob */
+    char dtype[8];              /* "U32" or "BF16" */
+    uint32_t shape[4], rank;
+    int32_t bits;               /* 0 when absent */
+} shrike_packed_tensor;
+int shrike_packed_layout_tensor(const shrike_packed_layout *layout, int layer, int expert,
+                                const char *role, shrike_packed_tensor *out);
+/* Model.routedExpertOffsets (sources/Shrike/Runtime/Inference/ModelExpertIO.swift:69-94): the
+ * nine (+ three) offsets from expert 0 of the layer, 0 for a role the blob lacks; EINVAL
+ * "is missing gate_bias" style when additive biases are expected and absent. */
+int shrike_packed_layout_expert_offsets(const shrike_packed_layout *layout, int layer,
+                                        int experts_have_additive_biases, shrike_expert_offsets *out);
+/* crossValidate (GTurboPackedExpertsLayoutV1.swift:166-199) against a manifest's dimensions
+ * and its file sizes ("packed_experts/<file>" paths). */
+int shrike_packed_layout_cross_validate(const shrike_packed_layout *layout, int manifest_num_layers,
+                                        int manifest_experts_per_layer, uint64_t manifest_expert_stride,
+                                        const char *const *manifest_paths, const uint64_t *manifest_sizes,
+                                        size_t manifest_file_count);
+
 #ifdef __cplusplus
 }
 #endif

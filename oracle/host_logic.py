@@ -4,7 +4,8 @@ the shipped implementation is the C++ in shrike_amd/csrc/host_logic.cpp and
 slot_cache.cpp, which the tests compare against these functions.
 
 Every function follows one reference function (cited in its docstring) and is pinned
-in tests/test_host_logic_oracle.py by the vectors the reference's own unit tests hold.
+in tests/test_host_logic_oracle.py and tests/test_packed_layout.py by the vectors the
+reference's own unit tests hold.
 All arithmetic here is integer; results are compared for equality.
 """
 from __future__ import annotations
@@ -682,3 +683,181 @@ class SlotCache:
     def counts(self):
         return dict(resident=self.slot_state.count(RESIDENT), loading=self.slot_state.count(LOADING),
                     pinned=sum(1 for p in self.slot_pins if p > 0))
+
+
+# ------------------------------------------------------------- packed experts layout
+
+LAYOUT_ALIGNMENT = 16384  # GTurboFormatV1.alignmentBytes, sources/ShrikeFormat/GTurboFormatV1.swift:7
+
+
+class LayoutInvalid(Exception):
+    """ShrikeFormatError.invalid(field:reason:)."""
+
+    def __init__(self, field_: str, reason: str):
+        super().__init__(f"{field_}: {reason}")
+        self.field, self.reason = field_, reason
+
+
+def _basename_fault(name: str):
+    """GTurboPathValidator.validateBasename, sources/ShrikeFormat/GTurboFormatV1.swift:58-77."""
+    if name == "" or name.startswith("/") or "\0" in name:
+        return "unsafe relative path"
+    if any(c in ("", ".", "..") for c in name.split("/")):
+        return "non-canonical path"
+    if "/" in name:
+        return "expected basename"
+    return None
+
+
+def _is_int(v) -> bool:
+    return isinstance(v, int) and not isinstance(v, bool)
+
+
+def decode_packed_layout(data: bytes) -> dict:
+    """GTurboPackedExpertsLayoutCodec.decode + GTurboV1StructuralValidator.validate
+    (sources/ShrikeFormat/GTurboPackedExpertsLayoutV1.swift:65-164) and the runtime view of
+    PackedExpertsLayoutReader.decode (sources/Shrike/Infrastructure/ModelIO/PackedExpertsLayout.swift:104-128):
+    layers by id, experts by logical id. Raises LayoutInvalid with the reference's reason."""
+    import json
+    try:
+        root = json.loads(data)
+        stride, num_layers, per_layer = root["expertStride"], root["numLayers"], root["expertsPerLayer"]
+        layers_in = root["layers"]
+        if not (_is_int(stride) and stride >= 0 and _is_int(num_layers) and _is_int(per_layer)
+                and isinstance(layers_in, list)):
+            raise TypeError("mistyped top-level key")
+        layers = []
+        for lj in layers_in:
+            experts = []
+            for ej in lj["experts"]:
+                tensors = {}
+                for name, tj in ej["tensors"].items():
+                    t = {"offset": tj["offset"], "size": tj["size"], "dtype": tj["dtype"], "shape": list(tj["shape"]),
+                         "bits": tj.get("bits")}
+                    if not (_is_int(t["offset"]) and t["offset"] >= 0 and _is_int(t["size"]) and t["size"] >= 0
+                            and isinstance(t["dtype"], str) and all(_is_int(d) and 0 <= d <= U32_MAX for d in t["shape"])
+                            and (t["bits"] is None or _is_int(t["bits"]))):
+                        raise TypeError("mistyped tensor")
+                    tensors[name] = t
+                e = {"expert": ej.get("expert"), "physicalRank": ej.get("physicalRank"), "offset": ej["offset"],
+                     "size": ej["size"], "tensors": tensors}
+                if not (_is_int(e["offset"]) and e["offset"] >= 0 and _is_int(e["size"]) and e["size"] >= 0
+                        and all(v is None or _is_int(v) for v in (e["expert"], e["physicalRank"]))):
+                    raise TypeError("mistyped expert")
+                experts.append(e)
+            if not (_is_int(lj["layer"]) and isinstance(lj["file"], str)):
+                raise TypeError("mistyped layer")
+            layers.append({"layer": lj["layer"], "file": lj["file"], "experts": experts})
+    except (ValueError, KeyError, TypeError, AttributeError) as exc:
+        raise LayoutInvalid("packed_experts/layout.json", str(exc))
+
+    if not (num_layers > 0 and per_layer > 0 and stride > 0 and stride % LAYOUT_ALIGNMENT == 0
+            and len(layers) == num_layers):
+        raise LayoutInvalid("layout", "invalid dimensions or stride")
+    layer_ids, layer_files = set(), set()
+    for layer in layers:
+        lid = layer["layer"]
+        if not (0 <= lid < num_layers) or lid in layer_ids:
+            raise LayoutInvalid("layout.layers", "duplicate or invalid layer")
+        layer_ids.add(lid)
+        fault = _basename_fault(layer["file"])
+        if fault:
+            raise LayoutInvalid(f"layout.layers[{lid}].file", fault)
+        key = "".join(chr(ord(c) + 32) if "A" <= c <= "Z" else c for c in layer["file"])
+        if key == "layout.json":
+            raise LayoutInvalid(f"layout.layers[{lid}].file", "reserved packed-expert filename")
+        if key in layer_files:
+            raise LayoutInvalid(f"layout.layers[{lid}].file", "duplicate layer filename")
+        layer_files.add(key)
+        experts = layer["experts"]
+        if len(experts) not in (per_layer, 0):
+            raise LayoutInvalid(f"layout.layers[{lid}].experts", "wrong expert count")
+        explicit = [e["expert"] is not None for e in experts]
+        if any(explicit) and not all(explicit):
+            raise LayoutInvalid(f"layout.layers[{lid}].experts",
+                                "expert ids must be either all explicit or all positional")
+        logical_ids, ranks, offsets = set(), set(), set()
+        for position, e in enumerate(experts):
+            logical = e["expert"] if e["expert"] is not None else position
+            physical = e["physicalRank"] if e["physicalRank"] is not None else logical
+            if (not (0 <= logical < per_layer and 0 <= physical < per_layer) or logical in logical_ids
+                    or physical in ranks or e["offset"] in offsets):
+                raise LayoutInvalid(f"layout.layers[{lid}].experts", "duplicate or invalid expert mapping")
+            logical_ids.add(logical), ranks.add(physical), offsets.add(e["offset"])
+            if physical * stride >= 1 << 64:
+                raise LayoutInvalid("expert.offset", "overflow")
+            if not (e["offset"] == physical * stride and e["size"] == stride):
+                raise LayoutInvalid(f"expert[{logical}]", "offset or size does not match physical rank")
+            ranges = []
+            for name, t in e["tensors"].items():
+                if not (t["dtype"] in ("U32", "BF16") and name != "" and t["size"] > 0 and len(t["shape"]) > 0
+                        and all(d > 0 for d in t["shape"]) and (t["bits"] is None or 0 < t["bits"] <= 32)):
+                    raise LayoutInvalid(f"expert[{logical}].tensors.{name}", "invalid dtype or shape")
+                end = t["offset"] + t["size"]
+                if end >= 1 << 64:
+                    raise LayoutInvalid(f"tensor.{name}.range", "overflow")
+                if end > e["size"]:
+                    raise LayoutInvalid(f"expert[{logical}].tensors.{name}", "range exceeds expert blob")
+                ranges.append((t["offset"], end, name))
+            ranges.sort(key=lambda r: (r[0], r[1]))
+            for a, b in zip(ranges, ranges[1:]):
+                if a[1] > b[0]:
+                    raise LayoutInvalid(f"expert[{logical}].tensors", f"overlapping ranges {a[2]} and {b[2]}")
+            e["logical"], e["physical"] = logical, physical
+    view = []
+    for layer in sorted(layers, key=lambda l: l["layer"]):
+        view.append({"layer": layer["layer"], "file": layer["file"],
+                     "experts": sorted(layer["experts"], key=lambda e: e["logical"])})
+    return {"expertStride": stride, "numLayers": num_layers, "expertsPerLayer": per_layer, "layers": view}
+
+
+def cross_validate_layout(layout: dict, num_layers: int, per_layer: int, stride: int, file_sizes: dict) -> None:
+    """GTurboV1StructuralValidator.crossValidate, GTurboPackedExpertsLayoutV1.swift:177-199."""
+    if (num_layers, per_layer, stride) != (layout["numLayers"], layout["expertsPerLayer"], layout["expertStride"]):
+        raise LayoutInvalid("manifest/layout", "dimension mismatch")
+    layer_size = layout["expertsPerLayer"] * layout["expertStride"]
+    for layer in layout["layers"]:
+        if layer["experts"] and file_sizes.get("packed_experts/" + layer["file"]) != layer_size:
+            raise LayoutInvalid("manifest.files.packed_experts/" + layer["file"], "missing or wrong layer size")
+
+
+OFFSET_ROLES = ["gate", "gate_scales", "gate_biases", "up", "up_scales", "up_biases", "down", "down_scales",
+                "down_biases", "gate_bias", "up_bias", "down_bias"]
+
+
+def routed_expert_offsets(layout: dict, layer: int, additive_biases: bool = False) -> list:
+    """Model.routedExpertOffsets, sources/Shrike/Runtime/Inference/ModelExpertIO.swift:69-94: offsets of
+    expert 0's sub-tensors in the order of MoEExpertOffsets' fields, 0 for a role the blob lacks."""
+    tensors = layout["layers"][layer]["experts"][0]["tensors"]
+    if additive_biases:
+        for role in ("gate_bias", "up_bias", "down_bias"):
+            if role not in tensors:
+                raise LayoutInvalid(f"layer {layer}", f"expert blob is missing {role}")
+    return [tensors[r]["offset"] & U32_MAX if r in tensors else 0 for r in OFFSET_ROLES]
+
+
+# ------------------------------------------------------------- parallel reader rules
+
+def reader_claim_slot(slots) -> int:
+    """shrike_expert_reader_claim_slot, sources/ShrikeKernelsC/expert_io.c:46-58: the oldest active slot
+    with an unclaimed read. slots: (active, sequence, next_index, count)."""
+    best = -1
+    for i, (active, sequence, next_index, count) in enumerate(slots):
+        if active and next_index < count and (best < 0 or sequence < slots[best][1]):
+            best = i
+    return best
+
+
+def reader_free_slot(slots) -> int:
+    """shrike_expert_reader_free_slot, expert_io.c:60-68."""
+    for i, s in enumerate(slots):
+        if not s[0]:
+            return i
+    return -1
+
+
+def reader_cancel_slot(count, next_index, outstanding, first_errno, ecanceled):
+    """shrike_expert_reader_cancel_slot, expert_io.c:70-80."""
+    if next_index >= count:
+        return count, next_index, outstanding, first_errno
+    return count, count, outstanding - (count - next_index), first_errno or ecanceled

@@ -122,14 +122,57 @@ class StreamingStatistics(C.Structure):
             "resident_slots", "loading_slots", "pinned_slots", "peak_loading_slots")]
 
 
+class ExpertBatchSlot(C.Structure):
+    _fields_ = [("active", C.c_int), ("sequence", C.c_uint64), ("next_index", C.c_size_t), ("count", C.c_size_t)]
+
+
+class ExpertBatchCancelState(C.Structure):
+    _fields_ = [("count", C.c_size_t), ("next_index", C.c_size_t), ("outstanding", C.c_size_t),
+                ("first_errno", C.c_int)]
+
+
+class PackedExpert(C.Structure):
+    _fields_ = [("expert", C.c_int32), ("physical_rank", C.c_int32), ("offset", C.c_uint64), ("size", C.c_uint64),
+                ("tensor_count", C.c_uint32)]
+
+
+class PackedTensor(C.Structure):
+    _fields_ = [("offset", C.c_uint64), ("size", C.c_uint64), ("dtype", C.c_char * 8), ("shape", C.c_uint32 * 4),
+                ("rank", C.c_uint32), ("bits", C.c_int32)]
+
+
 SIGNATURES = {
     "shrike_hip_last_error": (C.c_char_p, []),
+    "shrike_host_last_error": (C.c_char_p, []),
+    "shrike_expert_reader_create": (_VP, [C.c_char_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int)]),
+    "shrike_expert_reader_destroy": (None, [_VP]),
+    "shrike_expert_reader_fetch": (C.c_int, [_VP, C.POINTER(C.c_uint32), C.POINTER(C.c_void_p), C.c_size_t]),
+    "shrike_expert_reader_fetch_offsets": (C.c_int, [_VP, C.POINTER(C.c_uint64), C.POINTER(C.c_void_p), C.c_size_t]),
+    "shrike_expert_reader_threads": (C.c_int, [_VP]),
+    "shrike_expert_reader_batch_depth": (C.c_int, [_VP]),
+    "shrike_expert_reader_claim_slot": (C.c_int, [C.POINTER(ExpertBatchSlot), C.c_int]),
+    "shrike_expert_reader_free_slot": (C.c_int, [C.POINTER(ExpertBatchSlot), C.c_int]),
+    "shrike_expert_reader_cancel_slot": (None, [C.POINTER(ExpertBatchCancelState)]),
+    "shrike_packed_layout_decode": (_VP, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int)]),
+    "shrike_packed_layout_load": (_VP, [C.c_char_p, C.c_uint64, C.POINTER(C.c_int)]),
+    "shrike_packed_layout_destroy": (None, [_VP]),
+    "shrike_packed_layout_expert_stride": (C.c_uint64, [_VP]),
+    "shrike_packed_layout_num_layers": (C.c_int, [_VP]),
+    "shrike_packed_layout_experts_per_layer": (C.c_int, [_VP]),
+    "shrike_packed_layout_layer": (C.c_int, [_VP, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_char_p), C.POINTER(C.c_int)]),
+    "shrike_packed_layout_expert": (C.c_int, [_VP, C.c_int, C.c_int, C.POINTER(PackedExpert)]),
+    "shrike_packed_layout_tensor": (C.c_int, [_VP, C.c_int, C.c_int, C.c_char_p, C.POINTER(PackedTensor)]),
+    "shrike_packed_layout_expert_offsets": (C.c_int, [_VP, C.c_int, C.c_int, C.POINTER(ExpertOffsets)]),
+    "shrike_packed_layout_cross_validate": (C.c_int, [_VP, C.c_int, C.c_int, C.c_uint64, C.POINTER(C.c_char_p),
+                                                      C.POINTER(C.c_uint64), C.c_size_t]),
     "shrike_hip_init": (C.c_int, [C.c_int]),
     "shrike_expert_offsets_make": (_U64, [_U32, _U32, _U32, C.c_int, C.POINTER(ExpertOffsets)]),
     "shrike_parse_budget_bytes": (_I64, [C.c_char_p]),
     "shrike_expert_cache_slots": (_I32, [_U64, _I32, _I64]),
     "shrike_hip_pool_create": (_VP, [_U32, _U64, _U32, _U64, C.POINTER(C.c_int)]),
     "shrike_hip_pool_destroy": (None, [_VP]),
+    "shrike_hip_pool_fetch_experts": (C.c_int, [_VP, _VP, _VP, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), _U32, _U64,
+                                                _VP, _U64]),
     "shrike_hip_pool_slot_stride": (_U64, [_VP]),
     "shrike_hip_pool_cell_count": (_U32, [_VP]),
     "shrike_hip_pool_cell_ptr": (_VP, [_VP, _U32]),

@@ -3,6 +3,7 @@
 
 #include "../../include/shrike_host.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -57,6 +58,7 @@ struct shrike_hip_pool {
 extern "C" {
 
 const char *shrike_hip_last_error(void) { return g_last_error.c_str(); }
+const char *shrike_host_last_error(void) { return g_last_error.c_str(); }
 
 int shrike_hip_init(int device) {
     int count = 0;
@@ -234,6 +236,52 @@ int shrike_hip_pool_upload_async(shrike_hip_pool *pool, uint32_t cell, const voi
     SHRIKE_HIP(hipMemcpyAsync(shrike_hip_pool_cell_ptr(pool, cell), host_src, bytes, hipMemcpyHostToDevice,
                               as_stream(stream)));
     return 0;
+}
+
+int shrike_hip_pool_fetch_experts(shrike_hip_pool *pool, void *stream, shrike_expert_reader *reader,
+                                  const uint64_t *file_offsets, const uint32_t *cells, uint32_t count, uint64_t blob_bytes,
+                                  void *pinned_staging, uint64_t staging_bytes) {
+    SHRIKE_REQUIRE(pool && reader, "pool or reader is NULL");
+    if (count == 0) return 0;
+    SHRIKE_REQUIRE(file_offsets && cells && pinned_staging, "offsets, cells or staging is NULL");
+    SHRIKE_REQUIRE(blob_bytes > 0 && blob_bytes <= pool->stride, "%llu bytes do not fit a cell of %llu",
+                   (unsigned long long)blob_bytes, (unsigned long long)pool->stride);
+    SHRIKE_REQUIRE(staging_bytes / blob_bytes >= 2, "the staging buffer must hold two blobs of %llu bytes",
+                   (unsigned long long)blob_bytes);
+    for (uint32_t i = 0; i < count; ++i)
+        SHRIKE_REQUIRE(cells[i] < pool->cells, "expert cell %u out of range (%u cells)", cells[i], pool->cells);
+    const uint32_t per_half = uint32_t(std::min<uint64_t>(staging_bytes / blob_bytes / 2, count));
+    hipEvent_t copied[2] = {nullptr, nullptr};
+    bool pending[2] = {false, false};
+    int rc = 0;
+    for (int h = 0; h < 2 && rc == 0; ++h)
+        if (hipEventCreateWithFlags(&copied[h], hipEventDisableTiming) != hipSuccess) rc = hip_failed(hipGetLastError(), "hipEventCreate");
+    std::vector<void *> destinations(per_half);
+    uint32_t done = 0;
+    for (int h = 0; done < count && rc == 0; h ^= 1) {
+        const uint32_t n = std::min(per_half, count - done);
+        uint8_t *half = static_cast<uint8_t *>(pinned_staging) + uint64_t(h) * per_half * blob_bytes;
+        if (pending[h]) {  // the copies that last read this half
+            if (hipEventSynchronize(copied[h]) != hipSuccess) { rc = hip_failed(hipGetLastError(), "hipEventSynchronize"); break; }
+            pending[h] = false;
+        }
+        for (uint32_t i = 0; i < n; ++i) destinations[i] = half + uint64_t(i) * blob_bytes;
+        rc = shrike_expert_reader_fetch_offsets(reader, file_offsets + done, destinations.data(), n);
+        if (rc != 0) {
+            set_error("expert read failed: %s", strerror(rc));
+            break;
+        }
+        for (uint32_t i = 0; i < n && rc == 0; ++i)
+            rc = shrike_hip_pool_upload_async(pool, cells[done + i], destinations[i], blob_bytes, stream);
+        if (rc == 0 && hipEventRecord(copied[h], as_stream(stream)) != hipSuccess) rc = hip_failed(hipGetLastError(), "hipEventRecord");
+        pending[h] = rc == 0;
+        done += n;
+    }
+    // the staging buffer is the caller's again on return, also after a failure
+    if (hipStreamSynchronize(as_stream(stream)) != hipSuccess && rc == 0) rc = hip_failed(hipGetLastError(), "hipStreamSynchronize");
+    for (int h = 0; h < 2; ++h)
+        if (copied[h]) (void)hipEventDestroy(copied[h]);
+    return rc;
 }
 
 int shrike_hip_pool_table_publish(shrike_hip_pool *pool, uint32_t expert, uint32_t cell, uint32_t state,

@@ -4,6 +4,7 @@ into libshrikehip.so — nothing here computes a result in Python."""
 from __future__ import annotations
 
 import ctypes as C
+import os
 import errno
 
 import numpy as np
@@ -265,3 +266,158 @@ class SlotCache:
         e, w = np.zeros(max(1, self.experts_per_layer), np.uint32), np.zeros(max(1, self.experts_per_layer), np.uint64)
         n = capi.load().shrike_slot_cache_drain_publications(self._h, _vp(e), _vp(w), e.size)
         return list(zip(e[:n].tolist(), w[:n].tolist()))
+
+
+# --------------------------------------------------------------- parallel expert reader
+
+class ReadFailed(ShrikeError):
+    """ParallelExpertReader.Failure (sources/Shrike/Infrastructure/Streaming/ParallelExpertReader.swift)."""
+
+    def __init__(self, errno_: int, what: str):
+        super().__init__(f"{what}: {os.strerror(errno_)} (errno {errno_})")
+        self.errno = errno_
+
+
+class ParallelExpertReader:
+    """shrike_expert_reader with the reference wrapper's names: `threads` workers with a descriptor each,
+    up to `batch_depth` batches published at once, pread only."""
+
+    def __init__(self, path: str, expert_stride: int, threads: int = 4, batch_depth: int = 1,
+                 bypass_cache: bool = False):
+        err = C.c_int(0)
+        self.handle = capi.load().shrike_expert_reader_create(os.fsencode(path), expert_stride, threads, batch_depth,
+                                                              int(bypass_cache), C.byref(err))
+        if not self.handle:
+            raise ReadFailed(err.value, f"cannot open {path}")
+        self.expert_stride = expert_stride
+
+    def close(self):
+        if self.handle:
+            capi.load().shrike_expert_reader_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def thread_count(self) -> int:
+        return capi.load().shrike_expert_reader_threads(self.handle)
+
+    @property
+    def batch_depth(self) -> int:
+        return capi.load().shrike_expert_reader_batch_depth(self.handle)
+
+    @staticmethod
+    def _destinations(into):
+        return (C.c_void_p * len(into))(*[int(p) for p in into])
+
+    def fetch(self, experts, into) -> None:
+        """experts[i] * stride -> the address into[i] (each expert_stride bytes long)."""
+        if len(experts) != len(into):
+            raise ValueError("one destination per expert")
+        ids = (C.c_uint32 * len(experts))(*experts)
+        rc = capi.load().shrike_expert_reader_fetch(self.handle, ids, self._destinations(into), len(experts))
+        if rc:
+            raise ReadFailed(rc, "expert read failed")
+
+    def fetch_offsets(self, offsets, into) -> None:
+        if len(offsets) != len(into):
+            raise ValueError("one destination per offset")
+        offs = (C.c_uint64 * len(offsets))(*offsets)
+        rc = capi.load().shrike_expert_reader_fetch_offsets(self.handle, offs, self._destinations(into), len(offsets))
+        if rc:
+            raise ReadFailed(rc, "expert read failed")
+
+
+# --------------------------------------------------------------- packed experts layout
+
+class LayoutError(ShrikeError):
+    """ModelError.indexCorrupt / .missingFile of the layout reader, with the library's errno."""
+
+    def __init__(self, errno_: int, message: str):
+        super().__init__(message)
+        self.errno = errno_
+
+
+class PackedExpertsLayout:
+    """packed_experts/layout.json (sources/Shrike/Infrastructure/ModelIO/PackedExpertsLayout.swift:34-129)."""
+
+    def __init__(self, handle):
+        self.handle = handle
+
+    @staticmethod
+    def _made(handle, err):
+        if not handle:
+            raise LayoutError(err.value, capi.load().shrike_host_last_error().decode())
+        return PackedExpertsLayout(handle)
+
+    @classmethod
+    def decode(cls, data: bytes) -> "PackedExpertsLayout":
+        err = C.c_int(0)
+        return cls._made(capi.load().shrike_packed_layout_decode(data, len(data), C.byref(err)), err)
+
+    @classmethod
+    def load(cls, model_dir: str, max_bytes: int = 0) -> "PackedExpertsLayout":
+        err = C.c_int(0)
+        return cls._made(capi.load().shrike_packed_layout_load(os.fsencode(model_dir), max_bytes, C.byref(err)), err)
+
+    def close(self):
+        if self.handle:
+            capi.load().shrike_packed_layout_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def expert_stride(self) -> int:
+        return capi.load().shrike_packed_layout_expert_stride(self.handle)
+
+    @property
+    def num_layers(self) -> int:
+        return capi.load().shrike_packed_layout_num_layers(self.handle)
+
+    @property
+    def experts_per_layer(self) -> int:
+        return capi.load().shrike_packed_layout_experts_per_layer(self.handle)
+
+    def _check(self, rc):
+        if rc:
+            raise LayoutError(rc, capi.load().shrike_host_last_error().decode())
+
+    def layer(self, index: int) -> dict:
+        lid, file, count = C.c_int(0), C.c_char_p(), C.c_int(0)
+        self._check(capi.load().shrike_packed_layout_layer(self.handle, index, C.byref(lid), C.byref(file), C.byref(count)))
+        return {"layer": lid.value, "file": file.value.decode(), "expert_count": count.value}
+
+    def expert(self, layer: int, expert: int) -> dict:
+        out = capi.PackedExpert()
+        self._check(capi.load().shrike_packed_layout_expert(self.handle, layer, expert, C.byref(out)))
+        return {"expert": out.expert, "physical_rank": out.physical_rank, "offset": out.offset, "size": out.size,
+                "tensor_count": out.tensor_count}
+
+    def tensor(self, layer: int, expert: int, role: str):
+        out = capi.PackedTensor()
+        rc = capi.load().shrike_packed_layout_tensor(self.handle, layer, expert, role.encode(), C.byref(out))
+        if rc == 2:  # ENOENT: the blob has no such sub-tensor
+            return None
+        self._check(rc)
+        return {"offset": out.offset, "size": out.size, "dtype": out.dtype.decode(),
+                "shape": [out.shape[i] for i in range(min(out.rank, 4))], "bits": out.bits or None}
+
+    def expert_offsets(self, layer: int, additive_biases: bool = False) -> capi.ExpertOffsets:
+        out = capi.ExpertOffsets()
+        self._check(capi.load().shrike_packed_layout_expert_offsets(self.handle, layer, int(additive_biases), C.byref(out)))
+        return out
+
+    def cross_validate(self, num_layers: int, experts_per_layer: int, expert_stride: int, file_sizes: dict) -> None:
+        paths = (C.c_char_p * len(file_sizes))(*[k.encode() for k in file_sizes])
+        sizes = (C.c_uint64 * len(file_sizes))(*file_sizes.values())
+        self._check(capi.load().shrike_packed_layout_cross_validate(self.handle, num_layers, experts_per_layer,
+                                                                    expert_stride, paths, sizes, len(file_sizes)))

@@ -206,6 +206,17 @@ class ExpertPool:
                                                        stream.handle if stream else None, elapsed_nanos),
               "shrike_hip_pool_execute_plan")
 
+    def fetch_experts(self, reader, file_offsets, cells, blob_bytes: int, staging: "PinnedBuffer",
+                      stream: Stream | None = None) -> None:
+        """Blobs at file_offsets of the reader's layer file -> cells, through the pinned staging buffer.
+        `reader` is a shrike_amd.host.ParallelExpertReader created with stride blob_bytes."""
+        n = len(file_offsets)
+        offs = (C.c_uint64 * n)(*[int(o) for o in file_offsets])
+        cs = (C.c_uint32 * n)(*[int(c) for c in cells])
+        check(capi.load().shrike_hip_pool_fetch_experts(self.handle, stream.handle if stream else None, reader.handle,
+                                                        offs, cs, n, blob_bytes, staging.ptr, staging.nbytes),
+              "shrike_hip_pool_fetch_experts")
+
     def close(self) -> None:
         if self.handle:
             capi.load().shrike_hip_pool_destroy(self.handle)

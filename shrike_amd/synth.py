@@ -197,3 +197,62 @@ def quantize_affine(rows_f32: np.ndarray, bits: int, meta: int = META_BF16):
     if bits == 4:
         q = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)
     return np.ascontiguousarray(q), sb, bb
+
+
+# ------------------------------------------------------------------- packed experts directory
+
+_ROLE_OF = {"gate_w": "gate", "gate_s": "gate_scales", "gate_b": "gate_biases", "up_w": "up", "up_s": "up_scales",
+            "up_b": "up_biases", "down_w": "down", "down_s": "down_scales", "down_b": "down_biases",
+            "gate_ab": "gate_bias", "up_ab": "up_bias", "down_ab": "down_bias"}
+
+
+def packed_layout_tensors(d: int, f: int, bits: int = 4, additive_biases: bool = False) -> dict:
+    """The `tensors` object of one expert in packed_experts/layout.json for a synthetic blob: role names as
+    the runtime looks them up (sources/Shrike/Runtime/Inference/ModelExpertIO.swift:69-94), codes as "U32"
+    words with their bit width, metadata as "BF16" (the file format has no other 16-bit type)."""
+    off, _ = expert_offsets(d, f, bits, additive_biases)
+    out = {}
+    for name, rows, n in (("gate", f, d), ("up", f, d), ("down", d, f)):
+        out[_ROLE_OF[f"{name}_w"]] = {"offset": off[f"{name}_w"], "size": rows * n * bits // 8, "dtype": "U32",
+                                      "shape": [rows, n * bits // 32], "bits": bits}
+        for part in ("s", "b"):
+            out[_ROLE_OF[f"{name}_{part}"]] = {"offset": off[f"{name}_{part}"], "size": rows * (n // GROUP) * 2,
+                                               "dtype": "BF16", "shape": [rows, n // GROUP]}
+    if additive_biases:
+        for name, n in (("gate_ab", f), ("up_ab", f), ("down_ab", d)):
+            out[_ROLE_OF[name]] = {"offset": off[name], "size": n * 2, "dtype": "BF16", "shape": [n]}
+    return out
+
+
+def write_packed_experts(model_dir: str, layers: list, d: int, f: int, bits: int = 4, additive_biases: bool = False,
+                         physical_rank=None, alignment: int = 16384) -> dict:
+    """Writes <model_dir>/packed_experts/layout.json and one layer_NN.bin per populated layer
+    (sources/ShrikeFormat/GTurboPackedExpertsLayoutV1.swift:3-62). layers[l] is the list of that layer's
+    expert blobs by logical id, or [] for a dense layer. physical_rank(l, e) places expert e in the file
+    (identity by default). The file stride is the blob size rounded up to `alignment`. Returns the
+    layout as a dict."""
+    import json
+    import os
+    _, blob_bytes = expert_offsets(d, f, bits, additive_biases)
+    stride = (blob_bytes + alignment - 1) // alignment * alignment
+    per_layer = max(len(blobs) for blobs in layers)
+    root = os.path.join(model_dir, "packed_experts")
+    os.makedirs(root, exist_ok=True)
+    tensors = packed_layout_tensors(d, f, bits, additive_biases)
+    out_layers = []
+    for l, blobs in enumerate(layers):
+        name = f"layer_{l:02d}.bin"
+        experts = []
+        if blobs:
+            image = np.zeros(per_layer * stride, np.uint8)
+            for e, blob in enumerate(blobs):
+                rank = physical_rank(l, e) if physical_rank else e
+                image[rank * stride:rank * stride + blob.size] = blob
+                experts.append({"expert": e, "physicalRank": rank, "offset": rank * stride, "size": stride,
+                                "tensors": tensors})
+            image.tofile(os.path.join(root, name))
+        out_layers.append({"layer": l, "file": name, "experts": experts})
+    layout = {"expertStride": stride, "numLayers": len(layers), "expertsPerLayer": per_layer, "layers": out_layers}
+    with open(os.path.join(root, "layout.json"), "w") as fh:
+        json.dump(layout, fh, sort_keys=True)
+    return layout

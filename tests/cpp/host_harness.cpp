@@ -1,10 +1,12 @@
 // The reference's host-side unit tests, written against include/shrike.hpp the way the
 // reference writes them against its Swift classes. No GPU call is made: budget ladder,
-// grouping, sweep order, wave planner and slot cache run on the host. Exit code 0 = all passed.
+// grouping, sweep order, wave planner, slot cache, the packed-experts layout and the parallel reader run on the host. Exit code 0 = all passed.
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <optional>
+#include <string>
+#include <unistd.h>
 
 #include "shrike.hpp"
 
@@ -129,7 +131,64 @@ static void slotCache() {
     }
 }
 
+// PackedExpertsLayoutTests.swift:10-90 (the toy layout) and ParallelExpertReaderTests.swift:36-58, :132-158
+static void layoutAndReader() {
+    const char *tensors = "{\"gate\": {\"offset\": 0, \"size\": 4096, \"dtype\": \"U32\", \"shape\": [64, 64], \"bits\": 4},"
+                          " \"gate_scales\": {\"offset\": 4096, \"size\": 256, \"dtype\": \"BF16\", \"shape\": [64, 1]}}";
+    const std::string json = std::string("{\"expertStride\": 16384, \"numLayers\": 1, \"expertsPerLayer\": 2, \"layers\": [{\"layer\": 0,"
+        " \"file\": \"layer_00.bin\", \"experts\": [{\"expert\": 0, \"offset\": 0, \"size\": 16384, \"tensors\": ") + tensors
+        + "}, {\"expert\": 1, \"physicalRank\": 1, \"offset\": 16384, \"size\": 16384, \"tensors\": " + tensors + "}]}]}";
+    auto layout = PackedExpertsLayout::decode(json);
+    EXPECT(layout.expertStride() == 16384 && layout.numLayers() == 1 && layout.expertsPerLayer() == 2);
+    EXPECT(layout.file(0) == "layer_00.bin");
+    EXPECT(layout.expert(0, 0).offset == 0 && layout.expert(0, 0).size == 16384);
+    EXPECT(layout.subTensor(0, 0, "gate")->offset == 0 && layout.subTensor(0, 0, "gate_scales")->offset == 4096);
+    EXPECT(layout.expert(0, 1).offset == 16384 && layout.expert(0, 1).expert == 1);
+    EXPECT(!layout.subTensor(0, 0, "down"));
+    EXPECT(layout.routedExpertOffsets(0).gate_s_off == 4096 && layout.routedExpertOffsets(0).down_w_off == 0);
+    bool threw = false;
+    try { layout.expert(0, 2); } catch (const Error &e) { threw = std::string(e.what()).find("layer 0 has 2 experts; expert 2 is out of range") != std::string::npos; }
+    EXPECT(threw);
+    threw = false;
+    try { PackedExpertsLayout::decode("{\"expertStride\": 100, \"numLayers\": 1, \"expertsPerLayer\": 1, \"layers\": []}"); }
+    catch (const Error &e) { threw = e.code == EINVAL && std::string(e.what()).find("invalid dimensions or stride") != std::string::npos; }
+    EXPECT(threw);
+
+    // a file of 64 blocks, block e filled with e % 251; out-of-order ids with a repeat
+    const size_t stride = 4096;
+    char path[] = "/tmp/shrike_reader_XXXXXX";
+    const int fd = mkstemp(path);
+    EXPECT(fd >= 0);
+    std::vector<unsigned char> block(stride);
+    for (int e = 0; e < 64; ++e) {
+        std::fill(block.begin(), block.end(), static_cast<unsigned char>(e % 251));
+        EXPECT(write(fd, block.data(), stride) == ssize_t(stride));
+    }
+    close(fd);
+    {
+        ParallelExpertReader reader(path, stride, 4, 2);
+        EXPECT(reader.threadCount() == 4 && reader.batchDepth() == 2);
+        const std::vector<uint32_t> wanted = {63, 0, 17, 17, 40, 5, 62, 1};
+        std::vector<std::vector<unsigned char>> buffers(wanted.size(), std::vector<unsigned char>(stride));
+        std::vector<void *> into;
+        for (auto &b : buffers) into.push_back(b.data());
+        reader.fetch(wanted, into);
+        for (size_t i = 0; i < wanted.size(); ++i) EXPECT(buffers[i][0] == wanted[i] % 251 && buffers[i][stride - 1] == wanted[i] % 251);
+        reader.fetch(std::vector<uint32_t>{}, {});
+        threw = false;
+        try { reader.fetch(std::vector<uint32_t>{99}, {buffers[0].data()}); } catch (const ParallelExpertReader::Failure &e) { threw = e.code == EIO; }
+        EXPECT(threw);
+        EXPECT(ParallelExpertReader(path, stride, 0, 0).threadCount() == 1);
+        EXPECT(ParallelExpertReader(path, stride, 999, 9).threadCount() == 16);
+    }
+    unlink(path);
+    threw = false;
+    try { ParallelExpertReader missing("/nonexistent/shrike/experts.bin", 4096); } catch (const ParallelExpertReader::Failure &e) { threw = e.code == ENOENT; }
+    EXPECT(threw);
+}
+
 int main() {
+    layoutAndReader();
     budget();
     grouping();
     sweepOrder();
