@@ -375,6 +375,15 @@ int shrike_hip_prefill_reduce(void *stream, const void *d_route_partials, const 
                               void *d_h2, uint32_t query_count, uint32_t top_k, uint32_t d);
 /* residual_add_fp16 (RealForwardRunner.swift:4658-4665): hidden[i] = fp16(hidden[i] + delta[i]). */
 int shrike_hip_residual_add_f16(void *stream, void *d_hidden, const void *d_delta, uint64_t count);
+/* The producer of the path's input, RMSNorm.encodeResidualAddBF16W / encodeBF16W
+ * (residual_add_rmsnorm_bf16w and rmsnorm_bf16w, sources/Shrike/Metal/Primitives/rmsnorm.metal:70-130;
+ * called at RealForwardRunner.swift:2852-2858): per row, hidden = fp16(hidden + delta) in place
+ * (d_delta NULL: no add), then out = fp16(hidden * rsqrt(mean(hidden^2) + eps) * bf16 weight), the
+ * mean in fp32. The decode call is one row; `rows` rows of d elements are done a workgroup each.
+ * Bitwise equal to shrike_hip_residual_add_f16 followed by the norm alone, as in the reference. */
+int shrike_hip_residual_add_rmsnorm_bf16w(void *stream, void *d_hidden, const void *d_delta,
+                                          const void *d_weight, void *d_out, uint32_t d, float eps,
+                                          uint32_t rows);
 
 /* ----------------------------------------------------------------- plumbing
  * Device memory, streams, events and graphs for hosts without a HIP binding of

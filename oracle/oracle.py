@@ -228,6 +228,14 @@ def residual_add_f16(hidden, delta):
     return hidden
 
 
+def residual_add_rmsnorm_bf16w(hidden, delta, weight_bf16, eps):
+    """In place on `hidden` (fp16 bits); returns the normalised row (fp16 bits). delta None: rmsnorm only."""
+    out = np.empty_like(hidden)
+    lib().orc_residual_add_rmsnorm_bf16w(_p(hidden), _p(delta) if delta is not None else None, _p(weight_bf16), _p(out),
+                                         C.c_uint32(hidden.shape[0]), C.c_float(eps))
+    return out
+
+
 def cpu_layer_fp32(blobs, route_weights, off, x_f32, d, f, threads, bits=4, meta=META_BF16):
     out = np.zeros(d, np.float32)
     rw = np.ascontiguousarray(route_weights, np.float32)

@@ -483,6 +483,40 @@ void orc_residual_add_f16(uint16_t *hidden, const uint16_t *delta, size_t n) {
         hidden[i] = orc_f32_to_f16(orc_f16_to_f32(hidden[i]) + orc_f16_to_f32(delta[i]));
 }
 
+/* residual_add_rmsnorm_bf16w / rmsnorm_bf16w, sources/Shrike/Metal/Primitives/rmsnorm.metal:33-130:
+ * hidden[i] = half(hidden[i] + delta[i]) in place (delta == NULL: no add), then
+ * out[i] = half(hidden[i] * inv * weight[i]) with inv = 1/sqrt(mean(hidden^2) + eps) (mean and
+ * reciprocal square root taken in fp64 from the fp32 sum, rounded to fp32 once), the sum of squares in fp32. The order of that sum is this build's own (the reference leaves it to
+ * simd_sum): 256 threads, thread t takes the 8-element chunks t, t+256, ... with one fma chain,
+ * each 64-lane wave folds with the xor butterfly 32...1, the four wave sums are added in order. */
+void orc_residual_add_rmsnorm_bf16w(uint16_t *hidden, const uint16_t *delta, const uint16_t *weight_bf16,
+                                    uint16_t *out, uint32_t d, float eps) {
+    float acc[256];
+    if (delta) orc_residual_add_f16(hidden, delta, d);
+    for (uint32_t t = 0; t < 256; ++t) {
+        float a = 0.0f;
+        for (uint32_t c = t; c * 8u < d; c += 256u)
+            for (uint32_t j = 0; j < 8u && c * 8u + j < d; ++j) {
+                const float v = orc_f16_to_f32(hidden[c * 8u + j]);
+                a = fmaf(v, v, a);
+            }
+        acc[t] = a;
+    }
+    float total = 0.0f;
+    for (uint32_t w = 0; w < 4; ++w) {
+        float lane[64], next[64];
+        memcpy(lane, acc + 64u * w, sizeof lane);
+        for (uint32_t o = 32; o >= 1; o >>= 1) {
+            for (uint32_t l = 0; l < 64; ++l) next[l] = lane[l] + lane[l ^ o];
+            memcpy(lane, next, sizeof lane);
+        }
+        total = w == 0 ? lane[0] : total + lane[0];
+    }
+    const float inv = (float)(1.0 / sqrt((double)total / (double)d + (double)eps));
+    for (uint32_t i = 0; i < d; ++i)
+        out[i] = orc_f32_to_f16(orc_f16_to_f32(hidden[i]) * inv * orc_bf16_to_f32(weight_bf16[i]));
+}
+
 /* -------------------------------------------------------- CPU layer (timing) */
 
 typedef struct {

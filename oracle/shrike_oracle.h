@@ -141,6 +141,8 @@ void orc_prefill_reduce(const uint16_t *partials_f16, const uint16_t *weights_f1
                         uint32_t t, uint32_t top_k, uint32_t d, uint16_t *h2_f16);
 /* residual_add_fp16: sources/Shrike/Metal/Primitives/utility.metal:94-103 */
 void orc_residual_add_f16(uint16_t *hidden, const uint16_t *delta, size_t n);
+void orc_residual_add_rmsnorm_bf16w(uint16_t *hidden, const uint16_t *delta, const uint16_t *weight_bf16,
+                                    uint16_t *out, uint32_t d, float eps);
 
 /* ---- whole-layer timing helper for the CPU baseline (one task per expert,
  * sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:10-14 describes 6 threads). */

@@ -410,6 +410,15 @@ class Prefill:
               "shrike_hip_residual_add_f16")
 
 
+def residual_add_rmsnorm_bf16w(hidden, delta, weight, out, d: int, eps: float, rows: int = 1,
+                               stream: Stream | None = None) -> None:
+    """RMSNorm.encodeResidualAddBF16W (delta None: encodeBF16W): hidden += delta in place, out = the
+    normalised row the router, the shared expert and phase 1 read."""
+    check(capi.load().shrike_hip_residual_add_rmsnorm_bf16w(stream.handle if stream else None, ptr(hidden), ptr(delta),
+                                                            ptr(weight), ptr(out), d, eps, rows),
+          "shrike_hip_residual_add_rmsnorm_bf16w")
+
+
 class BatchedDecodeLayer:
     """One MoE layer for a batch of tokens whose experts stream through a slot pool smaller than
     the expert set: the runner's loop around the operators (RealForwardRunner.swift:4552-4686 with

@@ -323,3 +323,32 @@ def test_int4_gemv_against_committed_reference_vectors():
         y = O.int4_affine_gemv(w, s, b, x, rows, n, S.META_BF16).view(np.uint32)
         assert [int(v) for v in y[:16]] == case["head"], (rows, n)
         assert zlib.crc32(y.tobytes()) == case["crc32"], (rows, n)
+
+
+# ---------------------------------------------------------------- rmsnorm ahead of the router
+
+def test_residual_add_rmsnorm_against_the_definition():
+    """rmsnorm.metal:5-13, :96-130: hidden += delta in fp16; out = hidden * rsqrt(mean(hidden^2) + eps) * weight.
+    Pinned by the closed form on a constant row, by fp64 on random rows, and by the reference's statement
+    that the fused kernel equals residual_add_fp16 followed by the norm alone."""
+    eps = 1e-6
+    ones = S.f32_to_f16_bits(np.full(2048, 2.0, np.float32))
+    w = S.f32_to_bf16_bits(np.full(2048, 0.5, np.float32))
+    out = O.residual_add_rmsnorm_bf16w(ones.copy(), None, w, eps)
+    assert np.all(S.f16_bits_to_f32(out) == np.float32(np.float16(2.0 / np.sqrt(4.0 + eps) * 0.5)))
+    tree = S.SeedTree(0x5EED0051)
+    for d in (64, 2048, 2304, 2880, 4096):
+        hidden = S.activations_f16(tree, f"h.{d}", d)
+        delta = S.f32_to_f16_bits(tree.key(f"d.{d}").normal(d, std=0.5))
+        weight = S.f32_to_bf16_bits(tree.key(f"w.{d}").uniform(0.5, 1.5, d))
+        h = hidden.copy()
+        out = O.residual_add_rmsnorm_bf16w(h, delta, weight, eps)
+        summed = (S.f16_bits_to_f32(hidden) + S.f16_bits_to_f32(delta)).astype(np.float16)
+        assert np.array_equal(h, summed.view(np.uint16)), "the add rounds through fp16 storage"
+        x = summed.astype(np.float64)
+        want = x / np.sqrt(np.mean(x * x) + eps) * S.bf16_bits_to_f32(weight).astype(np.float64)
+        got = S.f16_bits_to_f32(out).astype(np.float64)
+        assert np.max(np.abs(got - want) / (np.abs(want) + 1e-3)) <= 1e-3  # one fp16 rounding of the result
+        two_step = O.residual_add_f16(hidden.copy(), delta)
+        assert np.array_equal(O.residual_add_rmsnorm_bf16w(two_step, None, weight, eps), out)
+        assert np.array_equal(two_step, h)

@@ -371,3 +371,26 @@ def test_batched_decode_through_a_pool_smaller_than_the_expert_set(gpu, bits, sl
     assert cache.statistics().hits > before
     again = layer.partials.download(np.uint16, t * k * d)
     assert np.array_equal(again, partials.reshape(-1))  # same bytes whatever cell an expert landed in
+
+
+@pytest.mark.parametrize("d,rows", [(2048, 1), (2304, 1), (2880, 3), (64, 5), (4096, 2), (2048, 512)])
+def test_residual_add_rmsnorm_bit_exact(gpu, d, rows):
+    """The producer of the path's input (rmsnorm.metal:96-130) against the oracle: the updated hidden rows
+    and the normalised rows bit for bit, with and without the residual add."""
+    tree = S.SeedTree(0x5EED0052)
+    eps = 1e-6
+    hidden = S.activations_f16(tree, "hidden", rows * d)
+    delta = S.f32_to_f16_bits(tree.key("delta").normal(rows * d, std=0.5))
+    weight = S.f32_to_bf16_bits(tree.key("weight").uniform(0.5, 1.5, d))
+    for with_delta in (True, False):
+        d_hidden, d_delta, d_weight, d_out = gpu.dev(hidden), gpu.dev(delta), gpu.dev(weight), gpu.empty(2 * rows * d)
+        gpu.residual_add_rmsnorm_bf16w(d_hidden, d_delta if with_delta else None, d_weight, d_out, d, eps, rows)
+        got_hidden, got_out = d_hidden.download(np.uint16, rows * d), d_out.download(np.uint16, rows * d)
+        for r in range(rows if rows <= 8 else 4):
+            h = hidden[r * d:(r + 1) * d].copy()
+            want = O.residual_add_rmsnorm_bf16w(h, delta[r * d:(r + 1) * d] if with_delta else None, weight, eps)
+            assert np.array_equal(got_hidden[r * d:(r + 1) * d], h)
+            assert np.array_equal(got_out[r * d:(r + 1) * d], want), f"row {r} of d={d}"
+    for bad_d in (20, 8192):  # not a multiple of 8; past the kernels' hidden-size ceiling
+        with pytest.raises(capi.ShrikeError, match="multiple of 8"):
+            gpu.residual_add_rmsnorm_bf16w(d_hidden, None, d_weight, d_out, bad_d, eps)
