@@ -51,8 +51,8 @@ __global__ __launch_bounds__(256) void k_residual_add_rmsnorm(uint16_t *hidden, 
     if ((threadIdx.x & 63u) == 0) s_partial[threadIdx.x >> 6] = acc;
     __syncthreads();
     const float total = __fadd_rn(__fadd_rn(__fadd_rn(s_partial[0], s_partial[1]), s_partial[2]), s_partial[3]);
-    // the mean and the reciprocal square root in fp64 (the fp32 division of this target is not the
-    // correctly rounded one), rounded to fp32 once
+    // the mean and the reciprocal square root in fp64, rounded to fp32 once: no dependence on how an
+    // fp32 division or square root is expanded
     const float inv = float(1.0 / sqrt(double(total) / double(d) + double(eps)));
 #pragma unroll
     for (int r = 0; r < kMine; ++r) {
