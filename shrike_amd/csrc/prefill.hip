@@ -57,23 +57,30 @@ __global__ __launch_bounds__(256) void k_prefill_scale_x(const uint16_t *hidden,
     dst[1] = make_float4(o[4], o[5], o[6], o[7]);
 }
 
+// A wave keeps ROWS fp16 router rows as fp32 in registers (MAXI 16-byte chunks a lane and row)
+// and walks a block of tokens two at a time: every x value fetched from L2 feeds ROWS rows, and
+// every logit is summed in the decode router's order (lane l: chunks l, l+64, ..., xor butterfly).
+template <int MAXI, int ROWS>
 __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits,
                                                             uint32_t query_count, uint32_t num_experts, uint32_t d) {
-    constexpr int MAXI = SHRIKE_MAX_HIDDEN / 8 / 64;  // 16-byte weight chunks a lane can own
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t e = blockIdx.x * 4u + wave;
-    if (e >= num_experts) return;
+    const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
+    const uint32_t e0 = (blockIdx.x * 4u + wave) * ROWS;
+    if (e0 >= num_experts) return;
     const uint32_t chunks = d / 8u;
-    float w[MAXI][8];
+    float w[ROWS][MAXI][8];
 #pragma unroll
-    for (int i = 0; i < MAXI; ++i) {
-        const uint32_t c = lane + 64u * i;
-        const uint4 v = *reinterpret_cast<const uint4 *>(weights + size_t(e) * d + size_t(c < chunks ? c : 0u) * 8u);
-        const uint32_t ww[4] = {v.x, v.y, v.z, v.w};
+    for (int r = 0; r < ROWS; ++r) {
+        const uint32_t e = min(e0 + uint32_t(r), num_experts - 1u);  // past the last row: a copy, never stored
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            w[i][2 * j] = f16_to_f32(uint16_t(ww[j]));
-            w[i][2 * j + 1] = f16_to_f32(uint16_t(ww[j] >> 16));
+        for (int i = 0; i < MAXI; ++i) {
+            const uint32_t c = lane + 64u * i;
+            const uint4 v = *reinterpret_cast<const uint4 *>(weights + size_t(e) * d + size_t(c < chunks ? c : 0u) * 8u);
+            const uint32_t ww[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                w[r][i][2 * j] = f16_to_f32(uint16_t(ww[j]));
+                w[r][i][2 * j + 1] = f16_to_f32(uint16_t(ww[j] >> 16));
+            }
         }
     }
     const uint32_t t0 = blockIdx.y * kFastTokenBlock;
@@ -81,7 +88,9 @@ __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weig
     for (uint32_t t = t0; t < t1; t += 2u) {
         const bool two = t + 1u < t1;
         const float *row[2] = {xs + size_t(t) * d, xs + size_t(two ? t + 1u : t) * d};
-        float acc[2] = {0.0f, 0.0f};
+        float acc[2][ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) acc[0][r] = acc[1][r] = 0.0f;
 #pragma unroll
         for (int i = 0; i < MAXI; ++i) {
             const uint32_t c = lane + 64u * i;
@@ -96,20 +105,37 @@ __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weig
                 for (int u = 0; u < 2; ++u) {
                     const float xv[8] = {x[u][0].x, x[u][0].y, x[u][0].z, x[u][0].w, x[u][1].x, x[u][1].y, x[u][1].z, x[u][1].w};
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) acc[u] = fmaf(w[i][j], xv[j], acc[u]);
+                    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) acc[u][r] = fmaf(w[r][i][j], xv[j], acc[u][r]);
                 }
             }
         }
 #pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) {
-            acc[0] = __fadd_rn(acc[0], __shfl_xor(acc[0], o));
-            acc[1] = __fadd_rn(acc[1], __shfl_xor(acc[1], o));
-        }
+        for (int o = 32; o >= 1; o >>= 1)
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                acc[0][r] = __fadd_rn(acc[0][r], __shfl_xor(acc[0][r], o));
+                acc[1][r] = __fadd_rn(acc[1][r], __shfl_xor(acc[1][r], o));
+            }
         if (lane == 0) {
-            logits[size_t(t) * num_experts + e] = acc[0];
-            if (two) logits[size_t(t + 1u) * num_experts + e] = acc[1];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                if (e0 + uint32_t(r) >= num_experts) break;
+                logits[size_t(t) * num_experts + e0 + r] = acc[0][r];
+                if (two) logits[size_t(t + 1u) * num_experts + e0 + r] = acc[1][r];
+            }
         }
     }
+}
+
+template <int MAXI, int ROWS>
+static void launch_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits, uint32_t query_count,
+                                      uint32_t num_experts, uint32_t d, hipStream_t s) {
+    const uint32_t per_block = 4u * ROWS;
+    hipLaunchKernelGGL((k_prefill_logits_f16<MAXI, ROWS>),
+                       dim3((num_experts + per_block - 1u) / per_block, (query_count + kFastTokenBlock - 1u) / kFastTokenBlock),
+                       dim3(256), 0, s, weights, xs, logits, query_count, num_experts, d);
 }
 
 // prefill.metal:441-563: one wave selects for one token.
@@ -140,11 +166,8 @@ struct GroupArgs {
     uint32_t *tile_count;
 };
 
-constexpr uint32_t kGroupLdsPairs = 49152;  // pairs whose expert ids (one byte each) fit the LDS copy
-
-__device__ __forceinline__ uint32_t pair_expert(const GroupArgs &a, const uint8_t *ids, bool in_lds, uint32_t i) {
-    return in_lds ? uint32_t(ids[i]) : a.indices[i];
-}
+constexpr uint32_t kGroupLdsPairs = 49152;   // pairs whose expert ids (one byte each) fit the LDS copy
+constexpr uint32_t kGroupLdsWeights = 16384;  // pairs whose fp16 weights are staged beside them
 
 // One launch, four experts a workgroup (one a wave). Every workgroup builds the whole
 // histogram for itself in LDS (the pairs are a few KB and sit in L2), so no count has to
@@ -155,15 +178,20 @@ __device__ __forceinline__ uint32_t pair_expert(const GroupArgs &a, const uint8_
 // (PrefillMoEGrouping.swift:323-332).
 __global__ __launch_bounds__(256) void k_group(GroupArgs a) {
     __shared__ uint32_t s_hist[SHRIKE_MAX_ROUTER_EXPERTS];
-    __shared__ uint8_t s_ids[kGroupLdsPairs];
+    __shared__ __align__(16) uint8_t s_ids[kGroupLdsPairs];
+    __shared__ uint16_t s_weights[kGroupLdsWeights];
     const bool in_lds = a.pairs <= kGroupLdsPairs;
+    // the placement loop below is one dependent step a 64 pairs: a global load inside it would
+    // cost its full latency every step
+    const bool weights_in_lds = a.pairs <= kGroupLdsWeights;
     s_hist[threadIdx.x] = 0u;
     __syncthreads();
-#pragma unroll 4
+#pragma unroll 16
     for (uint32_t i = threadIdx.x; i < a.pairs; i += 256u) {
         const uint32_t v = a.indices[i];
         if (v < a.num_experts) atomicAdd(&s_hist[v], 1u);
         if (in_lds) s_ids[i] = uint8_t(min(v, 255u));
+        if (weights_in_lds) s_weights[i] = a.weights[i];
     }
     __syncthreads();
     const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4u + (threadIdx.x >> 6);
@@ -206,15 +234,53 @@ __global__ __launch_bounds__(256) void k_group(GroupArgs a) {
         a.tiles[tiles_before + j] = t;
     }
     if (count == 0) return;
+    const uint32_t token_magic = 0xffffffffu / a.top_k + 1u;  // i / top_k == umulhi(i, magic) for i * top_k < 2^32
     uint32_t running = 0;
+    if (in_lds) {
+        // 1,024 pairs a step: a lane takes 16 neighbouring ids with one LDS read, flags the bytes equal
+        // to e, and a prefix sum over the lanes turns the per-lane counts into positions in index order
+        const uint32_t pattern = e * 0x01010101u;
+        for (uint32_t base = 0; base < a.pairs && running < count; base += 1024u) {
+            const uint32_t i0 = base + lane * 16u;
+            uint32_t match = 0;
+            if (i0 < a.pairs) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(s_ids + i0);
+                const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t x = words[w] ^ pattern;  // a zero byte where the id is e
+                    const uint32_t t = ~(((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x | 0x7f7f7f7fu);  // 0x80 in exactly those bytes
+                    match |= ((((t >> 7) * 0x01020408u) >> 24) & 0xfu) << (4 * w);
+                }
+                const uint32_t valid = a.pairs - i0;  // ids past the last pair are whatever the LDS held
+                if (valid < 16u) match &= (1u << valid) - 1u;
+            }
+            const uint32_t mine = __popc(match);
+            const uint32_t upto = wave_inclusive_scan_u32(mine, lane);
+            uint32_t at = offset + running + upto - mine;
+            while (match) {
+                const uint32_t i = i0 + uint32_t(__ffs(int(match)) - 1);
+                match &= match - 1u;
+                shrike_token_expert_pair p;
+                p.token = __umulhi(i, token_magic);
+                p.expert = e;
+                p.rank = i - p.token * a.top_k;
+                p.weight_bits_and_reserved = weights_in_lds ? s_weights[i] : a.weights[i];
+                if (at < offset + count) a.sorted[at] = p;  // ids the histogram did not count (out of range) never land
+                ++at;
+            }
+            running += uint32_t(__builtin_amdgcn_readlane(int(upto), 63));
+        }
+        return;
+    }
     const uint64_t below = (uint64_t(1) << lane) - 1u;
     for (uint32_t base = 0; base < a.pairs && running < count; base += 64u) {
         const uint32_t i = base + lane;
-        const bool mine = i < a.pairs && pair_expert(a, s_ids, in_lds, i) == e;
+        const bool mine = i < a.pairs && a.indices[i] == e;
         const uint64_t mask = __ballot(mine);
         if (mine) {
             shrike_token_expert_pair p;
-            p.token = i / a.top_k;
+            p.token = __umulhi(i, token_magic);
             p.expert = e;
             p.rank = i - p.token * a.top_k;
             p.weight_bits_and_reserved = a.weights[i];
@@ -361,9 +427,11 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
             hipLaunchKernelGGL(k_prefill_scale_x, dim3(uint32_t((slots + 255u) / 256u)), dim3(256), 0, s, a.hidden, a.effective_scale,
                                xs, query_count, d, hidden_stride_elements);
             SHRIKE_HIP(hipGetLastError());
-            hipLaunchKernelGGL(k_prefill_logits_f16, dim3((num_experts + 3u) / 4u, (query_count + kFastTokenBlock - 1u) / kFastTokenBlock),
-                               dim3(256), 0, s, static_cast<const uint16_t *>(d_weights), xs, d_logits_workspace, query_count,
-                               num_experts, d);
+            // two rows a wave: half the x traffic of one; more rows leave too few waves to hide the loads
+            const uint16_t *w16 = static_cast<const uint16_t *>(d_weights);
+            if (d <= 2048u) launch_prefill_logits_f16<4, 2>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
+            else if (d <= 3072u) launch_prefill_logits_f16<6, 2>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
+            else launch_prefill_logits_f16<8, 2>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
             break;
         }
         case 8: hipLaunchKernelGGL(k_prefill_logits<8>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;

@@ -27,4 +27,14 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
     return v;
 }
 
+// Inclusive prefix sum over the lanes of a wave, lane 0 first.
+__device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, uint32_t lane) {
+#pragma unroll
+    for (uint32_t o = 1; o < 64u; o <<= 1) {
+        const uint32_t below = __shfl_up(v, o);
+        v += lane >= o ? below : 0u;
+    }
+    return v;
+}
+
 }  // namespace shrike
