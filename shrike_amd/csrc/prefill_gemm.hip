@@ -21,6 +21,10 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kChunkK = 256;                 // k staged in LDS per step: four groups
+constexpr uint32_t kGroupsPerChunk = kChunkK / 64;
+constexpr uint32_t kStagePieces = kChunkK / 8;     // 16-byte pieces of one staged row
+constexpr uint32_t kStageRows = 256 / kStagePieces; // rows one pass of the workgroup stages
+constexpr uint32_t kStagePasses = kRowTile / kStageRows;
 constexpr uint32_t kLdsRow = kChunkK + 8;         // halves per staged row; the pad spreads the banks
 constexpr uint32_t kMaxMT = kRowTile / 32;        // 32-row MFMA tiles per row tile
 constexpr float kTwo24 = 16777216.0f;
@@ -127,12 +131,12 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     const uint32_t n0 = (blockIdx.y * 4u + wave) * (MODE == 0 ? 32u : 64u);
     const bool active = n0 < N;
 
-    // ---- A staging: thread -> (row = tid / 32 + 8 i, 16-byte piece = tid % 32)
-    const uint32_t piece = threadIdx.x & 31u, row0 = threadIdx.x >> 5;
-    const uint16_t *src_row[kMaxMT * 4];
+    // ---- A staging: thread -> (row = tid / kStagePieces + kStageRows i, 16-byte piece = tid % kStagePieces)
+    const uint32_t piece = threadIdx.x % kStagePieces, row0 = threadIdx.x / kStagePieces;
+    const uint16_t *src_row[kStagePasses];
 #pragma unroll
-    for (uint32_t i = 0; i < kMaxMT * 4; ++i) {
-        const uint32_t r = min(row0 + 8u * i, tile.rows - 1u);  // rows past the tile repeat its last row
+    for (uint32_t i = 0; i < kStagePasses; ++i) {
+        const uint32_t r = min(row0 + kStageRows * i, tile.rows - 1u);  // rows past the tile repeat its last row
         if (MODE == 0) {
             const uint32_t token = DENSE ? tile.pair_start + r : a.pairs[tile.pair_start + r].token;
             src_row[i] = a.hidden + size_t(token) * a.hidden_stride;
@@ -140,17 +144,17 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
             src_row[i] = a.act + (size_t(tile_index) * kRowTile + r) * a.f;
         }
     }
-    uint4 stage[kMaxMT * 4];
+    uint4 stage[kStagePasses];
     auto fetch = [&](uint32_t chunk) {
         const uint32_t k = chunk * kChunkK + piece * 8u;
 #pragma unroll
-        for (uint32_t i = 0; i < kMaxMT * 4; ++i)
-            if (i < mt_count * 4u && k < K) stage[i] = *reinterpret_cast<const uint4 *>(src_row[i] + k);
+        for (uint32_t i = 0; i < kStagePasses; ++i)
+            if (i * kStageRows < mt_count * 32u && k < K) stage[i] = *reinterpret_cast<const uint4 *>(src_row[i] + k);
     };
     auto commit = [&](uint32_t buf) {
 #pragma unroll
-        for (uint32_t i = 0; i < kMaxMT * 4; ++i) {
-            if (i >= mt_count * 4u) continue;
+        for (uint32_t i = 0; i < kStagePasses; ++i) {
+            if (i * kStageRows >= mt_count * 32u) continue;
             uint4 v = stage[i];
             if (BITS == 4) {  // (0,1,2,3,4,5,6,7) -> (0,4,1,5,2,6,3,7), to meet codes4
                 uint4 p;
@@ -160,7 +164,7 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
                 p.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
                 v = p;
             }
-            *reinterpret_cast<uint4 *>(&s_a[buf][row0 + 8u * i][piece * 8u]) = v;
+            *reinterpret_cast<uint4 *>(&s_a[buf][row0 + kStageRows * i][piece * 8u]) = v;
         }
     };
 
@@ -206,6 +210,17 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) total[nt][mt][i] = 0.0f;
 
+    // the rows' group sums for the bias term: their addresses hang on the pair records, so they are
+    // worked out here, far ahead of their use
+    const uint32_t *sums = MODE == 0 ? a.hidden_sums : a.act_sums;
+    const uint32_t *sum_row[kMaxMT];
+#pragma unroll
+    for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+        const uint32_t r = min(mt * 32u + col, tile.rows - 1u);
+        const uint32_t token = (MODE != 0) ? 0u : DENSE ? tile.pair_start + r : a.pairs[tile.pair_start + r].token;
+        sum_row[mt] = MODE == 0 ? sums + size_t(token) * G : sums + (size_t(tile_index) * kRowTile + r) * G;
+    }
+
     BRegs<BITS> cur[2], nxt[2];
     if (active) {
         load_b<BITS>(cur[0], bw[0], bs[0], 0, kb);
@@ -218,10 +233,10 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     for (uint32_t c = 0; c < chunks; ++c) {
         const uint32_t buf = c & 1u;
         if (c + 1u < chunks) fetch(c + 1u);
-        const uint32_t groups_here = min(4u, G - 4u * c);
+        const uint32_t groups_here = min(kGroupsPerChunk, G - kGroupsPerChunk * c);
         if (active) {
             for (uint32_t gi = 0; gi < groups_here; ++gi) {
-                const uint32_t g = 4u * c + gi;
+                const uint32_t g = kGroupsPerChunk * c + gi;
                 const uint32_t gn = min(g + 1u, G - 1u);
                 load_b<BITS>(nxt[0], bw[0], bs[0], gn, kb);
                 load_b<BITS>(nxt[1], bw[1], bs[1], gn, kb);
@@ -258,36 +273,55 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     }
     if (!active) return;
 
-    // ---- bias term: (group sums of the rows) x (group biases), sixteen k' = eight groups a step
+    // ---- bias term: (group sums of the rows) x (group biases), sixteen k' = eight groups an MFMA.
+    // The operands of four steps are fetched together, four values a load where the rows allow it.
     {
-        const uint32_t *sums = MODE == 0 ? a.hidden_sums : a.act_sums;
-        const uint32_t *sum_row[kMaxMT];
+        // a lane's four groups are one aligned 8- or 16-byte run when G is a multiple of 4 and the bias rows start aligned
+        const bool wide = (G & 3u) == 0u && ((reinterpret_cast<uintptr_t>(bb[0]) | reinterpret_cast<uintptr_t>(bb[1])) & 7u) == 0u;
+        for (uint32_t gbase = 0; gbase < G; gbase += 32u) {
+            Frag bfr[4][2], afr[4][kMaxMT];
 #pragma unroll
-        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
-            const uint32_t r = min(mt * 32u + col, tile.rows - 1u);
-            const uint32_t token = (MODE != 0) ? 0u : DENSE ? tile.pair_start + r : a.pairs[tile.pair_start + r].token;
-            sum_row[mt] = MODE == 0 ? sums + size_t(token) * G : sums + (size_t(tile_index) * kRowTile + r) * G;
-        }
-        for (uint32_t g0 = 0; g0 < G; g0 += 8u) {
-            const uint32_t gl = g0 + 4u * kb;  // this lane's four groups
-            Frag bfr[2], afr[kMaxMT];
+            for (uint32_t step = 0; step < 4; ++step) {
+                const uint32_t gl = gbase + 8u * step + 4u * kb;  // this lane's four groups
+                if (wide) {
+                    const bool on = gl < G;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const bool on = gl + j < G;
+                    for (int nt = 0; nt < 2; ++nt) {
+                        const uint2 b4 = on ? *reinterpret_cast<const uint2 *>(bb[nt] + gl) : make_uint2(0u, 0u);
+                        bfr[step][nt].u[0] = b4.x & 0xffffu; bfr[step][nt].u[1] = b4.x >> 16;
+                        bfr[step][nt].u[2] = b4.y & 0xffffu; bfr[step][nt].u[3] = b4.y >> 16;
+                    }
 #pragma unroll
-                for (int nt = 0; nt < 2; ++nt) {
-                    uint16_t bits = on ? bb[nt][gl + j] : uint16_t(0);
-                    if (a.meta == SHRIKE_META_BF16) bits = f32_to_f16(bf16_to_f32(bits));
-                    bfr[nt].u[j] = uint32_t(bits) * 0x00010001u;  // against (hi, lo)
+                    for (uint32_t mt = 0; mt < kMaxMT; ++mt)
+                        afr[step][mt].v = (on && mt < mt_count) ? *reinterpret_cast<const uint4 *>(sum_row[mt] + gl) : zero4();
+                } else {
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const bool on = gl + jj < G;
+#pragma unroll
+                        for (int nt = 0; nt < 2; ++nt) bfr[step][nt].u[jj] = on ? bb[nt][gl + jj] : 0u;
+#pragma unroll
+                        for (uint32_t mt = 0; mt < kMaxMT; ++mt) afr[step][mt].u[jj] = (on && mt < mt_count) ? sum_row[mt][gl + jj] : 0u;
+                    }
                 }
-#pragma unroll
-                for (uint32_t mt = 0; mt < kMaxMT; ++mt) afr[mt].u[j] = (on && mt < mt_count) ? sum_row[mt][gl + j] : 0u;
             }
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
+            for (uint32_t step = 0; step < 4; ++step) {
+                if (gbase + 8u * step >= G) break;
 #pragma unroll
-                for (uint32_t mt = 0; mt < kMaxMT; ++mt)
-                    if (mt < mt_count) total[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[mt].h, bfr[nt].h, total[nt][mt], 0, 0, 0);
+                for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {  // the bias as fp16, doubled against (hi, lo)
+                        uint16_t bits = uint16_t(bfr[step][nt].u[jj]);
+                        if (a.meta == SHRIKE_META_BF16) bits = f32_to_f16(bf16_to_f32(bits));
+                        bfr[step][nt].u[jj] = uint32_t(bits) * 0x00010001u;
+                    }
+#pragma unroll
+                    for (uint32_t mt = 0; mt < kMaxMT; ++mt)
+                        if (mt < mt_count)
+                            total[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[step][mt].h, bfr[step][nt].h, total[nt][mt], 0, 0, 0);
+                }
+            }
         }
     }
 
