@@ -15,6 +15,9 @@ struct RouterArgs {
     float *logits_out;
     SelectArgs sel;
     RouteLists lists;  // out_indices == nullptr: logits only
+    // several tokens in one launch (grid.y): token t reads hidden + t * token_stride, writes logits_out + t *
+    // num_experts and out_indices / out_weights + t * top_k, and counts arrivals in counter[t]; select only
+    uint32_t token_stride;
 };
 
 struct Phase1Args {
@@ -48,6 +51,9 @@ struct Phase2Args {
 };
 
 int launch_router(const RouterArgs &a, uint32_t router_bits, hipStream_t s);
+// the same for `tokens` tokens in one launch; a.counter must have a zeroed word for each
+constexpr uint32_t kRouterLaunchTokens = 16;  // up to here the one-launch router beats the three-launch prefill router
+int launch_router_tokens(const RouterArgs &a, uint32_t router_bits, uint32_t tokens, hipStream_t s);
 // router logit rows + the shared expert's gate/up rows in one grid
 int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, hipStream_t s);
 uint32_t phase1_blocks(uint32_t top_k, uint32_t f);

@@ -13,20 +13,30 @@ __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
     const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t e = blockIdx.x * 4u + wave;
     const bool select_too = a.lists.out_indices != nullptr;
-    if (e < a.sel.num_experts) router_row<RK>(a, e, lane, select_too);
+    // grid.y walks tokens (one in decode); the argument block stays as it is, the token's rows are locals
+    const size_t tok = blockIdx.y;
+    const uint16_t *hidden = a.hidden + tok * a.token_stride;
+    float *logits = a.logits_out + tok * a.sel.num_experts;
+    uint32_t *counter = a.counter + tok;
+    if (e < a.sel.num_experts) router_row<RK>(a, hidden, logits, e, lane, select_too);
     if (!select_too) return;  // logits only
     // The logits went out as write-through stores: once they are complete, the workgroup
     // counts itself in; the last to arrive reads all logits back past the caches.
     wait_stores();
     __syncthreads();
     if (threadIdx.x == 0)
-        s_last = __hip_atomic_fetch_add(a.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1u ? 1u : 0u;
+        s_last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1u ? 1u : 0u;
     __syncthreads();
     if (!s_last || wave != 0) return;
     __shared__ RouteScratch s_route;
+    SelectArgs sel = a.sel;
+    sel.logits = logits;
+    RouteLists lists = a.lists;
+    lists.out_indices = a.lists.out_indices + tok * a.sel.top_k;
+    lists.out_weights = a.lists.out_weights + tok * a.sel.top_k;
     uint32_t cell;
-    route_wave<true>(a.sel, a.lists, lane, true, cell, s_route);
-    if (lane == 0) __hip_atomic_store(a.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    route_wave<true>(sel, lists, lane, true, cell, s_route);
+    if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The head of the fused layer: the router's logit rows and, beside them in the same grid,
@@ -110,8 +120,11 @@ __global__ __launch_bounds__(64) void k_classify(ClassifyArgs a) {
     }
 }
 
-int launch_router(const RouterArgs &a, uint32_t router_bits, hipStream_t s) {
-    const dim3 grid((a.sel.num_experts + 3) / 4), block(256);
+int launch_router(const RouterArgs &a, uint32_t router_bits, hipStream_t s) { return launch_router_tokens(a, router_bits, 1, s); }
+
+int launch_router_tokens(const RouterArgs &a, uint32_t router_bits, uint32_t tokens, hipStream_t s) {
+    SHRIKE_REQUIRE(tokens == 1 || (a.lists.out_indices && !a.lists.residency), "router: several tokens select only");
+    const dim3 grid((a.sel.num_experts + 3) / 4, tokens), block(256);
     if (router_bits == 0) hipLaunchKernelGGL((k_router<0>), grid, block, 0, s, a);
     else if (router_bits == 8) hipLaunchKernelGGL((k_router<8>), grid, block, 0, s, a);
     else hipLaunchKernelGGL((k_router<4>), grid, block, 0, s, a);

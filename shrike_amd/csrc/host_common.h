@@ -36,9 +36,13 @@ inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s);
 
 // MoE.swift:41-216: the handle keeps the shape it was made for, the router's fp32
 // logits (routerLogits, MoE.swift:74) and the router's arrival counter.
+constexpr unsigned kCounterWords = 256;
+constexpr unsigned kRouterTokenCounters = 128;  // first of the per-token arrival counters
+
 struct shrike_hip_moe {
     shrike_moe_desc desc;
     int device;
     float *d_logits;        // fp32[SHRIKE_MAX_ROUTER_EXPERTS]
-    uint32_t *d_counter;    // u32[4], zero between launches
+    uint32_t *d_counter;    // u32[kCounterWords], zero between launches: [0] the router's arrivals, from
+                            // [kRouterTokenCounters] one word a token of the several-token router
 };

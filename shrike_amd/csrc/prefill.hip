@@ -419,6 +419,17 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
     a.sel.sigmoid = moe->desc.sigmoid_router_scores;
     a.sel.scaling = moe->desc.routed_scaling_factor;
     hipStream_t s = as_stream(stream);
+    if (query_count <= kRouterLaunchTokens) {
+        // a handful of tokens (decode for several sequences): the decode router's kernel with the tokens
+        // on the grid, one launch for logits and selection instead of three
+        a.logits_out = d_logits_workspace;
+        a.sel.logits = d_logits_workspace;
+        a.lists.out_indices = d_out_indices;
+        a.lists.out_weights = static_cast<uint16_t *>(d_out_weights);
+        a.counter = moe->d_counter + kRouterTokenCounters;
+        a.token_stride = hidden_stride_elements;
+        return launch_router_tokens(a, moe->desc.router_weight_bits, query_count, s);
+    }
     const dim3 grid((num_experts + 3u) / 4u, (query_count + kRouterTokenBlock - 1u) / kRouterTokenBlock);
     switch (moe->desc.router_weight_bits) {
         case 0: {

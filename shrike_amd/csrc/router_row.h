@@ -10,8 +10,10 @@ namespace shrike {
 // group-affine codes. The per-lane fused-multiply-add order and the xor butterfly are
 // fixed so that the fp32 logits are reproducible bit for bit (lane l takes chunks
 // l, l+64, ...).
+// hidden, logits: the token's activation row and its logit row (a.hidden, a.logits_out for one token)
 template <int RK>
-__device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint32_t lane, bool publish = false) {
+__device__ __forceinline__ void router_row(const RouterArgs &a, const uint16_t *hidden, float *logits, uint32_t e, uint32_t lane,
+                                           bool publish) {
     constexpr int E = RK == 0 ? 8 : RK == 8 ? 16 : 32;  // elements per 16-byte weight chunk
     constexpr int PIECES = E / 8;
     constexpr int MAXI = RK == 0 ? 8 : 4;
@@ -28,7 +30,7 @@ __device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint
         w[i] = *reinterpret_cast<const uint4 *>(row + 16u * cc);
 #pragma unroll
         for (int j = 0; j < PIECES; ++j) {
-            xv[i][j] = reinterpret_cast<const uint4 *>(a.hidden)[cc * PIECES + j];
+            xv[i][j] = reinterpret_cast<const uint4 *>(hidden)[cc * PIECES + j];
             ev[i][j] = reinterpret_cast<const uint4 *>(a.effective_scale)[cc * PIECES + j];
         }
         if (RK != 0) {
@@ -78,9 +80,14 @@ __device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint
     // publish: the logit is for another workgroup of the same launch and is written through to
     // device-coherent memory
     if (lane == 0) {
-        if (publish) __hip_atomic_store(a.logits_out + e, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else a.logits_out[e] = acc;
+        if (publish) __hip_atomic_store(logits + e, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else logits[e] = acc;
     }
+}
+
+template <int RK>
+__device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint32_t lane, bool publish = false) {
+    router_row<RK>(a, a.hidden, a.logits_out, e, lane, publish);
 }
 
 }  // namespace shrike

@@ -381,8 +381,8 @@ shrike_hip_moe *shrike_hip_moe_create(const shrike_moe_desc *desc, int *out_errn
     moe->d_logits = nullptr; moe->d_counter = nullptr;
     if (hipGetDevice(&moe->device) != hipSuccess
         || hipMalloc(reinterpret_cast<void **>(&moe->d_logits), sizeof(float) * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess
-        || hipMalloc(reinterpret_cast<void **>(&moe->d_counter), sizeof(uint32_t) * 4) != hipSuccess
-        || hipMemset(moe->d_counter, 0, sizeof(uint32_t) * 4) != hipSuccess
+        || hipMalloc(reinterpret_cast<void **>(&moe->d_counter), sizeof(uint32_t) * kCounterWords) != hipSuccess
+        || hipMemset(moe->d_counter, 0, sizeof(uint32_t) * kCounterWords) != hipSuccess
         || hipMemset(moe->d_logits, 0, sizeof(float) * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess) {
         set_error("device allocation for the MoE handle failed: %s", hipGetErrorString(hipGetLastError()));
         shrike_hip_moe_destroy(moe);
