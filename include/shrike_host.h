@@ -317,6 +317,87 @@ int shrike_packed_layout_cross_validate(const shrike_packed_layout *layout, int 
                                         const char *const *manifest_paths, const uint64_t *manifest_sizes,
                                         size_t manifest_file_count);
 
+/* ------------------------------------------------------- routed tile loop of a streamed prefill chunk */
+
+/* PrefillRoutedTileSchedulerConfig (sources/Shrike/Kernels/Prefill/MoE/PrefillRoutedTileScheduler.swift:46-96).
+ * make clamps as the reference's init does: depth >= 1, 1...16 experts a tile, 1...16 tiles a
+ * command buffer, lookahead 0 or 1 (reference defaults: 1, 8, 1, 0). */
+typedef struct {
+    int32_t max_pending_depth, tile_experts, tiles_per_command_buffer, fetch_lookahead;
+} shrike_tile_scheduler_config;
+void shrike_tile_scheduler_config_make(int max_pending_depth, int tile_experts, int tiles_per_command_buffer,
+                                       int fetch_lookahead, shrike_tile_scheduler_config *out);
+/* fitsSlotBudget (:63-66) and fitting (:71-91; 0 = nil, no configuration fits). */
+int shrike_tile_scheduler_fits_slot_budget(const shrike_tile_scheduler_config *config, int slot_count, int reserved_hits);
+int shrike_tile_scheduler_fitting(const shrike_tile_scheduler_config *config, int slot_count, int reserved_hits,
+                                  shrike_tile_scheduler_config *out);
+/* decide (:104-122). prefetchNext's avoidingSlots are the caller's pending slots, in their order.
+ * pending_depth < 0: the input's default (1 with a pending tile, else 0). */
+enum {
+    SHRIKE_TILE_ISSUE_WITHOUT_PENDING = 0,
+    SHRIKE_TILE_PREFETCH_NEXT = 1,
+    SHRIKE_TILE_DRAIN_NO_ASSIGNED_SLOTS = 2,   /* drainBeforeIssue(.pendingTileHasNoAssignedSlots) */
+    SHRIKE_TILE_DRAIN_PLAN_UNAVAILABLE = 3,    /* drainBeforeIssue(.avoidingSlotPlanUnavailable) */
+    SHRIKE_TILE_DRAIN_MAX_DEPTH = 4            /* drainBeforeIssue(.maxPendingDepthReached) */
+};
+int shrike_tile_scheduler_decide(const shrike_tile_scheduler_config *config, int has_pending_tile, int pending_depth,
+                                 size_t pending_assigned_slot_count, int avoiding_slot_plan_available);
+int shrike_tile_scheduler_plans_lookahead(const shrike_tile_scheduler_config *config, int index, int tile_count);
+int shrike_tile_scheduler_should_begin_lookahead(const shrike_tile_scheduler_config *config, int index, int tile_count,
+                                                 int avoiding_slot_plan_available);
+/* batchAction (:139-155) */
+enum { SHRIKE_TILE_BATCH_OPEN = 0, SHRIKE_TILE_BATCH_FULL = 1, SHRIKE_TILE_BATCH_LAST_TILE = 2 };
+typedef struct {
+    int32_t commit_before_append;   /* the tile's plan collides with a slot the open batch still holds */
+    int32_t commit_after_append;    /* SHRIKE_TILE_BATCH_* */
+} shrike_tile_batch_action;
+void shrike_tile_scheduler_batch_action(const shrike_tile_scheduler_config *config, int open_batch_tiles,
+                                        size_t open_batch_slot_count, int next_tile_plan_available, int is_last_tile,
+                                        shrike_tile_batch_action *out);
+
+/* PrefillRoutedTileDriver (sources/Shrike/Kernels/Prefill/MoE/PrefillRoutedTileSequencer.swift:3-24) as
+ * callbacks; those returning int give 0 or an error code, which ends the run. plan stores 0 in
+ * *available when no plan avoiding the batches' slots (and those of the begun tile
+ * avoiding_in_flight, -1 = none) fits the cache. */
+typedef struct {
+    void *context;
+    int (*open_batch_tiles)(void *context);
+    size_t (*open_batch_slot_count)(void *context);
+    int (*pending_depth)(void *context);
+    size_t (*pending_assigned_slot_count)(void *context);
+    int (*plan)(void *context, int tile, int avoiding_in_flight, int *available);
+    int (*begin)(void *context, int tile);
+    int (*abandon_plan)(void *context, int tile);
+    int (*encode)(void *context, int tile);
+    void (*commit_open_batch)(void *context);
+    int (*drain_oldest_batch)(void *context);
+    void (*abandon_begun_fetches)(void *context);
+} shrike_tile_driver;
+/* PrefillRoutedTileSequencer.run (:30-85): a tile is awaited and encoded only once its successor's
+ * fetch is in flight. On an error from a callback abandon_begun_fetches runs and the error returns. */
+int shrike_tile_sequencer_run(const shrike_tile_scheduler_config *config, int tile_count, const shrike_tile_driver *driver);
+
+/* PrefillChunkExpertProtection (sources/Shrike/Runtime/Inference/RealForwardRunner.swift:63-93): the chunk's
+ * routed experts still to come are protected from eviction; planning a tile clears its own.
+ * remaining: u8[experts_per_layer], 1 = protected. */
+void shrike_chunk_protection_init(const int32_t *routed_experts, size_t count, uint8_t *remaining, size_t experts_per_layer);
+void shrike_chunk_protection_planning(const int32_t *tile_experts, size_t count, uint8_t *remaining, size_t experts_per_layer);
+
+/* PrefillStreamedTileSlotLifetime (sources/Shrike/Kernels/Prefill/MoE/PrefillGroupedRoutedMoE.swift:388-424):
+ * a slot may not be planned again before the tile that holds it has completed. */
+typedef struct shrike_tile_lifetime shrike_tile_lifetime;
+enum {
+    SHRIKE_TILE_LIFETIME_INVALID = -1,
+    SHRIKE_TILE_LIFETIME_DUPLICATE_SLOTS = 1,
+    SHRIKE_TILE_LIFETIME_SLOT_REUSE = 2,      /* slotReuseBeforeCompletion; *conflicting_tile names the holder */
+    SHRIKE_TILE_LIFETIME_NOT_IN_FLIGHT = 3    /* completeWithoutInFlightTile */
+};
+shrike_tile_lifetime *shrike_tile_lifetime_create(void);
+void shrike_tile_lifetime_destroy(shrike_tile_lifetime *lifetime);
+int shrike_tile_lifetime_begin(shrike_tile_lifetime *lifetime, int tile_index, const int32_t *planned_slots, size_t count,
+                               int *conflicting_tile);
+int shrike_tile_lifetime_complete(shrike_tile_lifetime *lifetime, int tile_index);
+
 #ifdef __cplusplus
 }
 #endif

@@ -861,3 +861,110 @@ def reader_cancel_slot(count, next_index, outstanding, first_errno, ecanceled):
     if next_index >= count:
         return count, next_index, outstanding, first_errno
     return count, count, outstanding - (count - next_index), first_errno or ecanceled
+
+
+# ------------------------------------------------------------- routed tile loop of a streamed prefill chunk
+
+class TileConfig:
+    """PrefillRoutedTileSchedulerConfig, PrefillRoutedTileScheduler.swift:46-96."""
+
+    def __init__(self, max_pending_depth=1, tile_experts=8, tiles_per_command_buffer=1, fetch_lookahead=0):
+        self.max_pending_depth = max(1, max_pending_depth)
+        self.tile_experts = max(1, min(16, tile_experts))
+        self.tiles_per_command_buffer = max(1, min(16, tiles_per_command_buffer))
+        self.fetch_lookahead = max(0, min(1, fetch_lookahead))
+
+    def astuple(self):
+        return (self.max_pending_depth, self.tile_experts, self.tiles_per_command_buffer, self.fetch_lookahead)
+
+    @property
+    def _batches(self):
+        return self.max_pending_depth + 1
+
+    def fits_slot_budget(self, slot_count, reserved_hits=0):
+        if not (slot_count > 0 and reserved_hits >= 0):
+            return False
+        tiles = self._batches * self.tiles_per_command_buffer + self.fetch_lookahead
+        return tiles * self.tile_experts + reserved_hits <= slot_count
+
+    def fitting(self, slot_count, reserved_hits=0):
+        if not (slot_count > reserved_hits and reserved_hits >= 0):
+            return None
+        available = slot_count - reserved_hits
+        # Swift's `/` truncates toward zero; the numerator can be negative
+        q = int((available - self.fetch_lookahead * self.tile_experts) / (self._batches * self.tile_experts))
+        narrowed = TileConfig(self.max_pending_depth, self.tile_experts, max(1, min(self.tiles_per_command_buffer, q)),
+                              self.fetch_lookahead)
+        if narrowed.fits_slot_budget(slot_count, reserved_hits):
+            return narrowed
+        per_tile = available // (self._batches + self.fetch_lookahead)
+        if per_tile <= 0:
+            return None
+        return TileConfig(self.max_pending_depth, min(self.tile_experts, per_tile), 1, self.fetch_lookahead)
+
+
+def tile_decide(config, has_pending_tile, pending_assigned_slots, plan_available, pending_depth=None):
+    """PrefillRoutedTileScheduler.decide, :104-122. Returns (decision, reason or avoiding slots)."""
+    depth = max(0, pending_depth if pending_depth is not None else (1 if has_pending_tile else 0))
+    if not has_pending_tile:
+        return ("issueWithoutPending", None)
+    if depth > config.max_pending_depth:
+        return ("drainBeforeIssue", "maxPendingDepthReached")
+    if not pending_assigned_slots:
+        return ("drainBeforeIssue", "pendingTileHasNoAssignedSlots")
+    if not plan_available:
+        return ("drainBeforeIssue", "avoidingSlotPlanUnavailable")
+    return ("prefetchNext", list(pending_assigned_slots))
+
+
+def tile_batch_action(config, open_batch_tiles, open_batch_slots, next_plan_available, is_last_tile):
+    """PrefillRoutedTileScheduler.batchAction, :139-155. Returns (commitBeforeAppend, closeReason or None)."""
+    before = bool(open_batch_slots) and not next_plan_available
+    after = (0 if before else max(0, open_batch_tiles)) + 1
+    reason = "batchFull" if after >= config.tiles_per_command_buffer else "lastTile" if is_last_tile else None
+    return before, reason
+
+
+def tile_plans_lookahead(config, index, tile_count):
+    return config.fetch_lookahead > 0 and index + 1 < tile_count
+
+
+def tile_sequence(config, tile_count, driver):
+    """PrefillRoutedTileSequencer.run, PrefillRoutedTileSequencer.swift:30-104, over a driver object with the
+    protocol's members; an exception reaches abandon_begun_fetches and propagates."""
+    def issue(tile, plan_available):
+        decision, _ = tile_decide(config, driver.pending_depth > 0, driver.pending_assigned_slots, plan_available,
+                                  driver.pending_depth)
+        if decision == "drainBeforeIssue":
+            if plan_available:
+                driver.abandon_plan(tile)
+            driver.drain_oldest_batch()
+        driver.begin(tile)
+
+    try:
+        carried = None
+        for tile in range(tile_count):
+            is_last = tile == tile_count - 1
+            carried_fetch = carried == tile
+            carried = None
+            plan_available = True if carried_fetch else driver.plan(tile, None)
+            before, after = tile_batch_action(config, driver.open_batch_tiles, driver.open_batch_slots, plan_available, is_last)
+            if before:
+                driver.commit_open_batch()
+            if not carried_fetch:
+                issue(tile, plan_available)
+            if tile_plans_lookahead(config, tile, tile_count):
+                if driver.plan(tile + 1, tile):
+                    driver.begin(tile + 1)
+                    carried = tile + 1
+            driver.encode(tile)
+            if after is not None:
+                driver.commit_open_batch()
+            while driver.pending_depth + (1 if driver.open_batch_tiles > 0 else 0) > config.max_pending_depth:
+                driver.drain_oldest_batch()
+        driver.commit_open_batch()
+        while driver.pending_depth > 0:
+            driver.drain_oldest_batch()
+    except BaseException:
+        driver.abandon_begun_fetches()
+        raise

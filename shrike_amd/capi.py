@@ -141,8 +141,46 @@ class PackedTensor(C.Structure):
                 ("rank", C.c_uint32), ("bits", C.c_int32)]
 
 
+class TileSchedulerConfig(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("max_pending_depth", "tile_experts", "tiles_per_command_buffer", "fetch_lookahead")]
+
+
+class TileBatchAction(C.Structure):
+    _fields_ = [("commit_before_append", C.c_int32), ("commit_after_append", C.c_int32)]
+
+
+class TileDriver(C.Structure):
+    _fields_ = [("context", C.c_void_p),
+                ("open_batch_tiles", C.CFUNCTYPE(C.c_int, C.c_void_p)),
+                ("open_batch_slot_count", C.CFUNCTYPE(C.c_size_t, C.c_void_p)),
+                ("pending_depth", C.CFUNCTYPE(C.c_int, C.c_void_p)),
+                ("pending_assigned_slot_count", C.CFUNCTYPE(C.c_size_t, C.c_void_p)),
+                ("plan", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_int))),
+                ("begin", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int)),
+                ("abandon_plan", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int)),
+                ("encode", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int)),
+                ("commit_open_batch", C.CFUNCTYPE(None, C.c_void_p)),
+                ("drain_oldest_batch", C.CFUNCTYPE(C.c_int, C.c_void_p)),
+                ("abandon_begun_fetches", C.CFUNCTYPE(None, C.c_void_p))]
+
+
 SIGNATURES = {
     "shrike_hip_last_error": (C.c_char_p, []),
+    "shrike_tile_scheduler_config_make": (None, [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(TileSchedulerConfig)]),
+    "shrike_tile_scheduler_fits_slot_budget": (C.c_int, [C.POINTER(TileSchedulerConfig), C.c_int, C.c_int]),
+    "shrike_tile_scheduler_fitting": (C.c_int, [C.POINTER(TileSchedulerConfig), C.c_int, C.c_int, C.POINTER(TileSchedulerConfig)]),
+    "shrike_tile_scheduler_decide": (C.c_int, [C.POINTER(TileSchedulerConfig), C.c_int, C.c_int, C.c_size_t, C.c_int]),
+    "shrike_tile_scheduler_plans_lookahead": (C.c_int, [C.POINTER(TileSchedulerConfig), C.c_int, C.c_int]),
+    "shrike_tile_scheduler_should_begin_lookahead": (C.c_int, [C.POINTER(TileSchedulerConfig), C.c_int, C.c_int, C.c_int]),
+    "shrike_tile_scheduler_batch_action": (None, [C.POINTER(TileSchedulerConfig), C.c_int, C.c_size_t, C.c_int, C.c_int,
+                                                  C.POINTER(TileBatchAction)]),
+    "shrike_tile_sequencer_run": (C.c_int, [C.POINTER(TileSchedulerConfig), C.c_int, C.POINTER(TileDriver)]),
+    "shrike_chunk_protection_init": (None, [C.POINTER(C.c_int32), C.c_size_t, C.POINTER(C.c_uint8), C.c_size_t]),
+    "shrike_chunk_protection_planning": (None, [C.POINTER(C.c_int32), C.c_size_t, C.POINTER(C.c_uint8), C.c_size_t]),
+    "shrike_tile_lifetime_create": (_VP, []),
+    "shrike_tile_lifetime_destroy": (None, [_VP]),
+    "shrike_tile_lifetime_begin": (C.c_int, [_VP, C.c_int, C.POINTER(C.c_int32), C.c_size_t, C.POINTER(C.c_int)]),
+    "shrike_tile_lifetime_complete": (C.c_int, [_VP, C.c_int]),
     "shrike_host_last_error": (C.c_char_p, []),
     "shrike_expert_reader_create": (_VP, [C.c_char_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int)]),
     "shrike_expert_reader_destroy": (None, [_VP]),

@@ -421,3 +421,166 @@ class PackedExpertsLayout:
         sizes = (C.c_uint64 * len(file_sizes))(*file_sizes.values())
         self._check(capi.load().shrike_packed_layout_cross_validate(self.handle, num_layers, experts_per_layer,
                                                                     expert_stride, paths, sizes, len(file_sizes)))
+
+
+# --------------------------------------------------------------- routed tile loop of a streamed prefill chunk
+
+ISSUE_WITHOUT_PENDING, PREFETCH_NEXT, DRAIN_NO_ASSIGNED_SLOTS, DRAIN_PLAN_UNAVAILABLE, DRAIN_MAX_DEPTH = range(5)
+BATCH_OPEN, BATCH_FULL, BATCH_LAST_TILE = range(3)
+
+
+class TileSchedulerConfig:
+    """PrefillRoutedTileSchedulerConfig (PrefillRoutedTileScheduler.swift:46-96); the constructor clamps."""
+
+    def __init__(self, max_pending_depth=1, tile_experts=8, tiles_per_command_buffer=1, fetch_lookahead=0):
+        self.c = capi.TileSchedulerConfig()
+        capi.load().shrike_tile_scheduler_config_make(max_pending_depth, tile_experts, tiles_per_command_buffer,
+                                                      fetch_lookahead, C.byref(self.c))
+
+    def astuple(self):
+        return (self.c.max_pending_depth, self.c.tile_experts, self.c.tiles_per_command_buffer, self.c.fetch_lookahead)
+
+    def __eq__(self, other):
+        return isinstance(other, TileSchedulerConfig) and self.astuple() == other.astuple()
+
+    def __repr__(self):
+        return "TileSchedulerConfig(depth=%d, experts=%d, width=%d, lookahead=%d)" % self.astuple()
+
+    def fits_slot_budget(self, slot_count: int, reserved_hits: int = 0) -> bool:
+        return bool(capi.load().shrike_tile_scheduler_fits_slot_budget(C.byref(self.c), slot_count, reserved_hits))
+
+    def fitting(self, slot_count: int, reserved_hits: int = 0):
+        out = TileSchedulerConfig()
+        if not capi.load().shrike_tile_scheduler_fitting(C.byref(self.c), slot_count, reserved_hits, C.byref(out.c)):
+            return None
+        return out
+
+
+class TileScheduler:
+    """PrefillRoutedTileScheduler (PrefillRoutedTileScheduler.swift:98-156)."""
+
+    def __init__(self, config: TileSchedulerConfig | None = None):
+        self.config = config or TileSchedulerConfig()
+
+    def decide(self, has_pending_tile: bool, pending_assigned_slots, avoiding_slot_plan_available: bool, pending_depth=None):
+        """The decision code; for PREFETCH_NEXT the slots to avoid are pending_assigned_slots as given."""
+        return capi.load().shrike_tile_scheduler_decide(C.byref(self.config.c), int(has_pending_tile),
+                                                        -1 if pending_depth is None else pending_depth,
+                                                        len(pending_assigned_slots), int(avoiding_slot_plan_available))
+
+    def plans_lookahead(self, index: int, tile_count: int) -> bool:
+        return bool(capi.load().shrike_tile_scheduler_plans_lookahead(C.byref(self.config.c), index, tile_count))
+
+    def should_begin_lookahead(self, index: int, tile_count: int, avoiding_slot_plan_available: bool) -> bool:
+        return bool(capi.load().shrike_tile_scheduler_should_begin_lookahead(C.byref(self.config.c), index, tile_count,
+                                                                             int(avoiding_slot_plan_available)))
+
+    def batch_action(self, open_batch_tiles: int, open_batch_slots, next_tile_plan_available: bool, is_last_tile: bool):
+        out = capi.TileBatchAction()
+        capi.load().shrike_tile_scheduler_batch_action(C.byref(self.config.c), open_batch_tiles, len(open_batch_slots),
+                                                       int(next_tile_plan_available), int(is_last_tile), C.byref(out))
+        return bool(out.commit_before_append), out.commit_after_append
+
+
+class TileSequencer:
+    """PrefillRoutedTileSequencer.run over a Python driver object with the protocol's members
+    (PrefillRoutedTileSequencer.swift:3-24): properties open_batch_tiles, open_batch_slots, pending_depth,
+    pending_assigned_slots; methods plan(tile, avoiding_in_flight) -> bool, begin, abandon_plan, encode,
+    commit_open_batch, drain_oldest_batch, abandon_begun_fetches. An exception raised by the driver ends the
+    run, reaches abandon_begun_fetches first and is raised again from run()."""
+
+    def __init__(self, scheduler: TileScheduler):
+        self.scheduler = scheduler
+
+    def run(self, tile_count: int, driver) -> None:
+        raised = []
+
+        def guarded(fn):
+            def call(_ctx, *args):
+                try:
+                    fn(*args)
+                    return 0
+                except BaseException as exc:  # noqa: BLE001 - carried across the C frame
+                    raised.append(exc)
+                    return errno.ECANCELED
+            return call
+
+        def plan(_ctx, tile, avoiding, available):
+            try:
+                available[0] = int(bool(driver.plan(tile, None if avoiding < 0 else avoiding)))
+                return 0
+            except BaseException as exc:  # noqa: BLE001
+                raised.append(exc)
+                return errno.ECANCELED
+
+        T = capi.TileDriver
+        fields = dict(T._fields_)
+        d = T(None,
+              fields["open_batch_tiles"](lambda _c: driver.open_batch_tiles),
+              fields["open_batch_slot_count"](lambda _c: len(driver.open_batch_slots)),
+              fields["pending_depth"](lambda _c: driver.pending_depth),
+              fields["pending_assigned_slot_count"](lambda _c: len(driver.pending_assigned_slots)),
+              fields["plan"](plan),
+              fields["begin"](guarded(driver.begin)),
+              fields["abandon_plan"](guarded(driver.abandon_plan)),
+              fields["encode"](guarded(driver.encode)),
+              fields["commit_open_batch"](lambda _c: driver.commit_open_batch()),
+              fields["drain_oldest_batch"](guarded(driver.drain_oldest_batch)),
+              fields["abandon_begun_fetches"](lambda _c: driver.abandon_begun_fetches()))
+        rc = capi.load().shrike_tile_sequencer_run(C.byref(self.scheduler.config.c), tile_count, C.byref(d))
+        if raised:
+            raise raised[0]
+        if rc:
+            raise ShrikeError(f"tile sequencer failed with {rc}: {capi.last_error()}")
+
+
+class ChunkExpertProtection:
+    """PrefillChunkExpertProtection (RealForwardRunner.swift:63-93)."""
+
+    def __init__(self, routed_experts, experts_per_layer: int):
+        self._r = (C.c_uint8 * experts_per_layer)()
+        ids = (C.c_int32 * len(routed_experts))(*routed_experts)
+        capi.load().shrike_chunk_protection_init(ids, len(routed_experts), self._r, experts_per_layer)
+
+    @property
+    def remaining(self):
+        return [bool(v) for v in self._r]
+
+    def planning(self, tile_experts) -> None:
+        ids = (C.c_int32 * len(tile_experts))(*tile_experts)
+        capi.load().shrike_chunk_protection_planning(ids, len(tile_experts), self._r, len(self._r))
+
+
+class TileLifetimeError(ShrikeError):
+    """PrefillStreamedTileLifetimeError (PrefillGroupedRoutedMoE.swift:376-386)."""
+
+    def __init__(self, code, conflicting_tile, message):
+        super().__init__(message)
+        self.code, self.conflicting_tile = code, conflicting_tile
+
+
+class TileSlotLifetime:
+    """PrefillStreamedTileSlotLifetime (PrefillGroupedRoutedMoE.swift:388-424)."""
+
+    def __init__(self):
+        self._h = capi.load().shrike_tile_lifetime_create()
+
+    def __del__(self):
+        try:
+            if self._h:
+                capi.load().shrike_tile_lifetime_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    def begin(self, tile_index: int, planned_slots) -> None:
+        slots = (C.c_int32 * len(planned_slots))(*planned_slots)
+        other = C.c_int(-1)
+        rc = capi.load().shrike_tile_lifetime_begin(self._h, tile_index, slots, len(planned_slots), C.byref(other))
+        if rc:
+            raise TileLifetimeError(rc, other.value, capi.last_error())
+
+    def complete(self, tile_index: int) -> None:
+        rc = capi.load().shrike_tile_lifetime_complete(self._h, tile_index)
+        if rc:
+            raise TileLifetimeError(rc, -1, capi.last_error())
