@@ -15,6 +15,8 @@
 
 #include "../../include/shrike_host.h"
 
+#include <type_traits>
+
 namespace shrike {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -26,7 +28,7 @@ constexpr uint32_t kStagePieces = kChunkK / 8;     // 16-byte pieces of one stag
 constexpr uint32_t kStageRows = 256 / kStagePieces; // rows one pass of the workgroup stages
 constexpr uint32_t kStagePasses = kRowTile / kStageRows;
 constexpr uint32_t kLdsRow = kChunkK + 8;         // halves per staged row; the pad spreads the banks
-constexpr uint32_t kMaxMT = kRowTile / 32;        // 32-row MFMA tiles per row tile
+static_assert(kRowTile == 64, "a row tile is one or two 32-row MFMA tiles");
 constexpr float kTwo24 = 16777216.0f;
 
 struct FfnArgs {
@@ -107,28 +109,16 @@ __device__ __forceinline__ half8 b_step(const BRegs<BITS> &r, int s) {
 // MODE 0: gate and up rows n0..n0+31 of one expert against the gathered token rows, GLU,
 // fp16 activations out. MODE 1: down rows n0..n0+63 against the activations, fp16 partials
 // scattered to (token, rank).
-template <int BITS, int MODE, bool DENSE>
-__global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
-    __shared__ __align__(16) uint16_t s_a[2][kRowTile][kLdsRow];
-    const uint32_t tile_index = blockIdx.x;
-    shrike_row_tile tile;
-    if (DENSE) {
-        if (tile_index * kRowTile >= a.dense_rows) return;
-        tile.cell = 0;
-        tile.pair_start = tile_index * kRowTile;
-        tile.rows = min(kRowTile, a.dense_rows - tile.pair_start);
-        tile.expert = 0;
-    } else {
-        if (tile_index >= *a.tile_count) return;
-        tile = a.tiles[tile_index];
-        if (tile.cell == kSentinel || tile.rows == 0) return;
-    }
-
+// One row tile against one block of weight rows. MT = the tile's 32-row MFMA tiles, a template
+// parameter so that the main loop is straight-line code: the compiler is then free to put one
+// chain's matrix instructions beside another chain's vector work.
+template <int BITS, int MODE, bool DENSE, uint32_t MT>
+__device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile &tile, uint32_t tile_index,
+                                         uint16_t (&s_a)[2][kRowTile][kLdsRow]) {
     const uint32_t K = MODE == 0 ? a.d : a.f, N = MODE == 0 ? a.f : a.d;
     const uint32_t G = K / kGroup;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t col = lane & 31u, kb = lane >> 5;
-    const uint32_t mt_count = (tile.rows + 31u) / 32u;
     const uint32_t n0 = (blockIdx.y * 4u + wave) * (MODE == 0 ? 32u : 64u);
     const bool active = n0 < N;
 
@@ -150,12 +140,12 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
         const uint32_t k = chunk * kChunkK + piece * 8u;
 #pragma unroll
         for (uint32_t i = 0; i < kStagePasses; ++i)
-            if (i * kStageRows < mt_count * 32u && k < K) stage[i] = *reinterpret_cast<const uint4 *>(src_row[i] + k);
+            if (i * kStageRows < MT * 32u && k < K) stage[i] = *reinterpret_cast<const uint4 *>(src_row[i] + k);
     };
     auto commit = [&](uint32_t buf) {
 #pragma unroll
         for (uint32_t i = 0; i < kStagePasses; ++i) {
-            if (i * kStageRows >= mt_count * 32u) continue;
+            if (i * kStageRows >= MT * 32u) continue;
             uint4 v = stage[i];
             if (BITS == 4) {  // (0,1,2,3,4,5,6,7) -> (0,4,1,5,2,6,3,7), to meet codes4
                 uint4 p;
@@ -203,20 +193,20 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
         }
     }
 
-    f32x16 total[2][kMaxMT];
+    f32x16 total[2][MT];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (uint32_t mt = 0; mt < kMaxMT; ++mt)
+        for (uint32_t mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) total[nt][mt][i] = 0.0f;
 
     // the rows' group sums for the bias term: their addresses hang on the pair records, so they are
     // worked out here, far ahead of their use
     const uint32_t *sums = MODE == 0 ? a.hidden_sums : a.act_sums;
-    const uint32_t *sum_row[kMaxMT];
+    const uint32_t *sum_row[MT];
 #pragma unroll
-    for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+    for (uint32_t mt = 0; mt < MT; ++mt) {
         const uint32_t r = min(mt * 32u + col, tile.rows - 1u);
         const uint32_t token = (MODE != 0) ? 0u : DENSE ? tile.pair_start + r : a.pairs[tile.pair_start + r].token;
         sum_row[mt] = MODE == 0 ? sums + size_t(token) * G : sums + (size_t(tile_index) * kRowTile + r) * G;
@@ -225,72 +215,84 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     // A row's scales for the four groups of a staged chunk are one aligned 8-byte run when G is a
     // multiple of 4: they are then fetched a chunk ahead with one load instead of four two-byte ones
     // (every such load costs a cache-line look-up per lane, as each lane reads a row of its own).
+    // Decided from the tensors' start (the same for every lane, a row's scales being G * 2 bytes), so
+    // that the choice is uniform over the workgroup and each variant of the loop is straight-line code.
     static_assert(kGroupsPerChunk == 4, "a chunk's scales are read as four 16-bit values");
-    const bool wide_scales = (G & 3u) == 0u && ((reinterpret_cast<uintptr_t>(bs[0]) | reinterpret_cast<uintptr_t>(bs[1])) & 7u) == 0u;
-    const uint16_t *bs_each[2] = {wide_scales ? nullptr : bs[0], wide_scales ? nullptr : bs[1]};
+    const uint32_t scale_misalign = uint32_t((reinterpret_cast<uintptr_t>(bs[0]) | reinterpret_cast<uintptr_t>(bs[1])) & 7u);
+    const bool wide_scales = (G & 3u) == 0u && __builtin_amdgcn_readfirstlane(int(scale_misalign)) == 0;
     uint2 scales_cur[2] = {make_uint2(0u, 0u), make_uint2(0u, 0u)}, scales_nxt[2] = {make_uint2(0u, 0u), make_uint2(0u, 0u)};
     BRegs<BITS> cur[2], nxt[2];
-    if (active) {
-        load_b<BITS>(cur[0], bw[0], bs_each[0], 0, kb);
-        load_b<BITS>(cur[1], bw[1], bs_each[1], 0, kb);
-        if (wide_scales) {
-            scales_cur[0] = *reinterpret_cast<const uint2 *>(bs[0]);
-            scales_cur[1] = *reinterpret_cast<const uint2 *>(bs[1]);
-        }
-    }
     const uint32_t chunks = (K + kChunkK - 1u) / kChunkK;
-    fetch(0);
-    commit(0);
-    __syncthreads();
-    for (uint32_t c = 0; c < chunks; ++c) {
-        const uint32_t buf = c & 1u;
-        if (c + 1u < chunks) fetch(c + 1u);
-        const uint32_t groups_here = min(kGroupsPerChunk, G - kGroupsPerChunk * c);
-        if (active) {
-            if (wide_scales && c + 1u < chunks) {
-                scales_nxt[0] = reinterpret_cast<const uint2 *>(bs[0])[c + 1u];
-                scales_nxt[1] = reinterpret_cast<const uint2 *>(bs[1])[c + 1u];
+
+    // One group of 64 k: the next group's codes are put in flight, this group's are unpacked and
+    // multiplied, and the products are scaled into the totals.
+    auto group_step = [&](uint32_t c, uint32_t buf, uint32_t gi, auto wide_tag) {
+        constexpr bool WIDE = decltype(wide_tag)::value;
+        const uint32_t gn = min(kGroupsPerChunk * c + gi + 1u, G - 1u);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) load_b<BITS>(nxt[nt], bw[nt], WIDE ? nullptr : bs[nt], gn, kb);
+        half8 af[MT][4];
+#pragma unroll
+        for (uint32_t mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                af[mt][s] = *reinterpret_cast<const half8 *>(&s_a[buf][mt * 32u + col][gi * 64u + kb * 32u + s * 8u]);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            half8 bf[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) bf[s] = b_step<BITS>(cur[nt], s);
+            const uint32_t pair = gi < 2u ? scales_cur[nt].x : scales_cur[nt].y;
+            const uint16_t scale_bits = WIDE ? uint16_t(pair >> (16u * (gi & 1u))) : cur[nt].scale;
+            const float sc = meta_f32(scale_bits, a.meta) * kTwo24;
+#pragma unroll
+            for (uint32_t mt = 0; mt < MT; ++mt) {
+                f32x16 p = {0};
+#pragma unroll
+                for (int s = 0; s < 4; ++s) p = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt][s], bf[s], p, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) total[nt][mt][i] = fmaf(sc, p[i], total[nt][mt][i]);
             }
-            for (uint32_t gi = 0; gi < groups_here; ++gi) {
-                const uint32_t g = kGroupsPerChunk * c + gi;
-                const uint32_t gn = min(g + 1u, G - 1u);
-                load_b<BITS>(nxt[0], bw[0], bs_each[0], gn, kb);
-                load_b<BITS>(nxt[1], bw[1], bs_each[1], gn, kb);
-                half8 af[kMaxMT][4];
-#pragma unroll
-                for (uint32_t mt = 0; mt < kMaxMT; ++mt)
-#pragma unroll
-                    for (int s = 0; s < 4; ++s)
-                        if (mt < mt_count)
-                            af[mt][s] = *reinterpret_cast<const half8 *>(&s_a[buf][mt * 32u + col][gi * 64u + kb * 32u + s * 8u]);
-#pragma unroll
-                for (int nt = 0; nt < 2; ++nt) {
-                    half8 bf[4];
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) bf[s] = b_step<BITS>(cur[nt], s);
-                    const uint32_t pair = gi < 2u ? scales_cur[nt].x : scales_cur[nt].y;
-                    const uint16_t scale_bits = wide_scales ? uint16_t(pair >> (16u * (gi & 1u))) : cur[nt].scale;
-                    const float sc = meta_f32(scale_bits, a.meta) * kTwo24;
-#pragma unroll
-                    for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
-                        if (mt < mt_count) {
-                            f32x16 p = {0};
-#pragma unroll
-                            for (int s = 0; s < 4; ++s) p = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt][s], bf[s], p, 0, 0, 0);
-#pragma unroll
-                            for (int i = 0; i < 16; ++i) total[nt][mt][i] = fmaf(sc, p[i], total[nt][mt][i]);
-                        }
-                    }
-                }
-                cur[0] = nxt[0];
-                cur[1] = nxt[1];
-            }
-            scales_cur[0] = scales_nxt[0];
-            scales_cur[1] = scales_nxt[1];
         }
-        if (c + 1u < chunks) commit(buf ^ 1u);
+        cur[0] = nxt[0];
+        cur[1] = nxt[1];
+    };
+    auto main_loop = [&](auto wide_tag) {
+        constexpr bool WIDE = decltype(wide_tag)::value;
+        if (active) {
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                load_b<BITS>(cur[nt], bw[nt], WIDE ? nullptr : bs[nt], 0, kb);
+                if (WIDE) scales_cur[nt] = *reinterpret_cast<const uint2 *>(bs[nt]);
+            }
+        }
+        fetch(0);
+        commit(0);
         __syncthreads();
-    }
+        for (uint32_t c = 0; c < chunks; ++c) {
+            const uint32_t buf = c & 1u;
+            if (c + 1u < chunks) fetch(c + 1u);
+            if (active) {
+                if (WIDE) {  // G is a multiple of 4: every chunk is whole and its four groups are one block of code
+                    if (c + 1u < chunks) {
+                        scales_nxt[0] = reinterpret_cast<const uint2 *>(bs[0])[c + 1u];
+                        scales_nxt[1] = reinterpret_cast<const uint2 *>(bs[1])[c + 1u];
+                    }
+#pragma unroll
+                    for (uint32_t gi = 0; gi < kGroupsPerChunk; ++gi) group_step(c, buf, gi, wide_tag);
+                    scales_cur[0] = scales_nxt[0];
+                    scales_cur[1] = scales_nxt[1];
+                } else {
+                    const uint32_t groups_here = min(kGroupsPerChunk, G - kGroupsPerChunk * c);
+                    for (uint32_t gi = 0; gi < groups_here; ++gi) group_step(c, buf, gi, wide_tag);
+                }
+            }
+            if (c + 1u < chunks) commit(buf ^ 1u);
+            __syncthreads();
+        }
+    };
+    if (wide_scales) main_loop(std::true_type{});
+    else main_loop(std::false_type{});
     if (!active) return;
 
     // ---- bias term: (group sums of the rows) x (group biases), sixteen k' = eight groups an MFMA.
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
         // a lane's four groups are one aligned 8- or 16-byte run when G is a multiple of 4 and the bias rows start aligned
         const bool wide = (G & 3u) == 0u && ((reinterpret_cast<uintptr_t>(bb[0]) | reinterpret_cast<uintptr_t>(bb[1])) & 7u) == 0u;
         for (uint32_t gbase = 0; gbase < G; gbase += 32u) {
-            Frag bfr[4][2], afr[4][kMaxMT];
+            Frag bfr[4][2], afr[4][MT];
 #pragma unroll
             for (uint32_t step = 0; step < 4; ++step) {
                 const uint32_t gl = gbase + 8u * step + 4u * kb;  // this lane's four groups
@@ -312,8 +314,8 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
                         bfr[step][nt].u[2] = b4.y & 0xffffu; bfr[step][nt].u[3] = b4.y >> 16;
                     }
 #pragma unroll
-                    for (uint32_t mt = 0; mt < kMaxMT; ++mt)
-                        afr[step][mt].v = (on && mt < mt_count) ? *reinterpret_cast<const uint4 *>(sum_row[mt] + gl) : zero4();
+                    for (uint32_t mt = 0; mt < MT; ++mt)
+                        afr[step][mt].v = on ? *reinterpret_cast<const uint4 *>(sum_row[mt] + gl) : zero4();
                 } else {
 #pragma unroll
                     for (int jj = 0; jj < 4; ++jj) {
@@ -321,7 +323,7 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
 #pragma unroll
                         for (int nt = 0; nt < 2; ++nt) bfr[step][nt].u[jj] = on ? bb[nt][gl + jj] : 0u;
 #pragma unroll
-                        for (uint32_t mt = 0; mt < kMaxMT; ++mt) afr[step][mt].u[jj] = (on && mt < mt_count) ? sum_row[mt][gl + jj] : 0u;
+                        for (uint32_t mt = 0; mt < MT; ++mt) afr[step][mt].u[jj] = on ? sum_row[mt][gl + jj] : 0u;
                     }
                 }
             }
@@ -337,14 +339,12 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
                         bfr[step][nt].u[jj] = uint32_t(bits) * 0x00010001u;
                     }
 #pragma unroll
-                    for (uint32_t mt = 0; mt < kMaxMT; ++mt)
-                        if (mt < mt_count)
+                    for (uint32_t mt = 0; mt < MT; ++mt)
                             total[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[step][mt].h, bfr[step][nt].h, total[nt][mt], 0, 0, 0);
                 }
             }
         }
     }
-
     // ---- epilogue: lane holds (m = 32 mt + 8 (i / 4) + 4 kb + i % 4, n = n0 + col)
     const uint32_t n = n0 + col;
     if (MODE == 0) {
@@ -354,11 +354,11 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
             uab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.up_ab_off)[n]);
         }
 #pragma unroll
-        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+        for (uint32_t mt = 0; mt < MT; ++mt) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
-                if (mt < mt_count && m < tile.rows) {
+                if (m < tile.rows) {
                     float g = total[0][mt][i] + gab, u = total[1][mt][i] + uab;
                     if (DENSE && a.round_gate_up) {
                         g = f16_to_f32(f32_to_f16(g));
@@ -378,11 +378,11 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
             dab[1] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n + 32u]);
         }
 #pragma unroll
-        for (uint32_t mt = 0; mt < kMaxMT; ++mt) {
+        for (uint32_t mt = 0; mt < MT; ++mt) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
-                if (mt < mt_count && m < tile.rows) {
+                if (m < tile.rows) {
                     uint16_t *dst;
                     if (DENSE) {
                         dst = a.partials + size_t(tile.pair_start + m) * a.d + n;
@@ -401,6 +401,27 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
             }
         }
     }
+}
+
+template <int BITS, int MODE, bool DENSE>
+__global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
+    __shared__ __align__(16) uint16_t s_a[2][kRowTile][kLdsRow];
+    const uint32_t tile_index = blockIdx.x;
+    shrike_row_tile tile;
+    if (DENSE) {
+        if (tile_index * kRowTile >= a.dense_rows) return;
+        tile.cell = 0;
+        tile.pair_start = tile_index * kRowTile;
+        tile.rows = min(kRowTile, a.dense_rows - tile.pair_start);
+        tile.expert = 0;
+    } else {
+        if (tile_index >= *a.tile_count) return;
+        tile = a.tiles[tile_index];
+        if (tile.cell == kSentinel || tile.rows == 0) return;
+    }
+
+    if (tile.rows > 32u) ffn_tile<BITS, MODE, DENSE, 2>(a, tile, tile_index, s_a);
+    else ffn_tile<BITS, MODE, DENSE, 1>(a, tile, tile_index, s_a);
 }
 
 int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uint32_t n, uint32_t *out,
@@ -435,7 +456,6 @@ static Workspace workspace_layout(uint32_t query_count, uint32_t max_tiles, uint
 using namespace shrike;
 
 extern "C" {
-
 size_t shrike_hip_prefill_ffn_workspace_bytes(uint32_t query_count, uint32_t max_row_tiles, uint32_t d, uint32_t f) {
     return workspace_layout(query_count, max_row_tiles, d, f).total;
 }
