@@ -13,10 +13,15 @@
 //   RuntimeConfiguration (budget -> slots)            shrike::RuntimeConfiguration
 //   ParallelExpertReader (Infrastructure/Streaming)   shrike::ParallelExpertReader
 //   PackedExpertsLayout(Reader) (Infrastructure/ModelIO) shrike::PackedExpertsLayout
+//   PrefillRoutedTileScheduler / ...Sequencer / ...Driver shrike::PrefillRoutedTileScheduler, ...Sequencer, ...Driver
+//   ExpertLoadOperation, ExpertPrefetchRing           shrike::ExpertLoadOperation, shrike::ExpertPrefetchRing
 #pragma once
 
 #include <cerrno>
 #include <cstdint>
+#include <exception>
+#include <functional>
+#include <map>
 #include <optional>
 #include <stdexcept>
 #include <string>
@@ -462,6 +467,214 @@ struct PrefillMoE {
     static void encodeResidualAdd(Stream s, void *hidden, const void *delta, uint64_t count) {
         check(shrike_hip_residual_add_f16(s, hidden, delta, count));
     }
+};
+
+// PrefillRoutedTileSchedulerConfig / PrefillRoutedTileScheduler (PrefillRoutedTileScheduler.swift:46-155)
+struct PrefillRoutedTileSchedulerConfig : shrike_tile_scheduler_config {
+    explicit PrefillRoutedTileSchedulerConfig(int maxPendingDepth = 1, int tileExperts = 8, int tilesPerCommandBuffer = 1,
+                                              int fetchLookahead = 0) {
+        shrike_tile_scheduler_config_make(maxPendingDepth, tileExperts, tilesPerCommandBuffer, fetchLookahead, this);
+    }
+    bool fitsSlotBudget(int slotCount, int reservedHits = 0) const {
+        return shrike_tile_scheduler_fits_slot_budget(this, slotCount, reservedHits) != 0;
+    }
+    std::optional<PrefillRoutedTileSchedulerConfig> fitting(int slotCount, int reservedHits = 0) const {
+        PrefillRoutedTileSchedulerConfig out;
+        if (!shrike_tile_scheduler_fitting(this, slotCount, reservedHits, &out)) return std::nullopt;
+        return out;
+    }
+};
+
+struct PrefillRoutedTileScheduler {
+    PrefillRoutedTileSchedulerConfig config;
+    // SHRIKE_TILE_ISSUE_WITHOUT_PENDING ... SHRIKE_TILE_DRAIN_MAX_DEPTH; pendingDepth < 0 = the input's default
+    int decide(bool hasPendingTile, size_t pendingAssignedSlotCount, bool avoidingSlotPlanAvailable, int pendingDepth = -1) const {
+        return shrike_tile_scheduler_decide(&config, hasPendingTile, pendingDepth, pendingAssignedSlotCount, avoidingSlotPlanAvailable);
+    }
+    shrike_tile_batch_action batchAction(int openBatchTiles, size_t openBatchSlotCount, bool nextTilePlanAvailable, bool isLastTile) const {
+        shrike_tile_batch_action out;
+        shrike_tile_scheduler_batch_action(&config, openBatchTiles, openBatchSlotCount, nextTilePlanAvailable, isLastTile, &out);
+        return out;
+    }
+    bool shouldBeginLookahead(int index, int tileCount, bool avoidingSlotPlanAvailable) const {
+        return shrike_tile_scheduler_should_begin_lookahead(&config, index, tileCount, avoidingSlotPlanAvailable) != 0;
+    }
+};
+
+// PrefillRoutedTileDriver (PrefillRoutedTileSequencer.swift:3-24): what the sequencer drives. Methods may throw.
+struct PrefillRoutedTileDriver {
+    virtual ~PrefillRoutedTileDriver() = default;
+    virtual int openBatchTiles() = 0;
+    virtual size_t openBatchSlotCount() = 0;
+    virtual int pendingDepth() = 0;
+    virtual size_t pendingAssignedSlotCount() = 0;
+    virtual bool plan(int tile, std::optional<int> avoidingInFlight) = 0;
+    virtual void begin(int tile) = 0;
+    virtual void abandonPlan(int tile) = 0;
+    virtual void encode(int tile) = 0;
+    virtual void commitOpenBatch() = 0;
+    virtual void drainOldestBatch() = 0;
+    virtual void abandonBegunFetches() = 0;
+};
+
+// PrefillRoutedTileSequencer (PrefillRoutedTileSequencer.swift:26-104); a driver's exception crosses the C
+// boundary as a code and is rethrown here, after abandonBegunFetches has run.
+struct PrefillRoutedTileSequencer {
+    PrefillRoutedTileScheduler scheduler;
+    void run(int tileCount, PrefillRoutedTileDriver &driver) const {
+        Box box{&driver, nullptr};
+        shrike_tile_driver d = {};
+        d.context = &box;
+        d.open_batch_tiles = [](void *c) { return static_cast<Box *>(c)->driver->openBatchTiles(); };
+        d.open_batch_slot_count = [](void *c) { return static_cast<Box *>(c)->driver->openBatchSlotCount(); };
+        d.pending_depth = [](void *c) { return static_cast<Box *>(c)->driver->pendingDepth(); };
+        d.pending_assigned_slot_count = [](void *c) { return static_cast<Box *>(c)->driver->pendingAssignedSlotCount(); };
+        d.plan = [](void *c, int tile, int avoiding, int *available) {
+            return call(c, [&](PrefillRoutedTileDriver &drv) {
+                *available = drv.plan(tile, avoiding < 0 ? std::nullopt : std::optional<int>(avoiding)) ? 1 : 0;
+            });
+        };
+        d.begin = [](void *c, int tile) { return call(c, [&](PrefillRoutedTileDriver &drv) { drv.begin(tile); }); };
+        d.abandon_plan = [](void *c, int tile) { return call(c, [&](PrefillRoutedTileDriver &drv) { drv.abandonPlan(tile); }); };
+        d.encode = [](void *c, int tile) { return call(c, [&](PrefillRoutedTileDriver &drv) { drv.encode(tile); }); };
+        d.commit_open_batch = [](void *c) { static_cast<Box *>(c)->driver->commitOpenBatch(); };
+        d.drain_oldest_batch = [](void *c) { return call(c, [&](PrefillRoutedTileDriver &drv) { drv.drainOldestBatch(); }); };
+        d.abandon_begun_fetches = [](void *c) { static_cast<Box *>(c)->driver->abandonBegunFetches(); };
+        const int rc = shrike_tile_sequencer_run(&scheduler.config, tileCount, &d);
+        if (box.failure) std::rethrow_exception(box.failure);
+        check(rc);
+    }
+
+private:
+    struct Box {
+        PrefillRoutedTileDriver *driver;
+        std::exception_ptr failure;
+    };
+    template <class Body>
+    static int call(void *ctx, Body &&body) {
+        Box *b = static_cast<Box *>(ctx);
+        try {
+            body(*b->driver);
+            return 0;
+        } catch (...) {
+            b->failure = std::current_exception();
+            return EIO;
+        }
+    }
+};
+
+// ExpertLoadOperation (Infrastructure/Streaming/ExpertLoadOperation.swift:15-153): a shared handle
+class ExpertLoadOperation {
+public:
+    ExpertLoadOperation() : h_(shrike_load_operation_create()) {
+        if (!h_) throw Error(ENOMEM, "load operation");
+    }
+    ExpertLoadOperation(const ExpertLoadOperation &o) : h_(o.h_) { shrike_load_operation_retain(h_); }
+    ExpertLoadOperation &operator=(const ExpertLoadOperation &o) {
+        shrike_load_operation_retain(o.h_);
+        shrike_load_operation_release(h_);
+        h_ = o.h_;
+        return *this;
+    }
+    ~ExpertLoadOperation() { shrike_load_operation_release(h_); }
+    int state() const { return shrike_load_operation_state(h_); }
+    void markInFlight() { check(shrike_load_operation_mark_in_flight(h_)); }
+    void finish(int failure = 0) { check(shrike_load_operation_finish(h_, failure)); }
+    void wait() { check(shrike_load_operation_wait(h_)); }
+    bool wait(uint64_t untilNanos) { return shrike_load_operation_wait_until(h_, untilNanos) != 0; }
+    uint64_t completedNanos() const { return shrike_load_operation_completed_nanos(h_); }
+    shrike_load_operation *handle() const { return h_; }
+
+private:
+    shrike_load_operation *h_;
+};
+
+struct PrefetchClaimRefused {  // PreadExpertStreamer.swift:46-49
+    int expert, cell;
+};
+
+// ExpertPrefetchRing (Runtime/Inference/ExpertPrefetchRing.swift:42-352)
+class ExpertPrefetchRing {
+public:
+    using Drop = std::function<void(int layer, int expert, int cell)>;
+    using Issue = std::function<ExpertLoadOperation(const std::vector<int> &experts, const std::vector<int> &cells)>;
+    ExpertPrefetchRing(const std::vector<int> &cells, Drop drop) : drop_(std::move(drop)) {
+        int err = 0;
+        h_ = shrike_prefetch_ring_create(cells.data(), cells.size(),
+                                         [](void *c, int layer, int expert, int cell) { static_cast<ExpertPrefetchRing *>(c)->drop_(layer, expert, cell); },
+                                         this, &err);
+        if (!h_) throw Error(err, "invalid prefetch ring geometry");
+    }
+    ~ExpertPrefetchRing() { shrike_prefetch_ring_destroy(h_); }
+    ExpertPrefetchRing(const ExpertPrefetchRing &) = delete;
+    ExpertPrefetchRing &operator=(const ExpertPrefetchRing &) = delete;
+    void begin(int layer, const std::vector<int> &experts, const std::vector<int> &resident, const Issue &issue, bool deferred = false) {
+        struct Box {
+            const Issue *issue;
+            std::exception_ptr failure;
+            shrike_load_operation *handed;  // one reference that outlives the issue's own until the ring holds its
+        } box{&issue, nullptr, nullptr};
+        const int rc = shrike_prefetch_ring_begin(
+            h_, layer, experts.data(), experts.size(), resident.data(), resident.size(), deferred,
+            [](void *c, const int *e, const int *cells, size_t n, shrike_load_operation **out) -> int {
+                Box *b = static_cast<Box *>(c);
+                try {
+                    ExpertLoadOperation op = (*b->issue)(std::vector<int>(e, e + n), std::vector<int>(cells, cells + n));
+                    shrike_load_operation_retain(op.handle());
+                    b->handed = *out = op.handle();
+                    return 0;
+                } catch (const PrefetchClaimRefused &) {
+                    return SHRIKE_PREFETCH_CLAIM_REFUSED;
+                } catch (...) {
+                    b->failure = std::current_exception();
+                    return EIO;
+                }
+            },
+            &box);
+        shrike_load_operation_release(box.handed);
+        if (box.failure) std::rethrow_exception(box.failure);
+        check(rc);
+    }
+    std::map<int, int> readyCells(int layer, const std::vector<int> &experts, uint64_t joinNanos = 0) {
+        std::vector<int> e(experts.size() + 1), c(experts.size() + 1);
+        const size_t n = shrike_prefetch_ring_ready_cells(h_, layer, experts.data(), experts.size(), joinNanos, e.data(), c.data());
+        return zip(e, c, n);
+    }
+    void consume(int layer, const std::vector<int> &experts, const std::map<int, int> &freedCells) {
+        std::vector<int> fe, fc;
+        for (auto &kv : freedCells) {
+            fe.push_back(kv.first);
+            fc.push_back(kv.second);
+        }
+        shrike_prefetch_ring_consume(h_, layer, experts.data(), experts.size(), fe.data(), fc.data(), fe.size());
+    }
+    std::map<int, int> claimDemand(int layer, const std::vector<int> &experts) {
+        std::vector<int> e(experts.size() + 1), c(experts.size() + 1);
+        const size_t n = shrike_prefetch_ring_claim_demand(h_, layer, experts.data(), experts.size(), e.data(), c.data());
+        return zip(e, c, n);
+    }
+    void attachDemand(int layer, const std::vector<int> &experts, const ExpertLoadOperation &operation) {
+        shrike_prefetch_ring_attach_demand(h_, layer, experts.data(), experts.size(), operation.handle());
+    }
+    void unlease(int layer, const std::vector<int> &experts) { shrike_prefetch_ring_unlease(h_, layer, experts.data(), experts.size()); }
+    void noteDemandSubmission() { shrike_prefetch_ring_note_demand_submission(h_); }
+    bool noteHookFailure() { return shrike_prefetch_ring_note_hook_failure(h_) != 0; }
+    shrike_prefetch_statistics statistics() const {
+        shrike_prefetch_statistics st;
+        shrike_prefetch_ring_statistics(h_, &st);
+        return st;
+    }
+    int inFlightCount() const { return shrike_prefetch_ring_in_flight_count(h_); }
+    int leasedCount() const { return shrike_prefetch_ring_leased_count(h_); }
+
+private:
+    static std::map<int, int> zip(const std::vector<int> &k, const std::vector<int> &v, size_t n) {
+        std::map<int, int> out;
+        for (size_t i = 0; i < n; ++i) out[k[i]] = v[i];
+        return out;
+    }
+    shrike_prefetch_ring *h_;
+    Drop drop_;
 };
 
 }  // namespace shrike

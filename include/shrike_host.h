@@ -398,6 +398,73 @@ int shrike_tile_lifetime_begin(shrike_tile_lifetime *lifetime, int tile_index, c
                                int *conflicting_tile);
 int shrike_tile_lifetime_complete(shrike_tile_lifetime *lifetime, int tile_index);
 
+/* ------------------------------------------------------- load operations and the predictive prefetch ring */
+
+/* ExpertLoadOperation (sources/Shrike/Infrastructure/Streaming/ExpertLoadOperation.swift:3-153): one storage
+ * batch whose submission is independent from its completion. Reference counted: create returns one
+ * reference, the ring retains what is attached to its slots. finish(failure = 0) completes, any other
+ * value fails the operation with that code; mark_in_flight and finish return EALREADY where the
+ * reference traps a second start or a second completion. wait returns the failure code (0 = completed);
+ * wait_until returns 1 once the operation is terminal, 0 at the deadline (shrike_monotonic_nanos clock). */
+typedef struct shrike_load_operation shrike_load_operation;
+enum { SHRIKE_LOAD_SUBMITTED = 0, SHRIKE_LOAD_IN_FLIGHT = 1, SHRIKE_LOAD_COMPLETED = 2, SHRIKE_LOAD_FAILED = 3 };
+uint64_t shrike_monotonic_nanos(void);
+shrike_load_operation *shrike_load_operation_create(void);
+void shrike_load_operation_retain(shrike_load_operation *operation);
+void shrike_load_operation_release(shrike_load_operation *operation);
+int shrike_load_operation_state(shrike_load_operation *operation);
+int shrike_load_operation_mark_in_flight(shrike_load_operation *operation);
+int shrike_load_operation_finish(shrike_load_operation *operation, int failure);
+int shrike_load_operation_wait(shrike_load_operation *operation);
+int shrike_load_operation_wait_until(shrike_load_operation *operation, uint64_t deadline_nanos);
+uint64_t shrike_load_operation_submitted_nanos(shrike_load_operation *operation);
+uint64_t shrike_load_operation_started_nanos(shrike_load_operation *operation);
+uint64_t shrike_load_operation_completed_nanos(shrike_load_operation *operation);
+
+/* ExpertPrefetchStatistics (sources/Shrike/Runtime/Inference/ExpertPrefetchRing.swift:14-29), same fields. */
+typedef struct {
+    uint64_t issued, adopted, reclaimed, deferred, overlapped, late, joined, refused, failed, hook_failures,
+        begin_nanos, leased_peak;
+} shrike_prefetch_statistics;
+
+/* ExpertPrefetchRing (ExpertPrefetchRing.swift:42-352). The ring owns `cells` of the expert pool (distinct,
+ * at least one). drop(context, layer, expert, cell) removes a landing from its layer's residency table
+ * and runs with the ring locked. issue(context, experts, cells, count, &operation) submits one read
+ * of `count` experts into `cells` and returns 0 with the batch's operation (the ring retains it; the
+ * caller keeps its own reference), SHRIKE_PREFETCH_CLAIM_REFUSED when the pool already holds one of the
+ * experts (PrefetchClaimRefused: counted refused, begin returns 0), or an error code, which begin
+ * returns after rolling the slots back. Results that the reference returns as dictionaries come back
+ * as parallel arrays (room for as many entries as experts were passed), in slot order for ready_cells
+ * and completion_nanos and in the experts' order for claim_demand. */
+#define SHRIKE_PREFETCH_IN_FLIGHT_BUDGET 1            /* ExpertPrefetchRing.inFlightBudget (:49) */
+#define SHRIKE_PREFETCH_ATTACH_SPIN_NANOS 5000000ull  /* ExpertPrefetchRing.attachSpinNanos (:48) */
+#define SHRIKE_PREFETCH_CLAIM_REFUSED (-2)
+typedef struct shrike_prefetch_ring shrike_prefetch_ring;
+typedef void (*shrike_prefetch_drop)(void *context, int layer, int expert, int cell);
+typedef int (*shrike_prefetch_issue)(void *context, const int *experts, const int *cells, size_t count,
+                                     shrike_load_operation **out_operation);
+shrike_prefetch_ring *shrike_prefetch_ring_create(const int *cells, size_t count, shrike_prefetch_drop drop, void *drop_context,
+                                                  int *out_errno);                                            /* init (:95-102) */
+void shrike_prefetch_ring_destroy(shrike_prefetch_ring *ring);
+int shrike_prefetch_ring_begin(shrike_prefetch_ring *ring, int layer, const int *experts, size_t expert_count, const int *resident,
+                               size_t resident_count, int deferred, shrike_prefetch_issue issue, void *issue_context); /* begin (:108-164) */
+size_t shrike_prefetch_ring_ready_cells(shrike_prefetch_ring *ring, int layer, const int *experts, size_t expert_count,
+                                        uint64_t join_nanos, int *out_experts, int *out_cells);               /* readyCells (:171-212) */
+void shrike_prefetch_ring_consume(shrike_prefetch_ring *ring, int layer, const int *experts, size_t expert_count,
+                                  const int *freed_experts, const int *freed_cells, size_t freed_count);      /* consume (:232-252) */
+size_t shrike_prefetch_ring_claim_demand(shrike_prefetch_ring *ring, int layer, const int *experts, size_t expert_count,
+                                         int *out_experts, int *out_cells);                                   /* claimDemand (:257-282) */
+void shrike_prefetch_ring_attach_demand(shrike_prefetch_ring *ring, int layer, const int *experts, size_t expert_count,
+                                        shrike_load_operation *operation);                                    /* attachDemand (:284-291) */
+size_t shrike_prefetch_ring_completion_nanos(shrike_prefetch_ring *ring, int layer, const int *experts, size_t expert_count,
+                                             int *out_experts, uint64_t *out_nanos);                          /* completionNanos (:293-304) */
+void shrike_prefetch_ring_unlease(shrike_prefetch_ring *ring, int layer, const int *experts, size_t expert_count); /* :306-313 */
+void shrike_prefetch_ring_note_demand_submission(shrike_prefetch_ring *ring);                                 /* :315-319 */
+int shrike_prefetch_ring_note_hook_failure(shrike_prefetch_ring *ring);        /* 1 on the first failure (:322-327) */
+void shrike_prefetch_ring_statistics(shrike_prefetch_ring *ring, shrike_prefetch_statistics *out);
+int shrike_prefetch_ring_in_flight_count(shrike_prefetch_ring *ring);
+int shrike_prefetch_ring_leased_count(shrike_prefetch_ring *ring);
+
 #ifdef __cplusplus
 }
 #endif

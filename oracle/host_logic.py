@@ -968,3 +968,256 @@ def tile_sequence(config, tile_count, driver):
     except BaseException:
         driver.abandon_begun_fetches()
         raise
+
+
+# ------------------------------------------------------------------ load operations and the prefetch ring
+# (sources/Shrike/Infrastructure/Streaming/ExpertLoadOperation.swift:15-153,
+#  sources/Shrike/Runtime/Inference/ExpertPrefetchRing.swift:42-352). Pinned by the reference's own
+# ExpertPrefetchRingTests vectors.
+
+import threading as _threading
+import time as _time
+
+SUBMITTED, IN_FLIGHT, COMPLETED, FAILED = "submitted", "inFlight", "completed", "failed"
+
+
+class LoadOperation:
+    def __init__(self):
+        self._cond = _threading.Condition()
+        self.state, self.failure = SUBMITTED, None
+        self.submitted_nanos, self.started_nanos, self.completed_nanos = _time.monotonic_ns(), 0, 0
+
+    def mark_in_flight(self):
+        with self._cond:
+            assert self.state == SUBMITTED, "expert load operation started more than once"
+            self.state, self.started_nanos = IN_FLIGHT, _time.monotonic_ns()
+
+    def finish(self, failure=None):
+        with self._cond:
+            assert self.state in (SUBMITTED, IN_FLIGHT), "expert load operation completed more than once"
+            self.completed_nanos = _time.monotonic_ns()
+            self.state, self.failure = (FAILED, failure) if failure else (COMPLETED, None)
+            self._cond.notify_all()
+
+    def wait(self):
+        with self._cond:
+            while self.state in (SUBMITTED, IN_FLIGHT):
+                self._cond.wait()
+            if self.failure:
+                raise RuntimeError(self.failure)
+
+    def wait_until(self, deadline_nanos):
+        with self._cond:
+            while self.state in (SUBMITTED, IN_FLIGHT):
+                now = _time.monotonic_ns()
+                if now >= deadline_nanos:
+                    return False
+                self._cond.wait((deadline_nanos - now) / 1e9)
+            return True
+
+
+class ClaimRefused(Exception):
+    pass
+
+
+class _RingSlot:
+    def __init__(self, cell):
+        self.cell, self.layer, self.expert, self.operation, self.leased, self.demand = cell, -1, -1, None, False, False
+
+    @property
+    def in_flight(self):  # :60-71
+        if self.expert < 0:
+            return False
+        return self.operation is None or self.operation.state in (SUBMITTED, IN_FLIGHT)
+
+
+class PrefetchRing:
+    ATTACH_SPIN_NANOS, IN_FLIGHT_BUDGET = 5_000_000, 1
+
+    def __init__(self, cells, drop):
+        if not cells or len(set(cells)) != len(cells):
+            raise ValueError("invalid prefetch ring geometry")
+        self.slots = [_RingSlot(c) for c in cells]
+        self.drop, self.lock = drop, _threading.Lock()
+        self.stats = dict(issued=0, adopted=0, reclaimed=0, deferred=0, overlapped=0, late=0, joined=0, refused=0,
+                          failed=0, hook_failures=0, begin_nanos=0, leased_peak=0)
+
+    @property
+    def in_flight_count(self):
+        with self.lock:
+            return sum(1 for s in self.slots if s.in_flight)
+
+    @property
+    def leased_count(self):
+        with self.lock:
+            return sum(1 for s in self.slots if s.leased)
+
+    def _reclaim(self, keeping):  # :333-351
+        for s in self.slots:
+            if s.leased or s.layer == keeping or s.operation is None:
+                continue
+            if s.operation.state == COMPLETED:
+                self.drop(s.layer, s.expert, s.cell)
+                self.stats["reclaimed"] += 1
+                s.layer, s.expert, s.operation = -1, -1, None
+            elif s.operation.state == FAILED:
+                self.stats["failed"] += 1
+                s.layer, s.expert, s.operation = -1, -1, None
+
+    def begin(self, layer, experts, resident=(), deferred=False, issue=None):  # :108-164
+        started = _time.monotonic_ns()
+        try:
+            self.lock.acquire()
+            self._reclaim(layer)
+            active = {s.expert for s in self.slots if s.layer == layer and s.expert >= 0}
+            wanted = []
+            for e in experts:
+                if e not in resident and e not in active and e not in wanted:
+                    wanted.append(e)
+            free = [i for i, s in enumerate(self.slots) if s.expert < 0]
+            budget = max(0, self.IN_FLIGHT_BUDGET - sum(1 for s in self.slots if s.in_flight))
+            count = min(len(wanted), len(free), budget)
+            self.stats["refused"] += len(wanted) - count
+            if count == 0:
+                self.lock.release()
+                return
+            chosen, chosen_experts = free[:count], wanted[:count]
+            cells = [self.slots[i].cell for i in chosen]
+            for i, e in zip(chosen, chosen_experts):
+                self.slots[i].layer, self.slots[i].expert, self.slots[i].operation = layer, e, None
+            self.lock.release()
+            try:
+                operation = issue(chosen_experts, cells)
+            except BaseException as exc:
+                with self.lock:
+                    for i in chosen:
+                        self.slots[i].layer, self.slots[i].expert, self.slots[i].operation = -1, -1, None
+                    if isinstance(exc, ClaimRefused):
+                        self.stats["refused"] += count
+                        return
+                raise
+            with self.lock:
+                for i in chosen:
+                    self.slots[i].operation = operation
+                self.stats["issued"] += count
+                if deferred:
+                    self.stats["deferred"] += 1
+        finally:
+            self.stats["begin_nanos"] += _time.monotonic_ns() - started
+
+    def ready_cells(self, layer, experts, join_nanos=0):  # :171-212
+        requested = set(experts)
+        deadline = _time.monotonic_ns() + join_nanos if join_nanos > 0 else 0
+        result, joined_ops, late_ops = {}, set(), set()
+        self.lock.acquire()
+        try:
+            for s in self.slots:
+                if s.layer != layer or s.expert not in requested:
+                    continue
+                if s.in_flight:
+                    operation = self._attached(s)
+                    if operation is None:
+                        self.stats["late"] += 1
+                        continue
+                    self.lock.release()
+                    joined = deadline > 0 and operation.wait_until(deadline)
+                    if not joined:
+                        try:
+                            operation.wait()
+                        except RuntimeError:
+                            pass
+                    self.lock.acquire()
+                    (joined_ops if joined else late_ops).add(id(operation))
+                    if s.layer != layer or s.expert not in requested:
+                        continue
+                if s.operation is None:
+                    continue
+                if id(s.operation) in joined_ops:
+                    self.stats["joined"] += 1
+                elif id(s.operation) in late_ops:
+                    self.stats["late"] += 1
+                if s.operation.state == COMPLETED:
+                    result[s.expert] = s.cell
+                    s.leased = True
+            return result
+        finally:
+            self.lock.release()
+
+    def _attached(self, s):  # :216-228
+        if s.operation is not None:
+            return s.operation
+        layer, expert = s.layer, s.expert
+        deadline = _time.monotonic_ns() + self.ATTACH_SPIN_NANOS
+        while s.operation is None and _time.monotonic_ns() < deadline:
+            self.lock.release()
+            _time.sleep(50e-6)
+            self.lock.acquire()
+            if s.layer != layer or s.expert != expert:
+                return None
+        return s.operation
+
+    def consume(self, layer, experts, freed_cells):  # :232-252
+        with self.lock:
+            for s in self.slots:
+                if s.layer != layer or s.expert not in experts:
+                    continue
+                if s.expert in freed_cells:
+                    s.cell = freed_cells[s.expert]
+                else:
+                    self.drop(layer, s.expert, s.cell)
+                if not s.demand:
+                    self.stats["adopted"] += 1
+                s.layer, s.expert, s.operation, s.leased, s.demand = -1, -1, None, False, False
+
+    def claim_demand(self, layer, experts):  # :257-282
+        with self.lock:
+            self._reclaim(layer)
+            cells = {}
+            for e in experts:
+                own = next((s for s in self.slots if s.layer == layer and s.expert == e), None)
+                if own is not None:
+                    if own.leased or own.operation is None or own.operation.state != FAILED:
+                        continue
+                    self.stats["failed"] += 1
+                    own.operation = None
+                else:
+                    own = next((s for s in self.slots if s.expert < 0), None)
+                    if own is None:
+                        break
+                    own.layer, own.expert, own.operation = layer, e, None
+                own.leased = own.demand = True
+                cells[e] = own.cell
+            self.stats["leased_peak"] = max(self.stats["leased_peak"], sum(1 for s in self.slots if s.leased))
+            return cells
+
+    def attach_demand(self, layer, experts, operation):
+        with self.lock:
+            for s in self.slots:
+                if s.demand and s.layer == layer and s.expert in experts:
+                    s.operation = operation
+
+    def completion_nanos(self, layer, experts):
+        with self.lock:
+            return {s.expert: s.operation.completed_nanos for s in self.slots
+                    if s.layer == layer and s.expert in experts and s.operation is not None and s.operation.state == COMPLETED}
+
+    def unlease(self, layer, experts):
+        with self.lock:
+            for s in self.slots:
+                if s.layer == layer and s.expert in experts:
+                    s.leased = False
+
+    def note_demand_submission(self):
+        with self.lock:
+            if any(s.in_flight for s in self.slots):
+                self.stats["overlapped"] += 1
+
+    def note_hook_failure(self):
+        with self.lock:
+            self.stats["hook_failures"] += 1
+            return self.stats["hook_failures"] == 1
+
+    @property
+    def statistics(self):
+        with self.lock:
+            return dict(self.stats)

@@ -164,6 +164,15 @@ class TileDriver(C.Structure):
                 ("abandon_begun_fetches", C.CFUNCTYPE(None, C.c_void_p))]
 
 
+class PrefetchStatistics(C.Structure):
+    _fields_ = [(name, C.c_uint64) for name in ("issued", "adopted", "reclaimed", "deferred", "overlapped", "late", "joined",
+                                                "refused", "failed", "hook_failures", "begin_nanos", "leased_peak")]
+
+
+PREFETCH_DROP = C.CFUNCTYPE(None, C.c_void_p, C.c_int, C.c_int, C.c_int)
+PREFETCH_ISSUE = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_size_t, C.POINTER(C.c_void_p))
+
+
 SIGNATURES = {
     "shrike_hip_last_error": (C.c_char_p, []),
     "shrike_tile_scheduler_config_make": (None, [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(TileSchedulerConfig)]),
@@ -181,6 +190,37 @@ SIGNATURES = {
     "shrike_tile_lifetime_destroy": (None, [_VP]),
     "shrike_tile_lifetime_begin": (C.c_int, [_VP, C.c_int, C.POINTER(C.c_int32), C.c_size_t, C.POINTER(C.c_int)]),
     "shrike_tile_lifetime_complete": (C.c_int, [_VP, C.c_int]),
+    "shrike_monotonic_nanos": (C.c_uint64, []),
+    "shrike_load_operation_create": (_VP, []),
+    "shrike_load_operation_retain": (None, [_VP]),
+    "shrike_load_operation_release": (None, [_VP]),
+    "shrike_load_operation_state": (C.c_int, [_VP]),
+    "shrike_load_operation_mark_in_flight": (C.c_int, [_VP]),
+    "shrike_load_operation_finish": (C.c_int, [_VP, C.c_int]),
+    "shrike_load_operation_wait": (C.c_int, [_VP]),
+    "shrike_load_operation_wait_until": (C.c_int, [_VP, C.c_uint64]),
+    "shrike_load_operation_submitted_nanos": (C.c_uint64, [_VP]),
+    "shrike_load_operation_started_nanos": (C.c_uint64, [_VP]),
+    "shrike_load_operation_completed_nanos": (C.c_uint64, [_VP]),
+    "shrike_prefetch_ring_create": (_VP, [C.POINTER(C.c_int), C.c_size_t, PREFETCH_DROP, C.c_void_p, C.POINTER(C.c_int)]),
+    "shrike_prefetch_ring_destroy": (None, [_VP]),
+    "shrike_prefetch_ring_begin": (C.c_int, [_VP, C.c_int, C.POINTER(C.c_int), C.c_size_t, C.POINTER(C.c_int), C.c_size_t, C.c_int,
+                                             PREFETCH_ISSUE, C.c_void_p]),
+    "shrike_prefetch_ring_ready_cells": (C.c_size_t, [_VP, C.c_int, C.POINTER(C.c_int), C.c_size_t, C.c_uint64, C.POINTER(C.c_int),
+                                                      C.POINTER(C.c_int)]),
+    "shrike_prefetch_ring_consume": (None, [_VP, C.c_int, C.POINTER(C.c_int), C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                            C.c_size_t]),
+    "shrike_prefetch_ring_claim_demand": (C.c_size_t, [_VP, C.c_int, C.POINTER(C.c_int), C.c_size_t, C.POINTER(C.c_int),
+                                                       C.POINTER(C.c_int)]),
+    "shrike_prefetch_ring_attach_demand": (None, [_VP, C.c_int, C.POINTER(C.c_int), C.c_size_t, _VP]),
+    "shrike_prefetch_ring_completion_nanos": (C.c_size_t, [_VP, C.c_int, C.POINTER(C.c_int), C.c_size_t, C.POINTER(C.c_int),
+                                                           C.POINTER(C.c_uint64)]),
+    "shrike_prefetch_ring_unlease": (None, [_VP, C.c_int, C.POINTER(C.c_int), C.c_size_t]),
+    "shrike_prefetch_ring_note_demand_submission": (None, [_VP]),
+    "shrike_prefetch_ring_note_hook_failure": (C.c_int, [_VP]),
+    "shrike_prefetch_ring_statistics": (None, [_VP, C.POINTER(PrefetchStatistics)]),
+    "shrike_prefetch_ring_in_flight_count": (C.c_int, [_VP]),
+    "shrike_prefetch_ring_leased_count": (C.c_int, [_VP]),
     "shrike_host_last_error": (C.c_char_p, []),
     "shrike_expert_reader_create": (_VP, [C.c_char_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int)]),
     "shrike_expert_reader_destroy": (None, [_VP]),

@@ -584,3 +584,181 @@ class TileSlotLifetime:
         rc = capi.load().shrike_tile_lifetime_complete(self._h, tile_index)
         if rc:
             raise TileLifetimeError(rc, -1, capi.last_error())
+
+
+# ------------------------------------------------------------------ load operations and the prefetch ring
+
+LOAD_SUBMITTED, LOAD_IN_FLIGHT, LOAD_COMPLETED, LOAD_FAILED = 0, 1, 2, 3
+PREFETCH_CLAIM_REFUSED = -2
+
+
+def monotonic_nanos() -> int:
+    return int(capi.load().shrike_monotonic_nanos())
+
+
+class ExpertLoadOperation:
+    """ExpertLoadOperation (sources/Shrike/Infrastructure/Streaming/ExpertLoadOperation.swift:15-153): one
+    storage batch, submitted now and finished later by whoever reads it."""
+
+    def __init__(self):
+        self._h = capi.load().shrike_load_operation_create()
+        if not self._h:
+            raise MemoryError("load operation")
+
+    def __del__(self):
+        try:
+            if self._h:
+                capi.load().shrike_load_operation_release(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    @property
+    def state(self) -> int:
+        return capi.load().shrike_load_operation_state(self._h)
+
+    def mark_in_flight(self) -> None:
+        rc = capi.load().shrike_load_operation_mark_in_flight(self._h)
+        if rc:
+            raise ShrikeError(f"expert load operation started more than once (code {rc})")
+
+    def finish(self, failure: int = 0) -> None:
+        rc = capi.load().shrike_load_operation_finish(self._h, failure)
+        if rc:
+            raise ShrikeError(f"expert load operation completed more than once (code {rc})")
+
+    def wait(self) -> None:
+        rc = capi.load().shrike_load_operation_wait(self._h)
+        if rc:
+            raise ReadFailed(rc, "expert load operation")
+
+    def wait_until(self, deadline_nanos: int) -> bool:
+        return bool(capi.load().shrike_load_operation_wait_until(self._h, deadline_nanos))
+
+    @property
+    def submitted_nanos(self) -> int:
+        return int(capi.load().shrike_load_operation_submitted_nanos(self._h))
+
+    @property
+    def started_nanos(self) -> int:
+        return int(capi.load().shrike_load_operation_started_nanos(self._h))
+
+    @property
+    def completed_nanos(self) -> int:
+        return int(capi.load().shrike_load_operation_completed_nanos(self._h))
+
+
+class PrefetchClaimRefused(Exception):
+    """PrefetchClaimRefused (PreadExpertStreamer.swift:46-49): the pool already holds a predicted expert."""
+
+    def __init__(self, expert: int = -1, cell: int = -1):
+        super().__init__(f"prefetch claim refused: expert {expert}, cell {cell}")
+        self.expert, self.cell = expert, cell
+
+
+def _ints(values):
+    values = list(values)
+    return (C.c_int * max(1, len(values)))(*values), len(values)
+
+
+class ExpertPrefetchRing:
+    """ExpertPrefetchRing (sources/Shrike/Runtime/Inference/ExpertPrefetchRing.swift:42-352). `drop(layer, expert,
+    cell)` is called with the ring locked. `issue(experts, cells)` passed to begin returns the batch's
+    ExpertLoadOperation, raises PrefetchClaimRefused (counted, not propagated) or anything else
+    (propagated after the slots are rolled back)."""
+
+    _ISSUE_FAILED = 5  # EIO: the code that carries a Python exception across the C boundary
+
+    def __init__(self, cells, drop=None):
+        self._drop = drop or (lambda layer, expert, cell: None)
+        self._drop_c = capi.PREFETCH_DROP(lambda _ctx, layer, expert, cell: self._drop(layer, expert, cell))
+        arr, n = _ints(cells)
+        err = C.c_int(0)
+        self._h = capi.load().shrike_prefetch_ring_create(arr, n, self._drop_c, None, C.byref(err))
+        if not self._h:
+            raise ShrikeError("invalid prefetch ring geometry")  # ExpertPrefetchRing.swift:96-98
+
+    def __del__(self):
+        try:
+            if self._h:
+                capi.load().shrike_prefetch_ring_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    def begin(self, layer: int, experts, resident=(), deferred: bool = False, issue=None) -> None:
+        raised = []
+
+        def trampoline(_ctx, c_experts, c_cells, count, out_operation):
+            try:
+                operation = issue([c_experts[i] for i in range(count)], [c_cells[i] for i in range(count)])
+                out_operation[0] = operation._h
+                raised.append(operation)  # keeps the caller's reference alive until the ring holds its own
+                return 0
+            except PrefetchClaimRefused:
+                return PREFETCH_CLAIM_REFUSED
+            except BaseException as exc:  # carried across the C boundary
+                raised.append(exc)
+                return self._ISSUE_FAILED
+
+        e_arr, e_n = _ints(experts)
+        r_arr, r_n = _ints(resident)
+        rc = capi.load().shrike_prefetch_ring_begin(self._h, layer, e_arr, e_n, r_arr, r_n, 1 if deferred else 0,
+                                                    capi.PREFETCH_ISSUE(trampoline), None)
+        if rc:
+            for item in raised:
+                if isinstance(item, BaseException):
+                    raise item
+            raise ShrikeError(f"prefetch begin failed (code {rc})")
+
+    def ready_cells(self, layer: int, experts, join_nanos: int = 0) -> dict:
+        e_arr, e_n = _ints(experts)
+        out_e, out_c = (C.c_int * max(1, e_n))(), (C.c_int * max(1, e_n))()
+        n = capi.load().shrike_prefetch_ring_ready_cells(self._h, layer, e_arr, e_n, join_nanos, out_e, out_c)
+        return {out_e[i]: out_c[i] for i in range(n)}
+
+    def consume(self, layer: int, experts, freed_cells: dict) -> None:
+        e_arr, e_n = _ints(experts)
+        f_e, f_n = _ints(freed_cells.keys())
+        f_c, _ = _ints(freed_cells.values())
+        capi.load().shrike_prefetch_ring_consume(self._h, layer, e_arr, e_n, f_e, f_c, f_n)
+
+    def claim_demand(self, layer: int, experts) -> dict:
+        e_arr, e_n = _ints(experts)
+        out_e, out_c = (C.c_int * max(1, e_n))(), (C.c_int * max(1, e_n))()
+        n = capi.load().shrike_prefetch_ring_claim_demand(self._h, layer, e_arr, e_n, out_e, out_c)
+        return {out_e[i]: out_c[i] for i in range(n)}
+
+    def attach_demand(self, layer: int, experts, operation: ExpertLoadOperation) -> None:
+        e_arr, e_n = _ints(experts)
+        capi.load().shrike_prefetch_ring_attach_demand(self._h, layer, e_arr, e_n, operation._h)
+
+    def completion_nanos(self, layer: int, experts) -> dict:
+        e_arr, e_n = _ints(experts)
+        out_e, out_t = (C.c_int * max(1, e_n))(), (C.c_uint64 * max(1, e_n))()
+        n = capi.load().shrike_prefetch_ring_completion_nanos(self._h, layer, e_arr, e_n, out_e, out_t)
+        return {out_e[i]: int(out_t[i]) for i in range(n)}
+
+    def unlease(self, layer: int, experts) -> None:
+        e_arr, e_n = _ints(experts)
+        capi.load().shrike_prefetch_ring_unlease(self._h, layer, e_arr, e_n)
+
+    def note_demand_submission(self) -> None:
+        capi.load().shrike_prefetch_ring_note_demand_submission(self._h)
+
+    def note_hook_failure(self) -> bool:
+        return bool(capi.load().shrike_prefetch_ring_note_hook_failure(self._h))
+
+    @property
+    def statistics(self) -> dict:
+        st = capi.PrefetchStatistics()
+        capi.load().shrike_prefetch_ring_statistics(self._h, C.byref(st))
+        return {name: int(getattr(st, name)) for name, _ in capi.PrefetchStatistics._fields_}
+
+    @property
+    def in_flight_count(self) -> int:
+        return capi.load().shrike_prefetch_ring_in_flight_count(self._h)
+
+    @property
+    def leased_count(self) -> int:
+        return capi.load().shrike_prefetch_ring_leased_count(self._h)

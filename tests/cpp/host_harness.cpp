@@ -1,6 +1,7 @@
 // The reference's host-side unit tests, written against include/shrike.hpp the way the
 // reference writes them against its Swift classes. No GPU call is made: budget ladder,
 // grouping, sweep order, wave planner, slot cache, the packed-experts layout and the parallel reader run on the host. Exit code 0 = all passed.
+#include <array>
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -187,7 +188,116 @@ static void layoutAndReader() {
     EXPECT(threw);
 }
 
+// PrefillRoutedTileSchedulerTests / PrefillRoutedTileSequencerTests / ExpertPrefetchRingTests, a few cases each
+struct RecordingDriver : PrefillRoutedTileDriver {
+    std::vector<std::string> calls;
+    std::vector<int> open;
+    std::vector<std::vector<int>> pending;
+    int failingEncode = -1;
+    std::vector<int> slots(int tile) { return {2 * tile, 2 * tile + 1}; }
+    int openBatchTiles() override { return int(open.size()); }
+    size_t openBatchSlotCount() override { return 2 * open.size(); }
+    int pendingDepth() override { return int(pending.size()); }
+    size_t pendingAssignedSlotCount() override {
+        size_t n = 0;
+        for (auto &b : pending) n += b.size();
+        return n;
+    }
+    bool plan(int tile, std::optional<int> avoiding) override {
+        calls.push_back("plan" + std::to_string(tile) + (avoiding ? "/" + std::to_string(*avoiding) : ""));
+        return true;
+    }
+    void begin(int tile) override { calls.push_back("begin" + std::to_string(tile)); }
+    void abandonPlan(int tile) override { calls.push_back("abandonPlan" + std::to_string(tile)); }
+    void encode(int tile) override {
+        calls.push_back("encode" + std::to_string(tile));
+        if (tile == failingEncode) throw std::runtime_error("encode failed");
+        open.push_back(tile);
+    }
+    void commitOpenBatch() override {
+        if (open.empty()) return;
+        calls.push_back("commit");
+        std::vector<int> all;
+        for (int t : open)
+            for (int s : slots(t)) all.push_back(s);
+        pending.push_back(all);
+        open.clear();
+    }
+    void drainOldestBatch() override {
+        calls.push_back("drain");
+        if (!pending.empty()) pending.erase(pending.begin());
+    }
+    void abandonBegunFetches() override { calls.push_back("abandonBegun"); }
+};
+
+static void tileLoopAndRing() {
+    PrefillRoutedTileSchedulerConfig def;
+    auto fit = def.fitting(8);
+    EXPECT(fit && fit->max_pending_depth == 1 && fit->tile_experts == 4 && fit->tiles_per_command_buffer == 1);
+    EXPECT(!def.fitting(1));
+    EXPECT(PrefillRoutedTileSchedulerConfig(2, 4).fitsSlotBudget(16) && !PrefillRoutedTileSchedulerConfig(2, 8).fitsSlotBudget(16));
+    PrefillRoutedTileScheduler sch{PrefillRoutedTileSchedulerConfig(2, 4)};
+    EXPECT(sch.decide(false, 0, false) == SHRIKE_TILE_ISSUE_WITHOUT_PENDING);
+    EXPECT(sch.decide(true, 8, true, 2) == SHRIKE_TILE_PREFETCH_NEXT);
+    EXPECT(sch.decide(true, 2, true, 3) == SHRIKE_TILE_DRAIN_MAX_DEPTH);
+    {
+        RecordingDriver d;
+        PrefillRoutedTileSequencer{PrefillRoutedTileScheduler{PrefillRoutedTileSchedulerConfig(2, 8, 1, 1)}}.run(3, d);
+        const std::vector<std::string> want = {"plan0", "begin0", "plan1/0", "begin1", "encode0", "commit", "plan2/1", "begin2",
+                                               "encode1", "commit", "encode2", "commit", "drain", "drain", "drain"};
+        EXPECT(d.calls == want);
+    }
+    {
+        RecordingDriver d;
+        d.failingEncode = 0;
+        bool thrown = false;
+        try {
+            PrefillRoutedTileSequencer{PrefillRoutedTileScheduler{PrefillRoutedTileSchedulerConfig(2, 8, 1, 1)}}.run(3, d);
+        } catch (const std::runtime_error &e) {
+            thrown = std::string(e.what()) == "encode failed";
+        }
+        const std::vector<std::string> want = {"plan0", "begin0", "plan1/0", "begin1", "encode0", "abandonBegun"};
+        EXPECT(thrown && d.calls == want);
+    }
+    {
+        std::vector<std::array<int, 3>> drops;
+        ExpertPrefetchRing ring({10, 11, 12, 13}, [&](int l, int e, int c) { drops.push_back({l, e, c}); });
+        std::vector<std::vector<int>> issued;
+        ExpertLoadOperation first;
+        ring.begin(3, {7, 9, 11}, {}, [&](const std::vector<int> &e, const std::vector<int> &) { issued.push_back(e); return first; });
+        EXPECT(issued.size() == 1 && issued[0] == std::vector<int>{7} && ring.inFlightCount() == 1);
+        ring.begin(4, {1, 2}, {}, [&](const std::vector<int> &e, const std::vector<int> &) { issued.push_back(e); return ExpertLoadOperation(); });
+        EXPECT(issued.size() == 1 && ring.statistics().issued == 1);
+        first.markInFlight();
+        first.finish();
+        ring.begin(4, {1, 2}, {}, [&](const std::vector<int> &e, const std::vector<int> &) { issued.push_back(e); return ExpertLoadOperation(); });
+        EXPECT(issued.size() == 2 && issued[1] == std::vector<int>{1});
+        EXPECT(ring.statistics().issued == 2 && ring.statistics().reclaimed == 1 && drops.size() == 1 && drops[0][1] == 7);
+        // a refused claim is counted, an issue that throws rolls the slots back
+        ExpertPrefetchRing other({20, 21}, [](int, int, int) {});
+        other.begin(2, {1, 2}, {}, [](const std::vector<int> &e, const std::vector<int> &c) -> ExpertLoadOperation { throw PrefetchClaimRefused{e[0], c[0]}; });
+        EXPECT(other.statistics().refused == 2 && other.inFlightCount() == 0);
+        bool thrown = false;
+        try {
+            other.begin(2, {1}, {}, [](const std::vector<int> &, const std::vector<int> &) -> ExpertLoadOperation { throw std::runtime_error("reader refused"); });
+        } catch (const std::runtime_error &) {
+            thrown = true;
+        }
+        EXPECT(thrown && other.inFlightCount() == 0);
+        ExpertLoadOperation op;
+        other.begin(2, {1}, {}, [&](const std::vector<int> &, const std::vector<int> &) { return op; });
+        op.finish();
+        auto ready = other.readyCells(2, {1});
+        EXPECT(ready.size() == 1 && ready[1] == 20 && other.leasedCount() == 1);
+        other.consume(2, {1}, {{1, 77}});
+        EXPECT(other.statistics().adopted == 1 && other.leasedCount() == 0);
+        auto claimed = other.claimDemand(5, {4, 6, 8});
+        EXPECT(claimed.size() == 2 && claimed[4] == 77 && claimed[6] == 21);
+    }
+}
+
 int main() {
+    tileLoopAndRing();
     layoutAndReader();
     budget();
     grouping();
