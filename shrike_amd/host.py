@@ -440,6 +440,11 @@ class TileSchedulerConfig:
     def astuple(self):
         return (self.c.max_pending_depth, self.c.tile_experts, self.c.tiles_per_command_buffer, self.c.fetch_lookahead)
 
+    max_pending_depth = property(lambda self: self.c.max_pending_depth)
+    tile_experts = property(lambda self: self.c.tile_experts)
+    tiles_per_command_buffer = property(lambda self: self.c.tiles_per_command_buffer)
+    fetch_lookahead = property(lambda self: self.c.fetch_lookahead)
+
     def __eq__(self, other):
         return isinstance(other, TileSchedulerConfig) and self.astuple() == other.astuple()
 

@@ -492,3 +492,167 @@ class BatchedDecodeLayer:
             self.passes += 1
         pf.encode_reduce_token_major(self.partials, self.w, self.h2, t, k, d)
         return self.h2
+
+
+class StreamedPrefillLayer:
+    """One prefill chunk's routed experts streamed from a layer file through a pool smaller than the
+    chunk's expert set, sequenced the way the reference's ExpertStreamedTileDriver is
+    (RealForwardRunner.swift:4698-4866 under PrefillRoutedTileSequencer.run): the chunk's expert groups
+    are cut into tiles of `tile_experts`; a tile is planned against the slot cache (avoiding the cells
+    that open and pending batches and a fetch in flight still hold, protecting the experts the chunk
+    still needs), its misses are read by the parallel reader and copied to their cells on the upload
+    stream, and once they have landed the grouped FFN runs for exactly that tile's experts on the compute
+    stream. A batch of tiles is "committed" by recording an event and "drained" by waiting for it.
+    Everything numeric happens in libshrikehip; this class only sequences calls."""
+
+    def __init__(self, moe: MoE, pool: ExpertPool, cache, offsets, reader, file_offsets, blob_bytes: int,
+                 staging: PinnedBuffer, max_tokens: int, config):
+        d, ne, k = moe.desc.d, moe.desc.num_experts, moe.desc.top_k
+        fitted = config.fitting(cache.slot_count)
+        if fitted is None:
+            raise ShrikeError(f"no tile configuration fits {cache.slot_count} slots")
+        self.moe, self.pool, self.cache, self.off, self.config = moe, pool, cache, offsets, fitted
+        self.reader, self.file_offsets, self.blob_bytes, self.staging = reader, list(file_offsets), blob_bytes, staging
+        self.pf = Prefill(moe)
+        self.upload_stream = Stream()
+        self.idx, self.w = empty(4 * max_tokens * k), empty(2 * max_tokens * k)
+        self.router_ws = empty(self.pf.router_workspace_bytes(max_tokens, ne, d))
+        self.routes = GroupedRoutesDevice(max_tokens * k, ne)
+        self.partials = empty(2 * max_tokens * k * d)
+        self.ffn_ws = empty(self.pf.ffn_workspace_bytes(max_tokens, self.routes.max_row_tiles))
+        self.h2 = empty(2 * max_tokens * d)
+        self.trace = []  # (call, tile) in the order the sequencer made them
+
+    def run(self, router, hidden, t: int, stride: int):
+        from . import host as _host
+        m, pf = self.moe, self.pf
+        d, ne, k = m.desc.d, m.desc.num_experts, m.desc.top_k
+        compute = m.stream
+        pf.encode_block(router["weights"], router.get("scales"), router.get("biases"), hidden, router["eff_scale"],
+                        router["expert_scale"], router["bias"], self.idx, self.w, self.router_ws, t, ne, d, k, stride)
+        (compute.synchronize() if compute else synchronize())
+        ids, weights = self.idx.download(np.uint32, t * k), self.w.download(np.uint16, t * k)
+        # experts the pool already holds go first (PrefillSweepOrder.residentFirstBalanced), so the chunk's first
+        # tiles hit what the previous chunk left behind instead of evicting it
+        rows, last = {}, {}
+        for i, e in enumerate(ids.tolist()):
+            rows[e] = rows.get(e, 0) + 1
+            last[e] = i // k
+        resident = np.zeros(ne, np.uint8)
+        resident[self.cache.resident_experts()] = 1
+        order = _host.resident_first_balanced(rows, last, resident, self.cache.slot_count, self.config.tile_experts)
+        keys = _host.expert_sort_keys(order, ne)
+        sort_keys = empty(8 * ne).upload(keys)
+        grouped = _host.group_token_expert_pairs(_host.make_token_expert_pairs(ids, weights, t, k), t, k, ne,
+                                                 tile_expert_count=self.config.tile_experts, expert_sort_keys=keys)
+        self.grouped = grouped
+        layer = self
+
+        class Driver:
+            def __init__(self):
+                self.protection = _host.ChunkExpertProtection([int(g["expert"]) for g in grouped.groups], ne)
+                self.lifetime = _host.TileSlotLifetime()
+                self.kept, self.begun = {}, {}
+                self.open, self.pending = [], []  # open: (tile, slots, had misses, tile table); pending: (event, such entries)
+
+            def experts_of(self, tile):
+                tl = grouped.tiles[tile]
+                return [int(g["expert"]) for g in grouped.groups[int(tl["group_start"]): int(tl["group_start"]) + int(tl["group_count"])]]
+
+            open_batch_tiles = property(lambda self: len(self.open))
+            open_batch_slots = property(lambda self: [s for entry in self.open for s in entry[1]])
+            pending_depth = property(lambda self: len(self.pending))
+            pending_assigned_slots = property(lambda self: [s for _, batch in self.pending for entry in batch for s in entry[1]])
+
+            def _plan(self, tile, extra=()):
+                experts = self.experts_of(tile)
+                self.protection.planning(experts)
+                avoiding = set(self.open_batch_slots) | set(self.pending_assigned_slots) | set(extra)
+                return layer.cache.plan(experts, avoiding_slots=avoiding, protected_experts=self.protection.remaining)
+
+            def plan(self, tile, avoiding_in_flight):
+                layer.trace.append(("plan", tile))
+                extra = ()
+                if avoiding_in_flight is not None:
+                    extra = self.begun[avoiding_in_flight][0].assigned_slots
+                plan = self._plan(tile, extra)
+                if plan is not None:
+                    self.kept[tile] = plan
+                return plan is not None
+
+            def begin(self, tile):
+                layer.trace.append(("begin", tile))
+                plan = self.kept.pop(tile, None) or self._plan(tile)
+                if plan is None:
+                    raise ShrikeError(capi.last_error())
+                slots, experts = plan.assigned_slots, plan.experts
+                miss_slots = [slots[i] for i in plan.misses]
+                try:
+                    if miss_slots:
+                        layer.pool.fetch_experts(layer.reader, [layer.file_offsets[experts[i]] for i in plan.misses], miss_slots,
+                                                 layer.blob_bytes, layer.staging, layer.upload_stream)
+                except BaseException:
+                    layer.cache.abandon(plan)
+                    raise
+                layer.cache.complete(plan)
+                for expert, word in layer.cache.drain_publications():
+                    layer.pool.publish(expert, word & 0xFFFFFFFF, word >> 32, layer.upload_stream)
+                landed = Event()
+                landed.record(layer.upload_stream)
+                self.begun[tile] = (plan, landed)
+                if miss_slots:
+                    self.lifetime.begin(tile, miss_slots)
+
+            def abandon_plan(self, tile):
+                layer.trace.append(("abandonPlan", tile))
+                plan = self.kept.pop(tile, None)
+                if plan is not None:
+                    layer.cache.abandon(plan)
+
+            def encode(self, tile):
+                layer.trace.append(("encode", tile))
+                plan, landed = self.begun.pop(tile)
+                table = np.full(ne, (capi.EMPTY << 32) | SENTINEL, np.uint64)
+                for expert, slot in zip(plan.experts, plan.assigned_slots):
+                    table[expert] = (capi.RESIDENT << 32) | slot
+                landed.synchronize()  # the experts' bytes and words are in place; the table below is this tile's view
+                tile_table = empty(8 * ne).upload(table)
+                if compute:
+                    compute.wait_event(landed)
+                pf.group_pairs(layer.idx, layer.w, t, k, ne, layer.routes, expert_sort_keys=sort_keys, residency=tile_table)
+                pf.encode_grouped_expert_gemms(layer.pool, layer.off, layer.routes, hidden, stride, layer.partials,
+                                               layer.ffn_ws, t, k)
+                self.open.append((tile, list(plan.assigned_slots), bool(plan.misses), tile_table))
+
+            def commit_open_batch(self):
+                if not self.open:
+                    return
+                layer.trace.append(("commit", None))
+                done = Event()
+                done.record(compute)
+                self.pending.append((done, self.open))
+                self.open = []
+
+            def drain_oldest_batch(self):
+                layer.trace.append(("drain", None))
+                if not self.pending:
+                    return
+                done, batch = self.pending.pop(0)
+                done.synchronize()
+                for tile, _slots, missed, _table in batch:
+                    if missed:
+                        self.lifetime.complete(tile)
+
+            def abandon_begun_fetches(self):
+                layer.trace.append(("abandonBegun", None))
+                layer.upload_stream.synchronize()
+                self.begun.clear()
+                for plan in self.kept.values():
+                    layer.cache.abandon(plan)
+                self.kept.clear()
+
+        self.trace = []
+        driver = Driver()
+        _host.TileSequencer(_host.TileScheduler(self.config)).run(len(grouped.tiles), driver)
+        pf.encode_reduce_token_major(self.partials, self.w, self.h2, t, k, d)
+        return self.h2
