@@ -656,3 +656,83 @@ class StreamedPrefillLayer:
         _host.TileSequencer(_host.TileScheduler(self.config)).run(len(grouped.tiles), driver)
         pf.encode_reduce_token_major(self.partials, self.w, self.h2, t, k, d)
         return self.h2
+
+
+class DecodeLayerWithMisses:
+    """One token's routed experts when some of the selected experts are not in the pool: the runner's
+    speculative pass and agreed fixup (RealForwardRunner.swift:2226-2294, :5115-5162, :5262-5283) over this
+    build's operators. The classifier publishes four grids and a tagged readback; phase 1 runs for the hits
+    and phase 2 only when nothing missed; the host reads the miss list, agrees a cell for every miss (the
+    slot cache's plan for the selection: hits keep their cells, misses take victims outside it), writes the
+    agreed row (the sentinel at the hits), has the missing blobs copied into their cells, and the fixup runs
+    phase 1 over the agreed row and phase 2 over all positions, resolving a sentinel through that row.
+    Everything numeric happens in libshrikehip; this class only sequences calls."""
+
+    def __init__(self, moe: MoE, pool: ExpertPool, cache, offsets, host_store: PinnedBuffer, store_stride: int,
+                 expert_bytes: int):
+        k = moe.desc.top_k
+        self.moe, self.pool, self.cache, self.off = moe, pool, cache, offsets
+        self.store, self.store_stride, self.expert_bytes = host_store, store_stride, expert_bytes
+        self.upload_stream = Stream()
+        self.idx, self.w = empty(4 * 8), empty(2 * 8)
+        self.resolved, self.agreed = empty(4 * 8), empty(4 * 8)
+        self.hit_count, self.miss_count = empty(4), empty(4)
+        self.hit_pos, self.miss_pos, self.miss_exp = empty(32), empty(32), empty(32)
+        self.spec_args = empty(48)
+        self.predicted = empty(4 * 8).fill(0)  # the runner's prediction for the next layer rides in the readback
+        self.readback = PinnedBuffer(4 * (2 + 5 * k))
+        self.acts = empty(2 * k * moe.desc.f)
+        self.tag = 0
+        self.fixups = 0
+
+    def run(self, router, x, residual, y, hidden):
+        """router: dict(weights, scales, biases, eff_scale, expert_scale, bias). x: fp16[d] (the router's and
+        the experts' input), residual: fp16[d], y: fp16[d] out, hidden: fp16[d] updated in place."""
+        m = self.moe
+        d, f, ne, k = m.desc.d, m.desc.f, m.desc.num_experts, m.desc.top_k
+        compute = m.stream
+        m.encode_router(router["weights"], router.get("scales"), router.get("biases"), x, router["eff_scale"],
+                        router["expert_scale"], router["bias"], self.idx, self.w, ne, d, k)
+        self.tag = self.tag % 0xFFFF + 1
+        full = [1] * 12  # the operators below read only whether a grid's first word is zero
+        m.encode_residency_classification(self.idx, self.pool.table, self.hit_count, self.hit_pos, self.miss_count,
+                                          self.miss_pos, self.miss_exp, self.resolved, k, ne, full_grids=full,
+                                          spec_args=self.spec_args, host_readback=self.readback, tag=self.tag,
+                                          topk_weights=self.w, predicted=self.predicted)
+        spec = self.spec_args.ptr
+        m.encode_spec_phase1(self.pool, self.resolved, self.off, x, self.acts, d, f, k, indirect=spec)
+        m.encode_spec_phase2(self.pool, self.resolved, self.off, self.acts, self.w, residual, y, hidden, d, f, k,
+                             indirect=spec + 12)
+        (compute.synchronize() if compute else synchronize())
+        rb = self.readback.array.view(np.uint32)[: 2 + 5 * k].copy()  # counts, experts, weights, hit and miss positions, predictions
+        if np.any(rb >> 16 != self.tag):
+            raise ShrikeError("router readback carries another launch's tag")  # RouterHostReadback.swift
+        rb &= 0xFFFF
+        hits, misses = int(rb[0]), int(rb[1])
+        experts = rb[2:2 + k].tolist()
+        miss_positions = rb[2 + 3 * k: 2 + 3 * k + misses].tolist()
+        if misses == 0:
+            plan = self.cache.plan(experts)  # counts the hits, touches their recency
+            self.cache.complete(plan)
+            return
+        plan = self.cache.plan(experts)
+        if plan is None:
+            raise ShrikeError(capi.last_error())
+        if sorted(plan.misses) != sorted(miss_positions) or hits + misses != k:
+            self.cache.abandon(plan)
+            raise ShrikeError("the device's miss list and the slot cache disagree")
+        row = np.full(8, SENTINEL, np.uint32)
+        for i in plan.misses:
+            row[i] = plan.assigned_slots[i]
+        self.agreed.upload(row)
+        self.pool.execute_plan(self.cache, plan, self.store, self.store_stride, self.expert_bytes, self.upload_stream)
+        landed = Event()
+        landed.record(self.upload_stream)
+        if compute:
+            compute.wait_event(landed)
+        else:
+            landed.synchronize()
+        m.encode_spec_phase1(self.pool, self.agreed, self.off, x, self.acts, d, f, k, indirect=spec + 24)
+        m.encode_spec_phase2(self.pool, self.resolved, self.off, self.acts, self.w, residual, y, hidden, d, f, k,
+                             fallback_cells=self.agreed, indirect=spec + 36)
+        self.fixups += 1

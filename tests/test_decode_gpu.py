@@ -8,6 +8,7 @@ import pytest
 
 from oracle import oracle as O
 from shrike_amd import capi
+from shrike_amd import host as HL
 from shrike_amd import synth as S
 from tests.helpers import Layer, assert_ffn_close, assert_rel_close, f16
 
@@ -530,3 +531,49 @@ def test_batched_decode_operators_equal_the_single_token_ones(gpu, d, f, ne, k, 
     assert_ffn_close(all_acts[:k * f][live0], ref_acts[live0], "token 0 activations")
     ref_y = O.moe_phase2(blobs, off, np.ascontiguousarray(all_acts[:k * f]), h_w[:k].copy(), res_host[:d].copy(), d, f, bits, L.meta)
     assert_ffn_close(all_y[:d], ref_y, "token 0 y from the device's activations")
+
+
+@pytest.mark.parametrize("bits,resident_of_selection", [(4, 5), (8, 0), (4, 8)])
+def test_decode_with_misses_equals_the_resident_layer(gpu, bits, resident_of_selection):
+    """The speculative pass and the agreed fixup: a token whose selection is partly (or wholly) absent from a
+    12-cell pool gives the bytes of the all-resident layer; the next token over the same selection hits."""
+    d, f, ne, k, cells = 512, 256, 32, 8, 12
+    L = Layer(0x5EED0071 + bits, d, f, ne, k, bits=bits)
+    full = DeviceLayer(gpu, L)
+    residual = np.zeros(d, np.uint16)  # no shared expert: the fused layer's residual is zero
+    full.moe.encode_decode_layer(full.layer_args())
+    want_y, want_hidden = full.y.download(np.uint16, d), full.hidden.download(np.uint16, d)
+    want_idx = full.out_idx.download(np.uint32, k)
+    selection = want_idx.tolist()
+    others = [e for e in range(ne) if e not in selection]
+    resident = selection[:resident_of_selection] + others[: cells - resident_of_selection - 2]
+
+    small = DeviceLayer(gpu, L, cells=cells, resident=[])
+    small.moe.stream = gpu.Stream()
+    cache = HL.SlotCache(cells, ne)
+    store = gpu.PinnedBuffer(ne * L.stride)
+    for e in range(ne):
+        store.array[e * L.stride:(e + 1) * L.stride] = L.blobs[e]
+    warm = cache.plan(resident)
+    small.pool.execute_plan(cache, warm, store, L.stride, L.stride)
+    gpu.synchronize()
+    layer = gpu.DecodeLayerWithMisses(small.moe, small.pool, cache, small.off, store, L.stride, L.stride)
+    router = dict(weights=small.router_w, eff_scale=small.eff_scale, expert_scale=small.expert_scale, bias=small.logit_bias)
+    d_res = gpu.dev(residual)
+    layer.run(router, small.x, d_res, small.y, small.hidden)
+    small.moe.stream.synchronize()
+    assert np.array_equal(layer.idx.download(np.uint32, k), want_idx)
+    assert layer.fixups == (0 if resident_of_selection == k else 1)
+    assert np.array_equal(small.y.download(np.uint16, d), want_y)
+    assert np.array_equal(small.hidden.download(np.uint16, d), want_hidden)
+    st = cache.statistics(L.stride)
+    assert st.misses == len(resident) + (k - resident_of_selection) and st.loading_slots == 0
+    assert all(cache.entry(e) >> 32 == capi.RESIDENT for e in selection)
+    assert [small.pool.entry(e) for e in range(ne)] == [cache.entry(e) for e in range(ne)]
+    # the next token over the same selection: no fixup, the same bytes
+    small.hidden.upload(L.hidden)
+    layer.run(router, small.x, d_res, small.y, small.hidden)
+    small.moe.stream.synchronize()
+    assert layer.fixups == (0 if resident_of_selection == k else 1)
+    assert np.array_equal(small.y.download(np.uint16, d), want_y)
+    assert np.array_equal(small.hidden.download(np.uint16, d), want_hidden)
