@@ -433,6 +433,33 @@ def main():
             capi.check(capi.load().shrike_hip_probe_read(stream.handle, lay["pool"].bases, lay["pool"].stride, lay["res"].ptr,
                                                          K, off.gate_w_off, p1_bytes_per_cell, sink.ptr), "probe_read")
 
+    # the step ahead of the layer (residual add + RMS norm producing x): as a launch of its own, and in the
+    # prologue of the layer's first launch; both on a residual stream and an x buffer of their own
+    import ctypes as _C
+    tree_n = S.SeedTree(0x5EED0003)
+    hidden_n, x_n = rt.dev(S.activations_f16(tree_n, "hidden", D)), rt.empty(2 * D)
+    delta_n = rt.dev(S.f32_to_f16_bits(tree_n.key("delta").normal(D, std=0.05)))
+    weight_n = rt.dev(S.f32_to_bf16_bits(tree_n.key("weight").uniform(0.5, 1.5, D)))
+    normed_args = []
+    for lay in layers:
+        apart_a, fused_a = capi.DecodeLayerArgs(), capi.DecodeLayerArgs()
+        for dst in (apart_a, fused_a):
+            _C.memmove(_C.byref(dst), _C.byref(lay["args"]), _C.sizeof(dst))
+            dst.x, dst.hidden = x_n.ptr, hidden_n.ptr
+        fused_a.norm_delta, fused_a.norm_weight, fused_a.norm_eps = delta_n.ptr, weight_n.ptr, 1e-6
+        normed_args.append((apart_a, fused_a))
+
+    def norm_apart():
+        for apart_a, _ in normed_args:
+            rt.residual_add_rmsnorm_bf16w(hidden_n, delta_n, weight_n, x_n, D, 1e-6, 1, stream=stream)
+            moe.encode_decode_layer(apart_a)
+
+    def norm_fused():
+        for _, fused_a in normed_args:
+            moe.encode_decode_layer(fused_a)
+
+    g_norm_apart = capture(rt, capi, stream, norm_apart)
+    g_norm_fused = capture(rt, capi, stream, norm_fused)
     g_empty = capture(rt, capi, stream, empty_only)
     g_read = capture(rt, capi, stream, read_only)
     g_p12 = capture(rt, capi, stream, phase12)
@@ -451,7 +478,8 @@ def main():
     parts = {}
     for name, g, launches_per_layer in (("phase1+phase2 alternating", g_p12, 2), ("phase1", g_p1, 1), ("phase2", g_p2, 1), ("router_select_classify", g_rt, 1),
                                         ("shared_expert(2 launches)", g_sh, 1), ("empty launch of phase 1's grid", g_empty, 1),
-                                        ("read-only kernel over phase 1's bytes", g_read, 1)):
+                                        ("read-only kernel over phase 1's bytes", g_read, 1),
+                                        ("norm launch + layer (4 launches)", g_norm_apart, 4), ("layer with the norm in its first launch", g_norm_fused, 3)):
         time_graph(rt, capi, stream, g, 2)
         parts[name] = time_graph(rt, capi, stream, g, reps) / (reps * n_layers) * 1e3  # us per layer
 

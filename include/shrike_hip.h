@@ -269,6 +269,14 @@ typedef struct {
     void *acts;             /* fp16[top_k*f] */
     void *shared_scratch;   /* fp16[2*shared_f] */
     void *h1;               /* fp16[d] */
+    /* the step ahead of the layer fused into its first launch (residual_add_rmsnorm_bf16w,
+     * RealForwardRunner.swift:2852-2858, rmsnorm.metal:96-130): with norm_weight != NULL,
+     * x = half(half(hidden + norm_delta) * inv * norm_weight) is computed by the call and WRITTEN
+     * to x, and hidden ends as half(half(hidden + norm_delta) + y). norm_delta may be NULL (no add).
+     * Same bits as shrike_hip_residual_add_rmsnorm_bf16w followed by the layer without these fields. */
+    const void *norm_delta;   /* fp16[d] or NULL */
+    const void *norm_weight;  /* bf16[d] or NULL: no fused norm */
+    float norm_eps;
 } shrike_decode_layer_args;
 int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
                                 const shrike_decode_layer_args *args);

@@ -60,7 +60,8 @@ class DecodeLayerArgs(C.Structure):
         ("out_indices", C.c_void_p), ("out_weights", C.c_void_p),
         ("resolved_slots", C.c_void_p), ("hit_count", C.c_void_p), ("hit_positions", C.c_void_p),
         ("miss_count", C.c_void_p), ("miss_positions", C.c_void_p), ("miss_experts", C.c_void_p),
-        ("acts", C.c_void_p), ("shared_scratch", C.c_void_p), ("h1", C.c_void_p)]
+        ("acts", C.c_void_p), ("shared_scratch", C.c_void_p), ("h1", C.c_void_p),
+        ("norm_delta", C.c_void_p), ("norm_weight", C.c_void_p), ("norm_eps", C.c_float)]
 
 
 # name -> (restype, argtypes); every symbol include/shrike_hip.h declares

@@ -48,6 +48,16 @@ struct Phase2Args {
     uint32_t d, f, top_k, meta, ebias;
     const uint32_t *indirect, *io_status;
     uint32_t tokens;  // tokens > 1: grid.y walks tokens; residual, y and hidden rows are d apart
+    const uint16_t *delta;  // fp16[d] or null: hidden = half(half(hidden + delta) + y), the residual add of a norm fused ahead
+};
+
+// The residual add + RMS norm ahead of the layer, done by every workgroup of the head launch for itself:
+// x = norm(hidden + delta) * weight. hidden is read only (phase 2 applies the add); the first workgroup
+// stores x to x_out for the launches that follow.
+struct NormArgs {
+    const uint16_t *hidden, *delta, *weight;
+    uint16_t *x_out;
+    float eps;
 };
 
 int launch_router(const RouterArgs &a, uint32_t router_bits, hipStream_t s);
@@ -55,7 +65,8 @@ int launch_router(const RouterArgs &a, uint32_t router_bits, hipStream_t s);
 constexpr uint32_t kRouterLaunchTokens = 16;  // up to here the one-launch router beats the three-launch prefill router
 int launch_router_tokens(const RouterArgs &a, uint32_t router_bits, uint32_t tokens, hipStream_t s);
 // router logit rows + the shared expert's gate/up rows in one grid
-int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, hipStream_t s);
+// norm: null, or the norm to run in every workgroup's prologue (r.hidden and g.x are then not read)
+int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, const NormArgs *norm, hipStream_t s);
 uint32_t phase1_blocks(uint32_t top_k, uint32_t f);
 // shared_down_bits: 0 = none, else the shared down rows ride in the same grid (one chunk
 // column per lane only: nch_for(shared_f, bits) == 1)

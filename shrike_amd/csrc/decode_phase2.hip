@@ -39,6 +39,9 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     if (finisher) {
         if (residual_tok) res_bits = residual_tok[d0 + threadIdx.x];
         if (hidden_tok) hid_bits = hidden_tok[d0 + threadIdx.x];
+        // the residual add of a norm fused ahead of the layer (rmsnorm.metal:104-108) lands here
+        if (hidden_tok && a.delta)
+            hid_bits = f32_to_f16(__fadd_rn(f16_to_f32(hid_bits), f16_to_f32(a.delta[tok * a.d + d0 + threadIdx.x])));
     }
     if (!io_ready(a.io_status)) {  // moe.metal:1032-1035
         if (finisher) phase2_finish(y_tok, hidden_tok, d0 + threadIdx.x, res_bits, hid_bits);
@@ -293,6 +296,20 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
                    && g->hit_count && g->hit_positions && g->miss_count && g->miss_positions && g->miss_experts
                    && g->acts, "decodeLayer: pool, residency, x, y and the scratch buffers must be bound");
     SHRIKE_REQUIRE(g->pool_slot_stride % 16u == 0, "decodeLayer: pool slot stride must be a multiple of 16");
+    const bool normed = g->norm_weight != nullptr;
+    NormArgs norm = {};
+    if (normed) {  // x = rmsnorm(hidden + delta) * weight is this call's own first step; x is written
+        SHRIKE_REQUIRE(g->hidden, "decodeLayer: a fused norm reads hidden");
+        SHRIKE_REQUIRE(m.d % 8u == 0 && m.d <= SHRIKE_MAX_HIDDEN, "decodeLayer: d=%u is not a row the norm takes", m.d);
+        SHRIKE_REQUIRE(((reinterpret_cast<uintptr_t>(g->hidden) | reinterpret_cast<uintptr_t>(g->norm_delta)
+                         | reinterpret_cast<uintptr_t>(g->norm_weight) | reinterpret_cast<uintptr_t>(g->x)) & 15u) == 0,
+                       "decodeLayer: hidden, delta, norm weight and x must be 16-byte aligned");
+        norm.hidden = static_cast<const uint16_t *>(g->hidden);
+        norm.delta = static_cast<const uint16_t *>(g->norm_delta);
+        norm.weight = static_cast<const uint16_t *>(g->norm_weight);
+        norm.x_out = static_cast<uint16_t *>(const_cast<void *>(g->x));
+        norm.eps = g->norm_eps;
+    }
     hipStream_t s = as_stream(stream);
     const bool shared = g->shared_gate.weights != nullptr;
     const uint32_t sbits = g->shared_bits ? g->shared_bits : m.routed_weight_bits;
@@ -333,11 +350,15 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
     if (shared) {
         GemvArgs gu = {};
         fill_gemv_gate_up(gu, &g->shared_gate, &g->shared_up, gate_out, up_out, g->shared_f, m.d, m.meta_dtype, g->x);
-        if (int rc = launch_head(r, m.router_weight_bits, gu, sbits, s)) return rc;
+        if (int rc = launch_head(r, m.router_weight_bits, gu, sbits, normed ? &norm : nullptr, s)) return rc;
         fill_gemv_down(p1.shared_down, &g->shared_down, gate_out, up_out, g->h1, m.d, g->shared_f, m.meta_dtype,
                        m.activation, g->shared_scalar_gate);
         down_fused = nch_for(g->shared_f, sbits) == 1;
         residual = g->h1;
+    } else if (normed) {  // the head launch with router rows only
+        GemvArgs none = {};
+        none.n = m.d;
+        if (int rc = launch_head(r, m.router_weight_bits, none, sbits, &norm, s)) return rc;
     } else {
         if (int rc = launch_router(r, m.router_weight_bits, s)) return rc;
     }
@@ -353,6 +374,7 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
     p.residual = static_cast<const uint16_t *>(residual);
     p.y = static_cast<uint16_t *>(g->y); p.hidden = static_cast<uint16_t *>(g->hidden);
     p.d = m.d; p.f = m.f; p.top_k = m.top_k; p.meta = m.meta_dtype; p.ebias = m.expert_additive_biases;
+    p.delta = normed ? norm.delta : nullptr;
     return launch_phase2(p, m.routed_weight_bits, s);
 }
 

@@ -1,6 +1,7 @@
 // Router logits, top-k select and residency classification for gfx950, and the head
 // launch of the fused layer (router rows beside the shared expert's gate/up rows).
 #include "decode_launch.h"
+#include "rmsnorm_row.h"
 #include "router_row.h"
 
 namespace shrike {
@@ -40,14 +41,30 @@ __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
 }
 
 // The head of the fused layer: the router's logit rows and, beside them in the same grid,
-// the shared expert's gate and up rows. Neither depends on the other.
-template <int RK, int BITS, int NCH>
-__global__ __launch_bounds__(256) void k_head(RouterArgs r, GemvArgs g, uint32_t router_blocks) {
+// the shared expert's gate and up rows. Neither depends on the other. NORM: every workgroup first
+// computes the layer's input row itself (residual add + RMS norm, rmsnorm.metal:96-130) into LDS and
+// reads it from there; workgroup 0 also stores it for phase 1.
+template <int RK, int BITS, int NCH, bool NORM>
+__global__ __launch_bounds__(256) void k_head(RouterArgs r, GemvArgs g, uint32_t router_blocks, NormArgs n) {
+    __shared__ uint4 s_x[NORM ? SHRIKE_MAX_HIDDEN / 8 : 1];
+    __shared__ float s_partial[4];
+    // the norm runs behind the rows' own loads, which do not depend on it
+    auto normed_row = [&]() -> const uint4 * {
+        rmsnorm_row<false>(const_cast<uint16_t *>(n.hidden), n.delta, n.weight, blockIdx.x == 0 ? n.x_out : nullptr, s_x, r.d, n.eps,
+                           s_partial);
+        return s_x;
+    };
     if (blockIdx.x < router_blocks) {
         const uint32_t e = blockIdx.x * 4u + wave_index();
-        if (e < r.sel.num_experts) router_row<RK>(r, e, threadIdx.x & 63u);
+        if (e < r.sel.num_experts) {
+            if (NORM) router_row<RK>(r, [&] { return reinterpret_cast<const uint16_t *>(normed_row()); }, r.logits_out, e, threadIdx.x & 63u, false);
+            else router_row<RK>(r, e, threadIdx.x & 63u);
+        } else if (NORM) {
+            normed_row();  // the workgroup's barriers need every wave
+        }
     } else {
-        gemv_job<BITS, NCH>(g, blockIdx.x - router_blocks);
+        if (NORM) gemv_job<BITS, NCH>(g, blockIdx.x - router_blocks, normed_row);
+        else gemv_job<BITS, NCH>(g, blockIdx.x - router_blocks);
     }
 }
 
@@ -133,27 +150,42 @@ int launch_router_tokens(const RouterArgs &a, uint32_t router_bits, uint32_t tok
 }
 
 template <int RK, int BITS>
-static void launch_head_nch(const RouterArgs &r, const GemvArgs &g, uint32_t router_blocks, dim3 grid, hipStream_t s) {
+static void launch_head_nch(const RouterArgs &r, const GemvArgs &g, uint32_t router_blocks, dim3 grid, const NormArgs *norm,
+                            hipStream_t s) {
     const dim3 block(256);
-    switch (nch_for(g.n, BITS)) {
-        case 1: hipLaunchKernelGGL((k_head<RK, BITS, 1>), grid, block, 0, s, r, g, router_blocks); break;
-        case 2: hipLaunchKernelGGL((k_head<RK, BITS, 2>), grid, block, 0, s, r, g, router_blocks); break;
-        case 3: hipLaunchKernelGGL((k_head<RK, BITS, 3>), grid, block, 0, s, r, g, router_blocks); break;
-        default: hipLaunchKernelGGL((k_head<RK, BITS, 4>), grid, block, 0, s, r, g, router_blocks); break;
+    const NormArgs n = norm ? *norm : NormArgs{};
+    const uint32_t nch = nch_for(g.n, BITS);
+    if (norm) {
+        switch (nch) {
+            case 1: hipLaunchKernelGGL((k_head<RK, BITS, 1, true>), grid, block, 0, s, r, g, router_blocks, n); break;
+            case 2: hipLaunchKernelGGL((k_head<RK, BITS, 2, true>), grid, block, 0, s, r, g, router_blocks, n); break;
+            case 3: hipLaunchKernelGGL((k_head<RK, BITS, 3, true>), grid, block, 0, s, r, g, router_blocks, n); break;
+            default: hipLaunchKernelGGL((k_head<RK, BITS, 4, true>), grid, block, 0, s, r, g, router_blocks, n); break;
+        }
+    } else {
+        switch (nch) {
+            case 1: hipLaunchKernelGGL((k_head<RK, BITS, 1, false>), grid, block, 0, s, r, g, router_blocks, n); break;
+            case 2: hipLaunchKernelGGL((k_head<RK, BITS, 2, false>), grid, block, 0, s, r, g, router_blocks, n); break;
+            case 3: hipLaunchKernelGGL((k_head<RK, BITS, 3, false>), grid, block, 0, s, r, g, router_blocks, n); break;
+            default: hipLaunchKernelGGL((k_head<RK, BITS, 4, false>), grid, block, 0, s, r, g, router_blocks, n); break;
+        }
     }
 }
 
-int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, hipStream_t s) {
+// g.rows + g.rows_b == 0: router rows only (g.n must still be a valid row length)
+int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, const NormArgs *norm,
+                hipStream_t s) {
     const uint32_t router_blocks = (r.sel.num_experts + 3) / 4;
-    const dim3 grid(router_blocks + gemv_blocks(g.rows + g.rows_b, g.n, shared_bits));
+    const uint32_t shared_rows = g.rows + g.rows_b;
+    const dim3 grid(router_blocks + (shared_rows ? gemv_blocks(shared_rows, g.n, shared_bits) : 0u));
     if (shared_bits == 4) {
-        if (router_bits == 0) launch_head_nch<0, 4>(r, g, router_blocks, grid, s);
-        else if (router_bits == 8) launch_head_nch<8, 4>(r, g, router_blocks, grid, s);
-        else launch_head_nch<4, 4>(r, g, router_blocks, grid, s);
+        if (router_bits == 0) launch_head_nch<0, 4>(r, g, router_blocks, grid, norm, s);
+        else if (router_bits == 8) launch_head_nch<8, 4>(r, g, router_blocks, grid, norm, s);
+        else launch_head_nch<4, 4>(r, g, router_blocks, grid, norm, s);
     } else {
-        if (router_bits == 0) launch_head_nch<0, 8>(r, g, router_blocks, grid, s);
-        else if (router_bits == 8) launch_head_nch<8, 8>(r, g, router_blocks, grid, s);
-        else launch_head_nch<4, 8>(r, g, router_blocks, grid, s);
+        if (router_bits == 0) launch_head_nch<0, 8>(r, g, router_blocks, grid, norm, s);
+        else if (router_bits == 8) launch_head_nch<8, 8>(r, g, router_blocks, grid, norm, s);
+        else launch_head_nch<4, 8>(r, g, router_blocks, grid, norm, s);
     }
     SHRIKE_HIP(hipGetLastError());
     return 0;

@@ -9,6 +9,8 @@
 // so the loads stay back to back.
 #pragma once
 
+#include <type_traits>
+
 #include "device_utils.h"
 #include "host_common.h"
 
@@ -175,10 +177,16 @@ struct GemvArgs {
 
 constexpr uint32_t kGemvRowsPerWave = 4;
 
+struct NoXSource {  // gemv_job's input is a.x (or the GLU of gate_in and up_in)
+    __device__ const uint4 *operator()() const { return nullptr; }
+};
+
 // dequant_int4.metal:101-199 / dequant_int8.metal:66-107: y[row] = half(W[row,:] . x), the
 // work of workgroup `block` of a grid of 256-thread workgroups.
-template <int BITS, int NCH>
-__device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block) {
+// x_source(): called by every thread once the rows' own loads are in flight; returns the input row to read
+// in place of a.x, or null for a.x (it may first have to produce the row behind a barrier).
+template <int BITS, int NCH, class XSource>
+__device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block, XSource &&x_source) {
     typedef Chunk<BITS> C;
     const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t cpr = a.n * BITS / 128u, groups = a.n / kGroup, row_bytes = cpr * 16u;
@@ -192,7 +200,8 @@ __device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block) {
 
     // the input slice first: in-order load return must not hold it behind the rows
     SliceRegs<BITS, NCH> xin;
-    if (!a.gate_in && active) load_slice_regs<BITS, NCH>(xin, reinterpret_cast<const uint4 *>(a.x), cpr, col, true);
+    constexpr bool kPlainX = std::is_same<typename std::decay<XSource>::type, NoXSource>::value;
+    if (kPlainX && !a.gate_in && active) load_slice_regs<BITS, NCH>(xin, reinterpret_cast<const uint4 *>(a.x), cpr, col, true);
     uint16_t gate_bits = 0;
     if (a.scalar_gate) gate_bits = a.scalar_gate[0];
 
@@ -212,7 +221,10 @@ __device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block) {
                                 (second ? a.b_b : a.b_a) + size_t(local) * groups, cpr, col, on[j]);
         }
     }
-    if (a.gate_in) {
+    if (!kPlainX) {
+        const uint4 *x_row = x_source();
+        if (active) load_slice_regs<BITS, NCH>(xin, x_row, cpr, col, true);
+    } else if (a.gate_in) {
         // dequant_int4.metal:283-287: act = half(glu(gate, up)) once per workgroup, staged in LDS
         __shared__ uint4 act_l[SHRIKE_MAX_HIDDEN / 8];
         for (uint32_t p = threadIdx.x; p < a.n / 8u; p += 256u) {
@@ -245,6 +257,11 @@ __device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block) {
             (second ? a.y_b : a.y_a)[second ? row[j] - a.rows : row[j]] = yh;
         }
     }
+}
+
+template <int BITS, int NCH>
+__device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block) {
+    gemv_job<BITS, NCH>(a, block, NoXSource{});
 }
 
 inline uint32_t nch_for(uint32_t n, uint32_t bits) { return (n * bits / 128u + 63u) / 64u; }

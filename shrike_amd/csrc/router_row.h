@@ -11,8 +11,11 @@ namespace shrike {
 // fixed so that the fp32 logits are reproducible bit for bit (lane l takes chunks
 // l, l+64, ...).
 // hidden, logits: the token's activation row and its logit row (a.hidden, a.logits_out for one token)
-template <int RK>
-__device__ __forceinline__ void router_row(const RouterArgs &a, const uint16_t *hidden, float *logits, uint32_t e, uint32_t lane,
+// x_source(): called once the row's own loads are in flight; returns the activation row to read (it may
+// first have to produce it, e.g. a norm into LDS behind a barrier — then every wave of the workgroup
+// must come through here or call it by itself).
+template <int RK, class XSource>
+__device__ __forceinline__ void router_row(const RouterArgs &a, XSource &&x_source, float *logits, uint32_t e, uint32_t lane,
                                            bool publish) {
     constexpr int E = RK == 0 ? 8 : RK == 8 ? 16 : 32;  // elements per 16-byte weight chunk
     constexpr int PIECES = E / 8;
@@ -29,14 +32,19 @@ __device__ __forceinline__ void router_row(const RouterArgs &a, const uint16_t *
         const uint32_t cc = c < chunks ? c : 0u;
         w[i] = *reinterpret_cast<const uint4 *>(row + 16u * cc);
 #pragma unroll
-        for (int j = 0; j < PIECES; ++j) {
-            xv[i][j] = reinterpret_cast<const uint4 *>(hidden)[cc * PIECES + j];
-            ev[i][j] = reinterpret_cast<const uint4 *>(a.effective_scale)[cc * PIECES + j];
-        }
+        for (int j = 0; j < PIECES; ++j) ev[i][j] = reinterpret_cast<const uint4 *>(a.effective_scale)[cc * PIECES + j];
         if (RK != 0) {
             sc[i] = a.scales[size_t(e) * groups + cc * E / kGroup];
             bi[i] = a.biases[size_t(e) * groups + cc * E / kGroup];
         }
+    }
+    const uint16_t *hidden = x_source();
+#pragma unroll
+    for (int i = 0; i < MAXI; ++i) {
+        const uint32_t c = lane + 64u * i;
+        const uint32_t cc = c < chunks ? c : 0u;
+#pragma unroll
+        for (int j = 0; j < PIECES; ++j) xv[i][j] = reinterpret_cast<const uint4 *>(hidden)[cc * PIECES + j];
     }
     float acc = 0.0f;
 #pragma unroll
@@ -83,6 +91,12 @@ __device__ __forceinline__ void router_row(const RouterArgs &a, const uint16_t *
         if (publish) __hip_atomic_store(logits + e, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else logits[e] = acc;
     }
+}
+
+template <int RK>
+__device__ __forceinline__ void router_row(const RouterArgs &a, const uint16_t *hidden, float *logits, uint32_t e, uint32_t lane,
+                                           bool publish) {
+    router_row<RK>(a, [&] { return hidden; }, logits, e, lane, publish);
 }
 
 template <int RK>

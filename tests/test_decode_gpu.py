@@ -577,3 +577,45 @@ def test_decode_with_misses_equals_the_resident_layer(gpu, bits, resident_of_sel
     assert layer.fixups == (0 if resident_of_selection == k else 1)
     assert np.array_equal(small.y.download(np.uint16, d), want_y)
     assert np.array_equal(small.hidden.download(np.uint16, d), want_hidden)
+
+
+@pytest.mark.parametrize("d,f,ne,k,fs,rbits,bits,with_delta", [
+    (2048, 512, 64, 8, 512, 0, 4, True),     # the headline shape with fewer experts
+    (256, 128, 16, 4, 0, 0, 4, True),        # no shared expert: the head launch carries router rows only
+    (2880, 192, 32, 4, 0, 8, 8, False),      # ragged rows, affine router, no residual add
+    (512, 256, 32, 8, 256, 4, 4, True),
+])
+def test_decode_layer_with_the_norm_fused_ahead(gpu, d, f, ne, k, fs, rbits, bits, with_delta):
+    """residual_add_rmsnorm_bf16w in the head launch's prologue: x, routes, acts, y and the residual stream
+    equal, bit for bit, the stand-alone norm kernel followed by the layer."""
+    L = Layer(0x5EED0081 + d, d, f, ne, k, bits=bits, router_bits=rbits, shared_f=fs)
+    delta = S.f32_to_f16_bits(L.tree.key("norm.delta").normal(d, std=0.5))
+    weight = S.f32_to_bf16_bits(L.tree.key("norm.weight").uniform(0.5, 1.5, d))
+    eps = 1e-6
+    d_delta, d_weight = gpu.dev(delta), gpu.dev(weight)
+
+    apart = DeviceLayer(gpu, L)
+    gpu.residual_add_rmsnorm_bf16w(apart.hidden, d_delta if with_delta else None, d_weight, apart.x, d, eps, 1)
+    apart.moe.encode_decode_layer(apart.layer_args())
+
+    fused = DeviceLayer(gpu, L)
+    fused.x.fill(0x5A)
+    args = fused.layer_args()
+    args.norm_delta = d_delta.ptr if with_delta else None
+    args.norm_weight, args.norm_eps = d_weight.ptr, eps
+    fused.moe.encode_decode_layer(args)
+    gpu.synchronize()
+
+    want_hidden = L.hidden.copy()
+    want_x = O.residual_add_rmsnorm_bf16w(want_hidden, delta if with_delta else None, weight, eps)
+    assert np.array_equal(fused.x.download(np.uint16, d), want_x), "the normalised row differs from the oracle's"
+    for name, count, dtype in (("x", d, np.uint16), ("out_idx", k, np.uint32), ("out_w", k, np.uint16),
+                               ("acts", k * f, np.uint16), ("y", d, np.uint16), ("hidden", d, np.uint16)):
+        assert np.array_equal(getattr(fused, name).download(dtype, count), getattr(apart, name).download(dtype, count)), name
+    y = fused.y.download(np.uint16, d)
+    assert np.array_equal(fused.hidden.download(np.uint16, d), O.residual_add_f16(want_hidden, y))
+    # a second call on the same buffers is a second step of the residual stream, not a repeat of the first
+    fused.moe.encode_decode_layer(args)
+    gpu.residual_add_rmsnorm_bf16w(apart.hidden, d_delta if with_delta else None, d_weight, apart.x, d, eps, 1)
+    apart.moe.encode_decode_layer(apart.layer_args())
+    assert np.array_equal(fused.hidden.download(np.uint16, d), apart.hidden.download(np.uint16, d))
