@@ -32,9 +32,9 @@ __global__ __launch_bounds__(256) void k_prefill_logits(RouterArgs a, uint32_t q
 
 // The fp16 router's fast path. x * effective_scale is the same for every expert, so it is
 // formed once per token (k_prefill_scale_x, the product router_row forms per row); a wave
-// then keeps its expert's row in registers as fp32 and walks a block of tokens, two at a time.
-// The additions are router_row's, in router_row's order, so the logits are the same bits.
-constexpr uint32_t kFastTokenBlock = 32;
+// then keeps its experts' rows in registers and walks a block of tokens, the next token's x in flight
+// while one is multiplied. The additions are router_row's, in router_row's order, so the logits are
+// the same bits.
 
 __global__ __launch_bounds__(256) void k_prefill_scale_x(const uint16_t *hidden, const uint16_t *eff, float *xs,
                                                          uint32_t query_count, uint32_t d, uint32_t stride) {
@@ -57,84 +57,90 @@ __global__ __launch_bounds__(256) void k_prefill_scale_x(const uint16_t *hidden,
     dst[1] = make_float4(o[4], o[5], o[6], o[7]);
 }
 
-// A wave keeps ROWS fp16 router rows as fp32 in registers (MAXI 16-byte chunks a lane and row)
-// and walks a block of tokens two at a time: every x value fetched from L2 feeds ROWS rows, and
-// every logit is summed in the decode router's order (lane l: chunks l, l+64, ..., xor butterfly).
-template <int MAXI, int ROWS>
+// A wave keeps ROWS fp16 router rows in registers (MAXI 16-byte chunks a lane and row) and walks a
+// block of TOKENS tokens: every x value fetched from L2 feeds ROWS rows, and every logit is summed in
+// the decode router's order (lane l: chunks l, l+64, ..., xor butterfly).
+template <int MAXI, int ROWS, uint32_t TOKENS>
 __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits,
                                                             uint32_t query_count, uint32_t num_experts, uint32_t d) {
     const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t e0 = (blockIdx.x * 4u + wave) * ROWS;
     if (e0 >= num_experts) return;
     const uint32_t chunks = d / 8u;
-    float w[ROWS][MAXI][8];
+    // the rows stay packed: a multiply-add that takes its fp16 factor as it is (v_fma_mix_f32) widens it
+    // exactly, so the sums are those of converting first, and a row costs half the registers
+    uint4 w[ROWS][MAXI];
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
         const uint32_t e = min(e0 + uint32_t(r), num_experts - 1u);  // past the last row: a copy, never stored
 #pragma unroll
         for (int i = 0; i < MAXI; ++i) {
             const uint32_t c = lane + 64u * i;
-            const uint4 v = *reinterpret_cast<const uint4 *>(weights + size_t(e) * d + size_t(c < chunks ? c : 0u) * 8u);
-            const uint32_t ww[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                w[r][i][2 * j] = f16_to_f32(uint16_t(ww[j]));
-                w[r][i][2 * j + 1] = f16_to_f32(uint16_t(ww[j] >> 16));
-            }
+            w[r][i] = *reinterpret_cast<const uint4 *>(weights + size_t(e) * d + size_t(c < chunks ? c : 0u) * 8u);
         }
     }
-    const uint32_t t0 = blockIdx.y * kFastTokenBlock;
-    const uint32_t t1 = min(t0 + kFastTokenBlock, query_count);
-    for (uint32_t t = t0; t < t1; t += 2u) {
-        const bool two = t + 1u < t1;
-        const float *row[2] = {xs + size_t(t) * d, xs + size_t(two ? t + 1u : t) * d};
-        float acc[2][ROWS];
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r) acc[0][r] = acc[1][r] = 0.0f;
+    const uint32_t t0 = blockIdx.y * TOKENS;
+    const uint32_t t1 = min(t0 + TOKENS, query_count);
+    // one token a step, the next token's x in flight while this one is multiplied
+    float4 xa[MAXI][2], xb[MAXI][2];
+    auto fetch = [&](float4 (&x)[MAXI][2], uint32_t t) {
+        const float *row = xs + size_t(min(t, t1 - 1u)) * d;
 #pragma unroll
         for (int i = 0; i < MAXI; ++i) {
             const uint32_t c = lane + 64u * i;
-            if (c < chunks) {
-                float4 x[2][2];
+            const uint32_t cc = c < chunks ? c : 0u;
+            x[i][0] = reinterpret_cast<const float4 *>(row + size_t(cc) * 8u)[0];
+            x[i][1] = reinterpret_cast<const float4 *>(row + size_t(cc) * 8u)[1];
+        }
+    };
+    auto token = [&](const float4 (&x)[MAXI][2], uint32_t t) {
+        float acc[ROWS];
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    x[u][0] = reinterpret_cast<const float4 *>(row[u] + size_t(c) * 8u)[0];
-                    x[u][1] = reinterpret_cast<const float4 *>(row[u] + size_t(c) * 8u)[1];
-                }
+        for (int r = 0; r < ROWS; ++r) acc[r] = 0.0f;
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const float xv[8] = {x[u][0].x, x[u][0].y, x[u][0].z, x[u][0].w, x[u][1].x, x[u][1].y, x[u][1].z, x[u][1].w};
+        for (int i = 0; i < MAXI; ++i) {
+            if (lane + 64u * i < chunks) {
+                const float xv[8] = {x[i][0].x, x[i][0].y, x[i][0].z, x[i][0].w, x[i][1].x, x[i][1].y, x[i][1].z, x[i][1].w};
 #pragma unroll
-                    for (int r = 0; r < ROWS; ++r)
+                for (int r = 0; r < ROWS; ++r) {
+                    uint32_t ww[4] = {w[r][i].x, w[r][i].y, w[r][i].z, w[r][i].w};
+                    // the widening belongs to the multiply-add: keep it from being hoisted out of the token loop
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) acc[u][r] = fmaf(w[r][i][j], xv[j], acc[u][r]);
+                    for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(ww[q]));
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[r] = fmaf(f16_to_f32(uint16_t(ww[j / 2] >> (16 * (j % 2)))), xv[j], acc[r]);
                 }
             }
         }
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1)
 #pragma unroll
-            for (int r = 0; r < ROWS; ++r) {
-                acc[0][r] = __fadd_rn(acc[0][r], __shfl_xor(acc[0][r], o));
-                acc[1][r] = __fadd_rn(acc[1][r], __shfl_xor(acc[1][r], o));
-            }
+            for (int r = 0; r < ROWS; ++r) acc[r] = __fadd_rn(acc[r], __shfl_xor(acc[r], o));
         if (lane == 0) {
 #pragma unroll
-            for (int r = 0; r < ROWS; ++r) {
-                if (e0 + uint32_t(r) >= num_experts) break;
-                logits[size_t(t) * num_experts + e0 + r] = acc[0][r];
-                if (two) logits[size_t(t + 1u) * num_experts + e0 + r] = acc[1][r];
-            }
+            for (int r = 0; r < ROWS; ++r)
+                if (e0 + uint32_t(r) < num_experts) logits[size_t(t) * num_experts + e0 + r] = acc[r];
+        }
+    };
+    fetch(xa, t0);
+    for (uint32_t t = t0; t < t1; t += 2u) {
+        fetch(xb, t + 1u);
+        token(xa, t);
+        if (t + 1u < t1) {
+            fetch(xa, t + 2u);
+            token(xb, t + 1u);
         }
     }
 }
+
+constexpr uint32_t kLogitTokens = 8;  // tokens a wave walks with its rows: small blocks, many workgroups
 
 template <int MAXI, int ROWS>
 static void launch_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits, uint32_t query_count,
                                       uint32_t num_experts, uint32_t d, hipStream_t s) {
     const uint32_t per_block = 4u * ROWS;
-    hipLaunchKernelGGL((k_prefill_logits_f16<MAXI, ROWS>),
-                       dim3((num_experts + per_block - 1u) / per_block, (query_count + kFastTokenBlock - 1u) / kFastTokenBlock),
+    hipLaunchKernelGGL((k_prefill_logits_f16<MAXI, ROWS, kLogitTokens>),
+                       dim3((num_experts + per_block - 1u) / per_block, (query_count + kLogitTokens - 1u) / kLogitTokens),
                        dim3(256), 0, s, weights, xs, logits, query_count, num_experts, d);
 }
 
@@ -438,9 +444,9 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
             hipLaunchKernelGGL(k_prefill_scale_x, dim3(uint32_t((slots + 255u) / 256u)), dim3(256), 0, s, a.hidden, a.effective_scale,
                                xs, query_count, d, hidden_stride_elements);
             SHRIKE_HIP(hipGetLastError());
-            // two rows a wave: half the x traffic of one; more rows leave too few waves to hide the loads
+            // four packed rows a wave where they fit beside two tokens' x: a quarter of the x traffic of one row
             const uint16_t *w16 = static_cast<const uint16_t *>(d_weights);
-            if (d <= 2048u) launch_prefill_logits_f16<4, 2>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
+            if (d <= 2048u) launch_prefill_logits_f16<4, 4>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
             else if (d <= 3072u) launch_prefill_logits_f16<6, 2>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
             else launch_prefill_logits_f16<8, 2>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
             break;
