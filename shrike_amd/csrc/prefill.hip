@@ -57,15 +57,19 @@ __global__ __launch_bounds__(256) void k_prefill_scale_x(const uint16_t *hidden,
     dst[1] = make_float4(o[4], o[5], o[6], o[7]);
 }
 
-// A wave keeps ROWS fp16 router rows in registers (MAXI 16-byte chunks a lane and row) and walks a
-// block of TOKENS tokens: every x value fetched from L2 feeds ROWS rows, and every logit is summed in
-// the decode router's order (lane l: chunks l, l+64, ..., xor butterfly).
-template <int MAXI, int ROWS, uint32_t TOKENS>
+// A wave keeps ROWS fp16 router rows in registers (MAXI 16-byte chunks a lane and row); the workgroup
+// walks a block of TOKENS tokens, TPS of them a step: their x rows are staged once in LDS (the next
+// step's in flight while one is multiplied) for the four waves to read, and the TPS * ROWS sums of a step
+// go through the butterfly side by side. Every logit is summed in the decode router's order (lane l:
+// chunks l, l+64, ..., xor butterfly).
+template <int MAXI, int ROWS, uint32_t TOKENS, uint32_t TPS>
 __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits,
                                                             uint32_t query_count, uint32_t num_experts, uint32_t d) {
+    // chunk c = lane + 64 i of a row is two float4: half h of it sits at [(2 i + h) * 64 + lane], so that a
+    // wave's read of one half is one contiguous kilobyte
+    __shared__ float4 s_x[2][TPS][MAXI * 2 * 64];
     const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t e0 = (blockIdx.x * 4u + wave) * ROWS;
-    if (e0 >= num_experts) return;
     const uint32_t chunks = d / 8u;
     // the rows stay packed: a multiply-add that takes its fp16 factor as it is (v_fma_mix_f32) widens it
     // exactly, so the sums are those of converting first, and a row costs half the registers
@@ -81,65 +85,100 @@ __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weig
     }
     const uint32_t t0 = blockIdx.y * TOKENS;
     const uint32_t t1 = min(t0 + TOKENS, query_count);
-    // one token a step, the next token's x in flight while this one is multiplied
-    float4 xa[MAXI][2], xb[MAXI][2];
-    auto fetch = [&](float4 (&x)[MAXI][2], uint32_t t) {
-        const float *row = xs + size_t(min(t, t1 - 1u)) * d;
+    if (t0 >= t1) return;
+    constexpr int kStage = MAXI * 2 * 64 / 256;  // float4 a thread stages per token
+    static_assert(kStage >= 1 && kStage <= 4, "a thread stages one to four float4 a token");
+    const uint32_t quads = d / 4u;
+    auto quad = [&](int j) { return min(threadIdx.x + 256u * uint32_t(j), quads - 1u); };  // past the row: a copy, never stored
+    auto stage_load = [&](float4 (&st)[TPS][4], uint32_t t) {
 #pragma unroll
-        for (int i = 0; i < MAXI; ++i) {
-            const uint32_t c = lane + 64u * i;
-            const uint32_t cc = c < chunks ? c : 0u;
-            x[i][0] = reinterpret_cast<const float4 *>(row + size_t(cc) * 8u)[0];
-            x[i][1] = reinterpret_cast<const float4 *>(row + size_t(cc) * 8u)[1];
+        for (uint32_t u = 0; u < TPS; ++u) {
+            const float4 *row = reinterpret_cast<const float4 *>(xs + size_t(min(t + u, t1 - 1u)) * d);
+            st[u][0] = row[quad(0)];
+            if (kStage > 1) st[u][1] = row[quad(1)];
+            if (kStage > 2) st[u][2] = row[quad(2)];
+            if (kStage > 3) st[u][3] = row[quad(3)];
         }
     };
-    auto token = [&](const float4 (&x)[MAXI][2], uint32_t t) {
-        float acc[ROWS];
+    auto put = [&](uint32_t buf, uint32_t u, int j, float4 v) {
+        const uint32_t q = threadIdx.x + 256u * uint32_t(j);
+        const uint32_t c = q >> 1, h = q & 1u;
+        if (q < quads) s_x[buf][u][(2u * (c >> 6) + h) * 64u + (c & 63u)] = v;
+    };
+    auto stage_store = [&](const float4 (&st)[TPS][4], uint32_t buf) {
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) acc[r] = 0.0f;
+        for (uint32_t u = 0; u < TPS; ++u) {
+            put(buf, u, 0, st[u][0]);
+            if (kStage > 1) put(buf, u, 1, st[u][1]);
+            if (kStage > 2) put(buf, u, 2, st[u][2]);
+            if (kStage > 3) put(buf, u, 3, st[u][3]);
+        }
+    };
+    auto step = [&](uint32_t buf, uint32_t t) {
+        float acc[TPS][ROWS];
+#pragma unroll
+        for (uint32_t u = 0; u < TPS; ++u)
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) acc[u][r] = 0.0f;
 #pragma unroll
         for (int i = 0; i < MAXI; ++i) {
             if (lane + 64u * i < chunks) {
-                const float xv[8] = {x[i][0].x, x[i][0].y, x[i][0].z, x[i][0].w, x[i][1].x, x[i][1].y, x[i][1].z, x[i][1].w};
+                uint32_t ww[ROWS][4];
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
-                    uint32_t ww[4] = {w[r][i].x, w[r][i].y, w[r][i].z, w[r][i].w};
+                    ww[r][0] = w[r][i].x; ww[r][1] = w[r][i].y; ww[r][2] = w[r][i].z; ww[r][3] = w[r][i].w;
                     // the widening belongs to the multiply-add: keep it from being hoisted out of the token loop
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(ww[q]));
+                    for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(ww[r][q]));
+                }
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) acc[r] = fmaf(f16_to_f32(uint16_t(ww[j / 2] >> (16 * (j % 2)))), xv[j], acc[r]);
+                for (uint32_t u = 0; u < TPS; ++u) {
+                    const float4 x0 = s_x[buf][u][(2 * i) * 64 + lane], x1 = s_x[buf][u][(2 * i + 1) * 64 + lane];
+                    const float xv[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+                    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            acc[u][r] = fmaf(f16_to_f32(uint16_t(ww[r][j / 2] >> (16 * (j % 2)))), xv[j], acc[u][r]);
                 }
             }
         }
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1)
 #pragma unroll
-            for (int r = 0; r < ROWS; ++r) acc[r] = __fadd_rn(acc[r], __shfl_xor(acc[r], o));
+            for (uint32_t u = 0; u < TPS; ++u)
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) acc[u][r] = __fadd_rn(acc[u][r], __shfl_xor(acc[u][r], o));
         if (lane == 0) {
 #pragma unroll
-            for (int r = 0; r < ROWS; ++r)
-                if (e0 + uint32_t(r) < num_experts) logits[size_t(t) * num_experts + e0 + r] = acc[r];
+            for (uint32_t u = 0; u < TPS; ++u)
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r)
+                    if (t + u < t1 && e0 + uint32_t(r) < num_experts) logits[size_t(t + u) * num_experts + e0 + r] = acc[u][r];
         }
     };
-    fetch(xa, t0);
-    for (uint32_t t = t0; t < t1; t += 2u) {
-        fetch(xb, t + 1u);
-        token(xa, t);
-        if (t + 1u < t1) {
-            fetch(xa, t + 2u);
-            token(xb, t + 1u);
-        }
+    float4 staged[TPS][4];  // live across a step's arithmetic; handed to the lambdas as a parameter so it stays in registers
+    stage_load(staged, t0);
+    stage_store(staged, 0);
+    __syncthreads();
+    uint32_t buf = 0;
+    for (uint32_t t = t0; t < t1; t += TPS, buf ^= 1u) {
+        const bool more = t + TPS < t1;
+        if (more) stage_load(staged, t + TPS);
+        step(buf, t);
+        if (more) stage_store(staged, buf ^ 1u);
+        __syncthreads();
     }
 }
 
-constexpr uint32_t kLogitTokens = 8;  // tokens a wave walks with its rows: small blocks, many workgroups
+constexpr uint32_t kLogitTokens = 8;  // tokens a workgroup walks with its rows: small blocks, many workgroups
+constexpr uint32_t kLogitTokensPerStep = 2;
 
 template <int MAXI, int ROWS>
 static void launch_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits, uint32_t query_count,
                                       uint32_t num_experts, uint32_t d, hipStream_t s) {
     const uint32_t per_block = 4u * ROWS;
-    hipLaunchKernelGGL((k_prefill_logits_f16<MAXI, ROWS, kLogitTokens>),
+    hipLaunchKernelGGL((k_prefill_logits_f16<MAXI, ROWS, kLogitTokens, kLogitTokensPerStep>),
                        dim3((num_experts + per_block - 1u) / per_block, (query_count + kLogitTokens - 1u) / kLogitTokens),
                        dim3(256), 0, s, weights, xs, logits, query_count, num_experts, d);
 }
