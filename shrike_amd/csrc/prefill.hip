@@ -30,32 +30,10 @@ __global__ __launch_bounds__(256) void k_prefill_logits(RouterArgs a, uint32_t q
     }
 }
 
-// The fp16 router's fast path. x * effective_scale is the same for every expert, so it is
-// formed once per token (k_prefill_scale_x, the product router_row forms per row); a wave
-// then keeps its experts' rows in registers and walks a block of tokens, the next token's x in flight
-// while one is multiplied. The additions are router_row's, in router_row's order, so the logits are
-// the same bits.
-
-__global__ __launch_bounds__(256) void k_prefill_scale_x(const uint16_t *hidden, const uint16_t *eff, float *xs,
-                                                         uint32_t query_count, uint32_t d, uint32_t stride) {
-    const size_t slot = size_t(blockIdx.x) * 256u + threadIdx.x;  // eight elements each
-    const uint32_t per_row = d / 8u;
-    const uint32_t t = uint32_t(slot / per_row);
-    if (t >= query_count) return;
-    const uint32_t c = uint32_t(slot - size_t(t) * per_row);
-    const uint4 xv = *reinterpret_cast<const uint4 *>(hidden + size_t(t) * stride + size_t(c) * 8u);
-    const uint4 ev = *reinterpret_cast<const uint4 *>(eff + size_t(c) * 8u);
-    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, ew[4] = {ev.x, ev.y, ev.z, ev.w};
-    float o[8];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {  // moe.metal:357-358 (exact product)
-        o[2 * j] = __fmul_rn(f16_to_f32(uint16_t(xw[j])), bf16_to_f32(uint16_t(ew[j])));
-        o[2 * j + 1] = __fmul_rn(f16_to_f32(uint16_t(xw[j] >> 16)), bf16_to_f32(uint16_t(ew[j] >> 16)));
-    }
-    float4 *dst = reinterpret_cast<float4 *>(xs + size_t(t) * d + size_t(c) * 8u);
-    dst[0] = make_float4(o[0], o[1], o[2], o[3]);
-    dst[1] = make_float4(o[4], o[5], o[6], o[7]);
-}
+// The fp16 router's fast path. x * effective_scale is the same for every expert: a workgroup forms
+// the products (router_row's, moe.metal:357-358) once per token while staging the row in LDS, keeps its
+// experts' rows in registers and walks a block of tokens, the next step's rows in flight while one is
+// multiplied. The additions are router_row's, in router_row's order, so the logits are the same bits.
 
 // A wave keeps ROWS fp16 router rows in registers (MAXI 16-byte chunks a lane and row); the workgroup
 // walks a block of TOKENS tokens, TPS of them a step: their x rows are staged once in LDS (the next
@@ -63,8 +41,9 @@ __global__ __launch_bounds__(256) void k_prefill_scale_x(const uint16_t *hidden,
 // go through the butterfly side by side. Every logit is summed in the decode router's order (lane l:
 // chunks l, l+64, ..., xor butterfly).
 template <int MAXI, int ROWS, uint32_t TOKENS, uint32_t TPS>
-__global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits,
-                                                            uint32_t query_count, uint32_t num_experts, uint32_t d) {
+__global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weights, const uint16_t *hidden, uint32_t stride,
+                                                            const uint16_t *eff, float *logits, uint32_t query_count,
+                                                            uint32_t num_experts, uint32_t d) {
     // chunk c = lane + 64 i of a row is two float4: half h of it sits at [(2 i + h) * 64 + lane], so that a
     // wave's read of one half is one contiguous kilobyte
     __shared__ float4 s_x[2][TPS][MAXI * 2 * 64];
@@ -86,33 +65,40 @@ __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weig
     const uint32_t t0 = blockIdx.y * TOKENS;
     const uint32_t t1 = min(t0 + TOKENS, query_count);
     if (t0 >= t1) return;
-    constexpr int kStage = MAXI * 2 * 64 / 256;  // float4 a thread stages per token
-    static_assert(kStage >= 1 && kStage <= 4, "a thread stages one to four float4 a token");
-    const uint32_t quads = d / 4u;
-    auto quad = [&](int j) { return min(threadIdx.x + 256u * uint32_t(j), quads - 1u); };  // past the row: a copy, never stored
-    auto stage_load = [&](float4 (&st)[TPS][4], uint32_t t) {
+    // a thread stages kStage 8-element chunks of a token's row: fp16 x times bf16 effective scale, the
+    // exact fp32 product, two float4 a chunk
+    static_assert(MAXI % 4 == 0, "a workgroup of 256 threads stages 64 * MAXI chunks a token");
+    constexpr int kStage = MAXI / 4;
+    uint4 eff_c[kStage];
+#pragma unroll
+    for (int j = 0; j < kStage; ++j) eff_c[j] = reinterpret_cast<const uint4 *>(eff)[min(threadIdx.x + 256u * j, chunks - 1u)];
+    auto stage_load = [&](uint4 (&st)[TPS][kStage], uint32_t t) {
 #pragma unroll
         for (uint32_t u = 0; u < TPS; ++u) {
-            const float4 *row = reinterpret_cast<const float4 *>(xs + size_t(min(t + u, t1 - 1u)) * d);
-            st[u][0] = row[quad(0)];
-            if (kStage > 1) st[u][1] = row[quad(1)];
-            if (kStage > 2) st[u][2] = row[quad(2)];
-            if (kStage > 3) st[u][3] = row[quad(3)];
-        }
-    };
-    auto put = [&](uint32_t buf, uint32_t u, int j, float4 v) {
-        const uint32_t q = threadIdx.x + 256u * uint32_t(j);
-        const uint32_t c = q >> 1, h = q & 1u;
-        if (q < quads) s_x[buf][u][(2u * (c >> 6) + h) * 64u + (c & 63u)] = v;
-    };
-    auto stage_store = [&](const float4 (&st)[TPS][4], uint32_t buf) {
+            const uint4 *row = reinterpret_cast<const uint4 *>(hidden + size_t(min(t + u, t1 - 1u)) * stride);
 #pragma unroll
-        for (uint32_t u = 0; u < TPS; ++u) {
-            put(buf, u, 0, st[u][0]);
-            if (kStage > 1) put(buf, u, 1, st[u][1]);
-            if (kStage > 2) put(buf, u, 2, st[u][2]);
-            if (kStage > 3) put(buf, u, 3, st[u][3]);
+            for (int j = 0; j < kStage; ++j) st[u][j] = row[min(threadIdx.x + 256u * j, chunks - 1u)];  // past the row: a copy, never stored
         }
+    };
+    auto stage_store = [&](const uint4 (&st)[TPS][kStage], uint32_t buf) {
+#pragma unroll
+        for (uint32_t u = 0; u < TPS; ++u)
+#pragma unroll
+            for (int j = 0; j < kStage; ++j) {
+                const uint32_t c = threadIdx.x + 256u * j;
+                const uint4 xv = st[u][j], ev = eff_c[j];
+                const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, ew[4] = {ev.x, ev.y, ev.z, ev.w};
+                float o[8];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {  // moe.metal:357-358 (exact product)
+                    o[2 * q] = __fmul_rn(f16_to_f32(uint16_t(xw[q])), bf16_to_f32(uint16_t(ew[q])));
+                    o[2 * q + 1] = __fmul_rn(f16_to_f32(uint16_t(xw[q] >> 16)), bf16_to_f32(uint16_t(ew[q] >> 16)));
+                }
+                if (c < chunks) {
+                    s_x[buf][u][(2u * (c >> 6)) * 64u + (c & 63u)] = make_float4(o[0], o[1], o[2], o[3]);
+                    s_x[buf][u][(2u * (c >> 6) + 1u) * 64u + (c & 63u)] = make_float4(o[4], o[5], o[6], o[7]);
+                }
+            }
     };
     auto step = [&](uint32_t buf, uint32_t t) {
         float acc[TPS][ROWS];
@@ -157,7 +143,7 @@ __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weig
                     if (t + u < t1 && e0 + uint32_t(r) < num_experts) logits[size_t(t + u) * num_experts + e0 + r] = acc[u][r];
         }
     };
-    float4 staged[TPS][4];  // live across a step's arithmetic; handed to the lambdas as a parameter so it stays in registers
+    uint4 staged[TPS][kStage];  // live across a step's arithmetic; handed to the lambdas as a parameter so it stays in registers
     stage_load(staged, t0);
     stage_store(staged, 0);
     __syncthreads();
@@ -175,12 +161,12 @@ constexpr uint32_t kLogitTokens = 8;  // tokens a workgroup walks with its rows:
 constexpr uint32_t kLogitTokensPerStep = 2;
 
 template <int MAXI, int ROWS>
-static void launch_prefill_logits_f16(const uint16_t *weights, const float *xs, float *logits, uint32_t query_count,
-                                      uint32_t num_experts, uint32_t d, hipStream_t s) {
+static void launch_prefill_logits_f16(const uint16_t *weights, const uint16_t *hidden, uint32_t stride, const uint16_t *eff,
+                                      float *logits, uint32_t query_count, uint32_t num_experts, uint32_t d, hipStream_t s) {
     const uint32_t per_block = 4u * ROWS;
     hipLaunchKernelGGL((k_prefill_logits_f16<MAXI, ROWS, kLogitTokens, kLogitTokensPerStep>),
                        dim3((num_experts + per_block - 1u) / per_block, (query_count + kLogitTokens - 1u) / kLogitTokens),
-                       dim3(256), 0, s, weights, xs, logits, query_count, num_experts, d);
+                       dim3(256), 0, s, weights, hidden, stride, eff, logits, query_count, num_experts, d);
 }
 
 // prefill.metal:441-563: one wave selects for one token.
@@ -478,16 +464,14 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
     const dim3 grid((num_experts + 3u) / 4u, (query_count + kRouterTokenBlock - 1u) / kRouterTokenBlock);
     switch (moe->desc.router_weight_bits) {
         case 0: {
-            float *xs = d_logits_workspace + ((size_t(query_count) * num_experts + 3u) & ~size_t(3));
-            const size_t slots = size_t(query_count) * (d / 8u);
-            hipLaunchKernelGGL(k_prefill_scale_x, dim3(uint32_t((slots + 255u) / 256u)), dim3(256), 0, s, a.hidden, a.effective_scale,
-                               xs, query_count, d, hidden_stride_elements);
-            SHRIKE_HIP(hipGetLastError());
-            // four packed rows a wave where they fit beside two tokens' x: a quarter of the x traffic of one row
+            // four packed rows a wave where a row is four chunks a lane, two where it is up to eight
             const uint16_t *w16 = static_cast<const uint16_t *>(d_weights);
-            if (d <= 2048u) launch_prefill_logits_f16<4, 4>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
-            else if (d <= 3072u) launch_prefill_logits_f16<6, 2>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
-            else launch_prefill_logits_f16<8, 2>(w16, xs, d_logits_workspace, query_count, num_experts, d, s);
+            if (d <= 2048u)
+                launch_prefill_logits_f16<4, 4>(w16, a.hidden, hidden_stride_elements, a.effective_scale, d_logits_workspace, query_count,
+                                                num_experts, d, s);
+            else
+                launch_prefill_logits_f16<8, 2>(w16, a.hidden, hidden_stride_elements, a.effective_scale, d_logits_workspace, query_count,
+                                                num_experts, d, s);
             break;
         }
         case 8: hipLaunchKernelGGL(k_prefill_logits<8>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;
@@ -501,7 +485,8 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
 }
 
 size_t shrike_hip_prefill_router_workspace_bytes(uint32_t query_count, uint32_t num_experts, uint32_t d) {
-    return (((size_t(query_count) * num_experts + 3u) & ~size_t(3)) + size_t(query_count) * d) * sizeof(float);
+    (void)d;  // the fp32 logits alone: x times the effective scale is formed inside the logits kernel
+    return ((size_t(query_count) * num_experts + 3u) & ~size_t(3)) * sizeof(float);
 }
 
 uint32_t shrike_hip_group_max_row_tiles(uint64_t pair_count, uint32_t num_experts) {
