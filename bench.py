@@ -35,6 +35,9 @@ HBM_PEAK_GBPS = 8000.0
 # rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for the 453 MB
 # pool copies): 9,589,555 fetched + 8,192 written. profiles/decode_phase1_q35b_int4_hbm_traffic.txt
 PHASE1_TRAFFIC_BYTES = 9_597_747
+# The two grouped-FFN kernels of config 3's chunk, same method (profiles/prefill_chunk_q35b_int4_t512.txt):
+# gate/up 57,207.5 and down 25,509.4 FETCH_SIZE units (x2.0 KiB) fetched, 4,096 + 16,384 KiB written.
+PREFILL_FFN_TRAFFIC_BYTES = int(((57207.5 + 25509.4) * 2.0 + 4096 + 16384) * 1024)
 
 
 def build_layers(rt, capi, S, n_layers, meta, shared=True):
@@ -210,7 +213,7 @@ def prefill_main(args, rt, capi, S, meta):
         "roofline": {"bound": "hbm", "kernel": "k_grouped_ffn<4,0> + k_grouped_ffn<4,1> (gate/up + down of every row tile)",
                      "achieved": round(expert_bytes / (ffn_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(expert_bytes / (ffn_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "bytes_per_launch": expert_bytes,
-                     "us_per_launch": round(ffn_us, 2), "traffic": None,
+                     "us_per_launch": round(ffn_us, 2), "traffic": PREFILL_FFN_TRAFFIC_BYTES if T == 512 else None,
                      "mfma_tflops_on_pair_flops": round(flops / (ffn_us * 1e-6) / 1e12, 2)},
         "algorithmic_bytes_per_chunk": algorithmic, "pair_flops_per_chunk": flops,
     }

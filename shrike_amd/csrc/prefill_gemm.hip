@@ -113,13 +113,13 @@ __device__ __forceinline__ half8 b_step(const BRegs<BITS> &r, int s) {
 // parameter so that the main loop is straight-line code: the compiler is then free to put one
 // chain's matrix instructions beside another chain's vector work.
 template <int BITS, int MODE, bool DENSE, uint32_t MT>
-__device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile &tile, uint32_t tile_index,
+__device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile &tile, uint32_t tile_index, uint32_t col_block,
                                          uint16_t (&s_a)[2][kRowTile][kLdsRow]) {
     const uint32_t K = MODE == 0 ? a.d : a.f, N = MODE == 0 ? a.f : a.d;
     const uint32_t G = K / kGroup;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t col = lane & 31u, kb = lane >> 5;
-    const uint32_t n0 = (blockIdx.y * 4u + wave) * (MODE == 0 ? 32u : 64u);
+    const uint32_t n0 = (col_block * 4u + wave) * (MODE == 0 ? 32u : 64u);
     const bool active = n0 < N;
 
     // ---- A staging: thread -> (row = tid / kStagePieces + kStageRows i, 16-byte piece = tid % kStagePieces)
@@ -406,22 +406,33 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
 template <int BITS, int MODE, bool DENSE>
 __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     __shared__ __align__(16) uint16_t s_a[2][kRowTile][kLdsRow];
-    const uint32_t tile_index = blockIdx.x;
+    // Which (row tile, column block) this workgroup takes. Workgroups go to the chip's eight XCDs (each
+    // with an L2 of its own) round robin in launch order, so workgroup w runs on XCD w % 8 as that XCD's
+    // item w / 8. An expert's row tiles are neighbours in the tile table: an XCD takes a contiguous run
+    // of tiles with all their column blocks, so that the column blocks of a tile find its gathered rows,
+    // and the row tiles of an expert its codes, in the L2 that fetched them first.
+    const uint32_t column_blocks = gridDim.y;
+    const uint32_t tile_total = DENSE ? (a.dense_rows + kRowTile - 1u) / kRowTile : *a.tile_count;
+    const uint32_t w = blockIdx.y * gridDim.x + blockIdx.x;
+    const uint32_t xcd = w & 7u, item = w >> 3;
+    const uint32_t run = (tile_total + 7u) / 8u;  // tiles an XCD takes
+    if (item / column_blocks >= run) return;
+    const uint32_t tile_index = xcd * run + item / column_blocks, col_block = item % column_blocks;
     shrike_row_tile tile;
     if (DENSE) {
-        if (tile_index * kRowTile >= a.dense_rows) return;
+        if (tile_index >= tile_total) return;
         tile.cell = 0;
         tile.pair_start = tile_index * kRowTile;
         tile.rows = min(kRowTile, a.dense_rows - tile.pair_start);
         tile.expert = 0;
     } else {
-        if (tile_index >= *a.tile_count) return;
+        if (tile_index >= tile_total) return;
         tile = a.tiles[tile_index];
         if (tile.cell == kSentinel || tile.rows == 0) return;
     }
 
-    if (tile.rows > 32u) ffn_tile<BITS, MODE, DENSE, 2>(a, tile, tile_index, s_a);
-    else ffn_tile<BITS, MODE, DENSE, 1>(a, tile, tile_index, s_a);
+    if (tile.rows > 32u) ffn_tile<BITS, MODE, DENSE, 2>(a, tile, tile_index, col_block, s_a);
+    else ffn_tile<BITS, MODE, DENSE, 1>(a, tile, tile_index, col_block, s_a);
 }
 
 int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uint32_t n, uint32_t *out,
@@ -430,10 +441,11 @@ int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uin
 template <int BITS, bool DENSE>
 static int launch_ffn(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
     const dim3 block(256);
-    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0, DENSE>), dim3(max_tiles, (a.f + 127u) / 128u), block, 0, s, a);
+    const uint32_t grid_tiles = (max_tiles + 7u) & ~7u;  // whole runs for the kernel's XCD mapping
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0, DENSE>), dim3(grid_tiles, (a.f + 127u) / 128u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     if (int rc = launch_row_group_sums(a.act, a.f, max_tiles * kRowTile, a.f, const_cast<uint32_t *>(a.act_sums), a.tile_count, s)) return rc;
-    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1, DENSE>), dim3(max_tiles, (a.d + 255u) / 256u), block, 0, s, a);
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1, DENSE>), dim3(grid_tiles, (a.d + 255u) / 256u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     return 0;
 }
