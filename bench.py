@@ -190,7 +190,7 @@ def prefill_main(args, rt, capi, S, meta):
     timed(step, warm)
     ms = timed(step, steps)
     parts = {name: timed(fn, max(4, steps // 2)) * 1e3 for name, fn in
-             (("router (2 launches)", router), ("grouping (2 launches)", group), ("grouped FFN (4 launches)", ffn), ("reduce", reduce))}
+             (("router (2 launches)", router), ("grouping (1 launch)", group), ("grouped FFN (4 launches)", ffn), ("reduce", reduce))}
     rt.synchronize()
     counts = routes.counts.download(np.uint32, NE)
     tiles = int(routes.row_tile_count.download(np.uint32, 1)[0])
