@@ -177,26 +177,62 @@ private:
     shrike_packed_layout *h_;
 };
 
-// ExpertCachePlan (PreadExpertStreamer.swift:17-38)
+struct PrefetchClaimRefused {  // PreadExpertStreamer.swift:46-49
+    int expert, cell;
+};
+
+// ExpertCachePlan (PreadExpertStreamer.swift:17-38); assignedCells is the arena cell behind each
+// assigned slot, what expertCachePlanBuffers binds
 struct ExpertCachePlan {
     std::vector<int32_t> experts, assignedSlots;
     std::vector<uint64_t> assignedGenerations;
     std::vector<uint32_t> misses;
     uint32_t hits = 0;
     int32_t layer = 0;
+    std::vector<uint32_t> assignedCells, adopted;
+    std::map<int32_t, uint32_t> freedCells;
     shrike_expert_cache_plan raw() {
         return {uint32_t(experts.size()), layer, experts.data(), assignedSlots.data(), assignedGenerations.data(),
-                misses.data(), uint32_t(misses.size()), hits};
+                misses.data(), uint32_t(misses.size()), hits, nullptr, nullptr, 0, 0, nullptr, nullptr};
     }
 };
 
-// The cache planning of PreadExpertStreamer (PreadExpertStreamer.swift:405-543, :676-767)
+// ExpertCellArena's numbering and generations (ExpertCellArena.swift:16-29, :95-104)
+class CellArena {
+public:
+    explicit CellArena(uint32_t cellCount) {
+        int err = 0;
+        h_ = shrike_cell_arena_create(cellCount, &err);
+        if (!h_) throw Error(err, shrike_hip_last_error());
+    }
+    ~CellArena() { shrike_cell_arena_destroy(h_); }
+    CellArena(const CellArena &) = delete;
+    CellArena &operator=(const CellArena &) = delete;
+    uint32_t cellCount() const { return shrike_cell_arena_cell_count(h_); }
+    uint64_t cellGeneration(uint32_t cell) const { return shrike_cell_arena_generation(h_, cell); }
+    shrike_cell_arena *handle() const { return h_; }
+
+private:
+    shrike_cell_arena *h_;
+};
+
+// The cache planning of PreadExpertStreamer (PreadExpertStreamer.swift:405-543, :676-767) with its
+// landings and overflow slots (:815-1018)
 class SlotCache {
 public:
     SlotCache(uint32_t slotCount, uint32_t expertsPerLayer, uint32_t firstCell = 0, std::optional<double> slruProtectedShare = std::nullopt) {
         int err = 0;
         h_ = shrike_slot_cache_create(slotCount, expertsPerLayer, firstCell, slruProtectedShare ? SHRIKE_EVICT_SLRU : SHRIKE_EVICT_AGING_LFU,
                                       slruProtectedShare.value_or(0.0), &err);
+        if (!h_) throw Error(err, shrike_hip_last_error());
+    }
+    // the slots take cells firstCell ..< firstCell + slotCount of a shared arena, which must outlive the cache
+    SlotCache(CellArena &arena, uint32_t slotCount, uint32_t expertsPerLayer, uint32_t firstCell,
+              std::optional<double> slruProtectedShare = std::nullopt) {
+        int err = 0;
+        h_ = shrike_slot_cache_create_in_arena(arena.handle(), slotCount, expertsPerLayer, firstCell,
+                                               slruProtectedShare ? SHRIKE_EVICT_SLRU : SHRIKE_EVICT_AGING_LFU,
+                                               slruProtectedShare.value_or(0.0), &err);
         if (!h_) throw Error(err, shrike_hip_last_error());
     }
     ~SlotCache() { shrike_slot_cache_destroy(h_); }
@@ -207,20 +243,34 @@ public:
     std::optional<ExpertCachePlan> planExpertsCachedIfPossible(const std::vector<int32_t> &experts, int32_t layer = 0,
                                                                const std::vector<int32_t> &avoidingSlots = {},
                                                                const std::vector<uint8_t> *protectedExperts = nullptr,
-                                                               int64_t missesCounted = -1) {
+                                                               int64_t missesCounted = -1,
+                                                               const std::vector<int32_t> &gpuMissedExperts = {},
+                                                               const std::vector<int32_t> &leasedLandings = {}) {
         ExpertCachePlan p;
         const size_t n = experts.size();
         p.experts.resize(n);
         p.assignedSlots.resize(n);
         p.assignedGenerations.resize(n);
         p.misses.resize(n);
+        p.assignedCells.resize(n);
+        p.adopted.resize(n);
+        std::vector<int32_t> freedExperts(n);
+        std::vector<uint32_t> freedCells(n);
         shrike_expert_cache_plan raw = p.raw();
-        const int rc = shrike_slot_cache_plan(h_, experts.data(), uint32_t(n), layer, avoidingSlots.data(), uint32_t(avoidingSlots.size()),
-                                              protectedExperts ? protectedExperts->data() : nullptr,
-                                              protectedExperts ? uint32_t(protectedExperts->size()) : 0u, missesCounted, &raw);
+        raw.assigned_cells = p.assignedCells.data();
+        raw.adopted = p.adopted.data();
+        raw.freed_experts = freedExperts.data();
+        raw.freed_cells = freedCells.data();
+        const int rc = shrike_slot_cache_plan_with_landings(
+            h_, experts.data(), uint32_t(n), layer, avoidingSlots.data(), uint32_t(avoidingSlots.size()),
+            protectedExperts ? protectedExperts->data() : nullptr, protectedExperts ? uint32_t(protectedExperts->size()) : 0u,
+            gpuMissedExperts.data(), uint32_t(gpuMissedExperts.size()), leasedLandings.data(), uint32_t(leasedLandings.size()),
+            missesCounted, &raw);
         if (rc == ENOSPC) return std::nullopt;
         check(rc);
         p.misses.resize(raw.miss_count);
+        p.adopted.resize(raw.adopted_count);
+        for (uint32_t i = 0; i < raw.freed_count; ++i) p.freedCells[freedExperts[i]] = freedCells[i];
         p.hits = raw.hits;
         p.layer = raw.layer;
         return p;
@@ -258,6 +308,36 @@ public:
         return out;
     }
     uint64_t residencyEntry(uint32_t expert) { return shrike_slot_cache_entry(h_, expert); }
+
+    // landings, PreadExpertStreamer.swift:815-852, :1010-1018
+    bool claimLanding(int32_t expert, int64_t cell) { return shrike_slot_cache_claim_landing(h_, expert, cell) != 0; }
+    bool completeLanding(int32_t expert, int64_t cell) { return shrike_slot_cache_complete_landing(h_, expert, cell) != 0; }
+    void failLanding(int32_t expert, int64_t cell) { shrike_slot_cache_fail_landing(h_, expert, cell); }
+    void dropLanding(int32_t expert, int64_t cell) { shrike_slot_cache_drop_landing(h_, expert, cell); }
+    // the claims of beginPrefetch (:1034-1057); throws PrefetchClaimRefused when the pool holds a predicted expert
+    void claimPrefetch(const std::vector<int32_t> &experts, const std::vector<int64_t> &cells) {
+        if (experts.size() != cells.size()) throw Error(EINVAL, "prefetch experts and cells differ in count");
+        uint32_t refused = 0;
+        const int rc = shrike_slot_cache_claim_prefetch(h_, experts.data(), cells.data(), uint32_t(experts.size()), &refused);
+        if (rc == SHRIKE_PREFETCH_CLAIM_REFUSED) throw PrefetchClaimRefused{int(experts[refused]), int(cells[refused])};
+        check(rc);
+    }
+    // overflow slots, :860-893, :968-993; reserveOverflowSlot gives the cell
+    std::optional<uint32_t> reserveOverflowSlot(int32_t expert, const std::vector<int32_t> &protecting = {}) {
+        const int64_t cell = shrike_slot_cache_reserve_overflow_slot(h_, expert, protecting.data(), uint32_t(protecting.size()));
+        if (cell < 0) return std::nullopt;
+        return uint32_t(cell);
+    }
+    void abandonOverflowSlot(int32_t expert, int64_t cell) { shrike_slot_cache_abandon_overflow_slot(h_, expert, cell); }
+    // the completion of beginAgreedReads, :936-964
+    void finishAgreedReads(const std::vector<int32_t> &experts, const std::vector<int64_t> &cells, bool succeeded,
+                           uint64_t elapsedNanos = 0, uint64_t fetchNanos = 0) {
+        if (experts.size() != cells.size()) throw Error(EINVAL, "agreed reads' experts and cells differ in count");
+        check(shrike_slot_cache_finish_agreed_reads(h_, experts.data(), cells.data(), uint32_t(experts.size()), succeeded,
+                                                    elapsedNanos, fetchNanos));
+    }
+    int64_t slotCell(uint32_t slot) { return shrike_slot_cache_slot_cell(h_, slot); }
+    bool ownsCell(uint32_t cell) { return shrike_slot_cache_owns_cell(h_, cell) != 0; }
     // mirrors every changed residency word into the pool's device table, in order, on `s`
     void publishTo(ExpertPool &pool, Stream s, size_t expertsPerLayer) {
         std::vector<uint32_t> ids(expertsPerLayer);
@@ -587,10 +667,6 @@ public:
 
 private:
     shrike_load_operation *h_;
-};
-
-struct PrefetchClaimRefused {  // PreadExpertStreamer.swift:46-49
-    int expert, cell;
 };
 
 // ExpertPrefetchRing (Runtime/Inference/ExpertPrefetchRing.swift:42-352)

@@ -141,23 +141,46 @@ int shrike_row_tile_tables(const shrike_routed_expert_block *blocks, size_t bloc
 
 /* ---------------------------------------------------------------- slot cache */
 
+/* ExpertCellArena's numbering and generations
+ * (sources/Shrike/Infrastructure/Streaming/ExpertCellArena.swift:16-29, :95-104): every
+ * cell a residency word can name, the pool slots of every layer and the prefetch ring's
+ * cells alike, with one clock behind all generations. The cells' bytes are the HBM
+ * pool's; this object holds the numbering only. It must outlive the caches made in it. */
+typedef struct shrike_cell_arena shrike_cell_arena;
+shrike_cell_arena *shrike_cell_arena_create(uint32_t cell_count, int *out_errno);
+void shrike_cell_arena_destroy(shrike_cell_arena *arena);
+uint32_t shrike_cell_arena_cell_count(const shrike_cell_arena *arena);
+/* cellGeneration, ExpertCellArena.swift:95-98; 0 for a cell outside the arena. */
+uint64_t shrike_cell_arena_generation(const shrike_cell_arena *arena, uint32_t cell);
+
 /* The slot bookkeeping of PreadExpertStreamer
  * (sources/Shrike/Infrastructure/Streaming/PreadExpertStreamer.swift:405-543,
  * :676-767, :1085-1148): hit lookup, victim choice, loading/resident states, cell
- * generations, pins, statistics and the residency words. One lock guards it, as
- * in the reference. Slot s is pool cell first_cell + s. */
+ * generations, pins, statistics and the residency words; and the landings and overflow
+ * slots of :815-1018. One lock guards it, as in the reference. Slot s starts at pool cell
+ * first_cell + s; adopting a landing gives the slot the landing's cell. */
 typedef struct shrike_slot_cache shrike_slot_cache;
 
 /* ExpertEvictionPolicy, sources/Shrike/Runtime/Inference/Model.swift:22-41. */
 enum { SHRIKE_EVICT_AGING_LFU = 0, SHRIKE_EVICT_SLRU = 1 };
 
+/* A cache over an arena of its own, first_cell + slot_count cells long. */
 shrike_slot_cache *shrike_slot_cache_create(uint32_t slot_count, uint32_t experts_per_layer,
                                             uint32_t first_cell, int policy,
                                             double slru_protected_share, int *out_errno);
+/* PreadExpertStreamer.init(arena:cellRange:), PreadExpertStreamer.swift:309-319: the slots
+ * take cells first_cell ..< first_cell + slot_count of a shared arena. */
+shrike_slot_cache *shrike_slot_cache_create_in_arena(shrike_cell_arena *arena, uint32_t slot_count,
+                                                     uint32_t experts_per_layer, uint32_t first_cell,
+                                                     int policy, double slru_protected_share,
+                                                     int *out_errno);
 void shrike_slot_cache_destroy(shrike_slot_cache *cache);
 
-/* ExpertCachePlan. Arrays are caller-provided with room for expert_count entries;
- * experts is copied in by the plan call. */
+/* ExpertCachePlan, PreadExpertStreamer.swift:17-38. Arrays are caller-provided with room
+ * for expert_count entries; experts is copied in by the plan call. assigned_cells (the
+ * arena cell behind each assigned slot) is optional; adopted (indices into experts),
+ * freed_experts and freed_cells (freedCells as pairs) are needed only by a plan that is
+ * given leased landings, and may be NULL otherwise. */
 typedef struct {
     uint32_t expert_count;
     int32_t layer;
@@ -167,6 +190,12 @@ typedef struct {
     uint32_t *misses; /* indices into experts */
     uint32_t miss_count;
     uint32_t hits;
+    uint32_t *assigned_cells;
+    uint32_t *adopted;
+    uint32_t adopted_count;
+    uint32_t freed_count;
+    int32_t *freed_experts;
+    uint32_t *freed_cells;
 } shrike_expert_cache_plan;
 
 /* makeExpertCachePlan, PreadExpertStreamer.swift:405-543 (planExpertsCached /
@@ -178,6 +207,17 @@ int shrike_slot_cache_plan(shrike_slot_cache *cache, const int32_t *experts, uin
                            int32_t layer, const int32_t *avoiding_slots, uint32_t avoiding_count,
                            const uint8_t *protected_experts, uint32_t protected_count,
                            int64_t misses_counted, shrike_expert_cache_plan *plan);
+/* The same with gpuMissedExperts and leasedLandings (:499-515): a miss whose expert has a
+ * completed landing leased to the plan takes the landing's cell as its slot's cell and is
+ * a hit of the plan; the slot's former cell is reported in freed_cells for the ring to
+ * reuse, and the index is listed in adopted when the GPU had missed the expert. */
+int shrike_slot_cache_plan_with_landings(shrike_slot_cache *cache, const int32_t *experts,
+                                         uint32_t expert_count, int32_t layer,
+                                         const int32_t *avoiding_slots, uint32_t avoiding_count,
+                                         const uint8_t *protected_experts, uint32_t protected_count,
+                                         const int32_t *gpu_missed_experts, uint32_t gpu_missed_count,
+                                         const int32_t *leased_landings, uint32_t leased_count,
+                                         int64_t misses_counted, shrike_expert_cache_plan *plan);
 /* markPlanMissesResident + the success leg of finishPlanExecution
  * (PreadExpertStreamer.swift:1085-1105, :1070-1083): the plan's misses become
  * resident and are counted as one load batch. EIO when a generation changed. */
@@ -189,6 +229,46 @@ void shrike_slot_cache_abandon(shrike_slot_cache *cache, const shrike_expert_cac
 int shrike_slot_cache_pin(shrike_slot_cache *cache, const shrike_expert_cache_plan *plan);
 void shrike_slot_cache_unpin(shrike_slot_cache *cache, const int32_t *slots,
                              const uint64_t *generations, uint32_t count);
+
+/* cellIndexUnlocked, PreadExpertStreamer.swift:1135-1137: the arena cell behind a slot
+ * (-1 for a slot out of range), and ownsCell, :1021-1025. */
+int64_t shrike_slot_cache_slot_cell(shrike_slot_cache *cache, uint32_t slot);
+int shrike_slot_cache_owns_cell(shrike_slot_cache *cache, uint32_t cell);
+
+/* claimLanding, PreadExpertStreamer.swift:815-829: a ring cell claimed for a prediction's
+ * read, `loading` for the classifier and neither a hit nor a victim for a plan. 1 when
+ * claimed; 0 when the pool holds or is loading the expert, a landing for it exists,
+ * another landing holds the cell, or an argument is out of range. */
+int shrike_slot_cache_claim_landing(shrike_slot_cache *cache, int32_t expert, int64_t cell);
+/* completeLanding, :834-848: `resident` at the cell; 0 (nothing published) for a landing
+ * that was dropped, re-claimed, or overtaken by the pool's own read of the expert. */
+int shrike_slot_cache_complete_landing(shrike_slot_cache *cache, int32_t expert, int64_t cell);
+/* failLanding / dropLanding, :850-852, :1010-1018: the entry is emptied unless the pool
+ * owns the expert. */
+void shrike_slot_cache_fail_landing(shrike_slot_cache *cache, int32_t expert, int64_t cell);
+void shrike_slot_cache_drop_landing(shrike_slot_cache *cache, int32_t expert, int64_t cell);
+/* The claims of beginPrefetch, :1034-1057: every cell must be outside the pool (EINVAL,
+ * like an expert out of range); a refused claim drops the batch's earlier ones, stores
+ * its index and returns SHRIKE_PREFETCH_CLAIM_REFUSED. The caller issues the reads and
+ * reports each landing with complete_landing or fail_landing. */
+int shrike_slot_cache_claim_prefetch(shrike_slot_cache *cache, const int32_t *experts,
+                                     const int64_t *cells, uint32_t count, uint32_t *refused_index);
+
+/* reserveOverflowSlot, :860-893: a pool slot for a miss the ring could not house: the
+ * policy's victim among the slots not holding `protecting`, evicted and `loading` at its
+ * cell, on probation for SLRU. Returns the cell, or -1 when no slot is evictable or the
+ * pool already holds the expert. */
+int64_t shrike_slot_cache_reserve_overflow_slot(shrike_slot_cache *cache, int32_t expert,
+                                                const int32_t *protecting, uint32_t protecting_count);
+/* markOverflowResident, :968-976, and abandonOverflowSlot / emptyOverflowSlot, :980-993. */
+void shrike_slot_cache_mark_overflow_resident(shrike_slot_cache *cache, int32_t expert, int64_t cell);
+void shrike_slot_cache_abandon_overflow_slot(shrike_slot_cache *cache, int32_t expert, int64_t cell);
+/* The completion leg of beginAgreedReads, :936-964, :995-1002: on success every pool cell
+ * turns resident and every ring cell's landing completes, and the batch is counted; on
+ * failure the landings are dropped and the pool cells emptied. */
+int shrike_slot_cache_finish_agreed_reads(shrike_slot_cache *cache, const int32_t *experts,
+                                          const int64_t *cells, uint32_t count, int succeeded,
+                                          uint64_t elapsed_nanos, uint64_t fetch_nanos);
 
 /* ExpertStreamingStatistics, PreadExpertStreamer.swift:40-71 (the fields this
  * library maintains). */

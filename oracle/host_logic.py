@@ -449,21 +449,58 @@ class CachePlan:
     misses: list  # indices into experts
     hits: int
     layer: int = 0
+    adopted: list = field(default_factory=list)  # indices into experts
+    freed_cells: dict = field(default_factory=dict)  # expert -> the pool cell its swap gave back
+    assigned_cells: list = field(default_factory=list)
+
+
+class CellArena:
+    """ExpertCellArena's generations (ExpertCellArena.swift:95-104): one clock for all cells."""
+
+    def __init__(self, cell_count: int):
+        assert cell_count > 0
+        self.cell_count = cell_count
+        self.generations = [0] * cell_count
+        self.clock = 0
+
+    def cell_generation(self, cell):
+        return self.generations[cell]
+
+    def bump(self, cell):
+        self.clock += 1
+        self.generations[cell] = self.clock
+        return self.clock
+
+
+class ClaimRefusedByPool(Exception):
+    """PrefetchClaimRefused as beginPrefetch throws it (PreadExpertStreamer.swift:1050-1053)."""
+
+    def __init__(self, expert, cell):
+        super().__init__(f"prefetch claim refused: expert {expert}, cell {cell}")
+        self.expert, self.cell = expert, cell
 
 
 @dataclass
 class SlotCache:
     """The slot bookkeeping of PreadExpertStreamer (PreadExpertStreamer.swift:405-543,
     :676-767, :1085-1148) without the file reads: hits, victim choice (aging LFU then LRU, or
-    SLRU), loading/resident states, per-cell generations, pins, statistics and the residency
-    words. Landings, the prefetch ring and overflow slots are not modelled."""
+    SLRU), loading/resident states, arena-wide cell generations, pins, statistics and the
+    residency words; the landings a prefetch ring claims (:815-852, :1010-1018), their
+    adoption by a plan (:499-515) and the overflow slots of a decode route (:860-1002)."""
     slot_count: int
     experts_per_layer: int
     first_cell: int = 0
     slru_share: float | None = None  # None = aging LFU
+    arena: CellArena | None = None  # None = an arena of its own
 
     def __post_init__(self):
         n, e = self.slot_count, max(1, self.experts_per_layer)
+        if self.arena is None:
+            self.arena = CellArena(self.first_cell + n)
+        assert self.first_cell + n <= self.arena.cell_count
+        self.slot_cell = [self.first_cell + s for s in range(n)]
+        self.landings = {}  # expert -> [cell, resident, generation]
+        self.overflow_probation = set()
         self.slot_expert = [-1] * n
         self.slot_last_use = [0] * n
         self.slot_state = [EMPTY] * n
@@ -474,15 +511,35 @@ class SlotCache:
         self.protected_capacity = 0 if self.slru_share is None else max(1, int(self.slru_share * n + 0.5))
         self.use_count = [0] * e
         self.load_count = [0] * e
-        self.generation = [0] * n
-        self.generation_clock = 0  # ExpertCellArena.bumpCellGeneration, ExpertCellArena.swift:99-104
         self.use_clock = 0
         self.words = [residency_word(EMPTY, 0)] * self.experts_per_layer
         self.stats = dict(plans=0, requested=0, hits=0, misses=0, evictions=0, reloads=0,
                           read_operations=0, load_batches=0, peak_loading=0)
 
     def cell(self, slot):
-        return self.first_cell + slot
+        """cellIndexUnlocked, PreadExpertStreamer.swift:1135-1137."""
+        return self.slot_cell[slot]
+
+    def _generation(self, slot):
+        return self.arena.cell_generation(self.slot_cell[slot])
+
+    def _slot_of_cell(self, cell):
+        return self.slot_cell.index(cell) if cell in self.slot_cell else None
+
+    def owns_cell(self, cell):
+        return cell in self.slot_cell
+
+    def _demote(self, slot):
+        if self.slot_protected[slot]:
+            self.slot_protected[slot] = False
+            self.protected_count -= 1
+
+    def _record_expert_load(self, e):
+        """recordExpertLoadsUnlocked, PreadExpertStreamer.swift:1171-1179."""
+        if 0 <= e < len(self.load_count):
+            if self.load_count[e] > 0:
+                self.stats["reloads"] += 1
+            self.load_count[e] += 1
 
     def _publish(self, expert, cell, state):
         if 0 <= expert < self.experts_per_layer:
@@ -545,7 +602,8 @@ class SlotCache:
         self.protected_count -= 1
         self.slot_last_use[oldest] = clock
 
-    def plan(self, experts, layer=0, avoiding_slots=(), protected_experts=None, misses_counted=None):
+    def plan(self, experts, layer=0, avoiding_slots=(), protected_experts=None, misses_counted=None,
+             gpu_missed_experts=None, leased_landings=()):
         """makeExpertCachePlan, PreadExpertStreamer.swift:405-543; None when unplaceable."""
         assert len(experts) <= self.slot_count
         avoiding = {s for s in avoiding_slots if 0 <= s < self.slot_count}
@@ -585,8 +643,12 @@ class SlotCache:
         if self.slru_share is not None:
             for s in assigned:
                 if s >= 0 and not self.slot_protected[s]:
+                    if s in self.overflow_probation:
+                        self.overflow_probation.discard(s)
+                        continue
                     self._promote(s, clock)
         misses, v = [], 0
+        adopted, freed = [], {}
         for i, e in enumerate(experts):
             if assigned[i] != -1:
                 continue
@@ -597,17 +659,28 @@ class SlotCache:
             previous = self.slot_expert[slot]
             assigned[i] = slot
             reserved[slot] = True
-            if self.slot_protected[slot]:
-                self.slot_protected[slot] = False
-                self.protected_count -= 1
-            self.generation_clock += 1
-            self.generation[slot] = self.generation_clock
+            self._demote(slot)
+            self.overflow_probation.discard(slot)
+            cell = self.cell(slot)
+            self.arena.bump(cell)
             if previous >= 0:
-                self._publish(previous, self.cell(slot), EMPTY)
+                self._publish(previous, cell, EMPTY)
+            landing = self.landings.get(e) if e in leased_landings else None
+            if landing is not None and landing[1]:
+                del self.landings[e]
+                freed[e] = cell
+                self.slot_cell[slot] = landing[0]
+                self.slot_expert[slot] = e
+                self.slot_last_use[slot] = clock
+                self.slot_state[slot] = RESIDENT
+                self._record_expert_load(e)
+                if gpu_missed_experts is not None and e in gpu_missed_experts:
+                    adopted.append(i)
+                continue
             self.slot_expert[slot] = e
             self.slot_last_use[slot] = clock
             self.slot_state[slot] = LOADING
-            self._publish(e, self.cell(slot), LOADING)
+            self._publish(e, cell, LOADING)
             misses.append(i)
         counted = len(misses) if misses_counted is None else misses_counted
         self.stats["plans"] += 1
@@ -615,14 +688,14 @@ class SlotCache:
         self.stats["hits"] += len(experts) - counted
         self.stats["misses"] += counted
         self.stats["peak_loading"] = max(self.stats["peak_loading"], self.slot_state.count(LOADING))
-        return CachePlan(list(experts), assigned, [self.generation[s] for s in assigned], misses,
-                         len(experts) - len(misses), layer)
+        return CachePlan(list(experts), assigned, [self._generation(s) for s in assigned], misses,
+                         len(experts) - len(misses), layer, adopted, freed, [self.cell(s) for s in assigned])
 
     def complete(self, plan: CachePlan):
         """markPlanMissesResident + the success leg of finishPlanExecution,
         PreadExpertStreamer.swift:1085-1105, :1070-1083, :1150-1179."""
         for i in plan.misses:
-            if self.generation[plan.assigned_slots[i]] != plan.assigned_generations[i]:
+            if self._generation(plan.assigned_slots[i]) != plan.assigned_generations[i]:
                 raise RuntimeError("expert-cache cell generation changed during expert load")
         for i in plan.misses:
             s = plan.assigned_slots[i]
@@ -634,17 +707,13 @@ class SlotCache:
             self.stats["read_operations"] += len(plan.misses)
             self.stats["load_batches"] += 1
             for i in plan.misses:
-                e = plan.experts[i]
-                if 0 <= e < len(self.load_count):
-                    if self.load_count[e] > 0:
-                        self.stats["reloads"] += 1
-                    self.load_count[e] += 1
+                self._record_expert_load(plan.experts[i])
 
     def abandon(self, plan: CachePlan):
         """abandonExpertCachePlan / resetLoadingMissesUnlocked, PreadExpertStreamer.swift:1110-1128."""
         for i in plan.misses:
             s = plan.assigned_slots[i]
-            if not (0 <= s < self.slot_count and self.generation[s] == plan.assigned_generations[i]
+            if not (0 <= s < self.slot_count and self._generation(s) == plan.assigned_generations[i]
                     and self.slot_state[s] == LOADING):
                 continue
             self.slot_state[s] = EMPTY
@@ -663,7 +732,7 @@ class SlotCache:
         """pin, PreadExpertStreamer.swift:744-767; raises on a stale plan."""
         for i, e in enumerate(plan.experts):
             s = plan.assigned_slots[i]
-            if not (0 <= s < self.slot_count and self.generation[s] == plan.assigned_generations[i]
+            if not (0 <= s < self.slot_count and self._generation(s) == plan.assigned_generations[i]
                     and self.slot_expert[s] == e and self.slot_state[s] != EMPTY):
                 raise RuntimeError("expert-cache plan became stale before GPU pin")
         for s in plan.assigned_slots:
@@ -672,7 +741,7 @@ class SlotCache:
     def unpin(self, slots, generations):
         """unpin, PreadExpertStreamer.swift:769-778."""
         for s, g in zip(slots, generations):
-            if 0 <= s < self.slot_count and self.generation[s] == g:
+            if 0 <= s < self.slot_count and self._generation(s) == g:
                 assert self.slot_pins[s] > 0
                 self.slot_pins[s] -= 1
 
@@ -683,6 +752,120 @@ class SlotCache:
     def counts(self):
         return dict(resident=self.slot_state.count(RESIDENT), loading=self.slot_state.count(LOADING),
                     pinned=sum(1 for p in self.slot_pins if p > 0))
+
+    # ---- landings (a prefetch ring's cells outside the pool)
+
+    def claim_landing(self, expert, cell):
+        """claimLanding, PreadExpertStreamer.swift:815-829."""
+        if not (0 <= expert < self.experts_per_layer and 0 <= cell < self.arena.cell_count):
+            return False
+        if expert in self.landings or expert in self.slot_expert or any(l[0] == cell for l in self.landings.values()):
+            return False
+        self.landings[expert] = [cell, False, self.arena.bump(cell)]
+        self._publish(expert, cell, LOADING)
+        return True
+
+    def complete_landing(self, expert, cell):
+        """completeLanding, PreadExpertStreamer.swift:834-848."""
+        landing = self.landings.get(expert)
+        if landing is None or landing[0] != cell or landing[1] or self.arena.cell_generation(cell) != landing[2]:
+            return False
+        if expert in self.slot_expert:
+            del self.landings[expert]
+            return False
+        landing[1] = True
+        self._publish(expert, cell, RESIDENT)
+        return True
+
+    def drop_landing(self, expert, cell):
+        """dropLanding, PreadExpertStreamer.swift:1010-1018 (failLanding, :850-852, is the same)."""
+        landing = self.landings.get(expert)
+        if landing is None or landing[0] != cell:
+            return
+        del self.landings[expert]
+        if expert not in self.slot_expert:
+            self._publish(expert, cell, EMPTY)
+
+    fail_landing = drop_landing
+
+    def claim_prefetch(self, experts, cells):
+        """The claims of beginPrefetch, PreadExpertStreamer.swift:1034-1057."""
+        if len(experts) != len(cells):
+            raise ValueError("prefetch experts and cells differ in count")
+        if any(not 0 <= e < self.experts_per_layer for e in experts):
+            raise ValueError("invalid prefetched expert")
+        if any(self.owns_cell(c) for c in cells):
+            raise ValueError("a prefetch landing was offered a cell the pool owns")
+        landed = []
+        for e, c in zip(experts, cells):
+            if not self.claim_landing(e, c):
+                for pe, pc in landed:
+                    self.drop_landing(pe, pc)
+                raise ClaimRefusedByPool(e, c)
+            landed.append((e, c))
+
+    # ---- overflow slots (a decode route's misses the ring could not house)
+
+    def reserve_overflow_slot(self, expert, protecting=()):
+        """reserveOverflowSlot, PreadExpertStreamer.swift:860-893: the cell, or None."""
+        if not 0 <= expert < self.experts_per_layer or expert in self.slot_expert:
+            return None
+        reserved = [st == LOADING for st in self.slot_state]
+        for s in range(self.slot_count):
+            if self.slot_state[s] == RESIDENT and self.slot_expert[s] in protecting:
+                reserved[s] = True
+        victims = self._select_victims(1, reserved)
+        if victims is None:
+            return None
+        slot = victims[0]
+        self.overflow_probation.add(slot)
+        if self.slot_state[slot] == RESIDENT:
+            self.stats["evictions"] += 1
+        previous = self.slot_expert[slot]
+        self._demote(slot)
+        cell = self.cell(slot)
+        self.arena.bump(cell)
+        if previous >= 0:
+            self._publish(previous, cell, EMPTY)
+        self.slot_expert[slot] = expert
+        self.slot_last_use[slot] = self.use_clock
+        self.slot_state[slot] = LOADING
+        self._publish(expert, cell, LOADING)
+        return cell
+
+    def mark_overflow_resident(self, expert, cell):
+        """markOverflowResident, PreadExpertStreamer.swift:968-976."""
+        slot = self._slot_of_cell(cell)
+        if slot is None or self.slot_state[slot] != LOADING or self.slot_expert[slot] != expert:
+            return
+        self.slot_state[slot] = RESIDENT
+        self.slot_last_use[slot] = self.use_clock
+        self._publish(expert, cell, RESIDENT)
+
+    def abandon_overflow_slot(self, expert, cell):
+        """abandonOverflowSlot / emptyOverflowSlot, PreadExpertStreamer.swift:980-993."""
+        slot = self._slot_of_cell(cell)
+        if slot is None or self.slot_state[slot] != LOADING or self.slot_expert[slot] != expert:
+            return
+        self.slot_state[slot] = EMPTY
+        self.slot_expert[slot] = -1
+        self.overflow_probation.discard(slot)
+        self._publish(expert, cell, EMPTY)
+
+    def finish_agreed_reads(self, experts, cells, succeeded):
+        """The completion of beginAgreedReads, PreadExpertStreamer.swift:936-964, :995-1002."""
+        pool = [self.owns_cell(c) for c in cells]
+        for e, c, in_pool in zip(experts, cells, pool):
+            if succeeded:
+                self.mark_overflow_resident(e, c) if in_pool else self.complete_landing(e, c)
+            else:
+                self.abandon_overflow_slot(e, c) if in_pool else self.drop_landing(e, c)
+        if succeeded and experts:
+            self.stats["read_operations"] += len(experts)
+            self.stats["load_batches"] += 1
+            for e, in_pool in zip(experts, pool):
+                if in_pool:
+                    self._record_expert_load(e)
 
 
 # ------------------------------------------------------------- packed experts layout

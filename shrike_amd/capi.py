@@ -112,7 +112,10 @@ class RoutedExpertWave(C.Structure):
 class ExpertCachePlan(C.Structure):
     _fields_ = [("expert_count", C.c_uint32), ("layer", C.c_int32), ("experts", C.POINTER(C.c_int32)),
                 ("assigned_slots", C.POINTER(C.c_int32)), ("assigned_generations", C.POINTER(C.c_uint64)),
-                ("misses", C.POINTER(C.c_uint32)), ("miss_count", C.c_uint32), ("hits", C.c_uint32)]
+                ("misses", C.POINTER(C.c_uint32)), ("miss_count", C.c_uint32), ("hits", C.c_uint32),
+                ("assigned_cells", C.POINTER(C.c_uint32)), ("adopted", C.POINTER(C.c_uint32)),
+                ("adopted_count", C.c_uint32), ("freed_count", C.c_uint32),
+                ("freed_experts", C.POINTER(C.c_int32)), ("freed_cells", C.POINTER(C.c_uint32))]
 
 
 class StreamingStatistics(C.Structure):
@@ -338,6 +341,24 @@ SIGNATURES = {
     "shrike_row_tile_tables": (C.c_int, [C.POINTER(RoutedExpertBlock), C.c_size_t, _U32, _U32, _VP, _VP, _VP]),
     "shrike_slot_cache_create": (_VP, [_U32, _U32, _U32, C.c_int, C.c_double, C.POINTER(C.c_int)]),
     "shrike_slot_cache_destroy": (None, [_VP]),
+    "shrike_cell_arena_create": (_VP, [_U32, C.POINTER(C.c_int)]),
+    "shrike_cell_arena_destroy": (None, [_VP]),
+    "shrike_cell_arena_cell_count": (_U32, [_VP]),
+    "shrike_cell_arena_generation": (_U64, [_VP, _U32]),
+    "shrike_slot_cache_create_in_arena": (_VP, [_VP, _U32, _U32, _U32, C.c_int, C.c_double, C.POINTER(C.c_int)]),
+    "shrike_slot_cache_plan_with_landings": (C.c_int, [_VP, _VP, _U32, _I32, _VP, _U32, _VP, _U32, _VP, _U32, _VP, _U32,
+                                                       _I64, C.POINTER(ExpertCachePlan)]),
+    "shrike_slot_cache_slot_cell": (_I64, [_VP, _U32]),
+    "shrike_slot_cache_owns_cell": (C.c_int, [_VP, _U32]),
+    "shrike_slot_cache_claim_landing": (C.c_int, [_VP, _I32, _I64]),
+    "shrike_slot_cache_complete_landing": (C.c_int, [_VP, _I32, _I64]),
+    "shrike_slot_cache_fail_landing": (None, [_VP, _I32, _I64]),
+    "shrike_slot_cache_drop_landing": (None, [_VP, _I32, _I64]),
+    "shrike_slot_cache_claim_prefetch": (C.c_int, [_VP, _VP, _VP, _U32, C.POINTER(C.c_uint32)]),
+    "shrike_slot_cache_reserve_overflow_slot": (_I64, [_VP, _I32, _VP, _U32]),
+    "shrike_slot_cache_mark_overflow_resident": (None, [_VP, _I32, _I64]),
+    "shrike_slot_cache_abandon_overflow_slot": (None, [_VP, _I32, _I64]),
+    "shrike_slot_cache_finish_agreed_reads": (C.c_int, [_VP, _VP, _VP, _U32, C.c_int, _U64, _U64]),
     "shrike_slot_cache_plan": (C.c_int, [_VP, _VP, _U32, _I32, _VP, _U32, _VP, _U32, _I64, C.POINTER(ExpertCachePlan)]),
     "shrike_slot_cache_complete": (C.c_int, [_VP, C.POINTER(ExpertCachePlan), _U64, _U64]),
     "shrike_slot_cache_abandon": (None, [_VP, C.POINTER(ExpertCachePlan)]),

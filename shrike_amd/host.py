@@ -162,8 +162,14 @@ class CachePlan:
         self.slots_a = np.zeros(max(1, n), np.int32)
         self.gens_a = np.zeros(max(1, n), np.uint64)
         self.misses_a = np.zeros(max(1, n), np.uint32)
+        self.cells_a = np.zeros(max(1, n), np.uint32)
+        self.adopted_a = np.zeros(max(1, n), np.uint32)
+        self.freed_experts_a = np.zeros(max(1, n), np.int32)
+        self.freed_cells_a = np.zeros(max(1, n), np.uint32)
         self.c = capi.ExpertCachePlan(0, 0, _as(self.experts_a, C.c_int32), _as(self.slots_a, C.c_int32),
-                                      _as(self.gens_a, C.c_uint64), _as(self.misses_a, C.c_uint32), 0, 0)
+                                      _as(self.gens_a, C.c_uint64), _as(self.misses_a, C.c_uint32), 0, 0,
+                                      _as(self.cells_a, C.c_uint32), _as(self.adopted_a, C.c_uint32), 0, 0,
+                                      _as(self.freed_experts_a, C.c_int32), _as(self.freed_cells_a, C.c_uint32))
 
     @property
     def experts(self):
@@ -189,16 +195,65 @@ class CachePlan:
     def layer(self):
         return self.c.layer
 
+    @property
+    def assigned_cells(self):
+        """The arena cell behind each assigned slot (what expertCachePlanBuffers binds)."""
+        return self.cells_a[: self.c.expert_count].tolist()
+
+    @property
+    def adopted(self):
+        return self.adopted_a[: self.c.adopted_count].tolist()
+
+    @property
+    def freed_cells(self):
+        """freedCells: expert -> the pool cell its landing's swap gave back to the ring."""
+        n = self.c.freed_count
+        return dict(zip(self.freed_experts_a[:n].tolist(), self.freed_cells_a[:n].tolist()))
+
+
+class CellArena:
+    """ExpertCellArena's numbering and generations (ExpertCellArena.swift:16-29, :95-104); the cells' bytes
+    belong to the HBM pool."""
+
+    def __init__(self, cell_count: int):
+        err = C.c_int(0)
+        self._h = capi.load().shrike_cell_arena_create(cell_count, C.byref(err))
+        if not self._h:
+            raise ShrikeError(f"cell arena: {capi.last_error()}")
+        self.cell_count = cell_count
+
+    def cell_generation(self, cell: int) -> int:
+        if not 0 <= cell < self.cell_count:
+            raise IndexError("expert cell out of range")
+        return int(capi.load().shrike_cell_arena_generation(self._h, cell))
+
+    def close(self):
+        if self._h:
+            capi.load().shrike_cell_arena_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
 
 class SlotCache:
     """The slot bookkeeping of PreadExpertStreamer (PreadExpertStreamer.swift:405-543, :676-767)."""
 
-    def __init__(self, slot_count: int, experts_per_layer: int, first_cell: int = 0, slru_share=None):
+    def __init__(self, slot_count: int, experts_per_layer: int, first_cell: int = 0, slru_share=None,
+                 arena: "CellArena | None" = None):
         err = C.c_int(0)
         self.slot_count, self.experts_per_layer = slot_count, experts_per_layer
-        self._h = capi.load().shrike_slot_cache_create(slot_count, experts_per_layer, first_cell,
-                                                       0 if slru_share is None else 1,
-                                                       0.0 if slru_share is None else float(slru_share), C.byref(err))
+        self.arena = arena  # kept alive for as long as the cache
+        policy = (0 if slru_share is None else 1, 0.0 if slru_share is None else float(slru_share))
+        if arena is None:
+            self._h = capi.load().shrike_slot_cache_create(slot_count, experts_per_layer, first_cell, *policy,
+                                                           C.byref(err))
+        else:
+            self._h = capi.load().shrike_slot_cache_create_in_arena(arena._h, slot_count, experts_per_layer, first_cell,
+                                                                    *policy, C.byref(err))
         if not self._h:
             raise ShrikeError(f"slot cache: {capi.last_error()}")
 
@@ -213,15 +268,20 @@ class SlotCache:
         except Exception:
             pass
 
-    def plan(self, experts, layer=0, avoiding_slots=(), protected_experts=None, misses_counted=None):
+    def plan(self, experts, layer=0, avoiding_slots=(), protected_experts=None, misses_counted=None,
+             gpu_missed_experts=None, leased_landings=()):
         """planExpertsCachedIfPossible: None when the experts cannot be placed."""
         e = np.ascontiguousarray(experts, dtype=np.int32)
         avoid = np.ascontiguousarray(sorted(avoiding_slots), dtype=np.int32)
         prot = None if protected_experts is None else np.ascontiguousarray(np.asarray(protected_experts, dtype=np.uint8))
+        missed = np.ascontiguousarray(sorted(gpu_missed_experts or ()), dtype=np.int32)
+        leased = np.ascontiguousarray(sorted(leased_landings), dtype=np.int32)
         plan = CachePlan(e.size)
-        rc = capi.load().shrike_slot_cache_plan(self._h, _vp(e), e.size, layer, _vp(avoid) if avoid.size else None,
-                                                avoid.size, _vp(prot), 0 if prot is None else prot.size,
-                                                -1 if misses_counted is None else misses_counted, C.byref(plan.c))
+        rc = capi.load().shrike_slot_cache_plan_with_landings(
+            self._h, _vp(e), e.size, layer, _vp(avoid) if avoid.size else None, avoid.size, _vp(prot),
+            0 if prot is None else prot.size, _vp(missed) if missed.size else None, missed.size,
+            _vp(leased) if leased.size else None, leased.size, -1 if misses_counted is None else misses_counted,
+            C.byref(plan.c))
         if rc == errno.ENOSPC:
             return None
         capi.check(rc, "planExpertsCached")
@@ -248,6 +308,61 @@ class SlotCache:
     def unpin(self, slots, generations):
         s, g = np.ascontiguousarray(slots, np.int32), np.ascontiguousarray(generations, np.uint64)
         capi.load().shrike_slot_cache_unpin(self._h, _vp(s), _vp(g), s.size)
+
+    def slot_cell(self, slot: int) -> int:
+        """The arena cell behind a slot (cellIndexUnlocked, PreadExpertStreamer.swift:1135-1137)."""
+        return int(capi.load().shrike_slot_cache_slot_cell(self._h, slot))
+
+    def owns_cell(self, cell: int) -> bool:
+        return bool(capi.load().shrike_slot_cache_owns_cell(self._h, cell))
+
+    def claim_landing(self, expert: int, cell: int) -> bool:
+        """claimLanding, PreadExpertStreamer.swift:815-829."""
+        return bool(capi.load().shrike_slot_cache_claim_landing(self._h, expert, cell))
+
+    def complete_landing(self, expert: int, cell: int) -> bool:
+        """completeLanding, PreadExpertStreamer.swift:834-848."""
+        return bool(capi.load().shrike_slot_cache_complete_landing(self._h, expert, cell))
+
+    def fail_landing(self, expert: int, cell: int):
+        capi.load().shrike_slot_cache_fail_landing(self._h, expert, cell)
+
+    def drop_landing(self, expert: int, cell: int):
+        """dropLanding, PreadExpertStreamer.swift:1010-1018."""
+        capi.load().shrike_slot_cache_drop_landing(self._h, expert, cell)
+
+    def claim_prefetch(self, experts, cells):
+        """The claims of beginPrefetch (PreadExpertStreamer.swift:1034-1057): raises PrefetchClaimRefused when the
+        pool holds a predicted expert, ShrikeError for a cell the pool owns or an expert out of range."""
+        if len(experts) != len(cells):
+            raise ShrikeError("prefetch experts and cells differ in count")
+        e, c = np.ascontiguousarray(experts, np.int32), np.ascontiguousarray(cells, np.int64)
+        refused = C.c_uint32(0)
+        rc = capi.load().shrike_slot_cache_claim_prefetch(self._h, _vp(e), _vp(c), e.size, C.byref(refused))
+        if rc == PREFETCH_CLAIM_REFUSED:
+            raise PrefetchClaimRefused(int(e[refused.value]), int(c[refused.value]))
+        capi.check(rc, "beginPrefetch")
+
+    def reserve_overflow_slot(self, expert: int, protecting=()):
+        """reserveOverflowSlot, PreadExpertStreamer.swift:860-893: the cell, or None."""
+        p = np.ascontiguousarray(list(protecting), np.int32)
+        cell = capi.load().shrike_slot_cache_reserve_overflow_slot(self._h, expert, _vp(p) if p.size else None, p.size)
+        return None if cell < 0 else int(cell)
+
+    def mark_overflow_resident(self, expert: int, cell: int):
+        capi.load().shrike_slot_cache_mark_overflow_resident(self._h, expert, cell)
+
+    def abandon_overflow_slot(self, expert: int, cell: int):
+        """abandonOverflowSlot, PreadExpertStreamer.swift:980-993."""
+        capi.load().shrike_slot_cache_abandon_overflow_slot(self._h, expert, cell)
+
+    def finish_agreed_reads(self, experts, cells, succeeded: bool, elapsed_nanos: int = 0, fetch_nanos: int = 0):
+        """The completion of beginAgreedReads (PreadExpertStreamer.swift:936-964)."""
+        if len(experts) != len(cells):
+            raise ShrikeError("agreed reads' experts and cells differ in count")
+        e, c = np.ascontiguousarray(experts, np.int32), np.ascontiguousarray(cells, np.int64)
+        capi.check(capi.load().shrike_slot_cache_finish_agreed_reads(self._h, _vp(e), _vp(c), e.size, int(succeeded),
+                                                                     elapsed_nanos, fetch_nanos), "beginAgreedReads")
 
     def statistics(self, expert_stride_bytes: int = 0) -> capi.StreamingStatistics:
         st = capi.StreamingStatistics()
@@ -659,6 +774,51 @@ class PrefetchClaimRefused(Exception):
     def __init__(self, expert: int = -1, cell: int = -1):
         super().__init__(f"prefetch claim refused: expert {expert}, cell {cell}")
         self.expert, self.cell = expert, cell
+
+
+class ExpertIOScheduler:
+    """ExpertIOScheduler (sources/Shrike/Infrastructure/Streaming/ExpertLoadOperation.swift:166-219): a fixed
+    set of submission threads; a queued demand batch runs before any queued speculative one."""
+
+    DEMAND, SPECULATIVE = 0, 1
+
+    def __init__(self, worker_count: int = 4):
+        import collections
+        import threading
+        if worker_count <= 0:
+            raise ValueError("workerCount must be positive")
+        self._condition = threading.Condition()
+        self._queues = (collections.deque(), collections.deque())
+        self._closed = False
+        self._workers = [threading.Thread(target=self._run, name=f"Shrike.expert-io.{i}", daemon=True)
+                         for i in range(worker_count)]
+        for worker in self._workers:
+            worker.start()
+
+    def submit(self, work, priority: int = 0) -> None:
+        with self._condition:
+            if self._closed:
+                raise ShrikeError("the expert I/O scheduler is closed")
+            self._queues[priority].append(work)
+            self._condition.notify()
+
+    def _run(self):
+        while True:
+            with self._condition:
+                while not self._closed and not self._queues[0] and not self._queues[1]:
+                    self._condition.wait()
+                if not self._queues[0] and not self._queues[1]:
+                    return  # closed and drained
+                work = (self._queues[0] or self._queues[1]).popleft()
+            work()
+
+    def close(self) -> None:
+        """Runs what is queued, then ends the threads."""
+        with self._condition:
+            self._closed = True
+            self._condition.notify_all()
+        for worker in self._workers:
+            worker.join()
 
 
 def _ints(values):

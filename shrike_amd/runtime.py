@@ -11,6 +11,7 @@ import ctypes as C
 import numpy as np
 
 from . import capi
+from . import host as _host
 from .capi import (ACT_SILU, META_BF16, SENTINEL, DecodeLayerArgs, ExpertOffsets, MoEDesc,
                    PoolBases, Projection, ShrikeError, check)
 
@@ -723,7 +724,7 @@ class DecodeLayerWithMisses:
             raise ShrikeError("the device's miss list and the slot cache disagree")
         row = np.full(8, SENTINEL, np.uint32)
         for i in plan.misses:
-            row[i] = plan.assigned_slots[i]
+            row[i] = plan.assigned_cells[i]
         self.agreed.upload(row)
         self.pool.execute_plan(self.cache, plan, self.store, self.store_stride, self.expert_bytes, self.upload_stream)
         landed = Event()
@@ -736,3 +737,205 @@ class DecodeLayerWithMisses:
         m.encode_spec_phase2(self.pool, self.resolved, self.off, self.acts, self.w, residual, y, hidden, d, f, k,
                              fallback_cells=self.agreed, indirect=spec + 36)
         self.fixups += 1
+
+
+class AgreedDecodeLayer:
+    """One token's routed experts over a pool of fewer slots than experts plus a prefetch ring: the runner's
+    agreed layer (RealForwardRunner.swift:5262-5411) over this build's operators. Predictions are read ahead
+    into ring cells as landings; the classifier sees a landed prediction as resident at its ring cell. After
+    the speculative pass every miss of the classifier's list gets its cell: a landing the ring leased (no
+    read), a free ring cell claimed as a landing, or, when the ring has none, a pool slot reserved as an
+    overflow. The demand reads run on the storage threads; the fixup runs phase 1 over the agreed row and
+    phase 2 over all positions; then the plan swaps every leased cell into the pool by index and the freed
+    cells go back to the ring. All numerics happen in libshrikehip; this class sequences calls.
+
+    `cache` is a shrike_amd.host.SlotCache made in a CellArena as long as the pool, `ring` an
+    ExpertPrefetchRing over the cells behind the cache's slots (its drop callback must be this object's
+    `drop_landing`), `layer` the ring's key for this layer."""
+
+    JOIN_NANOS = 2_000_000
+
+    def __init__(self, moe: MoE, pool: ExpertPool, cache, ring, offsets, host_store: PinnedBuffer, store_stride: int,
+                 expert_bytes: int, scheduler, layer: int = 0):
+        k = moe.desc.top_k
+        self.moe, self.pool, self.cache, self.ring, self.off = moe, pool, cache, ring, offsets
+        self.store, self.store_stride, self.expert_bytes = host_store, store_stride, expert_bytes
+        self.scheduler, self.layer = scheduler, layer
+        self.upload_stream = Stream()
+        self.idx, self.w = empty(4 * 8), empty(2 * 8)
+        self.resolved, self.agreed = empty(4 * 8), empty(4 * 8)
+        self.hit_count, self.miss_count = empty(4), empty(4)
+        self.hit_pos, self.miss_pos, self.miss_exp = empty(32), empty(32), empty(32)
+        self.spec_args = empty(48)
+        self.predicted = empty(4 * 8).fill(0)
+        self.readback = PinnedBuffer(4 * (2 + 5 * k))
+        self.acts = empty(2 * k * moe.desc.f)
+        self.tag = 0
+        self.fixups = self.overflows = self.landed_hits = self.demand_reads = 0
+
+    def drop_landing(self, layer: int, expert: int, cell: int) -> None:
+        """The ring's reclaim of a landing no plan wanted (called with the ring locked)."""
+        if layer == self.layer:
+            self.cache.drop_landing(expert, cell)
+
+    def _copy(self, experts, cells):
+        """The reads: each expert's blob from the pinned store into its cell; returns when the bytes are in HBM."""
+        L = capi.load()
+        for expert, cell in zip(experts, cells):
+            check(L.shrike_hip_pool_upload_async(self.pool.handle, cell, self.store.ptr + expert * self.store_stride,
+                                                 self.expert_bytes, self.upload_stream.handle),
+                  "shrike_hip_pool_upload_async")
+        self.upload_stream.synchronize()
+
+    def _publish(self):
+        """The cache's changed residency words into the device table, in order, ahead of the next launch."""
+        for expert, word in self.cache.drain_publications():
+            self.pool.publish(expert, word & 0xFFFFFFFF, word >> 32, self.moe.stream)
+
+    def prefetch(self, predicted_experts) -> None:
+        """schedulePredictivePrefetch (RealForwardRunner.swift:474-494) with beginPrefetch as the ring's issue
+        (PreadExpertStreamer.swift:1034-1072): the predictions the pool lacks are claimed as landings in free
+        ring cells and read speculatively; a refused or failed issue is counted, never thrown into the decode."""
+        def issue(experts, cells):
+            self.cache.claim_prefetch(experts, cells)  # PrefetchClaimRefused passes through to the ring
+            operation = _host.ExpertLoadOperation()
+
+            def work():
+                operation.mark_in_flight()
+                try:
+                    self._copy(experts, cells)
+                    for expert, cell in zip(experts, cells):
+                        self.cache.complete_landing(expert, cell)
+                    operation.finish(0)
+                except Exception:
+                    for expert, cell in zip(experts, cells):
+                        self.cache.fail_landing(expert, cell)
+                    operation.finish(5)
+            self.scheduler.submit(work, _host.ExpertIOScheduler.SPECULATIVE)
+            return operation
+
+        try:
+            self.ring.begin(self.layer, list(predicted_experts), resident=self.cache.resident_experts(), issue=issue)
+        except Exception:
+            self.ring.note_hook_failure()
+
+    def run(self, router, x, residual, y, hidden):
+        """router: dict(weights, scales, biases, eff_scale, expert_scale, bias). x: fp16[d], residual: fp16[d],
+        y: fp16[d] out, hidden: fp16[d] updated in place."""
+        m = self.moe
+        d, f, ne, k = m.desc.d, m.desc.f, m.desc.num_experts, m.desc.top_k
+        compute = m.stream
+        self._publish()
+        m.encode_router(router["weights"], router.get("scales"), router.get("biases"), x, router["eff_scale"],
+                        router["expert_scale"], router["bias"], self.idx, self.w, ne, d, k)
+        self.tag = self.tag % 0xFFFF + 1
+        m.encode_residency_classification(self.idx, self.pool.table, self.hit_count, self.hit_pos, self.miss_count,
+                                          self.miss_pos, self.miss_exp, self.resolved, k, ne, full_grids=[1] * 12,
+                                          spec_args=self.spec_args, host_readback=self.readback, tag=self.tag,
+                                          topk_weights=self.w, predicted=self.predicted)
+        spec = self.spec_args.ptr
+        m.encode_spec_phase1(self.pool, self.resolved, self.off, x, self.acts, d, f, k, indirect=spec)
+        m.encode_spec_phase2(self.pool, self.resolved, self.off, self.acts, self.w, residual, y, hidden, d, f, k,
+                             indirect=spec + 12)
+        (compute.synchronize() if compute else synchronize())
+        rb = self.readback.array.view(np.uint32)[: 2 + 5 * k].copy()
+        if np.any(rb >> 16 != self.tag):
+            raise ShrikeError("router readback carries another launch's tag")
+        rb &= 0xFFFF
+        misses = int(rb[1])
+        experts = rb[2:2 + k].tolist()
+        miss_positions = rb[2 + 3 * k: 2 + 3 * k + misses].tolist()
+
+        # joinAgreedLandings, :5262-5267
+        leased = self.ring.ready_cells(self.layer, experts, self.JOIN_NANOS)
+        # agreeCells / agreeCell, :5273-5317
+        unleased = [experts[p] for p in miss_positions if experts[p] not in leased]
+        claimed = self.ring.claim_demand(self.layer, unleased)
+        read_experts, read_cells, overflow = [], [], {}
+        row = np.full(8, SENTINEL, np.uint32)
+        try:
+            for position in miss_positions:
+                expert = experts[position]
+                if expert in leased:
+                    row[position] = leased[expert]
+                    continue
+                if expert in claimed:
+                    if self.cache.claim_landing(expert, claimed[expert]):
+                        read_experts.append(expert)
+                        read_cells.append(claimed[expert])
+                        row[position] = claimed[expert]
+                        continue
+                    self.ring.consume(self.layer, [expert], {})
+                    del claimed[expert]
+                late = self.ring.ready_cells(self.layer, [expert], self.JOIN_NANOS)
+                if expert in late:
+                    leased[expert] = row[position] = late[expert]
+                    continue
+                cell = self.cache.reserve_overflow_slot(expert, protecting=experts)
+                if cell is None:
+                    raise ShrikeError(f"layer {self.layer} has no cell for expert {expert}")  # expertCacheUnplaceable
+                overflow[expert] = cell
+                read_experts.append(expert)
+                read_cells.append(cell)
+                row[position] = cell
+        except Exception:
+            # abandonAgreedContext, :5342-5349
+            self.ring.consume(self.layer, list(set(leased) | set(claimed)), {})
+            for expert, cell in overflow.items():
+                self.cache.abandon_overflow_slot(expert, cell)
+            raise
+        self.overflows += len(overflow)
+
+        # submitAgreedReads, :5319-5340 (beginAgreedReads, PreadExpertStreamer.swift:903-964)
+        operation = _host.ExpertLoadOperation()
+        if read_experts:
+            started = _host.monotonic_nanos()
+
+            def work():
+                operation.mark_in_flight()
+                fetch_started = _host.monotonic_nanos()
+                try:
+                    self._copy(read_experts, read_cells)
+                    landed = _host.monotonic_nanos()
+                    self.cache.finish_agreed_reads(read_experts, read_cells, True, landed - started, landed - fetch_started)
+                    operation.finish(0)
+                except Exception:
+                    self.cache.finish_agreed_reads(read_experts, read_cells, False)
+                    operation.finish(5)
+            self.scheduler.submit(work, _host.ExpertIOScheduler.DEMAND)
+            self.ring.attach_demand(self.layer, list(claimed), operation)
+            self.ring.note_demand_submission()
+            self.demand_reads += len(read_experts)
+        else:
+            operation.finish(0)
+
+        held = list(set(leased) | set(claimed))
+        if misses:
+            try:
+                operation.wait()  # the reference's fixup waits on the batch's event value instead of the host
+            except Exception:
+                self.ring.consume(self.layer, held, {})  # abandonPendingAgreedLayer, :5351-5355
+                raise ShrikeError(f"layer {self.layer}: an agreed read failed")
+            self.agreed.upload(row)
+            self._publish()
+            m.encode_spec_phase1(self.pool, self.agreed, self.off, x, self.acts, d, f, k, indirect=spec + 24)
+            m.encode_spec_phase2(self.pool, self.resolved, self.off, self.acts, self.w, residual, y, hidden, d, f, k,
+                                 fallback_cells=self.agreed, indirect=spec + 36)
+            self.fixups += 1
+
+        # planAgreedLayer, :5380-5411
+        miss_experts = [experts[p] for p in miss_positions]
+        plan = self.cache.plan(experts, gpu_missed_experts=miss_experts, leased_landings=held,
+                               misses_counted=len(read_experts))
+        if plan is None:
+            self.ring.unlease(self.layer, held)
+            raise ShrikeError(f"layer {self.layer}: the route does not fit its pool")
+        if plan.misses:
+            self.cache.abandon(plan)
+            self.ring.consume(self.layer, held, plan.freed_cells)
+            raise ShrikeError(f"layer {self.layer}: an agreed read did not land for experts "
+                              f"{[plan.experts[i] for i in plan.misses]}")
+        self.landed_hits += sum(1 for e in leased if e not in miss_experts)
+        self.ring.consume(self.layer, held, plan.freed_cells)
+        self._publish()
+        return plan

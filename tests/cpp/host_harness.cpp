@@ -98,6 +98,70 @@ static void wavePlanner() {
 }
 
 // PreadExpertStreamerTests+CachePlanning.swift:130-154, :225-270, :320-341
+// PreadExpertStreamerTests+Landing.swift: aSwapThenAnEvictionOfTheSameSlotPublishesEmptyOnceAtTheCell,
+// aPredictionThePoolHoldsRefusesTheBatch and anOverflowSlotIsAVictimOfThePoolLoadingAtItsCell
+static void landings() {
+    const auto word = [](uint32_t state, uint32_t cell) { return uint64_t(state) << 32 | cell; };
+    {
+        CellArena arena(4);
+        SlotCache c(arena, 2, 4, 0);
+        auto warm = c.planExpertsCached({0, 2});
+        c.markPlanMissesResident(warm);
+        const int64_t ring = 2;
+        c.claimPrefetch({1}, {ring});
+        EXPECT(c.completeLanding(1, ring));
+        EXPECT(c.residencyEntry(1) == word(SHRIKE_RESIDENCY_RESIDENT, 2));
+        auto swap = c.planExpertsCachedIfPossible({0, 1}, 0, {}, nullptr, -1, {}, {1});
+        EXPECT(swap && swap->hits == 2 && swap->misses.empty());
+        EXPECT(swap->assignedSlots == (std::vector<int32_t>{0, 1}));
+        EXPECT(swap->freedCells == (std::map<int32_t, uint32_t>{{1, 1}}));
+        EXPECT(swap->assignedGenerations == (std::vector<uint64_t>{1, 3}));
+        EXPECT(swap->assignedCells == (std::vector<uint32_t>{0, 2}));
+        EXPECT(arena.cellGeneration(1) == 4 && arena.cellGeneration(2) == 3);
+        EXPECT(c.residencyEntry(2) == word(SHRIKE_RESIDENCY_EMPTY, 0xffffffffu));
+        auto evict = c.planExpertsCached({3});
+        EXPECT(evict.assignedSlots == (std::vector<int32_t>{1}) && evict.assignedGenerations == (std::vector<uint64_t>{5}));
+        EXPECT(c.residencyEntry(3) == word(SHRIKE_RESIDENCY_LOADING, 2));
+        EXPECT(c.ownsCell(2) && !c.ownsCell(1) && c.slotCell(1) == 2);
+    }
+    {
+        CellArena arena(6);
+        SlotCache c(arena, 4, 4, 0);
+        auto warm = c.planExpertsCached({1});
+        c.markPlanMissesResident(warm);
+        bool refused = false;
+        try {
+            c.claimPrefetch({3, 1}, {4, 5});
+        } catch (const PrefetchClaimRefused &r) {
+            refused = r.expert == 1 && r.cell == 5;
+        }
+        EXPECT(refused);
+        EXPECT(c.residencyEntry(3) == word(SHRIKE_RESIDENCY_EMPTY, 0xffffffffu));
+        EXPECT(c.claimLanding(3, 4));
+        bool owned = false;
+        try {
+            c.claimPrefetch({2}, {0});
+        } catch (const Error &) {
+            owned = true;
+        }
+        EXPECT(owned);
+    }
+    {
+        CellArena arena(4);
+        SlotCache c(arena, 2, 4, 0);
+        auto warm = c.planExpertsCached({0, 1});
+        c.markPlanMissesResident(warm);
+        EXPECT(!c.reserveOverflowSlot(2, {0, 1}));
+        const auto cell = c.reserveOverflowSlot(2, {0, 5});
+        EXPECT(cell && *cell == 1);
+        EXPECT(c.claimLanding(3, 2));
+        c.finishAgreedReads({3, 2}, {2, int64_t(*cell)}, true);
+        EXPECT(c.residencyEntry(3) == word(SHRIKE_RESIDENCY_RESIDENT, 2));
+        EXPECT(c.residencyEntry(2) == word(SHRIKE_RESIDENCY_RESIDENT, *cell));
+        EXPECT(c.statistics().read_operations == 4);
+    }
+}
+
 static void slotCache() {
     {
         SlotCache c(4, 8);
@@ -304,6 +368,7 @@ int main() {
     sweepOrder();
     wavePlanner();
     slotCache();
+    landings();
     std::printf(failures ? "%d checks failed\n" : "all host checks passed\n", failures);
     return failures ? 1 : 0;
 }
