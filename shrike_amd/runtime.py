@@ -751,7 +751,8 @@ class AgreedDecodeLayer:
 
     `cache` is a shrike_amd.host.SlotCache made in a CellArena as long as the pool, `ring` an
     ExpertPrefetchRing over the cells behind the cache's slots (its drop callback must be this object's
-    `drop_landing`), `layer` the ring's key for this layer."""
+    `drop_landing`), `layer` this layer's key in the ring. A begin for another layer reclaims this layer's
+    finished landings that no route wanted, as in the runner."""
 
     JOIN_NANOS = 2_000_000
 
@@ -821,7 +822,7 @@ class AgreedDecodeLayer:
 
     def run(self, router, x, residual, y, hidden):
         """router: dict(weights, scales, biases, eff_scale, expert_scale, bias). x: fp16[d], residual: fp16[d],
-        y: fp16[d] out, hidden: fp16[d] updated in place."""
+        y: fp16[d] out, hidden: fp16[d] updated in place. Returns the route's plan."""
         m = self.moe
         d, f, ne, k = m.desc.d, m.desc.f, m.desc.num_experts, m.desc.top_k
         compute = m.stream

@@ -1,0 +1,98 @@
+"""Decode over a pool of fewer slots than experts with a prefetch ring beside it: a run of tokens, each
+with predictions for the next (some right, some wrong, some none), gives for every token the bytes of the
+layer with every expert resident, whichever way each selected expert reached HBM: a pool hit, a landed
+prediction, a demand read into a ring cell, or an overflow slot."""
+import numpy as np
+import pytest
+
+from shrike_amd import capi, host
+from shrike_amd import synth as S
+from tests.helpers import Layer
+from tests.test_decode_gpu import DeviceLayer
+
+pytestmark = pytest.mark.gpu
+
+
+def token_inputs(L, count):
+    tree = L.tree
+    return [(S.f32_to_f16_bits(tree.key(f"agreed.x.{i}").normal(L.d, std=1.0)),
+             S.f32_to_f16_bits(tree.key(f"agreed.hidden.{i}").normal(L.d, std=1.0))) for i in range(count)]
+
+
+@pytest.mark.parametrize("bits,slots,ring_cells,foresight", [(4, 10, 4, 0.75), (8, 8, 2, 0.5), (4, 9, 3, 0.0)])
+def test_agreed_layer_with_a_prefetch_ring_equals_the_resident_layer(gpu, bits, slots, ring_cells, foresight):
+    d, f, ne, k, tokens = 512, 256, 32, 8, 10
+    L = Layer(0x5EED0091 + bits + slots, d, f, ne, k, bits=bits)
+    inputs = token_inputs(L, tokens)
+
+    # every token over the layer with all experts resident: the bytes to match, and the routes to foresee
+    full = DeviceLayer(gpu, L)
+    want = []
+    for x, hidden in inputs:
+        full.x.upload(x)
+        full.hidden.upload(hidden)
+        full.moe.encode_decode_layer(full.layer_args())
+        gpu.synchronize()
+        want.append((full.out_idx.download(np.uint32, k).tolist(), full.y.download(np.uint16, d),
+                     full.hidden.download(np.uint16, d)))
+
+    small = DeviceLayer(gpu, L, cells=slots + ring_cells, resident=[])
+    small.moe.stream = gpu.Stream()
+    arena = host.CellArena(slots + ring_cells)
+    cache = host.SlotCache(slots, ne, 0, arena=arena)
+    store = gpu.PinnedBuffer(ne * L.stride)
+    for e in range(ne):
+        store.array[e * L.stride:(e + 1) * L.stride] = L.blobs[e]
+    scheduler = host.ExpertIOScheduler(2)
+    holder = {}
+    ring = host.ExpertPrefetchRing(list(range(slots, slots + ring_cells)),
+                                   drop=lambda layer, expert, cell: holder["layer"].drop_landing(layer, expert, cell))
+    layer = gpu.AgreedDecodeLayer(small.moe, small.pool, cache, ring, small.off, store, L.stride, L.stride, scheduler,
+                                  layer=3)
+    holder["layer"] = layer
+    router = dict(weights=small.router_w, eff_scale=small.eff_scale, expert_scale=small.expert_scale, bias=small.logit_bias)
+    residual = gpu.dev(np.zeros(d, np.uint16))  # no shared expert: the fused layer's residual is zero
+    rng = np.random.default_rng(bits * 100 + slots)
+
+    try:
+        for i, (x, hidden) in enumerate(inputs):
+            small.x.upload(x)
+            small.hidden.upload(hidden)
+            plan = layer.run(router, small.x, residual, small.y, small.hidden)
+            small.moe.stream.synchronize()
+            idx, y, hid = want[i]
+            assert layer.idx.download(np.uint32, k).tolist() == idx, f"token {i}: routes"
+            assert np.array_equal(small.y.download(np.uint16, d), y), f"token {i}: y"
+            assert np.array_equal(small.hidden.download(np.uint16, d), hid), f"token {i}: hidden"
+            # after the plan every selected expert is the pool's, at the cell its entry names
+            assert plan.misses == [] and sorted(plan.experts) == sorted(idx)
+            for e, cell in zip(plan.experts, plan.assigned_cells):
+                assert cache.entry(e) == capi.RESIDENT << 32 | cell and cache.owns_cell(cell)
+            assert [small.pool.entry(e) for e in range(ne)] == [cache.entry(e) for e in range(ne)]
+            assert ring.leased_count == 0
+            # the cells are a partition: the pool's slots and the ring's cells never overlap
+            pool_cells = sorted(cache.slot_cell(s) for s in range(slots))
+            assert len(set(pool_cells)) == slots and all(0 <= c < slots + ring_cells for c in pool_cells)
+            if i + 1 < tokens:
+                coming = want[i + 1][0]
+                right = [e for e in coming if rng.random() < foresight]
+                wrong = [int(e) for e in rng.choice(ne, 2, replace=False) if e not in coming]
+                # the next layer's begin comes first in a model: it reclaims this layer's finished landings
+                # that no route wanted, so the ring's cells come free again
+                ring.begin(4, [], issue=lambda experts, cells: None)
+                layer.prefetch(right + wrong)
+    finally:
+        scheduler.close()
+
+    st, ring_st = cache.statistics(L.stride), ring.statistics
+    assert st.loading_slots == 0 and st.pinned_slots == 0
+    assert st.requested_experts == tokens * k
+    assert layer.fixups >= 1  # the first token finds an empty pool
+    assert layer.demand_reads == st.misses
+    if foresight == 0.0:
+        assert layer.landed_hits == 0
+    else:
+        assert layer.landed_hits > 0, "no prediction landed ahead of its route"
+    assert ring_st["issued"] >= ring_st["adopted"]
+    print(f"\nbits {bits} slots {slots} ring {ring_cells}: fixups {layer.fixups}, demand reads {layer.demand_reads}, "
+          f"overflow {layer.overflows}, landed hits {layer.landed_hits}, ring {ring_st}")
