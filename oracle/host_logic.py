@@ -4,7 +4,8 @@ the shipped implementation is the C++ in shrike_amd/csrc/host_logic.cpp and
 slot_cache.cpp, which the tests compare against these functions.
 
 Every function follows one reference function (cited in its docstring) and is pinned
-in tests/test_host_logic_oracle.py and tests/test_packed_layout.py by the vectors the
+in tests/test_host_logic_oracle.py, tests/test_packed_layout.py, tests/test_tile_scheduler.py,
+tests/test_prefetch_ring.py and tests/test_slot_cache_landings.py by the vectors the
 reference's own unit tests hold.
 All arithmetic here is integer; results are compared for equality.
 """
