@@ -71,6 +71,12 @@ public:
         h_ = shrike_hip_pool_create(cellCount, expertStride, expertsPerLayer, chunkBytes, &err);
         if (!h_) throw Error(err, shrike_hip_last_error());
     }
+    // another layer's residency table over `arena`'s cells; `arena` must outlive it
+    ExpertPool(const ExpertPool &arena, uint32_t expertsPerLayer) {
+        int err = 0;
+        h_ = shrike_hip_pool_create_layer_view(arena.h_, expertsPerLayer, &err);
+        if (!h_) throw Error(err, shrike_hip_last_error());
+    }
     ~ExpertPool() { shrike_hip_pool_destroy(h_); }
     ExpertPool(const ExpertPool &) = delete;
     ExpertPool &operator=(const ExpertPool &) = delete;

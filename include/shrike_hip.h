@@ -94,6 +94,12 @@ typedef struct shrike_hip_pool shrike_hip_pool;
 shrike_hip_pool *shrike_hip_pool_create(uint32_t cells, uint64_t expert_stride,
                                         uint32_t num_experts, uint64_t chunk_bytes,
                                         int *out_errno);
+/* Another layer's residency table over the same cells: the arena is one for the model
+ * (ExpertCellArena.swift:3-8), every layer's streamer owns a range of its cells and a
+ * table of its own (PreadExpertStreamer.swift:309-352). The view shares the arena
+ * pool's cells and bases, must be destroyed before it, and takes every call a pool takes. */
+shrike_hip_pool *shrike_hip_pool_create_layer_view(const shrike_hip_pool *arena,
+                                                   uint32_t num_experts, int *out_errno);
 void shrike_hip_pool_destroy(shrike_hip_pool *pool);
 uint64_t shrike_hip_pool_slot_stride(const shrike_hip_pool *pool);
 uint32_t shrike_hip_pool_cell_count(const shrike_hip_pool *pool);

@@ -252,6 +252,7 @@ SIGNATURES = {
     "shrike_parse_budget_bytes": (_I64, [C.c_char_p]),
     "shrike_expert_cache_slots": (_I32, [_U64, _I32, _I64]),
     "shrike_hip_pool_create": (_VP, [_U32, _U64, _U32, _U64, C.POINTER(C.c_int)]),
+    "shrike_hip_pool_create_layer_view": (_VP, [_VP, _U32, C.POINTER(C.c_int)]),
     "shrike_hip_pool_destroy": (None, [_VP]),
     "shrike_hip_pool_fetch_experts": (C.c_int, [_VP, _VP, _VP, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), _U32, _U64,
                                                 _VP, _U64]),

@@ -53,6 +53,7 @@ struct shrike_hip_pool {
     shrike_pool_bases bases;
     uint64_t *d_table;
     std::vector<uint64_t> shadow;  // host copy of the table, updated at publish
+    bool owns_cells = true;        // false for a layer's table over another pool's cells
 };
 
 extern "C" {
@@ -207,10 +208,35 @@ shrike_hip_pool *shrike_hip_pool_create(uint32_t cells, uint64_t expert_stride, 
     return pool;
 }
 
+shrike_hip_pool *shrike_hip_pool_create_layer_view(const shrike_hip_pool *arena, uint32_t num_experts, int *out_errno) {
+    auto fail = [&](int code) -> shrike_hip_pool * { if (out_errno) *out_errno = code; return nullptr; };
+    if (!arena || num_experts == 0) {
+        set_error("a layer's residency table needs an arena and at least one expert");
+        return fail(EINVAL);
+    }
+    shrike_hip_pool *pool = new shrike_hip_pool();
+    pool->cells = arena->cells; pool->num_experts = num_experts; pool->stride = arena->stride;
+    pool->cells_per_chunk = arena->cells_per_chunk; pool->chunk_count = arena->chunk_count;
+    memcpy(pool->chunks, arena->chunks, sizeof(pool->chunks));
+    pool->bases = arena->bases;
+    pool->owns_cells = false;
+    pool->d_table = nullptr;
+    pool->shadow.assign(num_experts, uint64_t(SHRIKE_RESIDENCY_EMPTY) << 32 | SHRIKE_SLOT_SENTINEL);
+    if (hipMalloc(reinterpret_cast<void **>(&pool->d_table), sizeof(uint64_t) * num_experts) != hipSuccess
+        || hipMemcpy(pool->d_table, pool->shadow.data(), sizeof(uint64_t) * num_experts, hipMemcpyHostToDevice)
+               != hipSuccess) {
+        set_error("residency table allocation failed");
+        shrike_hip_pool_destroy(pool);
+        return fail(ENOMEM);
+    }
+    if (out_errno) *out_errno = 0;
+    return pool;
+}
+
 void shrike_hip_pool_destroy(shrike_hip_pool *pool) {
     if (!pool) return;
     for (void *c : pool->chunks)
-        if (c) (void)hipFree(c);
+        if (c && pool->owns_cells) (void)hipFree(c);
     if (pool->d_table) (void)hipFree(pool->d_table);
     delete pool;
 }

@@ -176,6 +176,21 @@ class ExpertPool:
         self.bases = L.shrike_hip_pool_bases(self.handle)
         self.table = L.shrike_hip_pool_residency_table(self.handle)
 
+    def layer_view(self, num_experts: int | None = None) -> "ExpertPool":
+        """Another layer's residency table over this pool's cells (one arena for the model, a table per layer);
+        this pool must outlive the view."""
+        err = C.c_int(0)
+        L = capi.load()
+        view = object.__new__(ExpertPool)
+        view.handle = L.shrike_hip_pool_create_layer_view(self.handle, num_experts or self.num_experts, C.byref(err))
+        if not view.handle:
+            raise ShrikeError(f"shrike_hip_pool_create_layer_view failed with {err.value}: {capi.last_error()}")
+        view.cells, view.num_experts = self.cells, num_experts or self.num_experts
+        view.stride, view.bases = self.stride, L.shrike_hip_pool_bases(view.handle)
+        view.table = L.shrike_hip_pool_residency_table(view.handle)
+        view._arena = self  # keeps the cells alive
+        return view
+
     def cell_ptr(self, cell: int) -> int:
         p = capi.load().shrike_hip_pool_cell_ptr(self.handle, cell)
         if not p:

@@ -96,3 +96,89 @@ def test_agreed_layer_with_a_prefetch_ring_equals_the_resident_layer(gpu, bits, 
     assert ring_st["issued"] >= ring_st["adopted"]
     print(f"\nbits {bits} slots {slots} ring {ring_cells}: fixups {layer.fixups}, demand reads {layer.demand_reads}, "
           f"overflow {layer.overflows}, landed hits {layer.landed_hits}, ring {ring_st}")
+
+
+def test_two_layers_share_one_arena_and_one_ring(gpu):
+    """The model's shape: one arena of cells (two layers' slot ranges and the ring's cells), a residency table
+    and a slot cache per layer, one ring for both. Each layer's begin reclaims the other's finished landings;
+    a landing swapped into one layer's pool hands that layer's freed cell to the ring, so cells migrate between
+    the layers' ranges while every token of both layers keeps the resident layers' bytes."""
+    d, f, ne, k, tokens = 512, 256, 32, 8, 8
+    slots, ring_cells = (10, 9), 3
+    cells = sum(slots) + ring_cells
+    layers = [Layer(0x5EED00A1, d, f, ne, k, bits=4), Layer(0x5EED00A2, d, f, ne, k, bits=4)]
+    inputs = [token_inputs(L, tokens) for L in layers]
+    want = []
+    for L, ins in zip(layers, inputs):
+        full, rows = DeviceLayer(gpu, L), []
+        for x, hidden in ins:
+            full.x.upload(x)
+            full.hidden.upload(hidden)
+            full.moe.encode_decode_layer(full.layer_args())
+            gpu.synchronize()
+            rows.append((full.out_idx.download(np.uint32, k).tolist(), full.y.download(np.uint16, d),
+                         full.hidden.download(np.uint16, d)))
+        want.append(rows)
+
+    arena_pool = gpu.ExpertPool(cells, layers[0].stride, ne)
+    pools = [arena_pool, arena_pool.layer_view()]
+    arena = host.CellArena(cells)
+    caches = [host.SlotCache(slots[0], ne, 0, arena=arena), host.SlotCache(slots[1], ne, slots[0], arena=arena)]
+    scheduler = host.ExpertIOScheduler(2)
+    agreed = []
+    ring = host.ExpertPrefetchRing(list(range(sum(slots), cells)),
+                                   drop=lambda layer, expert, cell: agreed[layer].drop_landing(layer, expert, cell))
+    devs, routers, stores = [], [], []
+    stream = gpu.Stream()
+    for index, L in enumerate(layers):
+        dev = DeviceLayer(gpu, L, resident=[], pool=pools[index])
+        dev.moe.stream = stream
+        store = gpu.PinnedBuffer(ne * L.stride)
+        for e in range(ne):
+            store.array[e * L.stride:(e + 1) * L.stride] = L.blobs[e]
+        agreed.append(gpu.AgreedDecodeLayer(dev.moe, pools[index], caches[index], ring, dev.off, store, L.stride, L.stride,
+                                            scheduler, layer=index))
+        routers.append(dict(weights=dev.router_w, eff_scale=dev.eff_scale, expert_scale=dev.expert_scale, bias=dev.logit_bias))
+        devs.append(dev)
+        stores.append(store)
+    residual = gpu.dev(np.zeros(d, np.uint16))
+    rng = np.random.default_rng(7)
+
+    def predictions(layer_index, token):
+        coming = want[layer_index][token][0]
+        right = [e for e in coming if rng.random() < 0.6]
+        return right + [int(e) for e in rng.choice(ne, 2, replace=False) if e not in coming]
+
+    try:
+        for t in range(tokens):
+            for index in (0, 1):
+                dev = devs[index]
+                x, hidden = inputs[index][t]
+                dev.x.upload(x)
+                dev.hidden.upload(hidden)
+                agreed[index].run(routers[index], dev.x, residual, dev.y, dev.hidden)
+                stream.synchronize()
+                idx, y, hid = want[index][t]
+                assert agreed[index].idx.download(np.uint32, k).tolist() == idx, f"token {t} layer {index}: routes"
+                assert np.array_equal(dev.y.download(np.uint16, d), y), f"token {t} layer {index}: y"
+                assert np.array_equal(dev.hidden.download(np.uint16, d), hid), f"token {t} layer {index}: hidden"
+                assert [pools[index].entry(e) for e in range(ne)] == [caches[index].entry(e) for e in range(ne)]
+                # the runner schedules the next layer's predictions while this layer's reads are behind it
+                following, at = (1, t) if index == 0 else (0, t + 1)
+                if at < tokens:
+                    agreed[following].prefetch(predictions(following, at))
+            owned = [caches[i].slot_cell(s) for i in (0, 1) for s in range(slots[i])]
+            assert len(set(owned)) == sum(slots), "two slots name one cell"
+            assert ring.leased_count == 0
+    finally:
+        scheduler.close()
+
+    moved = [sum(1 for s in range(slots[i]) if not (i * slots[0] <= caches[i].slot_cell(s) < slots[0] + i * slots[1]))
+             for i in (0, 1)]
+    hits = [a.landed_hits for a in agreed]
+    print(f"\ntwo layers: landed hits {hits}, slots now on cells outside their first range {moved}, "
+          f"overflow {[a.overflows for a in agreed]}, ring {ring.statistics}")
+    assert sum(hits) > 0 and sum(moved) > 0
+    for cache in caches:
+        st = cache.statistics()
+        assert st.loading_slots == 0 and st.requested_experts == tokens * k

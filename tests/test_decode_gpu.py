@@ -19,11 +19,11 @@ SENT = 0xFFFFFFFF
 class DeviceLayer:
     """Uploads a Layer: every expert resident in a pool, cell = a permutation of the expert id."""
 
-    def __init__(self, rt, layer: Layer, cells=None, chunk_bytes=0, resident=None, moe_kwargs=None):
+    def __init__(self, rt, layer: Layer, cells=None, chunk_bytes=0, resident=None, moe_kwargs=None, pool=None):
         self.rt, self.L = rt, layer
         L = layer
         cells = cells or L.ne
-        self.pool = rt.ExpertPool(cells, L.stride, L.ne, chunk_bytes)
+        self.pool = pool or rt.ExpertPool(cells, L.stride, L.ne, chunk_bytes)
         self.cell_of = {}
         resident = range(L.ne) if resident is None else resident
         for i, e in enumerate(resident):
