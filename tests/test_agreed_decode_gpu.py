@@ -182,3 +182,52 @@ def test_two_layers_share_one_arena_and_one_ring(gpu):
     for cache in caches:
         st = cache.statistics()
         assert st.loading_slots == 0 and st.requested_experts == tokens * k
+
+
+def test_a_failed_agreed_read_leaves_the_cache_and_the_ring_clean(gpu):
+    """A demand batch whose copies fail (forced from the host): the layer raises, the landings are dropped,
+    the overflow slots emptied and every lease returned; the same token then runs clean."""
+    d, f, ne, k, slots, ring_cells = 256, 128, 16, 4, 5, 2
+    L = Layer(0x5EED00B1, d, f, ne, k, bits=4)
+    full = DeviceLayer(gpu, L)
+    full.moe.encode_decode_layer(full.layer_args())
+    gpu.synchronize()
+    want = (full.out_idx.download(np.uint32, k).tolist(), full.y.download(np.uint16, d), full.hidden.download(np.uint16, d))
+
+    small = DeviceLayer(gpu, L, cells=slots + ring_cells, resident=[])
+    small.moe.stream = gpu.Stream()
+    cache = host.SlotCache(slots, ne, 0, arena=host.CellArena(slots + ring_cells))
+    store = gpu.PinnedBuffer(ne * L.stride)
+    for e in range(ne):
+        store.array[e * L.stride:(e + 1) * L.stride] = L.blobs[e]
+    scheduler = host.ExpertIOScheduler(1)
+    holder = {}
+    ring = host.ExpertPrefetchRing(list(range(slots, slots + ring_cells)),
+                                   drop=lambda layer, expert, cell: holder["layer"].drop_landing(layer, expert, cell))
+    layer = gpu.AgreedDecodeLayer(small.moe, small.pool, cache, ring, small.off, store, L.stride, L.stride, scheduler)
+    holder["layer"] = layer
+    router = dict(weights=small.router_w, eff_scale=small.eff_scale, expert_scale=small.expert_scale, bias=small.logit_bias)
+    residual = gpu.dev(np.zeros(d, np.uint16))
+    copy = layer._copy
+
+    def failing(experts, cells):
+        raise OSError(5, "forced read failure")
+    try:
+        layer._copy = failing
+        with pytest.raises(capi.ShrikeError, match="agreed read failed"):
+            layer.run(router, small.x, residual, small.y, small.hidden)
+        small.moe.stream.synchronize()
+        st = cache.statistics()
+        assert st.loading_slots == 0 and st.resident_slots == 0 and cache.resident_experts() == []
+        assert all(cache.entry(e) >> 32 == capi.EMPTY for e in range(ne))
+        assert ring.leased_count == 0 and ring.in_flight_count == 0
+        layer._copy = copy
+        small.hidden.upload(L.hidden)
+        plan = layer.run(router, small.x, residual, small.y, small.hidden)
+        small.moe.stream.synchronize()
+        assert plan.misses == [] and layer.idx.download(np.uint32, k).tolist() == want[0]
+        assert np.array_equal(small.y.download(np.uint16, d), want[1])
+        assert np.array_equal(small.hidden.download(np.uint16, d), want[2])
+        assert [small.pool.entry(e) for e in range(ne)] == [cache.entry(e) for e in range(ne)]
+    finally:
+        scheduler.close()
