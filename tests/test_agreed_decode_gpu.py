@@ -2,6 +2,8 @@
 with predictions for the next (some right, some wrong, some none), gives for every token the bytes of the
 layer with every expert resident, whichever way each selected expert reached HBM: a pool hit, a landed
 prediction, a demand read into a ring cell, or an overflow slot."""
+import time
+
 import numpy as np
 import pytest
 
@@ -11,6 +13,15 @@ from tests.helpers import Layer
 from tests.test_decode_gpu import DeviceLayer
 
 pytestmark = pytest.mark.gpu
+
+
+def wait_for_the_ring(ring, seconds=10.0):
+    """The speculative reads issued so far have landed (or failed): what the next token's classifier sees does
+    not hang on how fast the storage thread runs."""
+    deadline = time.monotonic() + seconds
+    while ring.in_flight_count and time.monotonic() < deadline:
+        time.sleep(0.0005)
+    assert ring.in_flight_count == 0, "a speculative read is still in flight"
 
 
 def token_inputs(L, count):
@@ -81,6 +92,7 @@ def test_agreed_layer_with_a_prefetch_ring_equals_the_resident_layer(gpu, bits, 
                 # that no route wanted, so the ring's cells come free again
                 ring.begin(4, [], issue=lambda experts, cells: None)
                 layer.prefetch(right + wrong)
+                wait_for_the_ring(ring)
     finally:
         scheduler.close()
 
@@ -167,6 +179,7 @@ def test_two_layers_share_one_arena_and_one_ring(gpu):
                 following, at = (1, t) if index == 0 else (0, t + 1)
                 if at < tokens:
                     agreed[following].prefetch(predictions(following, at))
+                    wait_for_the_ring(ring)
             owned = [caches[i].slot_cell(s) for i in (0, 1) for s in range(slots[i])]
             assert len(set(owned)) == sum(slots), "two slots name one cell"
             assert ring.leased_count == 0
