@@ -368,6 +368,26 @@ int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shri
                                    void *d_route_partials, void *d_workspace, size_t workspace_bytes,
                                    uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k);
 
+/* PrefillGroupedRoutedMoE.encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:846-922; kernels
+ * prefill_moe_affine_gemv_row_dev and its batched phases, prefill.metal:318-363, :647-728): the
+ * routed FFN of the sorted pairs [pair_start, pair_start + pair_count) only — one routed tile of
+ * a streamed chunk — with the experts' cells read from d_residency as it stands when the launch
+ * runs (NULL: the cells recorded at grouping time). Rows of other pairs are left untouched, and
+ * so are the rows of experts the table does not hold. The reference walks the range in
+ * microbatches of pair_microbatch_rows pairs through a scalar kernel; here the range goes through
+ * the grouped MFMA kernels in one pass, and *out_microbatches reports the count the reference
+ * returns. A range need not end at an expert's boundary. Arguments otherwise as for
+ * shrike_hip_prefill_grouped_ffn; the workspace may be shared between calls on one stream. */
+int shrike_hip_prefill_streamed_batched(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                        uint64_t pool_slot_stride, const shrike_expert_offsets *offsets,
+                                        const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles,
+                                        const uint64_t *d_residency, uint32_t pair_start,
+                                        uint32_t pair_count, uint32_t pair_microbatch_rows,
+                                        const void *d_hidden, uint32_t hidden_stride_elements,
+                                        void *d_route_partials, void *d_workspace, size_t workspace_bytes,
+                                        uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k,
+                                        uint32_t *out_microbatches);
+
 /* The shared expert for query_count tokens (RealForwardRunner.swift:4620-4647: the dense
  * int4/int8 QMMs of MPPPrefillInt4QMM + silu_mul_fp16) on the grouped kernel: h1[t, :] =
  * half(down . half(glu(half(gate . x_t), half(up . x_t)))), optionally * sigmoid(scalar_gate[0])

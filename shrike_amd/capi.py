@@ -323,6 +323,9 @@ SIGNATURES = {
     "shrike_hip_prefill_grouped_ffn": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, C.POINTER(ExpertOffsets),
                                                  C.POINTER(HipGroupedRoutes), _U32, _VP, _U32, _VP, _VP, C.c_size_t,
                                                  _U32, _U32, _U32, _U32]),
+    "shrike_hip_prefill_streamed_batched": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, C.POINTER(ExpertOffsets),
+                                                      C.POINTER(HipGroupedRoutes), _U32, _VP, _U32, _U32, _U32, _VP, _U32,
+                                                      _VP, _VP, C.c_size_t, _U32, _U32, _U32, _U32, C.POINTER(C.c_uint32)]),
     "shrike_hip_prefill_shared_expert_workspace_bytes": (C.c_size_t, [_U32, _U32, _U32]),
     "shrike_hip_prefill_shared_expert": (C.c_int, [_VP, _VP, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection),
                                                    _U32, _VP, _U32, _VP, _VP, _VP, C.c_size_t, _U32, _U32, _U32]),

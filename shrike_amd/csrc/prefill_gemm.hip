@@ -37,6 +37,8 @@ struct FfnArgs {
     shrike_expert_offsets off;
     const shrike_row_tile *tiles;
     const uint32_t *tile_count;
+    const uint64_t *residency;    // null, or the table that names the tiles' cells at this call
+    uint32_t pair_lo, pair_hi;    // the sorted pairs this call covers; rows of other pairs are left alone
     const shrike_token_expert_pair *pairs;
     const uint16_t *hidden;       // fp16[T, hidden_stride]
     uint32_t hidden_stride;
@@ -370,6 +372,9 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
             }
         }
     } else {
+        // a call over a range of the sorted pairs writes the rows of its pairs only
+        const uint32_t row_lo = DENSE ? 0u : max(a.pair_lo, tile.pair_start) - tile.pair_start;
+        const uint32_t row_hi = DENSE ? tile.rows : min(a.pair_hi, tile.pair_start + tile.rows) - tile.pair_start;
         float dab[2] = {0.0f, 0.0f};
         float gate_mul = 0.0f;
         if (DENSE && a.scalar_gate) gate_mul = 1.0f + expf(-f16_to_f32(a.scalar_gate[0]));
@@ -382,7 +387,7 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
-                if (m < tile.rows) {
+                if (m >= row_lo && m < row_hi) {
                     uint16_t *dst;
                     if (DENSE) {
                         dst = a.partials + size_t(tile.pair_start + m) * a.d + n;
@@ -428,7 +433,12 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     } else {
         if (tile_index >= tile_total) return;
         tile = a.tiles[tile_index];
+        if (a.residency) {  // moe.metal:136-146: a hit names its cell, anything else is the sentinel
+            const uint64_t word = a.residency[tile.expert];
+            tile.cell = uint32_t(word >> 32) == SHRIKE_RESIDENCY_RESIDENT ? uint32_t(word) : kSentinel;
+        }
         if (tile.cell == kSentinel || tile.rows == 0) return;
+        if (tile.pair_start + tile.rows <= a.pair_lo || tile.pair_start >= a.pair_hi) return;
     }
 
     if (tile.rows > 32u) ffn_tile<BITS, MODE, DENSE, 2>(a, tile, tile_index, col_block, s_a);
@@ -472,11 +482,11 @@ size_t shrike_hip_prefill_ffn_workspace_bytes(uint32_t query_count, uint32_t max
     return workspace_layout(query_count, max_row_tiles, d, f).total;
 }
 
-int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
-                                   uint64_t pool_slot_stride, const shrike_expert_offsets *offsets,
-                                   const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles, const void *d_hidden,
-                                   uint32_t hidden_stride_elements, void *d_route_partials, void *d_workspace,
-                                   size_t workspace_bytes, uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k) {
+static int grouped_ffn(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool, uint64_t pool_slot_stride,
+                       const shrike_expert_offsets *offsets, const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles,
+                       const uint64_t *d_residency, uint32_t pair_lo, uint32_t pair_hi, const void *d_hidden,
+                       uint32_t hidden_stride_elements, void *d_route_partials, void *d_workspace, size_t workspace_bytes,
+                       uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k) {
     SHRIKE_REQUIRE(moe && pool && offsets && routes, "grouped FFN: NULL argument");
     SHRIKE_REQUIRE(d == moe->desc.d && f == moe->desc.f, "grouped FFN: shape %ux%u differs from the handle's %ux%u", d, f, moe->desc.d, moe->desc.f);
     SHRIKE_REQUIRE(d % kGroup == 0 && f % kGroup == 0 && d > 0 && f > 0, "D and F must be positive multiples of 64");
@@ -487,7 +497,7 @@ int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shri
     SHRIKE_REQUIRE(reinterpret_cast<uintptr_t>(d_workspace) % 256u == 0, "grouped FFN: workspace must be 256-byte aligned");
     SHRIKE_REQUIRE(pool->cells_per_chunk > 0 && pool_slot_stride % 16u == 0, "grouped FFN: bad pool geometry");
     if (int rc = check_offsets(offsets, d, f, moe->desc.routed_weight_bits)) return rc;
-    if (max_row_tiles == 0 || query_count == 0) return 0;
+    if (max_row_tiles == 0 || query_count == 0 || pair_lo >= pair_hi) return 0;
     const Workspace w = workspace_layout(query_count, max_row_tiles, d, f);
     SHRIKE_REQUIRE(workspace_bytes >= w.total, "grouped FFN: workspace of %zu bytes, %zu needed", workspace_bytes, w.total);
     uint8_t *ws = static_cast<uint8_t *>(d_workspace);
@@ -497,6 +507,9 @@ int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shri
     a.off = *offsets;
     a.tiles = routes->row_tiles;
     a.tile_count = routes->row_tile_count;
+    a.residency = d_residency;
+    a.pair_lo = pair_lo;
+    a.pair_hi = pair_hi;
     a.pairs = static_cast<const shrike_token_expert_pair *>(routes->sorted_pairs);
     a.hidden = static_cast<const uint16_t *>(d_hidden);
     a.hidden_stride = hidden_stride_elements;
@@ -511,6 +524,36 @@ int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shri
     hipStream_t s = as_stream(stream);
     if (int rc = launch_row_group_sums(a.hidden, hidden_stride_elements, query_count, d, const_cast<uint32_t *>(a.hidden_sums), nullptr, s)) return rc;
     return moe->desc.routed_weight_bits == 8 ? launch_ffn<8, false>(a, max_row_tiles, s) : launch_ffn<4, false>(a, max_row_tiles, s);
+}
+
+int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                   uint64_t pool_slot_stride, const shrike_expert_offsets *offsets,
+                                   const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles, const void *d_hidden,
+                                   uint32_t hidden_stride_elements, void *d_route_partials, void *d_workspace,
+                                   size_t workspace_bytes, uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k) {
+    return grouped_ffn(moe, stream, pool, pool_slot_stride, offsets, routes, max_row_tiles, nullptr, 0u, 0xffffffffu, d_hidden,
+                       hidden_stride_elements, d_route_partials, d_workspace, workspace_bytes, query_count, d, f, top_k);
+}
+
+int shrike_hip_prefill_streamed_batched(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                        uint64_t pool_slot_stride, const shrike_expert_offsets *offsets,
+                                        const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles,
+                                        const uint64_t *d_residency, uint32_t pair_start, uint32_t pair_count,
+                                        uint32_t pair_microbatch_rows, const void *d_hidden, uint32_t hidden_stride_elements,
+                                        void *d_route_partials, void *d_workspace, size_t workspace_bytes,
+                                        uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k,
+                                        uint32_t *out_microbatches) {
+    if (out_microbatches) *out_microbatches = 0;
+    // PrefillGroupedRoutedMoE.swift:861-863: nothing to do is not an error
+    if (pair_count == 0 || pair_microbatch_rows == 0) return 0;
+    SHRIKE_REQUIRE(uint64_t(pair_start) + pair_count <= uint64_t(query_count) * top_k, "streamed batch: pairs %u..%llu leave the chunk's %llu",
+                   pair_start, (unsigned long long)pair_start + pair_count, (unsigned long long)query_count * top_k);
+    if (int rc = grouped_ffn(moe, stream, pool, pool_slot_stride, offsets, routes, max_row_tiles, d_residency, pair_start,
+                             pair_start + pair_count, d_hidden, hidden_stride_elements, d_route_partials, d_workspace,
+                             workspace_bytes, query_count, d, f, top_k))
+        return rc;
+    if (out_microbatches) *out_microbatches = (pair_count + pair_microbatch_rows - 1u) / pair_microbatch_rows;
+    return 0;
 }
 
 size_t shrike_hip_prefill_shared_expert_workspace_bytes(uint32_t query_count, uint32_t d, uint32_t f_shared) {

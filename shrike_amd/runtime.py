@@ -404,6 +404,22 @@ class Prefill:
             ptr(route_partials), ptr(workspace), workspace.nbytes, query_count, self.moe.desc.d, self.moe.desc.f, top_k),
             "shrike_hip_prefill_grouped_ffn")
 
+    def encode_streamed_batched(self, pool: ExpertPool, offsets, routes: GroupedRoutesDevice, hidden,
+                                hidden_stride_elements, route_partials, workspace: DeviceBuffer, query_count, top_k,
+                                pair_start: int, pair_count: int, residency=None, pair_microbatch_rows: int = 32,
+                                max_row_tiles=None) -> int:
+        """encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:846-922): the routed FFN of the sorted pairs
+        [pair_start, pair_start + pair_count) against `residency` (a device table, default the cells recorded at
+        grouping); returns the reference's microbatch count."""
+        count = C.c_uint32(0)
+        check(capi.load().shrike_hip_prefill_streamed_batched(
+            self.moe.handle, self._s(), pool.bases, pool.stride, C.byref(offsets), C.byref(routes.c),
+            routes.max_row_tiles if max_row_tiles is None else max_row_tiles, ptr(residency), pair_start, pair_count,
+            pair_microbatch_rows, ptr(hidden), hidden_stride_elements, ptr(route_partials), ptr(workspace),
+            workspace.nbytes, query_count, self.moe.desc.d, self.moe.desc.f, top_k, C.byref(count)),
+            "shrike_hip_prefill_streamed_batched")
+        return count.value
+
     def encode_shared_expert(self, gate, up, down, bits, hidden, hidden_stride_elements, h1, query_count, f_shared,
                              workspace: DeviceBuffer | None = None, scalar_gate=None):
         """The shared expert for every token of the chunk; returns the workspace it used."""

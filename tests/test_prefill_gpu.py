@@ -232,6 +232,57 @@ def test_one_pair_expert_leaves_other_rows_alone(gpu):
     assert np.all(guard.download(np.uint16, 64 * 512) == 0xD4D0)
 
 
+@pytest.mark.parametrize("bits,tile_experts", [(4, 3), (8, 16), (4, 1)])
+def test_streamed_batched_over_pair_ranges_equals_the_whole_chunk(gpu, bits, tile_experts):
+    """encodeStreamedBatched: the chunk's routed tiles (pair ranges of groupTokenExpertPairs' tiles) one call
+    each, against a residency table that holds the tile's experts only, give the partial rows of the one-pass
+    grouped FFN byte for byte, each call writing its own pairs' rows and no others; then a range cut through
+    an expert's rows."""
+    d, f, ne, k, t = 256, 128, 12, 3, 90
+    L = Layer(0x5EED0007 + bits, d, f, ne, k, bits=bits)
+    whole = PrefillCase(gpu, L, t)
+    want = whole.run()
+    pc = PrefillCase(gpu, L, t)
+    pairs = H.make_token_expert_pairs(pc.idx, pc.w, t, k)
+    grouped = H.group_token_expert_pairs(pairs, t, k, ne, tile_expert_count=tile_experts)
+    order = {(p.token, p.rank): i for i, p in enumerate(grouped.sorted_pairs)}
+    cells = pc.dl.cell_of
+    written = np.zeros((t, k), bool)
+    for group_start, group_count, pair_start, pair_count in grouped.tiles:
+        live = [g[0] for g in grouped.groups[group_start:group_start + group_count]]
+        table = np.full(ne, capi.EMPTY << 32 | 0xFFFFFFFF, np.uint64)
+        for e in live:
+            table[e] = capi.RESIDENT << 32 | cells[e]
+        batches = pc.pf.encode_streamed_batched(pc.dl.pool, pc.dl.off, pc.routes, pc.hidden, pc.stride, pc.partials, pc.ws,
+                                                t, k, pair_start, pair_count, residency=gpu.dev(table))
+        assert batches == -(-pair_count // 32)  # PrefillGroupedRoutedMoE.swift:864-921: microbatches of 32 pairs
+        gpu.synchronize()
+        got = pc.partials.download(np.uint16, t * k * d).reshape(t, k, d)
+        for (tok, rank), at in order.items():
+            if pair_start <= at < pair_start + pair_count:
+                written[tok, rank] = True
+        assert np.array_equal(got[written], want[written]), "a tile's rows differ from the one-pass result"
+        assert np.all(got[~written] == 0xD4D0), "a call wrote rows of pairs outside its range"
+    assert written.all()
+    # a range that starts and ends inside experts' rows, against the grouping's own cells
+    cut = PrefillCase(gpu, L, t)
+    lo, count = 17, 101
+    assert cut.pf.encode_streamed_batched(cut.dl.pool, cut.dl.off, cut.routes, cut.hidden, cut.stride, cut.partials, cut.ws,
+                                          t, k, lo, count, pair_microbatch_rows=8) == 13
+    gpu.synchronize()
+    got = cut.partials.download(np.uint16, t * k * d).reshape(t, k, d)
+    inside = np.zeros((t, k), bool)
+    for (tok, rank), at in order.items():
+        inside[tok, rank] = lo <= at < lo + count
+    assert np.array_equal(got[inside], want[inside]) and np.all(got[~inside] == 0xD4D0)
+    # nothing to do is not an error; a range past the chunk is
+    assert cut.pf.encode_streamed_batched(cut.dl.pool, cut.dl.off, cut.routes, cut.hidden, cut.stride, cut.partials, cut.ws,
+                                          t, k, 5, 0) == 0
+    with pytest.raises(capi.ShrikeError):
+        cut.pf.encode_streamed_batched(cut.dl.pool, cut.dl.off, cut.routes, cut.hidden, cut.stride, cut.partials, cut.ws,
+                                       t, k, t * k - 3, 4)
+
+
 def test_reduce_and_residual_bit_exact(gpu):
     rng = np.random.default_rng(12)
     for t, k, d in ((7, 8, 2048), (33, 4, 2880), (1, 1, 64)):
