@@ -542,6 +542,19 @@ struct PrefillGroupedRoutedMoE {
         check(shrike_hip_prefill_grouped_ffn(moe.handle(), s, pool.bases(), pool.stride(), &offsets, &routes, maxRowTiles, hidden,
                                              hiddenStrideElements, routePartials, workspace, workspaceSize, queryCount, d, f, topK));
     }
+    // encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:846-922): the sorted pairs [pairStart, pairStart + pairCount)
+    // against `residency` (device table, or null for the cells recorded at grouping); returns the microbatch count
+    static uint32_t encodeStreamedBatched(MoE &moe, Stream s, const ExpertPool &pool, const shrike_expert_offsets &offsets,
+                                          const shrike_hip_grouped_routes &routes, uint32_t maxRowTiles, const uint64_t *residency,
+                                          uint32_t pairStart, uint32_t pairCount, const void *hidden, uint32_t hiddenStrideElements,
+                                          void *routePartials, void *workspace, size_t workspaceSize, uint32_t queryCount,
+                                          uint32_t d, uint32_t f, uint32_t topK, uint32_t pairMicrobatchRows = 32) {
+        uint32_t microbatches = 0;
+        check(shrike_hip_prefill_streamed_batched(moe.handle(), s, pool.bases(), pool.stride(), &offsets, &routes, maxRowTiles,
+                                                  residency, pairStart, pairCount, pairMicrobatchRows, hidden, hiddenStrideElements,
+                                                  routePartials, workspace, workspaceSize, queryCount, d, f, topK, &microbatches));
+        return microbatches;
+    }
 };
 
 // PrefillMoE (PrefillMoE.swift:11-40)
