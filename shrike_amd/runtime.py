@@ -579,6 +579,8 @@ class StreamedPrefillLayer:
                                                  tile_expert_count=self.config.tile_experts, expert_sort_keys=keys)
         self.grouped = grouped
         layer = self
+        # one grouping for the chunk; every routed tile is then a pair range of it (encodeStreamedBatched)
+        pf.group_pairs(self.idx, self.w, t, k, ne, self.routes, expert_sort_keys=sort_keys)
 
         class Driver:
             def __init__(self):
@@ -617,12 +619,13 @@ class StreamedPrefillLayer:
                 plan = self.kept.pop(tile, None) or self._plan(tile)
                 if plan is None:
                     raise ShrikeError(capi.last_error())
-                slots, experts = plan.assigned_slots, plan.experts
+                slots, cells, experts = plan.assigned_slots, plan.assigned_cells, plan.experts
                 miss_slots = [slots[i] for i in plan.misses]
                 try:
                     if miss_slots:
-                        layer.pool.fetch_experts(layer.reader, [layer.file_offsets[experts[i]] for i in plan.misses], miss_slots,
-                                                 layer.blob_bytes, layer.staging, layer.upload_stream)
+                        layer.pool.fetch_experts(layer.reader, [layer.file_offsets[experts[i]] for i in plan.misses],
+                                                 [cells[i] for i in plan.misses], layer.blob_bytes, layer.staging,
+                                                 layer.upload_stream)
                 except BaseException:
                     layer.cache.abandon(plan)
                     raise
@@ -645,15 +648,15 @@ class StreamedPrefillLayer:
                 layer.trace.append(("encode", tile))
                 plan, landed = self.begun.pop(tile)
                 table = np.full(ne, (capi.EMPTY << 32) | SENTINEL, np.uint64)
-                for expert, slot in zip(plan.experts, plan.assigned_slots):
-                    table[expert] = (capi.RESIDENT << 32) | slot
+                for expert, cell in zip(plan.experts, plan.assigned_cells):
+                    table[expert] = (capi.RESIDENT << 32) | cell
                 landed.synchronize()  # the experts' bytes and words are in place; the table below is this tile's view
                 tile_table = empty(8 * ne).upload(table)
                 if compute:
                     compute.wait_event(landed)
-                pf.group_pairs(layer.idx, layer.w, t, k, ne, layer.routes, expert_sort_keys=sort_keys, residency=tile_table)
-                pf.encode_grouped_expert_gemms(layer.pool, layer.off, layer.routes, hidden, stride, layer.partials,
-                                               layer.ffn_ws, t, k)
+                tl = grouped.tiles[tile]
+                pf.encode_streamed_batched(layer.pool, layer.off, layer.routes, hidden, stride, layer.partials, layer.ffn_ws,
+                                           t, k, int(tl["pair_start"]), int(tl["pair_count"]), residency=tile_table)
                 self.open.append((tile, list(plan.assigned_slots), bool(plan.misses), tile_table))
 
             def commit_open_batch(self):
