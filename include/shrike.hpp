@@ -18,13 +18,17 @@
 #pragma once
 
 #include <cerrno>
+#include <condition_variable>
 #include <cstdint>
+#include <deque>
 #include <exception>
 #include <functional>
 #include <map>
+#include <mutex>
 #include <optional>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "shrike_hip.h"
@@ -686,6 +690,57 @@ public:
 
 private:
     shrike_load_operation *h_;
+};
+
+// ExpertIOScheduler (Infrastructure/Streaming/ExpertLoadOperation.swift:166-219): a fixed set of submission
+// threads; a queued demand batch runs before any queued speculative one. The destructor runs what is
+// queued, then joins the threads.
+class ExpertIOScheduler {
+public:
+    enum class Priority { demand, speculative };
+    explicit ExpertIOScheduler(int workerCount = 4) {
+        if (workerCount <= 0) throw Error(EINVAL, "workerCount must be positive");
+        for (int i = 0; i < workerCount; ++i) workers_.emplace_back([this] { run(); });
+    }
+    ~ExpertIOScheduler() {
+        {
+            std::lock_guard<std::mutex> held(lock_);
+            closed_ = true;
+        }
+        wake_.notify_all();
+        for (std::thread &worker : workers_) worker.join();
+    }
+    ExpertIOScheduler(const ExpertIOScheduler &) = delete;
+    ExpertIOScheduler &operator=(const ExpertIOScheduler &) = delete;
+    void submit(std::function<void()> work, Priority priority = Priority::demand) {
+        {
+            std::lock_guard<std::mutex> held(lock_);
+            if (closed_) throw Error(EINVAL, "the expert I/O scheduler is closed");
+            (priority == Priority::demand ? demand_ : speculative_).push_back(std::move(work));
+        }
+        wake_.notify_one();
+    }
+
+private:
+    void run() {
+        for (;;) {
+            std::function<void()> work;
+            {
+                std::unique_lock<std::mutex> held(lock_);
+                wake_.wait(held, [this] { return closed_ || !demand_.empty() || !speculative_.empty(); });
+                std::deque<std::function<void()>> &queue = demand_.empty() ? speculative_ : demand_;
+                if (queue.empty()) return;  // closed and drained
+                work = std::move(queue.front());
+                queue.pop_front();
+            }
+            work();
+        }
+    }
+    std::mutex lock_;
+    std::condition_variable wake_;
+    std::deque<std::function<void()>> demand_, speculative_;
+    std::vector<std::thread> workers_;
+    bool closed_ = false;
 };
 
 // ExpertPrefetchRing (Runtime/Inference/ExpertPrefetchRing.swift:42-352)

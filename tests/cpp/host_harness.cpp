@@ -162,6 +162,24 @@ static void landings() {
     }
 }
 
+// ExpertLoadOperation.swift:166-219: queued demand work runs ahead of queued speculative work
+static void ioScheduler() {
+    std::vector<int> order;
+    std::mutex guard;
+    {
+        std::mutex gate;
+        gate.lock();
+        ExpertIOScheduler scheduler(1);
+        scheduler.submit([&] { std::lock_guard<std::mutex> wait(gate); });  // holds the only worker while the queues fill
+        for (int i = 0; i < 3; ++i)
+            scheduler.submit([&, i] { std::lock_guard<std::mutex> g(guard); order.push_back(10 + i); }, ExpertIOScheduler::Priority::speculative);
+        for (int i = 0; i < 3; ++i)
+            scheduler.submit([&, i] { std::lock_guard<std::mutex> g(guard); order.push_back(i); });
+        gate.unlock();
+    }  // the destructor drains the queues
+    EXPECT(order == (std::vector<int>{0, 1, 2, 10, 11, 12}));
+}
+
 static void slotCache() {
     {
         SlotCache c(4, 8);
@@ -369,6 +387,7 @@ int main() {
     wavePlanner();
     slotCache();
     landings();
+    ioScheduler();
     std::printf(failures ? "%d checks failed\n" : "all host checks passed\n", failures);
     return failures ? 1 : 0;
 }
