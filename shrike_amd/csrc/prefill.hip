@@ -217,24 +217,44 @@ __global__ __launch_bounds__(256) void k_group(GroupArgs a) {
     const bool weights_in_lds = a.pairs <= kGroupLdsWeights;
     s_hist[threadIdx.x] = 0u;
     __syncthreads();
-#pragma unroll 16
-    for (uint32_t i = threadIdx.x; i < a.pairs; i += 256u) {
-        const uint32_t v = a.indices[i];
-        if (v < a.num_experts) atomicAdd(&s_hist[v], 1u);
-        if (in_lds) s_ids[i] = uint8_t(min(v, 255u));
-        if (weights_in_lds) s_weights[i] = a.weights[i];
+    // sixteen pairs a thread at a time: all their loads go out before the first is used (with the uses
+    // inside the loading loop every load was waited for on the spot, thirty-two round trips to L2 on end)
+    constexpr uint32_t kPairsAThread = 16;
+    for (uint32_t base = 0; base < a.pairs; base += 256u * kPairsAThread) {
+        uint32_t v[kPairsAThread];
+        uint16_t wv[kPairsAThread];
+#pragma unroll
+        for (uint32_t j = 0; j < kPairsAThread; ++j) {
+            const uint32_t i = min(base + j * 256u + threadIdx.x, a.pairs - 1u);
+            v[j] = a.indices[i];
+            wv[j] = a.weights[i];
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < kPairsAThread; ++j) {
+            const uint32_t i = base + j * 256u + threadIdx.x;
+            if (i >= a.pairs) continue;
+            if (v[j] < a.num_experts) atomicAdd(&s_hist[v[j]], 1u);
+            if (in_lds) s_ids[i] = uint8_t(min(v[j], 255u));
+            if (weights_in_lds) s_weights[i] = wv[j];
+        }
     }
     __syncthreads();
     const uint32_t lane = threadIdx.x & 63u, e = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (e >= a.num_experts) return;
+    // the keys and the residency word are fetched together, ahead of their use
     const uint64_t key = a.sort_keys ? a.sort_keys[e] : 0u;
+    const uint64_t word = a.residency ? a.residency[e] : 0u;
+    uint64_t other_key[SHRIKE_MAX_ROUTER_EXPERTS / 64u];
+#pragma unroll
+    for (uint32_t j = 0; j < SHRIKE_MAX_ROUTER_EXPERTS / 64u; ++j)
+        other_key[j] = a.sort_keys ? a.sort_keys[min(lane + 64u * j, a.num_experts - 1u)] : 0u;
     uint32_t offset = 0, tiles_before = 0, tiles_total = 0;
 #pragma unroll
     for (uint32_t j = 0; j < SHRIKE_MAX_ROUTER_EXPERTS / 64u; ++j) {
         const uint32_t other = lane + 64u * j;
         if (other >= a.num_experts) continue;
         const uint32_t c = s_hist[other];
-        const uint64_t k2 = a.sort_keys ? a.sort_keys[other] : 0u;
+        const uint64_t k2 = other_key[j];
         const bool before = k2 < key || (k2 == key && other < e);
         const uint32_t t = (c + kRowTile - 1u) / kRowTile;
         offset += before ? c : 0u;
@@ -251,10 +271,8 @@ __global__ __launch_bounds__(256) void k_group(GroupArgs a) {
         if (e == 0) *a.tile_count = tiles_total;
     }
     uint32_t cell = e;
-    if (a.residency) {  // moe.metal:136-146
-        const uint64_t word = a.residency[e];
+    if (a.residency)  // moe.metal:136-146
         cell = uint32_t(word >> 32) == SHRIKE_RESIDENCY_RESIDENT ? uint32_t(word) : kSentinel;
-    }
     const uint32_t my_tiles = (count + kRowTile - 1u) / kRowTile;
     for (uint32_t j = lane; j < my_tiles; j += 64u) {
         shrike_row_tile t;
