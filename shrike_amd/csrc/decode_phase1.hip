@@ -15,6 +15,7 @@ constexpr int kPhase1RowPairs = 4;  // (gate, up) row pairs per wave
 // memory (L2-resident) ahead of the row loads, so in-order load return never holds it back.
 template <int BITS, int NCH, int RP, bool ROUTE, int SBITS>
 __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
+    warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
     __shared__ uint32_t s_cell[SHRIKE_MAX_TOP_K];
     if (SBITS != 0 && blockIdx.x >= a.routed_blocks) {

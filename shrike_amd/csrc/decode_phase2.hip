@@ -19,6 +19,7 @@ __device__ __forceinline__ void phase2_finish(uint16_t *y, uint16_t *hidden, uin
 // load and reduces over lane segments. BATCH row groups are in flight per wave.
 template <int BITS, int NCH, int BATCH>
 __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
+    warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
     __shared__ float partial[SHRIKE_MAX_TOP_K][kPhase2Rows];
     if (a.indirect && a.indirect[0] == 0u) return;
@@ -103,7 +104,10 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
 }
 
 template <int BITS, int NCH>
-__global__ __launch_bounds__(256) void k_gemv(GemvArgs a) { gemv_job<BITS, NCH>(a, blockIdx.x); }
+__global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
+    warm_kernel_arguments(a);
+    gemv_job<BITS, NCH>(a, blockIdx.x);
+}
 
 template <int BITS, int NCH>
 static void launch_phase2_batch(const Phase2Args &a, dim3 grid, dim3 block, hipStream_t s) {

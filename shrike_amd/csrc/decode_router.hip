@@ -10,6 +10,7 @@ namespace shrike {
 // finishes last runs select (+ classify when a residency table is bound).
 template <int RK>
 __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
+    warm_kernel_arguments(a);
     __shared__ uint32_t s_last;
     const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t e = blockIdx.x * 4u + wave;
@@ -46,6 +47,9 @@ __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
 // reads it from there; workgroup 0 also stores it for phase 1.
 template <int RK, int BITS, int NCH, bool NORM>
 __global__ __launch_bounds__(256) void k_head(RouterArgs r, GemvArgs g, uint32_t router_blocks, NormArgs n) {
+    warm_kernel_arguments(r);
+    warm_kernel_arguments(g);
+    warm_kernel_arguments(n);
     __shared__ uint4 s_x[NORM ? SHRIKE_MAX_HIDDEN / 8 : 1];
     __shared__ float s_partial[4];
     // the norm runs behind the rows' own loads, which do not depend on it
@@ -83,6 +87,7 @@ struct ClassifyArgs {
 
 // moe.metal:194-231 with the readback of :158-181; lane p classifies position p.
 __global__ __launch_bounds__(64) void k_classify(ClassifyArgs a) {
+    warm_kernel_arguments(a);
     __shared__ uint32_t s_hit[SHRIKE_MAX_TOP_K], s_miss[SHRIKE_MAX_TOP_K];
     const uint32_t lane = threadIdx.x;
     const bool on = lane < a.top_k;

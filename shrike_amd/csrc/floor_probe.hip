@@ -15,6 +15,7 @@ constexpr uint32_t kProbeLoads = 4;
 
 __global__ __launch_bounds__(256) void k_probe_read(PoolArg pool, uint64_t stride, const uint32_t *cells, uint32_t cell_count,
                                                     uint64_t byte_offset, uint32_t waves_per_cell, uint32_t loads_per_cell, uint32_t *sink) {
+    warm_kernel_arguments(pool);
     const uint32_t lane = threadIdx.x & 63u, wave = blockIdx.x * 4u + wave_index();
     const uint32_t which = wave / waves_per_cell, part = wave % waves_per_cell;
     if (which >= cell_count) return;

@@ -16,6 +16,7 @@ constexpr uint32_t kRouterTokenBlock = 4;  // tokens a wave runs one expert row 
 // arithmetic is the decode router's, operand for operand.
 template <int RK>
 __global__ __launch_bounds__(256) void k_prefill_logits(RouterArgs a, uint32_t query_count, uint32_t stride, float *ws) {
+    warm_kernel_arguments(a);
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t e = blockIdx.x * 4u + wave;
     if (e >= a.sel.num_experts) return;
@@ -172,6 +173,7 @@ static void launch_prefill_logits_f16(const uint16_t *weights, const uint16_t *h
 // prefill.metal:441-563: one wave selects for one token.
 __global__ __launch_bounds__(256) void k_prefill_select(SelectArgs sel, const float *ws, uint32_t *out_indices,
                                                         uint16_t *out_weights, uint32_t query_count) {
+    warm_kernel_arguments(sel);
     __shared__ RouteScratch s_route[4];
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t t = blockIdx.x * 4u + wave;
@@ -208,6 +210,7 @@ constexpr uint32_t kGroupLdsWeights = 16384;  // pairs whose fp16 weights are st
 // equals the reference's sort by (sort key, expert, token, rank)
 // (PrefillMoEGrouping.swift:323-332).
 __global__ __launch_bounds__(256) void k_group(GroupArgs a) {
+    warm_kernel_arguments(a);
     __shared__ uint32_t s_hist[SHRIKE_MAX_ROUTER_EXPERTS];
     __shared__ __align__(16) uint8_t s_ids[kGroupLdsPairs];
     __shared__ uint16_t s_weights[kGroupLdsWeights];

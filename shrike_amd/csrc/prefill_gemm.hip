@@ -410,6 +410,7 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
 
 template <int BITS, int MODE, bool DENSE>
 __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
+    warm_kernel_arguments(a);
     __shared__ __align__(16) uint16_t s_a[2][kRowTile][kLdsRow];
     // Which (row tile, column block) this workgroup takes. Workgroups go to the chip's eight XCDs (each
     // with an L2 of its own) round robin in launch order, so workgroup w runs on XCD w % 8 as that XCD's
