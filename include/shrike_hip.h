@@ -175,6 +175,25 @@ int shrike_hip_moe_router(shrike_hip_moe *moe, void *stream, const void *d_weigh
                           uint32_t top_k);
 const float *shrike_hip_moe_router_logits(const shrike_hip_moe *moe);
 
+/* MoE.RouterOperands + MoE.encodeRouterPair, MoE.swift:403-459 (router_gemv_r4_pair and
+ * router_topk_select_k8_pair, moe.metal:383-408, :511-582; called at RealForwardRunner.swift:2861):
+ * this layer's router and a second one (the next layer's, as the prefetch probe) over the same
+ * activation row in one launch. The first router's logits, indices and weights are bit for bit
+ * shrike_hip_moe_router's. The second router's fp32 logits go to d_second_logits
+ * (fp32[num_experts], the reference's routerLogitsPair at its probe slot) or, when that is NULL,
+ * to the handle's own second buffer (shrike_hip_moe_router_pair_logits). */
+typedef struct {
+    const void *weights, *scales, *biases;      /* as for shrike_hip_moe_router */
+    const void *effective_scale, *logit_bias;   /* bf16[d], bf16[num_experts] */
+    uint32_t *out_indices;                      /* u32[top_k] */
+    void *out_weights;                          /* fp16[top_k] */
+} shrike_router_operands;
+int shrike_hip_moe_router_pair(shrike_hip_moe *moe, void *stream, const shrike_router_operands *first,
+                               const shrike_router_operands *second, const void *d_hidden,
+                               const void *d_per_expert_scale, uint32_t num_experts, uint32_t d,
+                               uint32_t top_k, float *d_second_logits);
+const float *shrike_hip_moe_router_pair_logits(const shrike_hip_moe *moe);
+
 /* MoE.encodeResidencyClassification, MoE.swift:552-610
  * (moe_classify_expert_residency_spec, moe.metal:194-231). `full_grids` are the
  * four full grids (12 words); d_spec_args receives the 12 published words: HIP
@@ -388,10 +407,12 @@ int shrike_hip_prefill_streamed_batched(shrike_hip_moe *moe, void *stream, const
                                         uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k,
                                         uint32_t *out_microbatches);
 
-/* The shared expert for query_count tokens (RealForwardRunner.swift:4620-4647: the dense
- * int4/int8 QMMs of MPPPrefillInt4QMM + silu_mul_fp16) on the grouped kernel: h1[t, :] =
- * half(down . half(glu(half(gate . x_t), half(up . x_t)))), optionally * sigmoid(scalar_gate[0])
- * — the roundings of shrike_hip_shared_expert, token by token. h1: fp16[query_count, d]. */
+/* The shared expert for query_count tokens (RealForwardRunner.swift:4387-4456: the dense
+ * int4/int8 QMMs of MPPPrefillInt4QMM + silu_mul_fp16, then encodeSigmoidScalarMulRows) on the
+ * grouped kernel: h1[t, :] = half(down . half(glu(half(gate . x_t), half(up . x_t)))) and, when
+ * d_scalar_gate is given, h1[t, :] = half(h1[t, :] * sigmoid(scalar_gate[t])) — ONE GATE A TOKEN,
+ * fp16[query_count], as shrike_hip_shared_scalar_gate_rows writes them. The roundings are those of
+ * shrike_hip_shared_expert, token by token. h1: fp16[query_count, d]. */
 size_t shrike_hip_prefill_shared_expert_workspace_bytes(uint32_t query_count, uint32_t d,
                                                         uint32_t f_shared);
 int shrike_hip_prefill_shared_expert(shrike_hip_moe *moe, void *stream, const shrike_projection *gate,
@@ -401,6 +422,18 @@ int shrike_hip_prefill_shared_expert(shrike_hip_moe *moe, void *stream, const sh
                                      const void *d_scalar_gate, void *d_workspace,
                                      size_t workspace_bytes, uint32_t query_count, uint32_t d,
                                      uint32_t f_shared);
+
+/* Elementwise.encodeScalarGateRows, sources/Shrike/Kernels/Primitives/Elementwise.swift:140-164
+ * (shared_scalar_gate_rows, moe.metal:1154-1193): the shared expert's scalar gate for a block of tokens,
+ * gate[t] = half(dequant8(gate_row) . x_t). gate_row is ONE 8-bit group-affine row (u8[d], 16-bit
+ * scale and bias per group of 64); x: fp16[rows, x_stride_elements]; d_gate: fp16[rows]. Eight partial
+ * sums added in order as in the reference. d must be a multiple of 64 (Elementwise.swift:148). */
+int shrike_hip_shared_scalar_gate_rows(void *stream, const shrike_projection *gate_row, uint32_t meta_dtype,
+                                       const void *d_x, uint32_t x_stride_elements, void *d_gate,
+                                       uint32_t rows, uint32_t d);
+/* Elementwise.encodeSigmoidScalarMulRows, Elementwise.swift:120-138 (sigmoid_scalar_mul_rows_fp16,
+ * moe.metal:1195-1207): y[t, i] = half(y[t, i] / (1 + exp(-gate[t]))) in place; y: fp16[rows, d]. */
+int shrike_hip_sigmoid_scalar_mul_rows(void *stream, void *d_y, const void *d_gate, uint32_t d, uint32_t rows);
 
 /* PrefillMoE.encodeReduceTokenMajor, sources/Shrike/Kernels/Prefill/MoE/PrefillMoE.swift:11-40
  * (prefill_moe_reduce_token_major, prefill.metal:624-645): h2[t, :] =

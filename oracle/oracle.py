@@ -62,10 +62,16 @@ def lib() -> C.CDLL:
     return _lib
 
 
-def ref_lib() -> C.CDLL | None:
-    """The reference's own int4_affine_gemv.c, compiled by oracle/Makefile; None if not built."""
+def ref_lib_path() -> str | None:
+    """Where oracle/Makefile put the reference's own int4_affine_gemv.c; None if it was not built."""
     path = os.path.join(_HERE, "_ref", "libshrike_ref.so")
-    return C.CDLL(path) if os.path.exists(path) else None
+    return path if os.path.exists(path) else None
+
+
+def ref_lib() -> C.CDLL | None:
+    """Loads that library (only the one CPU test that compares against it does)."""
+    path = ref_lib_path()
+    return C.CDLL(path) if path else None
 
 
 def _p(a: np.ndarray | None):
@@ -183,6 +189,21 @@ def shared_down(down, gate_f16, up_f16, d, f, bits=4, meta=META_BF16, act=ACT_SI
     lib().orc_shared_down(C.byref(dn), C.c_int(meta), C.c_int(bits), C.c_int(act), _p(gate_f16),
                           _p(up_f16), C.c_uint32(d), C.c_uint32(f), _p(scalar_gate_f16), _p(h1))
     return h1
+
+
+def shared_scalar_gate_rows(gate_proj, x_f16, rows, d, x_stride=None, meta=META_BF16):
+    """gate_proj: (w u8[d], s u16[d/64], b u16[d/64]) of the one 8-bit gate row; returns fp16 bits[rows]."""
+    out = np.empty(rows, np.uint16)
+    lib().orc_shared_scalar_gate_rows(_p(gate_proj[0]), _p(gate_proj[1]), _p(gate_proj[2]), C.c_int(meta), _p(x_f16),
+                                      C.c_uint32(d if x_stride is None else x_stride), C.c_uint32(rows),
+                                      C.c_uint32(d), _p(out))
+    return out
+
+
+def sigmoid_scalar_mul_rows(y_f16, gate_f16, d, rows):
+    """In place on y (fp16 bits [rows, d])."""
+    lib().orc_sigmoid_scalar_mul_rows(_p(y_f16), _p(gate_f16), C.c_uint32(d), C.c_uint32(rows))
+    return y_f16
 
 
 def router_logits(weights, scales, biases, kind, hidden_f16, eff_scale_bf16, num_experts, d,

@@ -351,6 +351,54 @@ void orc_shared_expert(const orc_proj *gate, const orc_proj *up, const orc_proj 
     free(g); free(u);
 }
 
+/* shared_scalar_gate_rows, sources/Shrike/Metal/MoE/moe.metal:1154-1193: gate[row] = half(W . x_row)
+ * for ONE 8-bit group-affine weight row against `rows` activation rows. Eight partial sums:
+ * partial p takes the groups p, p+8, ... in order; inside a group lane l of 32 owns elements
+ * 2l and 2l+1 (dot = q0*x0 + q1*x1, sum = x0 + x1; acc = fma(s, dot, acc); acc = fma(b, sum, acc));
+ * the 32 lane sums are folded (the reference leaves the order to simd_sum; here the butterfly
+ * v[l] += v[l^o], o = 1,2,4,8,16) and the eight partials are added in index order. */
+void orc_shared_scalar_gate_rows(const uint8_t *w, const uint16_t *scales, const uint16_t *biases, int meta,
+                                 const uint16_t *x_f16, uint32_t x_stride, uint32_t rows, uint32_t d,
+                                 uint16_t *gate_f16) {
+    const uint32_t groups = d / ORC_GROUP;
+    for (uint32_t r = 0; r < rows; ++r) {
+        const uint16_t *x = x_f16 + (size_t)r * x_stride;
+        float total = 0.0f;
+        for (uint32_t p = 0; p < 8; ++p) {
+            float lane[32], next[32];
+            for (uint32_t l = 0; l < 32; ++l) {
+                float acc = 0.0f;
+                for (uint32_t g = p; g < groups; g += 8) {
+                    const uint32_t i0 = g * ORC_GROUP + 2 * l;
+                    const float x0 = orc_f16_to_f32(x[i0]), x1 = orc_f16_to_f32(x[i0 + 1]);
+                    const float q0 = (float)w[i0] * x0, q1 = (float)w[i0 + 1] * x1;
+                    const float dot = q0 + q1, sum = x0 + x1;
+                    acc = fmaf(meta_to_f32(scales[g], meta), dot, acc);
+                    acc = fmaf(meta_to_f32(biases[g], meta), sum, acc);
+                }
+                lane[l] = acc;
+            }
+            for (uint32_t o = 1; o <= 16; o <<= 1) {
+                for (uint32_t l = 0; l < 32; ++l) next[l] = lane[l] + lane[l ^ o];
+                memcpy(lane, next, sizeof lane);
+            }
+            total += lane[0];
+        }
+        gate_f16[r] = orc_f32_to_f16(total);
+    }
+}
+
+/* sigmoid_scalar_mul_rows_fp16, moe.metal:1195-1207: y[row, i] = half(y[row, i] / (1 + exp(-gate[row]))). */
+void orc_sigmoid_scalar_mul_rows(uint16_t *y_f16, const uint16_t *gate_f16, uint32_t d, uint32_t rows) {
+    for (uint32_t r = 0; r < rows; ++r) {
+        const float g = orc_f16_to_f32(gate_f16[r]);
+        for (uint32_t i = 0; i < d; ++i) {
+            uint16_t *v = y_f16 + (size_t)r * d + i;
+            *v = orc_f32_to_f16(orc_f16_to_f32(*v) / (1.0f + expf(-g)));
+        }
+    }
+}
+
 /* ------------------------------------------------------------------- router */
 
 void orc_router_logits(const void *weights, const uint16_t *scales, const uint16_t *biases,

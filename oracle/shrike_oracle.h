@@ -113,6 +113,14 @@ void orc_shared_expert(const orc_proj *gate, const orc_proj *up, const orc_proj 
                        uint32_t f, const uint16_t *scalar_gate_f16 /* NULL = ungated */,
                        uint16_t *h1_f16);
 
+/* The per-row scalar gate of the shared expert for a block of tokens,
+ * sources/Shrike/Metal/MoE/moe.metal:1154-1207: one 8-bit weight row against `rows`
+ * activation rows (eight partial sums added in order, fp16 out), and y[row,:] *= sigmoid(gate[row]). */
+void orc_shared_scalar_gate_rows(const uint8_t *w, const uint16_t *scales, const uint16_t *biases, int meta,
+                                 const uint16_t *x_f16, uint32_t x_stride, uint32_t rows, uint32_t d,
+                                 uint16_t *gate_f16);
+void orc_sigmoid_scalar_mul_rows(uint16_t *y_f16, const uint16_t *gate_f16, uint32_t d, uint32_t rows);
+
 /* ---- router.
  * Logits: moe.metal:324-364 arithmetic (x = half(hidden) * bf16(effective_scale)).
  * The reference leaves the cross-lane summation order open (simd_sum, :362); this

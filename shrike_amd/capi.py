@@ -39,6 +39,11 @@ class Projection(C.Structure):
     _fields_ = [("weights", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p)]
 
 
+class RouterOperands(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("weights", "scales", "biases", "effective_scale", "logit_bias",
+                                          "out_indices", "out_weights")]
+
+
 class MoEDesc(C.Structure):
     _fields_ = [("d", C.c_uint32), ("f", C.c_uint32), ("num_experts", C.c_uint32),
                 ("top_k", C.c_uint32), ("routed_weight_bits", C.c_uint32),
@@ -269,6 +274,11 @@ SIGNATURES = {
     "shrike_hip_moe_router": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                         _U32, _U32, _U32]),
     "shrike_hip_moe_router_logits": (_VP, [_VP]),
+    "shrike_hip_moe_router_pair": (C.c_int, [_VP, _VP, C.POINTER(RouterOperands), C.POINTER(RouterOperands), _VP, _VP,
+                                             _U32, _U32, _U32, _VP]),
+    "shrike_hip_moe_router_pair_logits": (_VP, [_VP]),
+    "shrike_hip_shared_scalar_gate_rows": (C.c_int, [_VP, C.POINTER(Projection), _U32, _VP, _U32, _VP, _U32, _U32]),
+    "shrike_hip_sigmoid_scalar_mul_rows": (C.c_int, [_VP, _VP, _VP, _U32, _U32]),
     "shrike_hip_moe_classify": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _U32, _U32,
                                           C.POINTER(_U32), _VP, _VP, _U32, _VP, _VP]),
     "shrike_hip_moe_phase1_pool": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, _VP,

@@ -183,6 +183,9 @@ int check_shared(const shrike_projection *gate, const shrike_projection *up, con
     SHRIKE_REQUIRE(d % SHRIKE_GROUP_SIZE == 0 && f_shared % SHRIKE_GROUP_SIZE == 0 && f_shared > 0,
                    "sharedExpert: d=%u and f=%u must be multiples of %u", d, f_shared, SHRIKE_GROUP_SIZE);
     SHRIKE_REQUIRE(nch_for(d, bits) <= 4 && nch_for(f_shared, bits) <= 4, "sharedExpert: rows too long");
+    // the down projection stages half(glu(gate, up)) for the whole row in an LDS array of SHRIKE_MAX_HIDDEN halves
+    SHRIKE_REQUIRE(d <= SHRIKE_MAX_HIDDEN && f_shared <= SHRIKE_MAX_HIDDEN,
+                   "sharedExpert: d=%u or f=%u exceeds the activation ceiling %u", d, f_shared, SHRIKE_MAX_HIDDEN);
     return 0;
 }
 

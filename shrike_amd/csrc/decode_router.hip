@@ -6,17 +6,15 @@
 
 namespace shrike {
 
-// MoE.encodeRouter as one launch: four expert rows per workgroup, and the workgroup that
-// finishes last runs select (+ classify when a residency table is bound).
+// One workgroup's share of MoE.encodeRouter: four expert rows, and the workgroup that finishes last runs
+// select (+ classify when a residency table is bound). `tok` picks the token's rows, logits and counter.
 template <int RK>
-__global__ __launch_bounds__(256) void k_router(RouterArgs a) {
-    warm_kernel_arguments(a);
+__device__ __forceinline__ void router_block(const RouterArgs &a, size_t tok) {
     __shared__ uint32_t s_last;
     const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t e = blockIdx.x * 4u + wave;
     const bool select_too = a.lists.out_indices != nullptr;
-    // grid.y walks tokens (one in decode); the argument block stays as it is, the token's rows are locals
-    const size_t tok = blockIdx.y;
+    // the argument block stays as it is, the token's rows are locals
     const uint16_t *hidden = a.hidden + tok * a.token_stride;
     float *logits = a.logits_out + tok * a.sel.num_experts;
     uint32_t *counter = a.counter + tok;
@@ -39,6 +37,27 @@ __global__ __launch_bounds__(256) void k_router(RouterArgs a) {
     uint32_t cell;
     route_wave<true>(sel, lists, lane, true, cell, s_route);
     if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// MoE.encodeRouter as one launch; grid.y walks tokens (one in decode).
+template <int RK>
+__global__ __launch_bounds__(256) void k_router(RouterArgs a) {
+    warm_kernel_arguments(a);
+    router_block<RK>(a, blockIdx.y);
+}
+
+// MoE.encodeRouterPair (router_gemv_r4_pair + router_topk_select_k8_pair, moe.metal:383-408, :511-582): the
+// grid's second row is the second router over the same activation row, with logits, counter and outputs of
+// its own; the first row is k_router's work exactly.
+template <int RK>
+__global__ __launch_bounds__(256) void k_router_pair(RouterArgs first, RouterArgs second) {
+    if (blockIdx.y == 0) {
+        warm_kernel_arguments(first);
+        router_block<RK>(first, 0);
+    } else {
+        warm_kernel_arguments(second);
+        router_block<RK>(second, 0);
+    }
 }
 
 // The head of the fused layer: the router's logit rows and, beside them in the same grid,
@@ -154,6 +173,15 @@ int launch_router_tokens(const RouterArgs &a, uint32_t router_bits, uint32_t tok
     return 0;
 }
 
+int launch_router_pair(const RouterArgs &first, const RouterArgs &second, uint32_t router_bits, hipStream_t s) {
+    const dim3 grid((first.sel.num_experts + 3) / 4, 2), block(256);
+    if (router_bits == 0) hipLaunchKernelGGL((k_router_pair<0>), grid, block, 0, s, first, second);
+    else if (router_bits == 8) hipLaunchKernelGGL((k_router_pair<8>), grid, block, 0, s, first, second);
+    else hipLaunchKernelGGL((k_router_pair<4>), grid, block, 0, s, first, second);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
 template <int RK, int BITS>
 static void launch_head_nch(const RouterArgs &r, const GemvArgs &g, uint32_t router_blocks, dim3 grid, const NormArgs *norm,
                             hipStream_t s) {
@@ -243,6 +271,42 @@ int shrike_hip_moe_router(shrike_hip_moe *moe, void *stream, const void *d_weigh
 }
 
 const float *shrike_hip_moe_router_logits(const shrike_hip_moe *moe) { return moe ? moe->d_logits : nullptr; }
+
+int shrike_hip_moe_router_pair(shrike_hip_moe *moe, void *stream, const shrike_router_operands *first,
+                               const shrike_router_operands *second, const void *d_hidden, const void *d_per_expert_scale,
+                               uint32_t num_experts, uint32_t d, uint32_t top_k, float *d_second_logits) {
+    SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
+    if (int rc = check_router(moe, num_experts, d, top_k)) return rc;
+    SHRIKE_REQUIRE(first && second && d_hidden && d_per_expert_scale, "encodeRouterPair: operands, hidden and perExpertScale must be bound");
+    const shrike_router_operands *ops[2] = {first, second};
+    RouterArgs a[2] = {};
+    for (int i = 0; i < 2; ++i) {
+        const shrike_router_operands *o = ops[i];
+        SHRIKE_REQUIRE(o->weights && o->effective_scale && o->logit_bias, "encodeRouterPair: weights, effectiveScale and logitBias must be bound");
+        SHRIKE_REQUIRE(moe->desc.router_weight_bits == 0 || (o->scales && o->biases), "encodeRouterPair: affine router needs scales and biases");
+        SHRIKE_REQUIRE(o->out_indices && o->out_weights, "encodeRouterPair: outputs must be bound");
+        a[i].weights = o->weights;
+        a[i].scales = static_cast<const uint16_t *>(o->scales);
+        a[i].biases = static_cast<const uint16_t *>(o->biases);
+        a[i].hidden = static_cast<const uint16_t *>(d_hidden);
+        a[i].effective_scale = static_cast<const uint16_t *>(o->effective_scale);
+        a[i].d = d; a[i].meta = moe->desc.meta_dtype;
+        float *logits = i == 0 ? moe->d_logits : (d_second_logits ? d_second_logits : moe->d_logits + SHRIKE_MAX_ROUTER_EXPERTS);
+        a[i].counter = moe->d_counter + i; a[i].logits_out = logits;
+        a[i].sel.logits = logits;
+        a[i].sel.per_expert_scale = static_cast<const uint16_t *>(d_per_expert_scale);
+        a[i].sel.logit_bias = static_cast<const uint16_t *>(o->logit_bias);
+        a[i].sel.num_experts = num_experts; a[i].sel.top_k = top_k;
+        a[i].sel.sigmoid = moe->desc.sigmoid_router_scores; a[i].sel.scaling = moe->desc.routed_scaling_factor;
+        a[i].lists.out_indices = o->out_indices;
+        a[i].lists.out_weights = static_cast<uint16_t *>(o->out_weights);
+    }
+    return launch_router_pair(a[0], a[1], moe->desc.router_weight_bits, as_stream(stream));
+}
+
+const float *shrike_hip_moe_router_pair_logits(const shrike_hip_moe *moe) {
+    return moe ? moe->d_logits + SHRIKE_MAX_ROUTER_EXPERTS : nullptr;
+}
 
 int shrike_hip_moe_classify(shrike_hip_moe *moe, void *stream, const uint32_t *d_topk_indices,
                             const uint64_t *d_residency, uint32_t *d_hit_count, uint32_t *d_hit_positions,

@@ -241,3 +241,10 @@ int shrike_expert_reader_threads(const shrike_expert_reader *r) { return r ? int
 int shrike_expert_reader_batch_depth(const shrike_expert_reader *r) { return r ? r->depth : 0; }
 
 }  // extern "C"
+
+// library-internal: the byte count every read of this reader writes to its destination
+size_t shrike_expert_reader_stride_internal(const shrike_expert_reader *r) { return r ? r->stride : 0; }
+
+extern "C" {
+
+}  // extern "C"

@@ -42,7 +42,7 @@ constexpr unsigned kRouterTokenCounters = 128;  // first of the per-token arriva
 struct shrike_hip_moe {
     shrike_moe_desc desc;
     int device;
-    float *d_logits;        // fp32[SHRIKE_MAX_ROUTER_EXPERTS]
-    uint32_t *d_counter;    // u32[kCounterWords], zero between launches: [0] the router's arrivals, from
+    float *d_logits;        // fp32[2][SHRIKE_MAX_ROUTER_EXPERTS]: this layer's logits, then the paired router's
+    uint32_t *d_counter;    // u32[kCounterWords], zero between launches: [0] the router's arrivals ([1] the paired router's), from
                             // [kRouterTokenCounters] one word a token of the several-token router
 };

@@ -286,7 +286,8 @@ __global__ __launch_bounds__(256) void k_group(GroupArgs a) {
         a.tiles[tiles_before + j] = t;
     }
     if (count == 0) return;
-    const uint32_t token_magic = 0xffffffffu / a.top_k + 1u;  // i / top_k == umulhi(i, magic) for i * top_k < 2^32
+    // i / top_k == umulhi(i, magic) for i * top_k < 2^32; top_k == 1 would need magic 2^32, so it divides plainly below
+    const uint32_t token_magic = 0xffffffffu / a.top_k + 1u;
     uint32_t running = 0;
     if (in_lds) {
         // 1,024 pairs a step: a lane takes 16 neighbouring ids with one LDS read, flags the bytes equal
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(256) void k_group(GroupArgs a) {
                 const uint32_t i = i0 + uint32_t(__ffs(int(match)) - 1);
                 match &= match - 1u;
                 shrike_token_expert_pair p;
-                p.token = __umulhi(i, token_magic);
+                p.token = a.top_k == 1u ? i : __umulhi(i, token_magic);
                 p.expert = e;
                 p.rank = i - p.token * a.top_k;
                 p.weight_bits_and_reserved = weights_in_lds ? s_weights[i] : a.weights[i];
@@ -332,7 +333,7 @@ __global__ __launch_bounds__(256) void k_group(GroupArgs a) {
         const uint64_t mask = __ballot(mine);
         if (mine) {
             shrike_token_expert_pair p;
-            p.token = __umulhi(i, token_magic);
+            p.token = a.top_k == 1u ? i : __umulhi(i, token_magic);
             p.expert = e;
             p.rank = i - p.token * a.top_k;
             p.weight_bits_and_reserved = a.weights[i];
@@ -423,6 +424,58 @@ __global__ __launch_bounds__(256) void k_residual_add(uint16_t *hidden, const ui
     } else {
         for (uint64_t j = i; j < count; ++j) hidden[j] = f32_to_f16(__fadd_rn(f16_to_f32(hidden[j]), f16_to_f32(delta[j])));
     }
+}
+
+// shared_scalar_gate_rows, moe.metal:1154-1193: one 8-bit group-affine weight row against a block of token rows,
+// a workgroup a row. Eight partial sums as in the reference (its eight simdgroups of 32 lanes are the half-waves
+// here): partial p takes the groups p, p + 8, ..., lane l of its 32 the elements 2l and 2l + 1 of a group; the 32
+// lane sums fold by the butterfly 1, 2, 4, 8, 16 and the eight partials are added in index order.
+__global__ __launch_bounds__(256) void k_scalar_gate_rows(const uint8_t *w, const uint16_t *scales, const uint16_t *biases,
+                                                          uint32_t meta, const uint16_t *x, uint32_t x_stride, uint16_t *gate,
+                                                          uint32_t d) {
+    __shared__ float s_partial[8];
+    const uint32_t p = threadIdx.x >> 5, l = threadIdx.x & 31u;
+    const uint16_t *row = x + size_t(blockIdx.x) * x_stride;
+    float acc = 0.0f;
+    for (uint32_t g = p; g < d / kGroup; g += 8u) {
+        const uint32_t i0 = g * kGroup + 2u * l;
+        const uint32_t xw = *reinterpret_cast<const uint32_t *>(row + i0);
+        const uint16_t qw = *reinterpret_cast<const uint16_t *>(w + i0);
+        const float x0 = f16_to_f32(uint16_t(xw)), x1 = f16_to_f32(uint16_t(xw >> 16));
+        const float dot = __fadd_rn(__fmul_rn(float(qw & 0xffu), x0), __fmul_rn(float(qw >> 8), x1));
+        acc = fmaf(meta_f32(scales[g], meta), dot, acc);
+        acc = fmaf(meta_f32(biases[g], meta), __fadd_rn(x0, x1), acc);
+    }
+#pragma unroll
+    for (int o = 1; o <= 16; o <<= 1) acc = __fadd_rn(acc, __shfl_xor(acc, o));
+    if (l == 0) s_partial[p] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) total = __fadd_rn(total, s_partial[i]);
+        gate[blockIdx.x] = f32_to_f16(total);
+    }
+}
+
+// sigmoid_scalar_mul_rows_fp16, moe.metal:1195-1207: y[row, i] = half(y[row, i] / (1 + exp(-gate[row]))), eight
+// elements a thread.
+__global__ __launch_bounds__(256) void k_sigmoid_scalar_mul_rows(uint16_t *y, const uint16_t *gate, uint32_t d, uint32_t rows) {
+    const uint32_t per_row = d / 8u;
+    const uint64_t slot = uint64_t(blockIdx.x) * 256u + threadIdx.x;
+    if (slot >= uint64_t(rows) * per_row) return;
+    const uint32_t r = uint32_t(slot / per_row);
+    const float div = 1.0f + expf(-f16_to_f32(gate[r]));
+    uint4 v = *reinterpret_cast<const uint4 *>(y + slot * 8u);
+    uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint16_t lo = f32_to_f16(f16_to_f32(uint16_t(vw[j])) / div);
+        const uint16_t hi = f32_to_f16(f16_to_f32(uint16_t(vw[j] >> 16)) / div);
+        vw[j] = uint32_t(lo) | uint32_t(hi) << 16;
+    }
+    v.x = vw[0]; v.y = vw[1]; v.z = vw[2]; v.w = vw[3];
+    *reinterpret_cast<uint4 *>(y + slot * 8u) = v;
 }
 
 int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uint32_t n, uint32_t *out,
@@ -540,6 +593,33 @@ int shrike_hip_group_pairs(void *stream, const uint32_t *d_indices, const void *
     hipStream_t s = as_stream(stream);
     const dim3 grid((num_experts + 3u) / 4u);
     hipLaunchKernelGGL(k_group, grid, dim3(256), 0, s, a);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int shrike_hip_shared_scalar_gate_rows(void *stream, const shrike_projection *gate_row, uint32_t meta_dtype, const void *d_x,
+                                       uint32_t x_stride_elements, void *d_gate, uint32_t rows, uint32_t d) {
+    SHRIKE_REQUIRE(gate_row && gate_row->weights && gate_row->scales && gate_row->biases, "scalar gate rows: the gate row must be bound");
+    SHRIKE_REQUIRE(d_x && d_gate, "scalar gate rows: NULL buffer");
+    // Elementwise.swift:148
+    SHRIKE_REQUIRE(d > 0 && d % SHRIKE_GROUP_SIZE == 0, "shared_scalar_gate_rows drops the tail unless d is a multiple of 64");
+    SHRIKE_REQUIRE(x_stride_elements >= d && x_stride_elements % 2u == 0, "scalar gate rows: x stride is too small or odd");
+    SHRIKE_REQUIRE(meta_dtype <= SHRIKE_META_F16, "scalar gate rows: metaDtype=%u is not a known value", meta_dtype);
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(k_scalar_gate_rows, dim3(rows), dim3(256), 0, as_stream(stream), static_cast<const uint8_t *>(gate_row->weights),
+                       static_cast<const uint16_t *>(gate_row->scales), static_cast<const uint16_t *>(gate_row->biases), meta_dtype,
+                       static_cast<const uint16_t *>(d_x), x_stride_elements, static_cast<uint16_t *>(d_gate), d);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+int shrike_hip_sigmoid_scalar_mul_rows(void *stream, void *d_y, const void *d_gate, uint32_t d, uint32_t rows) {
+    SHRIKE_REQUIRE(d_y && d_gate, "sigmoid scalar mul rows: NULL buffer");
+    SHRIKE_REQUIRE(d % 8u == 0 && reinterpret_cast<uintptr_t>(d_y) % 16u == 0, "sigmoid scalar mul rows: d must be a multiple of 8 and y 16-byte aligned");
+    const uint64_t slots = uint64_t(rows) * (d / 8u);
+    if (slots == 0) return 0;
+    hipLaunchKernelGGL(k_sigmoid_scalar_mul_rows, dim3(uint32_t((slots + 255u) / 256u)), dim3(256), 0, as_stream(stream),
+                       static_cast<uint16_t *>(d_y), static_cast<const uint16_t *>(d_gate), d, rows);
     SHRIKE_HIP(hipGetLastError());
     return 0;
 }

@@ -53,7 +53,7 @@ struct FfnArgs {
     const uint16_t *dense_s[3], *dense_b[3];
     uint32_t dense_rows;
     uint32_t round_gate_up;        // gate and up pass through fp16 before the GLU (dequant_int4.metal:206-287)
-    const uint16_t *scalar_gate;   // fp16[1] or null: output * sigmoid(gate) (dequant_int4.metal:322-329)
+    const uint16_t *scalar_gate;   // fp16[rows] or null: row m's output * sigmoid(gate[m]) (moe.metal:1195-1207)
 };
 
 union Frag {
@@ -376,8 +376,6 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
         const uint32_t row_lo = DENSE ? 0u : max(a.pair_lo, tile.pair_start) - tile.pair_start;
         const uint32_t row_hi = DENSE ? tile.rows : min(a.pair_hi, tile.pair_start + tile.rows) - tile.pair_start;
         float dab[2] = {0.0f, 0.0f};
-        float gate_mul = 0.0f;
-        if (DENSE && a.scalar_gate) gate_mul = 1.0f + expf(-f16_to_f32(a.scalar_gate[0]));
         if (!DENSE && a.ebias) {
             dab[0] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n]);
             dab[1] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n + 32u]);
@@ -396,7 +394,8 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
                         dst = a.partials + (size_t(p.token) * a.top_k + p.rank) * a.d + n;
                     }
                     uint16_t y0 = f32_to_f16(total[0][mt][i] + dab[0]), y1 = f32_to_f16(total[1][mt][i] + dab[1]);
-                    if (DENSE && a.scalar_gate) {
+                    if (DENSE && a.scalar_gate) {  // one gate a token row (moe.metal:1195-1207)
+                        const float gate_mul = 1.0f + expf(-f16_to_f32(a.scalar_gate[tile.pair_start + m]));
                         y0 = f32_to_f16(f16_to_f32(y0) / gate_mul);
                         y1 = f32_to_f16(f16_to_f32(y1) / gate_mul);
                     }

@@ -56,6 +56,8 @@ struct shrike_hip_pool {
     bool owns_cells = true;        // false for a layer's table over another pool's cells
 };
 
+size_t shrike_expert_reader_stride_internal(const shrike_expert_reader *r);  // expert_io.cpp
+
 extern "C" {
 
 const char *shrike_hip_last_error(void) { return g_last_error.c_str(); }
@@ -274,6 +276,10 @@ int shrike_hip_pool_fetch_experts(shrike_hip_pool *pool, void *stream, shrike_ex
                    (unsigned long long)blob_bytes, (unsigned long long)pool->stride);
     SHRIKE_REQUIRE(staging_bytes / blob_bytes >= 2, "the staging buffer must hold two blobs of %llu bytes",
                    (unsigned long long)blob_bytes);
+    // the reader's workers write its own stride to every destination, and destinations sit blob_bytes apart
+    SHRIKE_REQUIRE(shrike_expert_reader_stride_internal(reader) == blob_bytes,
+                   "blob_bytes=%llu is not the stride the reader was created with (%llu)", (unsigned long long)blob_bytes,
+                   (unsigned long long)shrike_expert_reader_stride_internal(reader));
     for (uint32_t i = 0; i < count; ++i)
         SHRIKE_REQUIRE(cells[i] < pool->cells, "expert cell %u out of range (%u cells)", cells[i], pool->cells);
     const uint32_t per_half = uint32_t(std::min<uint64_t>(staging_bytes / blob_bytes / 2, count));
@@ -406,10 +412,10 @@ shrike_hip_moe *shrike_hip_moe_create(const shrike_moe_desc *desc, int *out_errn
     moe->desc = *desc;
     moe->d_logits = nullptr; moe->d_counter = nullptr;
     if (hipGetDevice(&moe->device) != hipSuccess
-        || hipMalloc(reinterpret_cast<void **>(&moe->d_logits), sizeof(float) * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess
+        || hipMalloc(reinterpret_cast<void **>(&moe->d_logits), sizeof(float) * 2u * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess
         || hipMalloc(reinterpret_cast<void **>(&moe->d_counter), sizeof(uint32_t) * kCounterWords) != hipSuccess
         || hipMemset(moe->d_counter, 0, sizeof(uint32_t) * kCounterWords) != hipSuccess
-        || hipMemset(moe->d_logits, 0, sizeof(float) * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess) {
+        || hipMemset(moe->d_logits, 0, sizeof(float) * 2u * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess) {
         set_error("device allocation for the MoE handle failed: %s", hipGetErrorString(hipGetLastError()));
         shrike_hip_moe_destroy(moe);
         return fail(ENOMEM);

@@ -288,6 +288,25 @@ class MoE:
             ptr(effective_scale), ptr(per_expert_scale), ptr(logit_bias), ptr(out_indices),
             ptr(out_weights), num_experts, d, top_k), "shrike_hip_moe_router")
 
+    def encode_router_pair(self, first: dict, second: dict, hidden, per_expert_scale, num_experts, d, top_k,
+                           second_logits=None):
+        """MoE.encodeRouterPair: first/second are dicts with weights, scales, biases, effective_scale, logit_bias,
+        out_indices, out_weights (device buffers; scales/biases None for fp16 rows)."""
+        def ops(o):
+            return capi.RouterOperands(*(ptr(o.get(n)) for n in ("weights", "scales", "biases", "effective_scale",
+                                                                   "logit_bias", "out_indices", "out_weights")))
+        a, b = ops(first), ops(second)
+        check(capi.load().shrike_hip_moe_router_pair(
+            self.handle, self._s(), C.byref(a), C.byref(b), ptr(hidden), ptr(per_expert_scale), num_experts, d, top_k,
+            ptr(second_logits)), "shrike_hip_moe_router_pair")
+
+    def pair_logits(self, num_experts: int) -> np.ndarray:
+        synchronize()
+        out = np.empty(num_experts, np.float32)
+        p = capi.load().shrike_hip_moe_router_pair_logits(self.handle)
+        check(capi.load().shrike_hip_memcpy_d2h(out.ctypes.data, p, out.nbytes), "memcpy_d2h")
+        return out
+
     def encode_residency_classification(self, topk, residency, hit_count, hit_positions, miss_count,
                                         miss_positions, miss_experts, resolved_slots, top_k, num_experts,
                                         full_grids=None, spec_args=None, host_readback=None, tag=0,
@@ -433,6 +452,17 @@ class Prefill:
             "shrike_hip_prefill_shared_expert")
         return workspace
 
+    def encode_scalar_gate_rows(self, gate_row, x, x_stride_elements, gate, rows, d):
+        """Elementwise.encodeScalarGateRows: gate_row is the (weights, scales, biases) of the one 8-bit row."""
+        g = Projection(ptr(gate_row[0]), ptr(gate_row[1]), ptr(gate_row[2]))
+        check(capi.load().shrike_hip_shared_scalar_gate_rows(self._s(), C.byref(g), self.moe.desc.meta_dtype, ptr(x),
+                                                             x_stride_elements, ptr(gate), rows, d),
+              "shrike_hip_shared_scalar_gate_rows")
+
+    def encode_sigmoid_scalar_mul_rows(self, y, gate, d, rows):
+        check(capi.load().shrike_hip_sigmoid_scalar_mul_rows(self._s(), ptr(y), ptr(gate), d, rows),
+              "shrike_hip_sigmoid_scalar_mul_rows")
+
     def encode_reduce_token_major(self, route_partials, route_weights, h2, query_count, top_k, d):
         check(capi.load().shrike_hip_prefill_reduce(self._s(), ptr(route_partials), ptr(route_weights), ptr(h2),
                                                     query_count, top_k, d), "shrike_hip_prefill_reduce")
@@ -476,6 +506,7 @@ class BatchedDecodeLayer:
         self.h2 = empty(2 * max_tokens * d)
         self.pass_table = empty(8 * ne)
         self.passes = 0
+        self.plan_log = []  # every batch of experts handed to the cache, in order
 
     def run(self, router, hidden, t: int, stride: int):
         """router: dict(weights, scales, biases, eff_scale, expert_scale, bias) of device buffers.
@@ -504,6 +535,7 @@ class BatchedDecodeLayer:
             plan = self.cache.plan(batch)
             if plan is None:
                 raise ShrikeError(capi.last_error())
+            self.plan_log.append(list(batch))
             if self.passes:
                 self.upload_stream.wait_event(served)  # the cells about to be overwritten were still being read
             self.pool.execute_plan(self.cache, plan, self.store, self.store_stride, self.expert_bytes, self.upload_stream)

@@ -93,7 +93,7 @@ def test_gemv_against_brute_force(rows, n, bits, meta):
         assert np.array_equal(O.int4_affine_gemv(w, s, b, x, rows, n, meta), got)
 
 
-@pytest.mark.skipif(O.ref_lib() is None, reason="oracle/_ref was not built (no reference checkout at build time)")
+@pytest.mark.skipif(O.ref_lib_path() is None, reason="oracle/_ref was not built (no reference checkout at build time)")
 @pytest.mark.parametrize("rows,n", [(2048, 512), (512, 2048), (128, 64), (2880, 2880), (1024, 2304)])
 def test_int4_gemv_bit_equal_to_the_reference_c(rows, n):
     rng = S.SeedTree(0x5EED0001).key(f"ref.{rows}.{n}")
@@ -352,3 +352,226 @@ def test_residual_add_rmsnorm_against_the_definition():
         two_step = O.residual_add_f16(hidden.copy(), delta)
         assert np.array_equal(O.residual_add_rmsnorm_bf16w(two_step, None, weight, eps), out)
         assert np.array_equal(two_step, h)
+
+
+# ------------------------------------------------------------ fp64 chains from the format's definition
+#
+# Everything below restates a function of the oracle in numpy fp64 from the DEFINITION of the format
+# (w = q * scale + bias per element, low nibble = even element) and of the layer (which value is rounded to
+# fp16 where, per the Metal sources cited), never from the oracle's own loops. A stage that rounds to fp16
+# can land one fp16 step away from the fp64 chain (an fp32 sum next to a rounding boundary), so chains are
+# held to a few fp16 steps of the vector's scale; each test also shows that a plausible mistake (operands
+# swapped, a term dropped, the gate left out) breaks the same bound.
+
+def dequant(w, s, b, rows, n, bits, meta):
+    """[rows, n] fp64 weights from the format's definition."""
+    w = np.ascontiguousarray(w).reshape(rows, n * bits // 8)
+    q = np.stack([w & 0xF, w >> 4], axis=2).reshape(rows, n) if bits == 4 else w
+    sf = S.meta_to_f32(np.ascontiguousarray(s).reshape(-1), meta).astype(np.float64).reshape(rows, n // 64)
+    bf = S.meta_to_f32(np.ascontiguousarray(b).reshape(-1), meta).astype(np.float64).reshape(rows, n // 64)
+    return q.astype(np.float64) * np.repeat(sf, 64, axis=1) + np.repeat(bf, 64, axis=1)
+
+
+def h(v):
+    """One fp16 rounding, back in fp64."""
+    with np.errstate(over="ignore"):
+        return np.asarray(v, np.float64).astype(np.float16).astype(np.float64)
+
+
+def glu64(g, u, act):
+    if act == O.ACT_SILU:
+        return g / (1.0 + np.exp(-g)) * u
+    if act == O.ACT_GELU_TANH:  # moe.metal:98-105
+        return 0.5 * g * (1.0 + np.tanh(np.clip(0.7978845608028654 * (g + 0.044715 * g ** 3), -20, 20))) * u
+    gc, uc = np.minimum(g, 7.0), np.clip(u, -7.0, 7.0)  # moe.metal:280-288
+    return gc / (1.0 + np.exp(-1.702 * gc)) * (uc + 1.0)
+
+
+def close_in_f16_steps(got_bits, want64, steps, what):
+    """|got - want| <= steps * (one fp16 step at the vector's largest magnitude)."""
+    got = f16(got_bits).astype(np.float64)
+    scale = max(float(np.max(np.abs(want64))), 1e-3)
+    step = 2.0 ** (np.floor(np.log2(scale)) - 10)
+    worst = float(np.max(np.abs(got - want64)))
+    return worst <= steps * step, f"{what}: worst |diff| {worst:.3e} vs {steps} fp16 steps of {step:.3e}"
+
+
+def shared_chain(sh, x64, d, fs, bits, meta, act, gate_bits=None, swap=False, drop_gate=False):
+    """dequant_int4.metal:177-179 (the GEMVs write half), :283-287 (act = half(glu)), :322-329 (gated tail)."""
+    wg, wu, wd = (dequant(*sh[n], r, c, bits, meta) for n, r, c in (("gate", fs, d), ("up", fs, d), ("down", d, fs)))
+    g, u = h(wg @ x64), h(wu @ x64)
+    if swap:
+        g, u = u, g
+    y = h(wd @ h(glu64(g, u, act)))
+    if gate_bits is not None and not drop_gate:
+        y = h(y / (1.0 + np.exp(-float(f16(gate_bits)[0]))))
+    return g, u, y
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("d,fs", [(256, 128), (2048, 512)])
+@pytest.mark.parametrize("gated", [False, True])
+def test_shared_expert_against_fp64_chain(bits, d, fs, gated):
+    tree = S.SeedTree(0x5EED0A10 + bits + d)
+    meta = S.META_BF16
+    sh = {n: S.affine_matrix(tree.key(f"shared.{n}"), r, c, bits, meta)
+          for n, r, c in (("gate", fs, d), ("up", fs, d), ("down", d, fs))}
+    x = S.activations_f16(tree, "x", d)
+    gate_bits = S.f32_to_f16_bits(np.array([-0.4], np.float32)) if gated else None
+    g64, u64, y64 = shared_chain(sh, f16(x).astype(np.float64), d, fs, bits, meta, O.ACT_SILU, gate_bits)
+    g, u = O.shared_gate_up(sh["gate"], sh["up"], x, d, fs, bits=bits, meta=meta)
+    ok, msg = close_in_f16_steps(g, g64, 1, "gate rows")
+    assert ok, msg
+    ok, msg = close_in_f16_steps(u, u64, 1, "up rows")
+    assert ok, msg
+    assert not np.array_equal(g, u)
+    # the down stage alone from the oracle's own gate/up: one rounding of act, one of y (and one more when gated)
+    y_from = O.shared_down(sh["down"], g, u, d, fs, bits=bits, meta=meta, scalar_gate_f16=gate_bits)
+    wd = dequant(*sh["down"], d, fs, bits, meta)
+    y_stage = h(wd @ h(glu64(f16(g).astype(np.float64), f16(u).astype(np.float64), O.ACT_SILU)))
+    if gated:
+        y_stage = h(y_stage / (1.0 + np.exp(-float(f16(gate_bits)[0]))))
+    ok, msg = close_in_f16_steps(y_from, y_stage, 2, "down from given gate/up")
+    assert ok, msg
+    # the whole chain; the composition equals its two halves
+    y = O.shared_expert(sh["gate"], sh["up"], sh["down"], x, d, fs, bits=bits, meta=meta, scalar_gate_f16=gate_bits)
+    assert np.array_equal(y, y_from)
+    ok, msg = close_in_f16_steps(y, y64, 3, "shared expert")
+    assert ok, msg
+    # what the bound catches
+    _, _, swapped = shared_chain(sh, f16(x).astype(np.float64), d, fs, bits, meta, O.ACT_SILU, gate_bits, swap=True)
+    assert not close_in_f16_steps(y, swapped, 3, "")[0], "gate and up swapped must not pass"
+    if gated:
+        _, _, ungated = shared_chain(sh, f16(x).astype(np.float64), d, fs, bits, meta, O.ACT_SILU, gate_bits, drop_gate=True)
+        assert not close_in_f16_steps(y, ungated, 3, "")[0], "a dropped scalar gate must not pass"
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("act", [O.ACT_SILU, O.ACT_GELU_TANH, O.ACT_CLAMPED_SWIGLU])
+@pytest.mark.parametrize("additive", [False, True])
+def test_routed_phases_against_fp64_chain(bits, act, additive):
+    """moe.metal:261-288 (additive biases ahead of the GLU, clamped SwiGLU), :829 (acts are half), :933-939
+    (partial = half weight * (down + bias); y = half(residual + sum in rank order)), :889-893 (hidden += y)."""
+    d, f, k = 192, 128, 3
+    meta = S.META_BF16
+    tree = S.SeedTree(0x5EED0A20 + bits + 16 * act + int(additive))
+    blobs = [S.expert_blob(tree, f"e{e}", d, f, bits, meta, additive) for e in range(k)]
+    off, _ = O.expert_offsets(d, f, bits, additive)
+    soff, _ = S.expert_offsets(d, f, bits, additive)
+    x = S.activations_f16(tree, "x", d)
+    x64 = f16(x).astype(np.float64)
+    acts = O.moe_phase1(blobs, off, x, d, f, bits=bits, meta=meta, act=act, additive_biases=additive)
+    w_bits = S.f32_to_f16_bits(np.array([0.5, 0.3, 0.2], np.float32))
+    residual = S.activations_f16(tree, "residual", d)
+    hidden = S.activations_f16(tree, "hidden", d)
+    hidden_out = hidden.copy()
+    y = O.moe_phase2(blobs, off, acts, w_bits, residual, d, f, bits=bits, meta=meta, additive_biases=additive,
+                     hidden_f16=hidden_out)
+
+    def ab(blob, name, n):
+        return S.bf16_bits_to_f32(blob[soff[name]:soff[name] + 2 * n].view(np.uint16)).astype(np.float64)
+
+    def chain(bias_after_glu=False, drop_down_bias=False):
+        acc = f16(residual).astype(np.float64)
+        all_acts = []
+        for e in range(k):
+            v = S.blob_views(blobs[e], d, f, bits, additive)
+            g, u = dequant(*v["gate"], f, d, bits, meta) @ x64, dequant(*v["up"], f, d, bits, meta) @ x64
+            if additive and not bias_after_glu:
+                g, u = g + ab(blobs[e], "gate_ab", f), u + ab(blobs[e], "up_ab", f)
+            a = glu64(g, u, act)
+            if additive and bias_after_glu:
+                a = a + ab(blobs[e], "gate_ab", f)
+            a = h(a)
+            all_acts.append(a)
+            down = dequant(*v["down"], d, f, bits, meta) @ a
+            if additive and not drop_down_bias:
+                down = down + ab(blobs[e], "down_ab", d)
+            acc = acc + float(f16(w_bits)[e]) * down
+        return np.concatenate(all_acts), h(acc)
+
+    a64, y64 = chain()
+    ok, msg = close_in_f16_steps(acts, a64, 1, "acts")
+    assert ok, msg
+    ok, msg = close_in_f16_steps(y, y64, 2, "y")
+    assert ok, msg
+    assert np.array_equal(hidden_out, (f16(hidden) + f16(y)).astype(np.float16).view(np.uint16))
+    if additive:
+        wrong_acts, _ = chain(bias_after_glu=True)
+        assert not close_in_f16_steps(acts, wrong_acts, 1, "")[0], "the bias added after the GLU must not pass"
+        _, wrong_y = chain(drop_down_bias=True)
+        assert not close_in_f16_steps(y, wrong_y, 2, "")[0], "a dropped down bias must not pass"
+    # a sentinel position keeps its acts and adds nothing (moe.metal:986, :1037-1038)
+    keep = np.full(k * f, 0x3555, np.uint16)
+    part = O.moe_phase1([blobs[0], None, blobs[2]], off, x, d, f, bits=bits, meta=meta, act=act,
+                        additive_biases=additive, acts=keep.copy())
+    assert np.array_equal(part[f:2 * f], keep[f:2 * f]) and np.array_equal(part[:f], acts[:f])
+
+
+@pytest.mark.parametrize("kind", [O.ROUTER_F16, O.ROUTER_AFFINE8, O.ROUTER_AFFINE4])
+def test_router_logits_with_effective_scale_against_fp64(kind):
+    """moe.metal:324-364: logit = sum (q*s + b) * (half(hidden) * bf16(effective_scale))."""
+    e, d = 48, 704
+    tree = S.SeedTree(0x5EED0A30 + kind)
+    dense = tree.key("w").normal(e * d, std=0.02).reshape(e, d)
+    x = S.activations_f16(tree, "x", d)
+    eff = S.f32_to_bf16_bits(tree.key("eff").uniform(0.25, 1.75, d))
+    xs = f16(x).astype(np.float64) * S.bf16_bits_to_f32(eff).astype(np.float64)
+    if kind == O.ROUTER_F16:
+        w = S.f32_to_f16_bits(dense.reshape(-1)).reshape(e, d)
+        got = O.router_logits(w, None, None, kind, x, eff, e, d)
+        ref = f16(w).astype(np.float64).reshape(e, d) @ xs
+    else:
+        wq, ws, wb = S.quantize_affine(dense.astype(np.float32), kind)
+        got = O.router_logits(wq, ws, wb, kind, x, eff, e, d)
+        ref = dequant(wq, ws, wb, e, d, kind, S.META_BF16) @ xs
+    bound = 1e-5 * np.abs(ref).max() + 1e-6
+    assert np.abs(got - ref).max() <= bound
+    plain = (f16(w).astype(np.float64).reshape(e, d) if kind == O.ROUTER_F16
+             else dequant(wq, ws, wb, e, d, kind, S.META_BF16)) @ f16(x).astype(np.float64)
+    assert np.abs(got - plain).max() > 100 * bound, "ignoring the effective scale must not pass"
+
+
+def test_cpu_layer_against_fp64_chain():
+    """CPUExpertFFN.swift:102-140 over several experts, one task each: out += w_e * down_e(silu(gate_e x) * up_e x),
+    everything in fp32 with no fp16 rounding between the stages; any thread count gives the same bits."""
+    d, f, n = 256, 128, 5
+    tree = S.SeedTree(0x5EED0A40)
+    blobs = [S.expert_blob(tree, f"e{e}", d, f, 4) for e in range(n)]
+    off, _ = O.expert_offsets(d, f, 4)
+    x = tree.key("x").normal(d).astype(np.float32)
+    rw = np.array([0.4, 0.25, 0.2, 0.1, 0.05], np.float32)
+    want = np.zeros(d, np.float64)
+    for e in range(n):
+        v = S.blob_views(blobs[e], d, f, 4)
+        g = dequant(*v["gate"], f, d, 4, S.META_BF16) @ x.astype(np.float64)
+        u = dequant(*v["up"], f, d, 4, S.META_BF16) @ x.astype(np.float64)
+        want += float(rw[e]) * (dequant(*v["down"], d, f, 4, S.META_BF16) @ (g / (1.0 + np.exp(-g)) * u))
+    outs = [O.cpu_layer_fp32(blobs, rw, off, x, d, f, threads) for threads in (1, 3, 8)]
+    assert np.abs(outs[0] - want).max() <= 2e-4 * max(1.0, np.abs(want).max())  # CPUExpertFFNTests.swift:69-113
+    assert all(np.array_equal(o.view(np.uint32), outs[0].view(np.uint32)) for o in outs[1:])
+    dropped = O.cpu_layer_fp32(blobs[:4], rw[:4], off, x, d, f, 2)
+    assert np.abs(dropped - want).max() > 2e-4 * max(1.0, np.abs(want).max()), "a dropped expert must not pass"
+
+
+@pytest.mark.parametrize("d", [2048, 2304, 192])
+def test_per_row_scalar_gate_against_fp64(d):
+    """moe.metal:1154-1207: gate[row] = half(dequant8(W) . x_row); y[row, :] = half(y[row, :] * sigmoid(gate[row]))."""
+    rows, stride = 7, d + 24
+    tree = S.SeedTree(0x5EED0A50 + d)
+    w, s, b = S.affine_matrix(tree.key("gate.row"), 1, d, 8, S.META_BF16)
+    x = S.activations_f16(tree, "x", rows * stride)
+    gate = O.shared_scalar_gate_rows((w, s, b), x, rows, d, x_stride=stride)
+    xm = f16(x).astype(np.float64).reshape(rows, stride)[:, :d]
+    want = xm @ dequant(w, s, b, 1, d, 8, S.META_BF16)[0]
+    assert np.all(np.abs(f16(gate) - want) <= 1e-3 * np.abs(want) + 1e-4), "one fp16 rounding of an fp32 sum"
+    assert len(set(gate.tolist())) == rows, "every row has its own gate"
+    y = S.activations_f16(tree, "y", rows * d)
+    out = O.sigmoid_scalar_mul_rows(y.copy(), gate, d, rows)
+    sig = 1.0 / (1.0 + np.exp(-f16(gate).astype(np.float64)))
+    want_y = h(f16(y).astype(np.float64).reshape(rows, d) * sig[:, None])
+    diff = np.abs(f16(out).astype(np.float64).reshape(rows, d) - want_y)
+    assert np.all(diff <= np.abs(want_y) * 2.0 ** -10 + 1e-7)
+    one_gate = h(f16(y).astype(np.float64).reshape(rows, d) * sig[0])
+    assert np.max(np.abs(f16(out).astype(np.float64).reshape(rows, d) - one_gate)) > 1e-2, \
+        "row 0's gate applied to every row must not pass"

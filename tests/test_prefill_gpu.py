@@ -78,7 +78,8 @@ def expected_row_tiles(groups, cell_of):
 
 
 @pytest.mark.parametrize("t,k,ne,mode", [(512, 8, 256, "plain"), (512, 8, 256, "keys"), (37, 3, 17, "plain"), (64, 4, 32, "residency"),
-                                         (1, 8, 256, "plain"), (300, 2, 4, "keys"), (0, 8, 16, "plain")])
+                                         (1, 8, 256, "plain"), (300, 2, 4, "keys"), (0, 8, 16, "plain"),
+                                         (200, 1, 32, "plain"), (5000, 1, 7, "keys")])  # one expert a token: the token index is the pair index
 def test_device_grouping_equals_host_grouping(gpu, t, k, ne, mode):
     idx, w = random_routes(t * 131 + k, t, k, ne)
     keys = None
@@ -351,20 +352,36 @@ def test_prefill_layer_at_full_size_agrees_with_the_decode_kernels(gpu):
         assert_rel_close(out[tok], dl.y.download(np.uint16, d), f"token {tok}: prefill h2 vs decode y", tol=2e-3)
 
 
-@pytest.mark.parametrize("d,fs,bits,t,gated", [(2048, 512, 4, 20, False), (2304, 1024, 8, 16, True), (192, 320, 4, 70, False), (128, 64, 8, 1, True)])
+@pytest.mark.parametrize("d,fs,bits,t,gated", [(2048, 512, 4, 20, False), (2048, 512, 4, 70, True), (2304, 1024, 8, 16, True),
+                                              (192, 320, 4, 70, False), (128, 64, 8, 1, True)])
 def test_shared_expert_for_a_token_block(gpu, d, fs, bits, t, gated):
+    """The chunk's shared expert with ONE SCALAR GATE A TOKEN (RealForwardRunner.swift:4438-4456): the gate row's
+    GEMV for every token (moe.metal:1154-1193) bit for bit against the oracle, then h1[t] = shared(x_t) * sigmoid(gate[t])
+    against the oracle token by token; the two-launch form (ungated block, then sigmoid_scalar_mul_rows) gives the same."""
     L = Layer(0x5EED0007, d, 64, 4, 2, bits=bits, shared_f=fs, shared_bits=bits)
     dl = DeviceLayer(gpu, L, resident=[])
     pf = gpu.Prefill(dl.moe)
-    x = token_rows(L, t, d + 8)
+    stride = d + 8
+    x = token_rows(L, t, stride)
+    dx = gpu.dev(x)
     h1 = gpu.dev(np.full(t * d, 0xD4D0, np.uint16))
-    gate_bits = S.f32_to_f16_bits(np.array([0.37], np.float32)) if gated else None
-    pf.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, gpu.dev(x), d + 8, h1, t, fs,
-                            scalar_gate=gpu.dev(gate_bits) if gated else None)
+    gates = None
+    d_gates = None
+    if gated:
+        gate_row = S.affine_matrix(L.tree.key("shared.scalar_gate"), 1, d, 8, L.meta)
+        d_gates = gpu.empty(2 * t).fill(0xFF)
+        pf.encode_scalar_gate_rows(tuple(gpu.dev(a) for a in gate_row), dx, stride, d_gates, t, d)
+        gates = d_gates.download(np.uint16, t)
+        want_gates = O.shared_scalar_gate_rows(gate_row, x, t, d, x_stride=stride, meta=L.meta)
+        assert np.array_equal(gates, want_gates), "the per-row gate differs from the oracle in bits"
+        assert t == 1 or len(set(gates.tolist())) > 1
+    pf.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, dx, stride, h1, t, fs,
+                            scalar_gate=d_gates)
     gpu.synchronize()
     got = h1.download(np.uint16, t * d).reshape(t, d)
     for tok in range(t):
-        xt = np.ascontiguousarray(x[tok * (d + 8):tok * (d + 8) + d])
+        xt = np.ascontiguousarray(x[tok * stride:tok * stride + d])
+        gate_bits = gates[tok:tok + 1].copy() if gated else None
         ref = O.shared_expert(L.shared["gate"], L.shared["up"], L.shared["down"], xt, d, fs, bits=bits, meta=L.meta,
                               scalar_gate_f16=gate_bits)
         # gate/up -> fp16 -> act -> fp16 -> down -> fp16 (-> gate -> fp16): whole chain, the reference's metric
@@ -376,14 +393,27 @@ def test_shared_expert_for_a_token_block(gpu, d, fs, bits, t, gated):
                                         one, d, fs, scalar_gate=gpu.dev(gate_bits) if gated else None)
             gpu.synchronize()
             assert_rel_close(got[tok], one.download(np.uint16, d), f"token {tok} vs the decode operator", tol=2e-3 if gated else 1e-3)
+    if gated:
+        # the reference's two kernels: the ungated block, then y[t, :] *= sigmoid(gate[t]) in place
+        plain = gpu.dev(np.full(t * d, 0xD4D0, np.uint16))
+        pf.encode_shared_expert(dl.shared["gate"], dl.shared["up"], dl.shared["down"], bits, dx, stride, plain, t, fs)
+        ungated = plain.download(np.uint16, t * d)
+        pf.encode_sigmoid_scalar_mul_rows(plain, d_gates, d, t)
+        gpu.synchronize()
+        assert np.array_equal(plain.download(np.uint16, t * d).reshape(t, d), got), "fused and two-launch gating differ"
+        # the elementwise kernel against the oracle: the device's exp may differ from libm's in the last bit
+        assert_ffn_close(plain.download(np.uint16, t * d), O.sigmoid_scalar_mul_rows(ungated.copy(), gates, d, t), "sigmoid rows")
 
 
-@pytest.mark.parametrize("bits,slots,slru", [(8, 16, None), (4, 8, 0.5)])
-def test_batched_decode_through_a_pool_smaller_than_the_expert_set(gpu, bits, slots, slru):
-    """Config 5 in small: 12 sequences, top-4 of 48 experts, a pool of 16 (or 8) cells; the experts
+@pytest.mark.parametrize("d,f,ne,k,t,bits,slots,slru", [
+    (256, 128, 48, 4, 12, 8, 16, None), (256, 128, 48, 4, 12, 4, 8, 0.5),
+    (2304, 1024, 256, 8, 16, 8, 64, None),  # config 5 as it is stated: Kimi-Linear shape, 16 sequences, 64 of 256 cells
+])
+def test_batched_decode_through_a_pool_smaller_than_the_expert_set(gpu, d, f, ne, k, t, bits, slots, slru):
+    """Config 5: several sequences, one token each, through a pool smaller than the expert set; the experts
     stream from pinned host memory in passes. Routes are bit-exact, every partial row matches the
-    oracle stage by stage, the statistics count what happened, and a second step hits the cache."""
-    d, f, ne, k, t = 256, 128, 48, 4, 12
+    oracle stage by stage, the statistics (and so the miss rate) equal the slot-cache restatement's over the
+    same plans, and a second step hits the cache."""
     L = Layer(0x5EED0005, d, f, ne, k, bits=bits)
     dl = DeviceLayer(gpu, L, cells=slots, resident=[])
     dl.moe.stream = gpu.Stream()
@@ -420,6 +450,18 @@ def test_batched_decode_through_a_pool_smaller_than_the_expert_set(gpu, bits, sl
     layer.run(router, hidden, t, d)
     dl.moe.stream.synchronize()
     assert cache.statistics().hits > before
+    # the miss rate over both steps is the slot-cache restatement's over the same plans
+    twin = H.SlotCache(slots, ne, slru_share=slru)
+    for batch in layer.plan_log:
+        twin.load(batch)
+    st, ts = cache.statistics(L.stride), twin.stats
+    assert (st.plans, st.requested_experts, st.hits, st.misses, st.evictions, st.reloads) == tuple(
+        ts[n] for n in ("plans", "requested", "hits", "misses", "evictions", "reloads"))
+    assert [cache.entry(e) for e in range(ne)] == list(twin.words)
+    miss_rate = st.misses / st.requested_experts
+    print(f"\n[config 5] d={d} f={f} E={ne} K={k} tokens={t} cells={slots}: {used} distinct experts a step, "
+          f"{layer.passes} passes, miss rate over two steps {miss_rate:.3f}")
+    assert 0.0 < miss_rate < 1.0
     again = layer.partials.download(np.uint16, t * k * d)
     assert np.array_equal(again, partials.reshape(-1))  # same bytes whatever cell an expert landed in
 
