@@ -306,6 +306,22 @@ typedef struct {
 int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
                                 const shrike_decode_layer_args *args);
 
+/* The decode layer for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). NO COUNTERPART IN THE REFERENCE. Same kernels and same
+ * results as shrike_hip_moe_decode_layer, but no handle (shrike_hip_moe_create allocates): the
+ * description is passed by value, and the router logits, the route lists, the activations and the
+ * shared expert's intermediate rows live in a 96 KiB static device array that each GPU the library
+ * runs on holds until the process ends. In `args` the caller binds the inputs (router, pool,
+ * residency, shared projections, x, hidden) and the outputs (y, hidden, out_indices, out_weights);
+ * the scratch fields (resolved_slots, hit_*, miss_*, acts, shared_scratch, h1) may be NULL and then
+ * come from the static array (a caller that reads the miss lists binds those). Limits: f <= 4096,
+ * shared_f <= 4096, d <= SHRIKE_MAX_HIDDEN; larger sizes are EINVAL. The call allocates nothing and
+ * calls no allocating routine once shrike_hip_init() has run on the device (otherwise its first call
+ * on a device looks the array's address up, which must not happen under capture). All calls on one
+ * GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
+int shrike_hip_moe_decode_layer_noalloc(const shrike_moe_desc *desc, void *stream,
+                                        const shrike_decode_layer_args *args);
+
 /* ------------------------------------------------------- measurement aids
  * No counterpart in the reference. An empty launch of `workgroups` x 256 threads, and a
  * kernel that only reads bytes [byte_offset, byte_offset + bytes_per_cell) of each pool cell

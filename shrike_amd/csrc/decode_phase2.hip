@@ -1,6 +1,8 @@
 // Phase 2 of the routed decode layer for gfx950 (down matvec per selected expert, weighted
 // combine, residual, hidden += y: moe.metal:889-941, :1008-1057), the dense group-affine
 // GEMV of the shared expert, and the fused-layer entry point.
+#include <mutex>
+
 #include "decode_launch.h"
 
 namespace shrike {
@@ -187,6 +189,45 @@ int check_shared(const shrike_projection *gate, const shrike_projection *up, con
     SHRIKE_REQUIRE(d <= SHRIKE_MAX_HIDDEN && f_shared <= SHRIKE_MAX_HIDDEN,
                    "sharedExpert: d=%u or f=%u exceeds the activation ceiling %u", d, f_shared, SHRIKE_MAX_HIDDEN);
     return 0;
+}
+
+// ---- the static scratch of the allocation-free layer entry point
+//
+// 96 KiB of device memory that every GPU the library runs on holds until the process ends. Layout (bytes):
+// fp32 logits[256] at 0; the route lists (resolved cells, hit/miss counts, positions, experts) at 1024;
+// fp16 acts[8 * 4096] at 2048; the shared expert's fp16 gate and up rows [2 * 4096] behind them; fp16 h1[4096].
+constexpr uint32_t kNoAllocMaxF = 4096, kNoAllocMaxSharedF = 4096;
+constexpr size_t kScratchLists = 1024, kScratchActs = 2048;
+constexpr size_t kScratchShared = kScratchActs + size_t(SHRIKE_MAX_TOP_K) * kNoAllocMaxF * 2u;
+constexpr size_t kScratchH1 = kScratchShared + 2u * kNoAllocMaxSharedF * 2u;
+constexpr size_t kScratchBytes = kScratchH1 + size_t(SHRIKE_MAX_HIDDEN) * 2u;
+static_assert(kScratchBytes <= 96u * 1024u, "the static scratch is stated as 96 KiB");
+static __device__ __align__(256) unsigned char scratch[96u * 1024u];
+
+// In host code `scratch` is only a handle for the symbol; the array's device address differs from GPU to GPU and is
+// looked up once per device, with that device current.
+constexpr int kMaxDevices = 64;
+static unsigned char *g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+static int layer_scratch(unsigned char **out) {
+    int device = -1;
+    SHRIKE_HIP(hipGetDevice(&device));
+    SHRIKE_REQUIRE(device >= 0 && device < kMaxDevices, "device %d is past the %d this library keeps scratch for", device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void *ptr = nullptr;
+        SHRIKE_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        SHRIKE_REQUIRE(ptr != nullptr, "the static scratch has no address on device %d", device);
+        g_scratch_ptr[device] = static_cast<unsigned char *>(ptr);
+    }
+    *out = g_scratch_ptr[device];
+    return 0;
+}
+
+int init_layer_scratch() {
+    unsigned char *ptr = nullptr;
+    return layer_scratch(&ptr);
 }
 
 }  // namespace shrike
@@ -383,6 +424,35 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
     p.d = m.d; p.f = m.f; p.top_k = m.top_k; p.meta = m.meta_dtype; p.ebias = m.expert_additive_biases;
     p.delta = normed ? norm.delta : nullptr;
     return launch_phase2(p, m.routed_weight_bits, s);
+}
+
+// The same layer for callers that cannot allocate: no handle (making one allocates), no scratch from the caller.
+// The kernels are the ones above; the logits, the route lists, the activations and the shared expert's
+// intermediate rows live in the static array. Calls that overlap on one GPU race on it.
+int shrike_hip_moe_decode_layer_noalloc(const shrike_moe_desc *desc, void *stream, const shrike_decode_layer_args *g) {
+    if (int rc = check_moe_desc(desc)) return rc;
+    SHRIKE_REQUIRE(g != nullptr, "args is NULL");
+    SHRIKE_REQUIRE(desc->f <= kNoAllocMaxF, "decodeLayerNoAlloc: f=%u exceeds the static scratch's %u", desc->f, kNoAllocMaxF);
+    SHRIKE_REQUIRE(g->shared_gate.weights == nullptr || g->shared_f <= kNoAllocMaxSharedF,
+                   "decodeLayerNoAlloc: sharedF=%u exceeds the static scratch's %u", g->shared_f, kNoAllocMaxSharedF);
+    unsigned char *base = nullptr;
+    if (int rc = layer_scratch(&base)) return rc;
+    shrike_hip_moe moe = {};
+    moe.desc = *desc;
+    moe.d_logits = reinterpret_cast<float *>(base);
+    moe.d_counter = nullptr;  // the fused layer selects in the second launch's prologue: no arrival counter
+    shrike_decode_layer_args a = *g;
+    uint32_t *lists = reinterpret_cast<uint32_t *>(base + kScratchLists);
+    if (!a.resolved_slots) a.resolved_slots = lists;
+    if (!a.hit_positions) a.hit_positions = lists + 8;
+    if (!a.miss_positions) a.miss_positions = lists + 16;
+    if (!a.miss_experts) a.miss_experts = lists + 24;
+    if (!a.hit_count) a.hit_count = lists + 32;
+    if (!a.miss_count) a.miss_count = lists + 33;
+    if (!a.acts) a.acts = base + kScratchActs;
+    if (!a.shared_scratch) a.shared_scratch = base + kScratchShared;
+    if (!a.h1) a.h1 = base + kScratchH1;
+    return shrike_hip_moe_decode_layer(&moe, stream, &a);
 }
 
 }  // extern "C"

@@ -32,6 +32,11 @@ int hip_failed(hipError_t err, const char *what);  // records the error, returns
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
+int check_moe_desc(const shrike_moe_desc *desc);  // runtime.hip
+// decode_phase2.hip: looks up, for the current device, the address of the static scratch array of
+// shrike_hip_moe_decode_layer_noalloc (once per device; later calls return at once)
+int init_layer_scratch();
+
 }  // namespace shrike
 
 // MoE.swift:41-216: the handle keeps the shape it was made for, the router's fp32

@@ -56,6 +56,29 @@ struct shrike_hip_pool {
     bool owns_cells = true;        // false for a layer's table over another pool's cells
 };
 
+namespace shrike {
+
+// MoE.init's preconditions (MoE.swift:113-116 and the kernels' own ceilings); EINVAL with the cause recorded.
+int check_moe_desc(const shrike_moe_desc *desc) {
+    SHRIKE_REQUIRE(desc != nullptr, "desc is NULL");
+    SHRIKE_REQUIRE(desc->routed_weight_bits == 4 || desc->routed_weight_bits == 8, "routedWeightBits=%u not in {4, 8}",
+                   desc->routed_weight_bits);
+    SHRIKE_REQUIRE(desc->router_weight_bits == 0 || desc->router_weight_bits == 4 || desc->router_weight_bits == 8,
+                   "routerWeightBits=%u not in {0 (fp16), 4, 8}", desc->router_weight_bits);
+    SHRIKE_REQUIRE(desc->top_k >= 1 && desc->top_k <= SHRIKE_MAX_TOP_K, "topK=%u not in 1...%u", desc->top_k, SHRIKE_MAX_TOP_K);
+    SHRIKE_REQUIRE(desc->d != 0 && desc->d <= SHRIKE_MAX_HIDDEN && desc->d % SHRIKE_GROUP_SIZE == 0,
+                   "d=%u must be a multiple of %u and at most %u", desc->d, SHRIKE_GROUP_SIZE, SHRIKE_MAX_HIDDEN);
+    SHRIKE_REQUIRE(desc->f != 0 && desc->f % SHRIKE_GROUP_SIZE == 0, "f=%u must be a positive multiple of %u", desc->f,
+                   SHRIKE_GROUP_SIZE);
+    SHRIKE_REQUIRE(desc->num_experts >= desc->top_k && desc->num_experts <= SHRIKE_MAX_ROUTER_EXPERTS,
+                   "numExperts=%u must be in topK...%u", desc->num_experts, SHRIKE_MAX_ROUTER_EXPERTS);
+    SHRIKE_REQUIRE(desc->meta_dtype <= SHRIKE_META_F16 && desc->activation <= SHRIKE_ACT_CLAMPED_SWIGLU,
+                   "metaDtype=%u or activation=%u is not a known value", desc->meta_dtype, desc->activation);
+    return 0;
+}
+
+}  // namespace shrike
+
 size_t shrike_expert_reader_stride_internal(const shrike_expert_reader *r);  // expert_io.cpp
 
 extern "C" {
@@ -74,7 +97,7 @@ int shrike_hip_init(int device) {
         set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
         return ENODEV;
     }
-    return 0;
+    return shrike::init_layer_scratch();  // the allocation-free layer's static scratch, found once per device
 }
 
 uint64_t shrike_expert_offsets_make(uint32_t d, uint32_t f, uint32_t bits, int additive_biases,
@@ -382,32 +405,7 @@ uint64_t shrike_hip_pool_table_entry(const shrike_hip_pool *pool, uint32_t exper
 
 shrike_hip_moe *shrike_hip_moe_create(const shrike_moe_desc *desc, int *out_errno) {
     auto fail = [&](int code) -> shrike_hip_moe * { if (out_errno) *out_errno = code; return nullptr; };
-    if (!desc) { set_error("desc is NULL"); return fail(EINVAL); }
-    // MoE.swift:113-116
-    if (desc->routed_weight_bits != 4 && desc->routed_weight_bits != 8) {
-        set_error("routedWeightBits=%u not in {4, 8}", desc->routed_weight_bits); return fail(EINVAL);
-    }
-    if (desc->router_weight_bits != 0 && desc->router_weight_bits != 4 && desc->router_weight_bits != 8) {
-        set_error("routerWeightBits=%u not in {0 (fp16), 4, 8}", desc->router_weight_bits); return fail(EINVAL);
-    }
-    if (desc->top_k < 1 || desc->top_k > SHRIKE_MAX_TOP_K) {
-        set_error("topK=%u not in 1...%u", desc->top_k, SHRIKE_MAX_TOP_K); return fail(EINVAL);
-    }
-    if (desc->d == 0 || desc->d > SHRIKE_MAX_HIDDEN || desc->d % SHRIKE_GROUP_SIZE) {
-        set_error("d=%u must be a multiple of %u and at most %u", desc->d, SHRIKE_GROUP_SIZE, SHRIKE_MAX_HIDDEN);
-        return fail(EINVAL);
-    }
-    if (desc->f == 0 || desc->f % SHRIKE_GROUP_SIZE) {
-        set_error("f=%u must be a positive multiple of %u", desc->f, SHRIKE_GROUP_SIZE); return fail(EINVAL);
-    }
-    if (desc->num_experts < desc->top_k || desc->num_experts > SHRIKE_MAX_ROUTER_EXPERTS) {
-        set_error("numExperts=%u must be in topK...%u", desc->num_experts, SHRIKE_MAX_ROUTER_EXPERTS);
-        return fail(EINVAL);
-    }
-    if (desc->meta_dtype > SHRIKE_META_F16 || desc->activation > SHRIKE_ACT_CLAMPED_SWIGLU) {
-        set_error("metaDtype=%u or activation=%u is not a known value", desc->meta_dtype, desc->activation);
-        return fail(EINVAL);
-    }
+    if (int rc = shrike::check_moe_desc(desc)) return fail(rc);
     shrike_hip_moe *moe = new shrike_hip_moe();
     moe->desc = *desc;
     moe->d_logits = nullptr; moe->d_counter = nullptr;
