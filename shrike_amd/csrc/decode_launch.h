@@ -15,6 +15,7 @@ struct RouterArgs {
     float *logits_out;
     SelectArgs sel;
     RouteLists lists;  // out_indices == nullptr: logits only
+    RouteEntry *route_table;  // head launch of the fused layer: one entry per expert beside the logit (lists.residency read)
     // several tokens in one launch (grid.y): token t reads hidden + t * token_stride, writes logits_out + t *
     // num_experts and out_indices / out_weights + t * top_k, and counts arrivals in counter[t]; select only
     uint32_t token_stride;
@@ -30,10 +31,12 @@ struct Phase1Args {
     uint32_t d, f, top_k, meta, act, ebias;
     const uint32_t *indirect, *io_status;
     uint32_t tokens, x_stride;  // tokens > 1: grid.y walks tokens; x rows x_stride elements apart
-    // fused layer only: route from the logits of the previous launch (sel.logits != nullptr),
-    // and run the shared expert's down projection in workgroups past `routed_blocks`
+    // fused layer only: every wave selects from the route table the previous launch left, the shared expert's down
+    // projection runs in workgroups past `routed_blocks`, and one more workgroup behind those writes the route lists
     SelectArgs sel;
     RouteLists lists;
+    const RouteEntry *route_table;
+    uint32_t lists_block;  // set by launch_phase1: the workgroup that writes the route lists
     uint32_t routed_blocks;
     GemvArgs shared_down;
 };

@@ -17,7 +17,17 @@ template <int BITS, int NCH, int RP, bool ROUTE, int SBITS>
 __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
-    __shared__ uint32_t s_cell[SHRIKE_MAX_TOP_K];
+    if (ROUTE && blockIdx.x == a.lists_block) {
+        // the workgroup behind all others: one wave selects once more and writes what the host and phase 2 read
+        // (indices, weights, hit and miss lists, resolved cells); nobody in this launch waits for it
+        if (threadIdx.x < 64u) {
+            const TableSelect t = select_from_table(a.route_table, a.sel.num_experts, a.sel.top_k, threadIdx.x, a.sel.top_k);
+            uint32_t my_cell;
+            finish_routes(a.sel, a.lists, threadIdx.x, true, t.mine, t.my_key, t.my_raw, bf16_to_f32(uint16_t(t.my_gain)),
+                          t.my_cell, my_cell);
+        }
+        return;
+    }
     if (SBITS != 0 && blockIdx.x >= a.routed_blocks) {
         gemv_job<SBITS == 0 ? 4 : SBITS, 1>(a.shared_down, blockIdx.x - a.routed_blocks);
         return;
@@ -37,21 +47,18 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     const uint32_t k = in_range ? pair0 / a.f : 0u;
     const uint32_t f0 = pair0 - k * a.f;
 
-    SliceRegs<BITS, NCH> xr;
-    load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
-
     uint32_t cell = kSentinel;
+    SliceRegs<BITS, NCH> xr;
     if (ROUTE) {
-        if (wave == 0) {
-            __shared__ RouteScratch s_route;
-            uint32_t my_cell;
-            route_wave<false>(a.sel, a.lists, lane, blockIdx.x == 0, my_cell, s_route);
-            if (lane < a.top_k) s_cell[lane] = my_cell;
-        }
-        __syncthreads();
-        if (in_range) cell = s_cell[k];
-    } else if (in_range) {
-        cell = resolved_tok[k];
+        // every wave selects for itself, in registers, from the table the previous launch left: no barrier, and the
+        // table's loads go out ahead of the activation slice's (loads return in order)
+        // (a wave stops at the round that names its own position's expert)
+        const TableSelect t = select_from_table(a.route_table, a.sel.num_experts, a.sel.top_k, lane, k);
+        load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
+        if (in_range) cell = uint32_t(__builtin_amdgcn_readlane(int(t.my_cell), int(k)));
+    } else {
+        load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
+        if (in_range) cell = resolved_tok[k];
     }
     if (cell == kSentinel) return;  // moe.metal:986, and waves past the last row
     const uint8_t *base = cell_base_uniform(a.pool, cell, a.stride);
@@ -114,17 +121,19 @@ int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t sha
                        "phase1: the shared down rows ride along only in the routed launch and with one chunk column per lane");
         extra = gemv_blocks(a.shared_down.rows, a.shared_down.n, shared_down_bits);
     }
-    const dim3 grid(a.routed_blocks + extra, a.tokens ? a.tokens : 1u);
+    Phase1Args b = a;
+    b.lists_block = routing ? a.routed_blocks + extra : 0xffffffffu;
+    const dim3 grid(a.routed_blocks + extra + (routing ? 1u : 0u), a.tokens ? a.tokens : 1u);
     if (bits == 4) {
-        if (!routing) launch_phase1_nch<4, false, 0>(a, grid, s);
-        else if (shared_down_bits == 0) launch_phase1_nch<4, true, 0>(a, grid, s);
-        else if (shared_down_bits == 4) launch_phase1_nch<4, true, 4>(a, grid, s);
-        else launch_phase1_nch<4, true, 8>(a, grid, s);
+        if (!routing) launch_phase1_nch<4, false, 0>(b, grid, s);
+        else if (shared_down_bits == 0) launch_phase1_nch<4, true, 0>(b, grid, s);
+        else if (shared_down_bits == 4) launch_phase1_nch<4, true, 4>(b, grid, s);
+        else launch_phase1_nch<4, true, 8>(b, grid, s);
     } else {
-        if (!routing) launch_phase1_nch<8, false, 0>(a, grid, s);
-        else if (shared_down_bits == 0) launch_phase1_nch<8, true, 0>(a, grid, s);
-        else if (shared_down_bits == 4) launch_phase1_nch<8, true, 4>(a, grid, s);
-        else launch_phase1_nch<8, true, 8>(a, grid, s);
+        if (!routing) launch_phase1_nch<8, false, 0>(b, grid, s);
+        else if (shared_down_bits == 0) launch_phase1_nch<8, true, 0>(b, grid, s);
+        else if (shared_down_bits == 4) launch_phase1_nch<8, true, 4>(b, grid, s);
+        else launch_phase1_nch<8, true, 8>(b, grid, s);
     }
     SHRIKE_HIP(hipGetLastError());
     return 0;

@@ -195,12 +195,14 @@ int check_shared(const shrike_projection *gate, const shrike_projection *up, con
 //
 // 96 KiB of device memory that every GPU the library runs on holds until the process ends. Layout (bytes):
 // fp32 logits[256] at 0; the route lists (resolved cells, hit/miss counts, positions, experts) at 1024;
-// fp16 acts[8 * 4096] at 2048; the shared expert's fp16 gate and up rows [2 * 4096] behind them; fp16 h1[4096].
+// fp16 acts[8 * 4096] at 2048; the shared expert's fp16 gate and up rows [2 * 4096] behind them; fp16 h1[4096];
+// the route table (16 bytes an expert, 256 experts) last.
 constexpr uint32_t kNoAllocMaxF = 4096, kNoAllocMaxSharedF = 4096;
 constexpr size_t kScratchLists = 1024, kScratchActs = 2048;
 constexpr size_t kScratchShared = kScratchActs + size_t(SHRIKE_MAX_TOP_K) * kNoAllocMaxF * 2u;
 constexpr size_t kScratchH1 = kScratchShared + 2u * kNoAllocMaxSharedF * 2u;
-constexpr size_t kScratchBytes = kScratchH1 + size_t(SHRIKE_MAX_HIDDEN) * 2u;
+constexpr size_t kScratchRoute = kScratchH1 + size_t(SHRIKE_MAX_HIDDEN) * 2u;  // RouteEntry[256]
+constexpr size_t kScratchBytes = kScratchRoute + size_t(SHRIKE_MAX_ROUTER_EXPERTS) * sizeof(RouteEntry);
 static_assert(kScratchBytes <= 96u * 1024u, "the static scratch is stated as 96 KiB");
 static __device__ __align__(256) unsigned char scratch[96u * 1024u];
 
@@ -378,7 +380,9 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
     r.sel.logit_bias = static_cast<const uint16_t *>(g->logit_bias);
     r.sel.num_experts = m.num_experts; r.sel.top_k = m.top_k;
     r.sel.sigmoid = m.sigmoid_router_scores; r.sel.scaling = m.routed_scaling_factor;
-    // r.lists stays empty: launch 1 writes logits only
+    // launch 1 writes the logits and, beside each, the expert's route entry; no list yet
+    r.lists.residency = g->residency;
+    r.route_table = moe->d_route;
 
     Phase1Args p1 = {};
     fill_pool(p1.pool, g->pool);
@@ -391,6 +395,7 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
     p1.lists.residency = g->residency; p1.lists.hit_count = g->hit_count; p1.lists.hit_positions = g->hit_positions;
     p1.lists.miss_count = g->miss_count; p1.lists.miss_positions = g->miss_positions;
     p1.lists.miss_experts = g->miss_experts; p1.lists.resolved_slots = g->resolved_slots;
+    p1.route_table = moe->d_route;
     p1.routed_blocks = phase1_blocks(m.top_k, m.f);
 
     const void *residual = nullptr;
@@ -403,12 +408,10 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
                        m.activation, g->shared_scalar_gate);
         down_fused = nch_for(g->shared_f, sbits) == 1;
         residual = g->h1;
-    } else if (normed) {  // the head launch with router rows only
+    } else {  // the head launch with router rows only
         GemvArgs none = {};
         none.n = m.d;
-        if (int rc = launch_head(r, m.router_weight_bits, none, sbits, &norm, s)) return rc;
-    } else {
-        if (int rc = launch_router(r, m.router_weight_bits, s)) return rc;
+        if (int rc = launch_head(r, m.router_weight_bits, none, sbits, normed ? &norm : nullptr, s)) return rc;
     }
     if (int rc = launch_phase1(p1, m.routed_weight_bits, true, down_fused ? sbits : 0u, s)) return rc;
     if (shared && !down_fused) {
@@ -441,6 +444,7 @@ int shrike_hip_moe_decode_layer_noalloc(const shrike_moe_desc *desc, void *strea
     moe.desc = *desc;
     moe.d_logits = reinterpret_cast<float *>(base);
     moe.d_counter = nullptr;  // the fused layer selects in the second launch's prologue: no arrival counter
+    moe.d_route = reinterpret_cast<RouteEntry *>(base + kScratchRoute);
     shrike_decode_layer_args a = *g;
     uint32_t *lists = reinterpret_cast<uint32_t *>(base + kScratchLists);
     if (!a.resolved_slots) a.resolved_slots = lists;

@@ -80,8 +80,13 @@ __global__ __launch_bounds__(256) void k_head(RouterArgs r, GemvArgs g, uint32_t
     if (blockIdx.x < router_blocks) {
         const uint32_t e = blockIdx.x * 4u + wave_index();
         if (e < r.sel.num_experts) {
-            if (NORM) router_row<RK>(r, [&] { return reinterpret_cast<const uint16_t *>(normed_row()); }, r.logits_out, e, threadIdx.x & 63u, false);
-            else router_row<RK>(r, e, threadIdx.x & 63u);
+            // what the expert's route entry needs beside the logit: fetched beside the row, used behind it
+            const uint16_t bias_bits = r.sel.logit_bias[e], gain_bits = r.sel.per_expert_scale[e];
+            const uint64_t word = r.lists.residency ? r.lists.residency[e] : 0;
+            float logit;
+            if (NORM) logit = router_row<RK>(r, [&] { return reinterpret_cast<const uint16_t *>(normed_row()); }, r.logits_out, e, threadIdx.x & 63u, false);
+            else logit = router_row<RK>(r, e, threadIdx.x & 63u);
+            if (r.route_table && (threadIdx.x & 63u) == 0) write_route_entry(r.route_table, e, logit, bias_bits, gain_bits, word, r.sel.sigmoid);
         } else if (NORM) {
             normed_row();  // the workgroup's barriers need every wave
         }

@@ -197,6 +197,13 @@ __device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block, XSou
     const uint32_t total = a.rows + a.rows_b;
     const uint32_t first = (block * 4u + wave) * kGemvRowsPerWave * rpl;
     const bool active = first < total;
+    // The two row sets' pointers, pinned in scalar registers: picking between the FIELDS of the argument block by a
+    // per-lane condition would otherwise become a vector load of the chosen pointer from constant memory, a
+    // dependent memory round trip ahead of every row load and every store.
+    const uint8_t *w_a = a.w_a, *w_b = a.w_b;
+    const uint16_t *s_a = a.s_a, *s_b = a.s_b, *b_a = a.b_a, *b_b = a.b_b;
+    uint16_t *y_a = a.y_a, *y_b = a.y_b;
+    asm volatile("" : "+s"(w_a), "+s"(w_b), "+s"(s_a), "+s"(s_b), "+s"(b_a), "+s"(b_b), "+s"(y_a), "+s"(y_b));
 
     // the input slice first: in-order load return must not hold it behind the rows
     SliceRegs<BITS, NCH> xin;
@@ -216,29 +223,25 @@ __device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block, XSou
             const uint32_t rr = on[j] ? row[j] : 0u;
             const bool second = rr >= a.rows;
             const uint32_t local = second ? rr - a.rows : rr;
-            load_row<BITS, NCH>(rows[j], (second ? a.w_b : a.w_a) + size_t(local) * row_bytes,
-                                (second ? a.s_b : a.s_a) + size_t(local) * groups,
-                                (second ? a.b_b : a.b_a) + size_t(local) * groups, cpr, col, on[j]);
+            load_row<BITS, NCH>(rows[j], (second ? w_b : w_a) + size_t(local) * row_bytes,
+                                (second ? s_b : s_a) + size_t(local) * groups,
+                                (second ? b_b : b_a) + size_t(local) * groups, cpr, col, on[j]);
         }
     }
     if (!kPlainX) {
         const uint4 *x_row = x_source();
         if (active) load_slice_regs<BITS, NCH>(xin, x_row, cpr, col, true);
     } else if (a.gate_in) {
-        // dequant_int4.metal:283-287: act = half(glu(gate, up)) once per workgroup, staged in LDS
+        // dequant_int4.metal:283-287: act = half(glu(gate, up)) once per workgroup, staged in LDS; a thread takes
+        // pairs of neighbours, so that a short row still spreads over the whole workgroup
         __shared__ uint4 act_l[SHRIKE_MAX_HIDDEN / 8];
-        for (uint32_t p = threadIdx.x; p < a.n / 8u; p += 256u) {
-            const uint4 gv = reinterpret_cast<const uint4 *>(a.gate_in)[p];
-            const uint4 uv = reinterpret_cast<const uint4 *>(a.up_in)[p];
-            const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
-            uint32_t o[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const uint16_t lo = f32_to_f16(glu_rt(f16_to_f32(uint16_t(gw[t])), f16_to_f32(uint16_t(uw[t])), a.act));
-                const uint16_t hi = f32_to_f16(glu_rt(f16_to_f32(uint16_t(gw[t] >> 16)), f16_to_f32(uint16_t(uw[t] >> 16)), a.act));
-                o[t] = uint32_t(lo) | (uint32_t(hi) << 16);
-            }
-            act_l[p] = make_uint4(o[0], o[1], o[2], o[3]);
+        uint32_t *act_w = reinterpret_cast<uint32_t *>(act_l);
+        for (uint32_t p = threadIdx.x; p < a.n / 2u; p += 256u) {
+            const uint32_t gw = reinterpret_cast<const uint32_t *>(a.gate_in)[p];
+            const uint32_t uw = reinterpret_cast<const uint32_t *>(a.up_in)[p];
+            const uint16_t lo = f32_to_f16(glu_rt(f16_to_f32(uint16_t(gw)), f16_to_f32(uint16_t(uw)), a.act));
+            const uint16_t hi = f32_to_f16(glu_rt(f16_to_f32(uint16_t(gw >> 16)), f16_to_f32(uint16_t(uw >> 16)), a.act));
+            act_w[p] = uint32_t(lo) | (uint32_t(hi) << 16);
         }
         __syncthreads();
         if (active) load_slice_regs<BITS, NCH>(xin, act_l, cpr, col, true);
@@ -247,14 +250,23 @@ __device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block, XSou
     typename C::X x[NCH];
     float xs[NCH];
     unpack_slices<BITS, NCH>(xin, x, xs);
+    // what the rows' epilogue shares is formed once: the gate's divisor, and the segment's last lane by a mask
+    // (a segment is a power of two lanes)
+    const bool gated = a.scalar_gate != nullptr;
+    const float gate_div = gated ? 1.0f + expf(-f16_to_f32(gate_bits)) : 1.0f;
+    const bool writer_lane = (lane & (seg - 1u)) == seg - 1u;
+    float sums[kGemvRowsPerWave];
+#pragma unroll
+    for (uint32_t j = 0; j < kGemvRowsPerWave; ++j) sums[j] = row_partial<BITS, NCH>(rows[j], x, xs, a.meta);
+#pragma unroll
+    for (uint32_t j = 0; j < kGemvRowsPerWave; ++j) sums[j] = seg_sum(sums[j], seg);  // four independent chains
 #pragma unroll
     for (uint32_t j = 0; j < kGemvRowsPerWave; ++j) {
-        const float v = seg_sum(row_partial<BITS, NCH>(rows[j], x, xs, a.meta), seg);
-        if (on[j] && (lane % seg) == seg - 1u) {
+        if (on[j] && writer_lane) {
             const bool second = row[j] >= a.rows;
-            uint16_t yh = f32_to_f16(v);
-            if (a.scalar_gate) yh = f32_to_f16(f16_to_f32(yh) / (1.0f + expf(-f16_to_f32(gate_bits))));
-            (second ? a.y_b : a.y_a)[second ? row[j] - a.rows : row[j]] = yh;
+            uint16_t yh = f32_to_f16(sums[j]);
+            if (gated) yh = f32_to_f16(f16_to_f32(yh) / gate_div);
+            (second ? y_b : y_a)[second ? row[j] - a.rows : row[j]] = yh;
         }
     }
 }
@@ -295,6 +307,19 @@ struct RouteLists {  // outputs of select + classify; residency == nullptr: sele
 };
 
 __device__ __forceinline__ float sigmoidf_(float v) { return 1.0f / (1.0f + expf(-v)); }
+// The selection score of one expert (moe.metal:436-440) as an unsigned key: a larger score is a larger key, 0 marks
+// what can never be taken (NaN and -inf; the reference's slots start at -inf, index 0).
+__device__ __forceinline__ uint32_t score_key(float raw, float bias, uint32_t sigmoid) {
+    float s = (sigmoid ? sigmoidf_(raw) : raw) + bias;
+    s = s + 0.0f;  // -0 and +0 tie
+    const uint32_t u = __float_as_uint(s);
+    const uint32_t ord = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    return (s == s && s > -INFINITY) ? ord : 0u;
+}
+__device__ __forceinline__ float key_score(uint32_t key) {
+    return key == 0u ? -INFINITY : __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
 template <bool COHERENT>
 __device__ __forceinline__ float load_logit(const float *p) {
     return COHERENT ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *p;
@@ -315,6 +340,10 @@ struct RouteScratch {
     float raw[256];
 };
 
+__device__ __forceinline__ void finish_routes(const SelectArgs &a, const RouteLists &out, uint32_t lane, bool write_lists,
+                                              uint32_t mine, uint32_t my_key, float my_raw, float my_gain,
+                                              uint32_t cell_of_mine, uint32_t &my_cell);
+
 template <bool COHERENT>
 __device__ void route_wave(const SelectArgs &a, const RouteLists &out, uint32_t lane, bool write_lists,
                            uint32_t &my_cell, RouteScratch &lds) {
@@ -333,11 +362,7 @@ __device__ void route_wave(const SelectArgs &a, const RouteLists &out, uint32_t 
         const uint64_t word = out.residency ? out.residency[ee] : 0;
         // moe.metal:136-146: a hit names its cell, anything else is the sentinel
         cellv[j] = (uint32_t(word >> 32) == SHRIKE_RESIDENCY_RESIDENT) ? uint32_t(word) : kSentinel;
-        float s = (a.sigmoid ? sigmoidf_(raw[j]) : raw[j]) + bias;
-        s = s + 0.0f;  // -0 and +0 tie
-        const uint32_t u = __float_as_uint(s);
-        const uint32_t ord = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-        key[j] = (on && s == s && s > -INFINITY) ? ord : 0u;
+        key[j] = on ? score_key(raw[j], bias, a.sigmoid) : 0u;
     }
     const uint32_t K = a.top_k;
     // Every lane parks its four candidates in LDS; after the rounds lane p fetches position
@@ -406,14 +431,22 @@ __device__ void route_wave(const SelectArgs &a, const RouteLists &out, uint32_t 
             if (lane == r) { mine = win; my_key = top; }
         }
     }
-    const float my_score = my_key == 0u ? -INFINITY
-        : __uint_as_float((my_key & 0x80000000u) ? (my_key & 0x7fffffffu) : ~my_key);
-    const bool on = lane < K;
     const float my_gain = bf16_to_f32(uint16_t(s_gain[mine]));
     const uint32_t cell_of_mine = s_cellv[mine];
+    finish_routes(a, out, lane, write_lists, mine, my_key, a.sigmoid ? s_raw[mine] : 0.0f, my_gain, cell_of_mine, my_cell);
+}
+
+// The second half of the select (moe.metal:460-490) and the classification (moe.metal:121-151) for a wave whose lane
+// p < top_k holds position p's expert `mine`, its score key, raw logit, gain and residency-resolved cell.
+__device__ __forceinline__ void finish_routes(const SelectArgs &a, const RouteLists &out, uint32_t lane, bool write_lists,
+                                              uint32_t mine, uint32_t my_key, float my_raw, float my_gain,
+                                              uint32_t cell_of_mine, uint32_t &my_cell) {
+    const uint32_t K = a.top_k;
+    const float my_score = key_score(my_key);
+    const bool on = lane < K;
     float weight;
     if (a.sigmoid) {  // moe.metal:460-474
-        const float orig = on ? sigmoidf_(s_raw[mine]) : 0.0f;
+        const float orig = on ? sigmoidf_(my_raw) : 0.0f;
         float sum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {  // rank order, as the reference adds them
@@ -459,6 +492,98 @@ __device__ void route_wave(const SelectArgs &a, const RouteLists &out, uint32_t 
         out.hit_count[0] = __popcll(hit_mask);
         out.miss_count[0] = __popcll(miss_mask);
     }
+}
+
+// ---- the route table of the fused layer
+//
+// The layer's first launch leaves one 16-byte entry per expert: everything the selection needs, already combined
+// (score key with the bias folded in, the cell the residency word resolves to, the raw logit and the gain). The
+// second launch's waves then select from 4 KB written a moment ago instead of gathering four cold per-layer
+// arrays, and need no arithmetic before the first comparison.
+struct RouteEntry {
+    uint32_t key, cell;
+    float raw;
+    uint32_t gain;  // bf16 bits of per_expert_scale
+};
+
+__device__ __forceinline__ void write_route_entry(RouteEntry *table, uint32_t e, float raw, uint16_t bias_bits,
+                                                  uint16_t gain_bits, uint64_t word, uint32_t sigmoid) {
+    uint4 v;
+    v.x = score_key(raw, bf16_to_f32(bias_bits), sigmoid);
+    // moe.metal:136-146: a hit names its cell, anything else is the sentinel
+    v.y = (uint32_t(word >> 32) == SHRIKE_RESIDENCY_RESIDENT) ? uint32_t(word) : kSentinel;
+    v.z = __float_as_uint(raw);
+    v.w = gain_bits;
+    *reinterpret_cast<uint4 *>(table + e) = v;
+}
+
+// What the select leaves in a wave: lane p < top_k holds position p's expert and its entry.
+struct TableSelect {
+    uint32_t mine, my_key, my_cell, my_gain;
+    float my_raw;
+};
+
+// moe.metal:419-458 over the route table, by one wave, all in registers. Lane l holds experts 4l .. 4l+3 and first
+// sorts its four by key, descending, equals in index order (exchanges of neighbours only, so the sort is stable). A
+// round then looks at the heads alone: the wave's maximum, the ballot of the lanes whose head holds it, the lowest
+// such lane (the lowest index, moe.metal:443-449), whose head's entry is read across by lane index and popped. The
+// full 32-bit key is compared, so the order is exact. Positions that find nothing left take expert 0 with score
+// -inf, as the reference's initial slots do.
+// last_round (uniform): the last position the caller needs; later rounds are skipped.
+__device__ __forceinline__ TableSelect select_from_table(const RouteEntry *table, uint32_t num_experts, uint32_t K,
+                                                         uint32_t lane, uint32_t last_round) {
+    uint32_t key[4], cellv[4], rawv[4], gainv[4], idx[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint4 v = reinterpret_cast<const uint4 *>(table)[lane * 4u + j];
+        idx[j] = lane * 4u + j;
+        key[j] = idx[j] < num_experts ? v.x : 0u;
+        cellv[j] = v.y; rawv[j] = v.z; gainv[j] = v.w;
+    }
+    TableSelect r;
+    // what a position with nothing left to take names: expert 0
+    r.mine = 0; r.my_key = 0;
+    r.my_cell = uint32_t(__builtin_amdgcn_readfirstlane(int(cellv[0])));
+    r.my_gain = uint32_t(__builtin_amdgcn_readfirstlane(int(gainv[0])));
+    r.my_raw = __uint_as_float(uint32_t(__builtin_amdgcn_readfirstlane(int(rawv[0]))));
+    auto exchange = [&](int a, int b) {  // neighbours a < b: the later one moves ahead only when strictly larger
+        const bool swap = key[b] > key[a];
+        uint32_t t;
+        t = key[a]; key[a] = swap ? key[b] : t; key[b] = swap ? t : key[b];
+        t = cellv[a]; cellv[a] = swap ? cellv[b] : t; cellv[b] = swap ? t : cellv[b];
+        t = idx[a]; idx[a] = swap ? idx[b] : t; idx[b] = swap ? t : idx[b];
+        t = rawv[a]; rawv[a] = swap ? rawv[b] : t; rawv[b] = swap ? t : rawv[b];
+        t = gainv[a]; gainv[a] = swap ? gainv[b] : t; gainv[b] = swap ? t : gainv[b];
+    };
+    exchange(0, 1); exchange(2, 3); exchange(1, 2); exchange(0, 1); exchange(2, 3); exchange(1, 2);
+#pragma unroll
+    for (int round = 0; round < 8; ++round) {
+        if (uint32_t(round) < K && uint32_t(round) <= last_round) {
+            const uint32_t top = wave_max_u32(key[0]);
+            if (top != 0u) {  // uniform
+                const int win = __ffsll((long long)__ballot(key[0] == top)) - 1;
+                const uint32_t widx = uint32_t(__builtin_amdgcn_readlane(int(idx[0]), win));
+                const uint32_t wcell = uint32_t(__builtin_amdgcn_readlane(int(cellv[0]), win));
+                const uint32_t wraw = uint32_t(__builtin_amdgcn_readlane(int(rawv[0]), win));
+                const uint32_t wgain = uint32_t(__builtin_amdgcn_readlane(int(gainv[0]), win));
+                const bool me = lane == uint32_t(win);
+#pragma unroll
+                for (int j = 0; j < 3; ++j) {
+                    key[j] = me ? key[j + 1] : key[j];
+                    cellv[j] = me ? cellv[j + 1] : cellv[j];
+                    idx[j] = me ? idx[j + 1] : idx[j];
+                    rawv[j] = me ? rawv[j + 1] : rawv[j];
+                    gainv[j] = me ? gainv[j + 1] : gainv[j];
+                }
+                key[3] = me ? 0u : key[3];
+                if (lane == uint32_t(round)) {
+                    r.mine = widx; r.my_key = top; r.my_cell = wcell; r.my_gain = wgain;
+                    r.my_raw = __uint_as_float(wraw);
+                }
+            }
+        }
+    }
+    return r;
 }
 
 }  // namespace shrike

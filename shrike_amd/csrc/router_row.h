@@ -13,10 +13,10 @@ namespace shrike {
 // hidden, logits: the token's activation row and its logit row (a.hidden, a.logits_out for one token)
 // x_source(): called once the row's own loads are in flight; returns the activation row to read (it may
 // first have to produce it, e.g. a norm into LDS behind a barrier — then every wave of the workgroup
-// must come through here or call it by itself).
+// must come through here or call it by itself). Returns the logit (in every lane).
 template <int RK, class XSource>
-__device__ __forceinline__ void router_row(const RouterArgs &a, XSource &&x_source, float *logits, uint32_t e, uint32_t lane,
-                                           bool publish) {
+__device__ __forceinline__ float router_row(const RouterArgs &a, XSource &&x_source, float *logits, uint32_t e, uint32_t lane,
+                                            bool publish) {
     constexpr int E = RK == 0 ? 8 : RK == 8 ? 16 : 32;  // elements per 16-byte weight chunk
     constexpr int PIECES = E / 8;
     constexpr int MAXI = RK == 0 ? 8 : 4;
@@ -91,17 +91,18 @@ __device__ __forceinline__ void router_row(const RouterArgs &a, XSource &&x_sour
         if (publish) __hip_atomic_store(logits + e, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else logits[e] = acc;
     }
+    return acc;  // every lane holds the sum
 }
 
 template <int RK>
-__device__ __forceinline__ void router_row(const RouterArgs &a, const uint16_t *hidden, float *logits, uint32_t e, uint32_t lane,
-                                           bool publish) {
-    router_row<RK>(a, [&] { return hidden; }, logits, e, lane, publish);
+__device__ __forceinline__ float router_row(const RouterArgs &a, const uint16_t *hidden, float *logits, uint32_t e, uint32_t lane,
+                                            bool publish) {
+    return router_row<RK>(a, [&] { return hidden; }, logits, e, lane, publish);
 }
 
 template <int RK>
-__device__ __forceinline__ void router_row(const RouterArgs &a, uint32_t e, uint32_t lane, bool publish = false) {
-    router_row<RK>(a, a.hidden, a.logits_out, e, lane, publish);
+__device__ __forceinline__ float router_row(const RouterArgs &a, uint32_t e, uint32_t lane, bool publish = false) {
+    return router_row<RK>(a, a.hidden, a.logits_out, e, lane, publish);
 }
 
 }  // namespace shrike

@@ -403,6 +403,9 @@ uint64_t shrike_hip_pool_table_entry(const shrike_hip_pool *pool, uint32_t exper
 
 // --------------------------------------------------------------------- moe
 
+constexpr size_t kLogitsBytes = sizeof(float) * 2u * SHRIKE_MAX_ROUTER_EXPERTS;  // this layer's logits and the paired router's
+constexpr size_t kRouteBytes = 16u * SHRIKE_MAX_ROUTER_EXPERTS;                   // the fused layer's route table
+
 shrike_hip_moe *shrike_hip_moe_create(const shrike_moe_desc *desc, int *out_errno) {
     auto fail = [&](int code) -> shrike_hip_moe * { if (out_errno) *out_errno = code; return nullptr; };
     if (int rc = shrike::check_moe_desc(desc)) return fail(rc);
@@ -410,14 +413,15 @@ shrike_hip_moe *shrike_hip_moe_create(const shrike_moe_desc *desc, int *out_errn
     moe->desc = *desc;
     moe->d_logits = nullptr; moe->d_counter = nullptr;
     if (hipGetDevice(&moe->device) != hipSuccess
-        || hipMalloc(reinterpret_cast<void **>(&moe->d_logits), sizeof(float) * 2u * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess
+        || hipMalloc(reinterpret_cast<void **>(&moe->d_logits), kLogitsBytes + kRouteBytes) != hipSuccess
         || hipMalloc(reinterpret_cast<void **>(&moe->d_counter), sizeof(uint32_t) * kCounterWords) != hipSuccess
         || hipMemset(moe->d_counter, 0, sizeof(uint32_t) * kCounterWords) != hipSuccess
-        || hipMemset(moe->d_logits, 0, sizeof(float) * 2u * SHRIKE_MAX_ROUTER_EXPERTS) != hipSuccess) {
+        || hipMemset(moe->d_logits, 0, kLogitsBytes + kRouteBytes) != hipSuccess) {
         set_error("device allocation for the MoE handle failed: %s", hipGetErrorString(hipGetLastError()));
         shrike_hip_moe_destroy(moe);
         return fail(ENOMEM);
     }
+    moe->d_route = reinterpret_cast<shrike::RouteEntry *>(reinterpret_cast<unsigned char *>(moe->d_logits) + kLogitsBytes);
     if (out_errno) *out_errno = 0;
     return moe;
 }
