@@ -47,13 +47,16 @@ __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
 // Sum over aligned lane segments of `seg` lanes (seg in {1,2,4,8,16,32,64}); every
 // lane of a segment's last 16-lane row ends up holding the segment sum, and for
 // seg <= 16 every lane of the segment does. Callers read lane (segment end - 1).
+// A step that does not apply keeps v by a select, not by a branch: with a segment length known only at run time the
+// six steps stay one straight run of instructions (a taken scalar branch a step costs more than the step).
 __device__ __forceinline__ float seg_sum(float v, uint32_t seg) {
-    if (seg >= 2) v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
-    if (seg >= 4) v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
-    if (seg >= 8) v += dpp_f32<0x141>(v);  // row_half_mirror
-    if (seg >= 16) v += dpp_f32<0x140>(v); // row_mirror
-    if (seg >= 32) v += dpp_f32<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
-    if (seg >= 64) v += dpp_f32<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+    float t;
+    t = v + dpp_f32<0xB1>(v); v = seg >= 2 ? t : v;          // quad_perm [1,0,3,2]
+    t = v + dpp_f32<0x4E>(v); v = seg >= 4 ? t : v;          // quad_perm [2,3,0,1]
+    t = v + dpp_f32<0x141>(v); v = seg >= 8 ? t : v;         // row_half_mirror
+    t = v + dpp_f32<0x140>(v); v = seg >= 16 ? t : v;        // row_mirror
+    t = v + dpp_f32<0x142, 0xA>(v); v = seg >= 32 ? t : v;   // row_bcast15 into rows 1 and 3
+    t = v + dpp_f32<0x143, 0xC>(v); v = seg >= 64 ? t : v;   // row_bcast31 into rows 2 and 3
     return v;
 }
 __device__ __forceinline__ float wave_sum(float v) {
