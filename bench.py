@@ -5,21 +5,32 @@ A step is one MoE-layer decode for one token at the 35B-A3B int4 shape (hidden 2
 256 routed experts of intermediate 512, top-8, one shared expert of intermediate 512,
 fp16 router, group-64 affine int4 with 16-bit scale/bias): router -> top-k -> slot
 resolve -> shared expert -> gate/up matvec + SiLU-multiply -> down matvec + weighted
-combine. Consecutive steps walk a stack of layers whose expert pools sit at distinct
-addresses and together exceed the 256 MB Infinity Cache, so every step streams its
-experts from HBM. The stack is captured once in a HIP graph and replayed.
+combine. Consecutive steps walk a stack of 40 layers whose expert pools sit at distinct
+addresses (18 GB, far past the 256 MB Infinity Cache), and the activation vector rotates
+over four variants so that a layer picks other experts from one pass to the next: every
+step streams its experts from HBM. Runs of layers are captured in HIP graphs.
+
+Timing: W warm-up steps, then REGIONS regions of exactly K steps each, every region
+bracketed by HIP events on the launch stream; `ms_per_step` is the median region / K
+(minimum and maximum are reported beside it).
 
 Prints ONE JSON line. `value` is expert bytes read per second (8 routed + 1 shared
-expert = 15,925,248 B per step) with all inputs resident in HBM; `ms_per_step` carries
-the per-layer time. `roofline` prices the dominant kernel (phase 1) against 8 TB/s;
-`cpu_baseline` times the CPU oracle's fp32 port of the same layer on this host.
+expert = 15,925,248 B per step) with all inputs resident in HBM. `roofline` prices the
+dominant kernel of the timed layer (its second launch) against 8 TB/s; `cpu_baseline`
+times the CPU oracle's fp32 port on this host (the layer on several cores, and one
+expert on one core); `secondary` carries the other workloads of the benchmark
+definition (ragged prefill chunk, gpt-oss-shape batch, Kimi-shape batch through a
+64-of-256 pool), each measured by the same run.
 """
 from __future__ import annotations
 
 import argparse
 import ctypes as C
+import gc
 import json
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -31,13 +42,22 @@ if ROOT not in sys.path:
 
 D, F, NE, K, FS, BITS = 2048, 512, 256, 8, 512, 4
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes of one routed gate/up launch read from the FETCH_SIZE and WRITE_SIZE counters (two
-# rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for the 453 MB
-# pool copies): 9,589,555 fetched + 8,192 written. profiles/decode_phase1_q35b_int4_hbm_traffic.txt
-PHASE1_TRAFFIC_BYTES = 9_597_747
-# The two grouped-FFN kernels of config 3's chunk, same method (profiles/prefill_chunk_q35b_int4_t512.txt):
-# gate/up 57,207.5 and down 25,509.4 FETCH_SIZE units (x2.0 KiB) fetched, 4,096 + 16,384 KiB written.
-PREFILL_FFN_TRAFFIC_BYTES = int(((57207.5 + 25509.4) * 2.0 + 4096 + 16384) * 1024)
+REGIONS = 15          # timed regions; the median is reported
+X_VARIANTS = 4        # activation vectors in rotation
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def profile_figure(filename: str, key: str):
+    """A figure from a tracked rocprofv3 summary: the first line `key: <number>`; None when absent."""
+    try:
+        with open(os.path.join(PROFILES, filename)) as fh:
+            for line in fh:
+                m = re.match(r"\s*" + re.escape(key) + r"\s*:\s*([0-9][0-9_,.]*)", line)
+                if m:
+                    return int(float(m.group(1).replace(",", "").replace("_", "")))
+    except OSError:
+        pass
+    return None
 
 
 def build_layers(rt, capi, S, n_layers, meta, shared=True):
@@ -58,7 +78,7 @@ def build_layers(rt, capi, S, n_layers, meta, shared=True):
     # (sources/Shrike/Runtime/Inference/RealForwardRunner.swift:754-825)
     scratch = {name: rt.empty(size) for name, size in dict(idx=32, w=16, res=32, hc=4, hp=32, mc=4, mp=32, me=32,
                                                            acts=2 * K * F, ss=4 * FS, h1=2 * D, y=2 * D).items()}
-    x = rt.dev(S.activations_f16(tree, "layer.x", D))
+    xs = [rt.dev(S.activations_f16(tree, "layer.x" if v == 0 else f"layer.x.{v}", D)) for v in range(X_VARIANTS)]
     for l in range(n_layers):
         pool = rt.ExpertPool(NE, stride, NE)
         if l == 0:
@@ -69,7 +89,7 @@ def build_layers(rt, capi, S, n_layers, meta, shared=True):
             capi.check(capi.load().shrike_hip_memcpy_d2d(pool.cell_ptr(0), first_pool.cell_ptr(0), NE * pool.stride), "d2d")
         for e in range(NE):
             pool.publish(e, e, capi.RESIDENT)
-        lay = dict(pool=pool, x=x, **scratch)
+        lay = dict(pool=pool, x=xs[0], xs=xs, **scratch)
         lay["router"] = rt.dev(S.router_f16(tree, f"layer.{l}.router.w", NE, D))
         lay["shared"] = {n: tuple(rt.dev(t) for t in S.affine_matrix(tree.key(f"layer.{l}.shared.{n}"), r, c, BITS, meta))
                          for n, r, c in (("gate", FS, D), ("up", FS, D), ("down", D, FS))}
@@ -86,6 +106,12 @@ def build_layers(rt, capi, S, n_layers, meta, shared=True):
         a.miss_positions, a.miss_experts = lay["mp"].ptr, lay["me"].ptr
         a.acts, a.shared_scratch, a.h1 = lay["acts"].ptr, lay["ss"].ptr, lay["h1"].ptr
         lay["args"] = a
+        lay["args_x"] = [a]
+        for v in range(1, X_VARIANTS):  # the same layer over another activation vector
+            b = capi.DecodeLayerArgs()
+            C.memmove(C.byref(b), C.byref(a), C.sizeof(b))
+            b.x = xs[v].ptr
+            lay["args_x"].append(b)
         layers.append(lay)
     rt.synchronize()
     keep = (ones_d, ones_e, zeros_e, hidden, blobs)
@@ -114,9 +140,65 @@ def time_graph(rt, capi, stream, graph, launches):
     return start.elapsed_ms(stop)
 
 
+def median_of_regions(rt, capi, stream, graph, launches, regions=REGIONS):
+    """ms per launch of `graph`: the median over `regions` event-bracketed regions of `launches` launches each."""
+    events = [rt.Event() for _ in range(regions + 1)]
+    stream.synchronize()
+    events[0].record(stream)
+    for r in range(regions):
+        for _ in range(launches):
+            capi.check(capi.load().shrike_hip_graph_launch(graph, stream.handle), "graph_launch")
+        events[r + 1].record(stream)
+    events[-1].synchronize()
+    return statistics.median(events[r].elapsed_ms(events[r + 1]) for r in range(regions)) / launches
+
+
+class LayerWalk:
+    """Exactly-K-step regions over the layer stack: a region is a run of graph launches that covers K consecutive
+    layers (wrapping round the stack), each launch over the next activation variant. Graphs are captured once per
+    (variant, first layer, layer count)."""
+
+    def __init__(self, rt, capi, moe, stream, layers):
+        self.rt, self.capi, self.moe, self.stream, self.layers = rt, capi, moe, stream, layers
+        self.graphs = {}
+        self.at, self.variant = 0, 0
+
+    def graph(self, variant, first, count):
+        key = (variant, first, count)
+        if key not in self.graphs:
+            def body():
+                for lay in self.layers[first:first + count]:
+                    self.moe.encode_decode_layer(lay["args_x"][variant])
+            self.graphs[key] = capture(self.rt, self.capi, self.stream, body)
+        return self.graphs[key]
+
+    def enqueue(self, steps):
+        """Enqueues exactly `steps` layers, continuing where the last call stopped."""
+        n = len(self.layers)
+        while steps > 0:
+            count = min(steps, n - self.at)
+            g = self.graph(self.variant, self.at, count)
+            self.capi.check(self.capi.load().shrike_hip_graph_launch(g, self.stream.handle), "graph_launch")
+            self.at = (self.at + count) % n
+            self.variant = (self.variant + 1) % X_VARIANTS
+            steps -= count
+
+    def plan(self, steps, regions):
+        """Captures what `regions` regions of `steps` steps will launch, so that no capture falls into a timed region."""
+        at, variant = self.at, self.variant
+        n = len(self.layers)
+        for _ in range(regions):
+            left = steps
+            while left > 0:
+                count = min(left, n - at)
+                self.graph(variant, at, count)
+                at, variant, left = (at + count) % n, (variant + 1) % X_VARIANTS, left - count
+
+
 def cpu_baseline(S, blobs, sample_layers, meta):
     """The oracle's fp32 port of the layer (one task per expert, as
-    sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:10-14 describes) on this host's cores."""
+    sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:10-14 describes) on this host's cores, and config 1 of the
+    benchmark definition: one routed expert for one token on one core."""
     from oracle import oracle as O
     off, _ = O.expert_offsets(D, F, BITS)
     cores = min(K + 1, len(os.sched_getaffinity(0)))
@@ -128,17 +210,28 @@ def cpu_baseline(S, blobs, sample_layers, meta):
     for i in range(sample_layers):
         picks = rng.choice(NE, K + 1, replace=False)
         O.cpu_layer_fp32([blobs[int(e)] for e in picks], weights, off, x, D, F, cores, bits=BITS, meta=meta)
-    dt = time.perf_counter() - t0
-    per_layer = dt / sample_layers
+    per_layer = (time.perf_counter() - t0) / sample_layers
     expert_bytes = (K + 1) * 1_769_472
+    # config 1: one expert, one token, one core (sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:102-140)
+    singles = max(8, sample_layers // 2)
+    out = np.zeros(D, np.float32)
+    picks = rng.choice(NE, singles, replace=True)
+    t0 = time.perf_counter()
+    for e in picks:
+        O.cpu_expert_ffn_accumulate(blobs[int(e)], off, x, D, F, 0.125, out, bits=BITS, meta=meta)
+    per_expert = (time.perf_counter() - t0) / singles
     return {"value": round(expert_bytes / per_layer / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
             "us_per_layer": round(per_layer * 1e6, 1),
             "sample": f"{sample_layers} layer evaluations of 9 experts (8 routed + 1 shared-sized) drawn from the "
                       f"256-expert pool, fp32 scalar C port of shrike_int4_affine_gemv + CPUExpertFFN.accumulate, "
-                      f"{cores} threads, gcc -O2"}
+                      f"{cores} threads, gcc -O2",
+            "config1": {"workload": "config 1: one routed expert SwiGLU FFN for one token (hidden 2048, intermediate 512, int4)",
+                        "cores": 1, "us_per_expert": round(per_expert * 1e6, 1),
+                        "value": round(1_769_472 / per_expert / 1e9, 3), "unit": "GB/s", "bytes_per_expert": 1_769_472,
+                        "sample": f"{singles} experts drawn from the pool, one thread"}}
 
 
-def prefill_main(args, rt, capi, S, meta):
+def prefill_workload(args, rt, capi, S, meta):
     """Config 3: one ragged prefill chunk of T tokens through router -> grouping -> grouped expert FFN
     -> reduce, top-8 of 256 int4 experts with a Zipf skew injected through the router's logit-bias
     operand. Steps alternate between layers with their own pools so the experts stream from HBM."""
@@ -176,20 +269,23 @@ def prefill_main(args, rt, capi, S, meta):
     def step(lay):
         router(lay); group(lay); ffn(lay); reduce(lay)
 
-    def timed(fn, n):
-        start, stop = rt.Event(), rt.Event()
+    def timed(fn, n, regions=1):
+        times = []
         stream.synchronize()
-        start.record(stream)
-        for i in range(n):
-            fn(layers[i % n_layers])
-        stop.record(stream)
-        stop.synchronize()
-        return start.elapsed_ms(stop) / n
+        for _ in range(regions):
+            start, stop = rt.Event(), rt.Event()
+            start.record(stream)
+            for i in range(n):
+                fn(layers[i % n_layers])
+            stop.record(stream)
+            stop.synchronize()
+            times.append(start.elapsed_ms(stop) / n)
+        return statistics.median(times)
 
-    steps, warm = max(1, args.steps // 40), max(1, args.warmup // 40)
+    steps, warm = max(6, args.steps // 40), max(3, args.warmup // 40)
     timed(step, warm)
-    ms = timed(step, steps)
-    parts = {name: timed(fn, max(4, steps // 2)) * 1e3 for name, fn in
+    ms = timed(step, steps, regions=5)
+    parts = {name: timed(fn, max(6, steps // 2), regions=3) * 1e3 for name, fn in
              (("router (2 launches)", router), ("grouping (1 launch)", group), ("grouped FFN (4 launches)", ffn), ("reduce", reduce))}
     rt.synchronize()
     counts = routes.counts.download(np.uint32, NE)
@@ -200,7 +296,8 @@ def prefill_main(args, rt, capi, S, meta):
     algorithmic = expert_bytes + 2 * T * D * 2 + T * K * 16
     flops = T * K * 6 * D * F
     ffn_us = parts["grouped FFN (4 launches)"]
-    out = {
+    traffic = profile_figure("prefill_chunk_q35b_int4_t512.txt", "hbm_bytes_per_chunk_grouped_ffn") if T == 512 else None
+    return {
         "metric": "ragged prefill chunk through the routed experts: tokens/s (ms per chunk in ms_per_step), 35B-A3B int4 shape",
         "value": round(T / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 x u4 -> f32",
@@ -213,19 +310,18 @@ def prefill_main(args, rt, capi, S, meta):
         "roofline": {"bound": "hbm", "kernel": "k_grouped_ffn<4,0> + k_grouped_ffn<4,1> (gate/up + down of every row tile)",
                      "achieved": round(expert_bytes / (ffn_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(expert_bytes / (ffn_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "bytes_per_launch": expert_bytes,
-                     "us_per_launch": round(ffn_us, 2), "traffic": PREFILL_FFN_TRAFFIC_BYTES if T == 512 else None,
+                     "us_per_launch": round(ffn_us, 2), "traffic": traffic,
                      "mfma_tflops_on_pair_flops": round(flops / (ffn_us * 1e-6) / 1e12, 2)},
         "algorithmic_bytes_per_chunk": algorithmic, "pair_flops_per_chunk": flops,
     }
-    print(json.dumps(out))
 
 
-def gptoss_main(args, rt, capi, S, meta):
+def gptoss_workload(args, rt, capi, S, meta, bits):
     """Config 4: a batch of 4 independent tokens through 24 stacked gpt-oss-20B-shape layers (hidden 2880,
-    32 experts of intermediate 2880, top-4, int4 or int8 codes): router -> grouping -> grouped FFN -> reduce
-    per layer, every layer with its own pool."""
+    32 experts of intermediate 2880, top-4, int4 or int8 codes): router -> resolve -> phase 1 -> phase 2 with the
+    token dimension on the grid, every layer with its own pool."""
     d = f = 2880
-    ne, k, t, bits, n_layers = 32, 4, 4, args.bits, min(args.layers, 24)
+    ne, k, t, n_layers = 32, 4, 4, min(args.layers, 24)
     tree = S.SeedTree(0x5EED0004)
     off, stride = rt.expert_offsets(d, f, bits)
     blobs = [S.expert_blob(tree, f"layer.0.expert.{e}", d, f, bits, meta) for e in range(ne)]
@@ -241,6 +337,7 @@ def gptoss_main(args, rt, capi, S, meta):
             pool.publish(e, e, capi.RESIDENT)
         pools.append(pool)
         routers.append(rt.dev(S.router_f16(tree, f"layer.{l}.router.w", ne, d)))
+    del blobs
     moe = rt.MoE(d, f, ne, k, routed_bits=bits, router_bits=0, meta=meta)
     stream = rt.Stream()
     moe.stream = stream
@@ -270,11 +367,10 @@ def gptoss_main(args, rt, capi, S, meta):
 
     all_layers()
     stream.synchronize()
-    used = sum(len(set(idx.download(np.uint32, t * k).tolist())) for _ in range(1))  # last layer's distinct experts
     graph = capture(rt, capi, stream, all_layers)
     reps = max(2, args.steps // 200)
     time_graph(rt, capi, stream, graph, max(1, args.warmup // 200))
-    ms = time_graph(rt, capi, stream, graph, reps) / reps
+    ms = median_of_regions(rt, capi, stream, graph, reps, regions=7)
     # distinct experts differ per layer (own router); count them from one eager pass per layer
     distinct = []
     for l in range(n_layers):
@@ -282,7 +378,8 @@ def gptoss_main(args, rt, capi, S, meta):
         stream.synchronize()
         distinct.append(len(set(idx.download(np.uint32, t * k).tolist())))
     expert_bytes = sum(distinct) * stride
-    print(json.dumps({
+    capi.check(capi.load().shrike_hip_graph_destroy(graph), "graph_destroy")
+    return {
         "metric": "gpt-oss-20B-shape MoE layers, 4 tokens: us per layer (ms per 24-layer stack in ms_per_step)",
         "value": round(expert_bytes / (ms * 1e-3) / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": reps, "warmup": max(1, args.warmup // 200),
         "ms_per_step": round(ms, 5), "us_per_layer": round(ms * 1e3 / n_layers, 2), "higher_is_better": True, "scaling": "weak",
@@ -292,10 +389,10 @@ def gptoss_main(args, rt, capi, S, meta):
                    "distinct_experts_per_layer": distinct, "expert_bytes_per_stack": expert_bytes,
                    "pair_bytes_per_stack": n_layers * t * k * stride, "meta_dtype": args.meta},
         "GBps_on_pair_bytes": round(n_layers * t * k * stride / (ms * 1e-3) / 1e9, 2),
-        "hbm_peak_frac_on_expert_bytes": round(expert_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}))
+        "hbm_peak_frac_on_expert_bytes": round(expert_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
 
 
-def kimi_main(args, rt, capi, S, meta):
+def kimi_workload(args, rt, capi, S, meta):
     """Config 5: 16 sequences, one token each, Kimi-Linear-48B shape (hidden 2304, 256 int8 experts of
     intermediate 1024, top-8, shared expert 1024); the pool holds 64 of the 256 experts and misses are copied
     from pinned host memory on a side stream. Reports the miss rate, the wall time per step and the host->device rate."""
@@ -338,7 +435,7 @@ def kimi_main(args, rt, capi, S, meta):
     dt = time.perf_counter() - t0
     st = cache.statistics(stride)
     req, miss, read, plans = st.requested_experts - base[0], st.misses - base[1], st.bytes_read - base[2], st.plans - base[3]
-    print(json.dumps({
+    return {
         "metric": "Kimi-Linear-48B-shape MoE decode, 16 sequences through a 64-of-256 slot pool: ms per step (wall clock, misses included)",
         "value": round(t / (dt / steps), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
         "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -347,22 +444,193 @@ def kimi_main(args, rt, capi, S, meta):
                                f"pool of {slots} cells, misses from pinned host memory on a side stream",
                    "passes_per_step": round(plans / steps, 2)},
         "miss_rate": round(miss / max(1, req), 4), "experts_requested_per_step": round(req / steps, 1),
-        "host_to_device_GBps": round(read / dt / 1e9, 2), "bytes_copied_per_step": int(read / steps)}))
+        "host_to_device_GBps": round(read / dt / 1e9, 2), "bytes_copied_per_step": int(read / steps)}
+
+
+def decode_workload(args, rt, capi, S, meta):
+    from shrike_amd import probes
+    n_layers = args.layers
+    layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta, shared=not args.no_shared)
+    moe = rt.MoE(D, F, NE, K, routed_bits=BITS, router_bits=0, meta=meta)
+    stream = rt.Stream()
+    moe.stream = stream
+
+    def all_layers():
+        for lay in layers:
+            moe.encode_decode_layer(lay["args"])
+
+    all_layers()  # eager pass: fills every layer's routing scratch
+    stream.synchronize()
+
+    # ---- the headline: exactly K steps a region, REGIONS regions, median
+    steps, warm = max(1, args.steps), max(0, args.warmup)
+    walk = LayerWalk(rt, capi, moe, stream, layers)
+    walk.plan(warm, 1)
+    walk.enqueue(warm)
+    walk.plan(steps, REGIONS)
+    events = [rt.Event() for _ in range(REGIONS + 1)]
+    stream.synchronize()
+    rt.synchronize()
+    events[0].record(stream)
+    for r in range(REGIONS):
+        walk.enqueue(steps)
+        events[r + 1].record(stream)
+    events[-1].synchronize()
+    rt.synchronize()
+    region_ms = [events[r].elapsed_ms(events[r + 1]) for r in range(REGIONS)]
+    ms_per_step = statistics.median(region_ms) / steps
+    # the experts a pass over the stack touches, per activation variant (routes differ from variant to variant)
+    distinct = set()
+    for v in range(X_VARIANTS):
+        for l, lay in enumerate(layers):
+            moe.encode_decode_layer_launches(lay["args_x"][v], 3)
+            stream.synchronize()
+            distinct.update((l, int(e)) for e in lay["idx"].download(np.uint32, K))
+
+    # ---- the layer's launches one at a time (each in a graph of its own over the whole stack), the split operators
+    # and the two floors, for the per-kernel figures
+    def launches(mask):
+        def body():
+            for lay in layers:
+                moe.encode_decode_layer_launches(lay["args"], mask)
+        return body
+
+    def phase1_only():
+        for lay in layers:
+            moe.encode_spec_phase1(lay["pool"], lay["res"], off, lay["x"], lay["acts"], D, F, K)
+
+    def phase2_only():
+        for lay in layers:
+            moe.encode_spec_phase2(lay["pool"], lay["res"], off, lay["acts"], lay["w"], lay["h1"], lay["y"], None, D, F, K)
+
+    def router_only():
+        for lay in layers:
+            a = lay["args"]
+            moe.encode_router(a.router_weights, None, None, a.x, a.effective_scale, a.per_expert_scale, a.logit_bias,
+                              a.out_indices, a.out_weights, NE, D, K)
+
+    def shared_only():
+        for lay in layers:
+            sh = lay["shared"]
+            moe.encode_shared_expert(sh["gate"], sh["up"], sh["down"], BITS, lay["x"], lay["ss"], lay["h1"], D, FS)
+
+    # the floors a launch is bounded by on this part: a launch with nothing to do, and a kernel that only
+    # reads the bytes phase 1 reads (gate + up sub-tensors of the same eight cells) with no arithmetic
+    sink = rt.empty(4)
+    p1_blocks = K * F // 4 // 4
+    p1_bytes_per_cell = 2 * (F * D // 2 + 2 * F * (D // 64) * 2)
+
+    def empty_only():
+        for lay in layers:
+            probes.check(probes.load().shrike_probe_empty_launch(stream.handle, p1_blocks, sink.ptr), "probe_empty_launch")
+
+    def read_only():
+        for lay in layers:
+            probes.check(probes.load().shrike_probe_read(stream.handle, lay["pool"].bases, lay["pool"].stride, lay["res"].ptr,
+                                                         K, off.gate_w_off, p1_bytes_per_cell, sink.ptr), "probe_read")
+
+    # the step ahead of the layer (residual add + RMS norm producing x): as a launch of its own, and in the
+    # prologue of the layer's first launch; both on a residual stream and an x buffer of their own
+    tree_n = S.SeedTree(0x5EED0003)
+    hidden_n, x_n = rt.dev(S.activations_f16(tree_n, "hidden", D)), rt.empty(2 * D)
+    delta_n = rt.dev(S.f32_to_f16_bits(tree_n.key("delta").normal(D, std=0.05)))
+    weight_n = rt.dev(S.f32_to_bf16_bits(tree_n.key("weight").uniform(0.5, 1.5, D)))
+    normed_args = []
+    for lay in layers:
+        apart_a, fused_a = capi.DecodeLayerArgs(), capi.DecodeLayerArgs()
+        for dst in (apart_a, fused_a):
+            C.memmove(C.byref(dst), C.byref(lay["args"]), C.sizeof(dst))
+            dst.x, dst.hidden = x_n.ptr, hidden_n.ptr
+        fused_a.norm_delta, fused_a.norm_weight, fused_a.norm_eps = delta_n.ptr, weight_n.ptr, 1e-6
+        normed_args.append((apart_a, fused_a))
+
+    def norm_apart():
+        for apart_a, _ in normed_args:
+            rt.residual_add_rmsnorm_bf16w(hidden_n, delta_n, weight_n, x_n, D, 1e-6, 1, stream=stream)
+            moe.encode_decode_layer(apart_a)
+
+    def norm_fused():
+        for _, fused_a in normed_args:
+            moe.encode_decode_layer(fused_a)
+
+    reps = max(2, min(10, steps // n_layers))
+    parts = {}
+    for name, body in (("launch 1: router rows + route entries + shared gate/up rows (k_head)", launches(1)),
+                       ("launch 2: select + routed gate/up rows + shared down rows (k_phase1, routing)", launches(2)),
+                       ("launch 3: routed down rows + combine (k_phase2)", launches(4)),
+                       ("operator: phase 1 alone (no routing, no shared rows)", phase1_only),
+                       ("operator: phase 2 alone", phase2_only),
+                       ("operator: router + select + classify", router_only),
+                       ("operator: shared expert (2 launches)", shared_only),
+                       ("floor: empty launch of phase 1's grid", empty_only),
+                       ("floor: read-only kernel over phase 1's routed bytes", read_only),
+                       ("norm launch + layer (4 launches)", norm_apart),
+                       ("layer with the norm in its first launch", norm_fused)):
+        g = capture(rt, capi, stream, body)
+        time_graph(rt, capi, stream, g, 2)
+        parts[name] = median_of_regions(rt, capi, stream, g, reps, regions=7) / n_layers * 1e3  # us per layer
+        capi.check(capi.load().shrike_hip_graph_destroy(g), "graph_destroy")
+
+    expert_bytes = (K + 1) * stride  # 15,925,248
+    total_bytes = expert_bytes + NE * D * 2 + 2 * D * 2
+    routed_gate_up = K * 2 * (F * D // 2 + 2 * F * (D // 64) * 2)      # gate+up codes, scales and biases of 8 experts
+    shared_down = D * FS // 2 + 2 * D * (FS // 64) * 2                  # the shared expert's down rows ride in launch 2
+    launch2_bytes = routed_gate_up + (0 if args.no_shared else shared_down)
+    launch2_us = parts["launch 2: select + routed gate/up rows + shared down rows (k_phase1, routing)"]
+    alone_us = parts["operator: phase 1 alone (no routing, no shared rows)"]
+    value = expert_bytes / (ms_per_step * 1e-3) / 1e9
+    kernel = "k_phase1<4,1,4,true,4>"
+    out = {
+        "metric": "MoE-layer decode: HBM GB/s on expert bytes (us per layer in ms_per_step), 35B-A3B int4 shape",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": round(ms_per_step, 6), "us_per_layer": round(ms_per_step * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (seeded SplitMix64: uniform int4 codes, |N(0,0.02)| scales, N(0,1) fp16 activations)",
+        "config": {"workload": "config 2: full MoE layer decode, 1 token, hidden 2048, top-8 of 256 int4 experts "
+                               "(intermediate 512, group 64) + 1 shared expert, fp16 router, all slots resident",
+                   "stacked_layers": n_layers, "pool_bytes_total": n_layers * NE * stride,
+                   "activation_variants": X_VARIANTS,
+                   "expert_bytes_touched_by_a_pass_over_every_variant": len(distinct) * stride,
+                   "meta_dtype": args.meta, "launches_per_layer": 3, "hip_graph": True},
+        "timing": {"regions": REGIONS, "steps_per_region": steps, "statistic": "median",
+                   "us_per_layer_min": round(min(region_ms) / steps * 1e3, 3),
+                   "us_per_layer_max": round(max(region_ms) / steps * 1e3, 3)},
+        "hbm_peak_frac_on_expert_bytes": round(value / HBM_PEAK_GBPS, 4),
+        "expert_bytes_per_step": expert_bytes, "total_bytes_per_step": total_bytes,
+        "kernel_us_per_layer": {k: round(v, 3) for k, v in parts.items()},
+        "roofline": {"bound": "hbm", "kernel": kernel + " (the layer's second launch: every wave selects from the route entries, "
+                                               "routed gate/up matvec + SiLU-multiply, shared expert's down rows)",
+                     "achieved": round(launch2_bytes / (launch2_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(launch2_bytes / (launch2_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "bytes_per_launch": launch2_bytes, "us_per_launch": round(launch2_us, 3),
+                     "traffic": profile_figure("decode_phase1_q35b_int4_hbm_traffic.txt", "hbm_bytes_per_launch"),
+                     "standalone_operator": {"kernel": "k_phase1<4,1,4,false,0> (gate/up rows alone)", "bytes_per_launch": routed_gate_up,
+                                             "us_per_launch": round(alone_us, 3),
+                                             "frac": round(routed_gate_up / (alone_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
+                     "floors_us": {"empty_launch": round(parts["floor: empty launch of phase 1's grid"], 3),
+                                   "read_only_same_bytes": round(parts["floor: read-only kernel over phase 1's routed bytes"], 3)}},
+        "setup_seconds": round(gen_s, 1),
+    }
+    if args.cpu_sample > 0:
+        out["cpu_baseline"] = cpu_baseline(S, keep[4], args.cpu_sample, meta)
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
-    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--steps", type=int, default=400, help="layer decodes per timed region (the run times 15 regions)")
+    ap.add_argument("--warmup", type=int, default=80)
     ap.add_argument("--layers", type=int, default=40, help="stacked layers with their own pools (40 x 453 MB)")
     ap.add_argument("--meta", choices=["f16", "bf16"], default="f16")
     ap.add_argument("--cpu-sample", type=int, default=60, help="layer evaluations timed on the CPU (0 = skip)")
     ap.add_argument("--no-shared", action="store_true", help="diagnostic: leave the shared expert out of the layer")
+    ap.add_argument("--no-secondary", action="store_true", help="the headline workload alone")
     ap.add_argument("--workload", choices=["decode", "prefill", "gptoss", "kimi"], default="decode",
-                    help="decode: the headline metric (config 2); prefill: the ragged 512-token chunk (config 3); "
-                         "gptoss: 4 tokens through 24 gpt-oss-shape layers (config 4); kimi: 16 sequences through a "
-                         "64-cell pool fed from pinned host memory (config 5)")
+                    help="decode: the headline metric (config 2) with the other workloads in its `secondary` block; "
+                         "prefill: the ragged 512-token chunk (config 3) alone; gptoss: 4 tokens through 24 gpt-oss-shape "
+                         "layers (config 4) alone; kimi: 16 sequences through a 64-cell pool fed from pinned host memory "
+                         "(config 5) alone")
     ap.add_argument("--bits", type=int, choices=[4, 8], default=4, help="gptoss: code width")
     ap.add_argument("--tokens", type=int, default=512, help="prefill: tokens in the chunk")
     args = ap.parse_args()
@@ -377,143 +645,28 @@ def main():
     rt.init(0)
     meta = S.META_F16 if args.meta == "f16" else S.META_BF16
     if args.workload == "prefill":
-        return prefill_main(args, rt, capi, S, meta)
+        return print(json.dumps(prefill_workload(args, rt, capi, S, meta)))
     if args.workload == "gptoss":
-        return gptoss_main(args, rt, capi, S, meta)
+        return print(json.dumps(gptoss_workload(args, rt, capi, S, meta, args.bits)))
     if args.workload == "kimi":
-        return kimi_main(args, rt, capi, S, meta)
-    n_layers = args.layers
-    layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta, shared=not args.no_shared)
-    moe = rt.MoE(D, F, NE, K, routed_bits=BITS, router_bits=0, meta=meta)
-    stream = rt.Stream()
-    moe.stream = stream
-
-    def all_layers():
-        for lay in layers:
-            moe.encode_decode_layer(lay["args"])
-
-    all_layers()  # eager pass: fills every layer's routing scratch
-    stream.synchronize()
-    g_layer = capture(rt, capi, stream, all_layers)
-
-    def phase1_only():
-        for lay in layers:
-            moe.encode_spec_phase1(lay["pool"], lay["res"], off, lay["x"], lay["acts"], D, F, K)
-
-    def phase2_only():
-        for lay in layers:
-            moe.encode_spec_phase2(lay["pool"], lay["res"], off, lay["acts"], lay["w"], lay["h1"], lay["y"], None, D, F, K)
-
-    def router_only():
-        a0 = layers[0]["args"]
-        for lay in layers:
-            a = lay["args"]
-            moe.encode_router(a.router_weights, None, None, a.x, a.effective_scale, a.per_expert_scale, a.logit_bias,
-                              a.out_indices, a.out_weights, NE, D, K)
-
-    def shared_only():
-        for lay in layers:
-            sh = lay["shared"]
-            moe.encode_shared_expert(sh["gate"], sh["up"], sh["down"], BITS, lay["x"], lay["ss"], lay["h1"], D, FS)
-
-    def phase12():
-        for lay in layers:
-            moe.encode_spec_phase1(lay["pool"], lay["res"], off, lay["x"], lay["acts"], D, F, K)
-            moe.encode_spec_phase2(lay["pool"], lay["res"], off, lay["acts"], lay["w"], lay["h1"], lay["y"], None, D, F, K)
-
-    # the floors phase 1 is bounded by on this part: a launch with nothing to do, and a kernel that only
-    # reads the bytes phase 1 reads (gate + up sub-tensors of the same eight cells) with no arithmetic
-    sink = rt.empty(4)
-    p1_blocks = K * F // 4 // 4
-    p1_bytes_per_cell = 2 * (F * D // 2 + 2 * F * (D // 64) * 2)
-
-    def empty_only():
-        for lay in layers:
-            capi.check(capi.load().shrike_hip_probe_empty_launch(stream.handle, p1_blocks, sink.ptr), "probe_empty_launch")
-
-    def read_only():
-        for lay in layers:
-            capi.check(capi.load().shrike_hip_probe_read(stream.handle, lay["pool"].bases, lay["pool"].stride, lay["res"].ptr,
-                                                         K, off.gate_w_off, p1_bytes_per_cell, sink.ptr), "probe_read")
-
-    # the step ahead of the layer (residual add + RMS norm producing x): as a launch of its own, and in the
-    # prologue of the layer's first launch; both on a residual stream and an x buffer of their own
-    import ctypes as _C
-    tree_n = S.SeedTree(0x5EED0003)
-    hidden_n, x_n = rt.dev(S.activations_f16(tree_n, "hidden", D)), rt.empty(2 * D)
-    delta_n = rt.dev(S.f32_to_f16_bits(tree_n.key("delta").normal(D, std=0.05)))
-    weight_n = rt.dev(S.f32_to_bf16_bits(tree_n.key("weight").uniform(0.5, 1.5, D)))
-    normed_args = []
-    for lay in layers:
-        apart_a, fused_a = capi.DecodeLayerArgs(), capi.DecodeLayerArgs()
-        for dst in (apart_a, fused_a):
-            _C.memmove(_C.byref(dst), _C.byref(lay["args"]), _C.sizeof(dst))
-            dst.x, dst.hidden = x_n.ptr, hidden_n.ptr
-        fused_a.norm_delta, fused_a.norm_weight, fused_a.norm_eps = delta_n.ptr, weight_n.ptr, 1e-6
-        normed_args.append((apart_a, fused_a))
-
-    def norm_apart():
-        for apart_a, _ in normed_args:
-            rt.residual_add_rmsnorm_bf16w(hidden_n, delta_n, weight_n, x_n, D, 1e-6, 1, stream=stream)
-            moe.encode_decode_layer(apart_a)
-
-    def norm_fused():
-        for _, fused_a in normed_args:
-            moe.encode_decode_layer(fused_a)
-
-    g_norm_apart = capture(rt, capi, stream, norm_apart)
-    g_norm_fused = capture(rt, capi, stream, norm_fused)
-    g_empty = capture(rt, capi, stream, empty_only)
-    g_read = capture(rt, capi, stream, read_only)
-    g_p12 = capture(rt, capi, stream, phase12)
-    g_p1 = capture(rt, capi, stream, phase1_only)
-    g_p2 = capture(rt, capi, stream, phase2_only)
-    g_rt = capture(rt, capi, stream, router_only)
-    g_sh = capture(rt, capi, stream, shared_only)
-
-    steps = max(n_layers, args.steps // n_layers * n_layers)
-    warm = max(n_layers, args.warmup // n_layers * n_layers)
-    time_graph(rt, capi, stream, g_layer, warm // n_layers)
-    ms = time_graph(rt, capi, stream, g_layer, steps // n_layers)
-    ms_per_step = ms / steps
-
-    reps = max(1, steps // n_layers // 2)
-    parts = {}
-    for name, g, launches_per_layer in (("phase1+phase2 alternating", g_p12, 2), ("phase1", g_p1, 1), ("phase2", g_p2, 1), ("router_select_classify", g_rt, 1),
-                                        ("shared_expert(2 launches)", g_sh, 1), ("empty launch of phase 1's grid", g_empty, 1),
-                                        ("read-only kernel over phase 1's bytes", g_read, 1),
-                                        ("norm launch + layer (4 launches)", g_norm_apart, 4), ("layer with the norm in its first launch", g_norm_fused, 3)):
-        time_graph(rt, capi, stream, g, 2)
-        parts[name] = time_graph(rt, capi, stream, g, reps) / (reps * n_layers) * 1e3  # us per layer
-
-    expert_bytes = (K + 1) * stride  # 15,925,248
-    total_bytes = expert_bytes + NE * D * 2 + 2 * D * 2
-    p1_bytes = K * 2 * (F * D // 2 + 2 * F * (D // 64) * 2)  # gate+up codes, scales and biases of 8 experts
-    p1_us = parts["phase1"]
-    value = expert_bytes / (ms_per_step * 1e-3) / 1e9
-    out = {
-        "metric": "MoE-layer decode: HBM GB/s on expert bytes (us per layer in ms_per_step), 35B-A3B int4 shape",
-        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warm,
-        "ms_per_step": round(ms_per_step, 6), "us_per_layer": round(ms_per_step * 1e3, 3),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic (seeded SplitMix64: uniform int4 codes, |N(0,0.02)| scales, N(0,1) fp16 activations)",
-        "config": {"workload": "config 2: full MoE layer decode, 1 token, hidden 2048, top-8 of 256 int4 experts "
-                               "(intermediate 512, group 64) + 1 shared expert, fp16 router, all slots resident",
-                   "stacked_layers": n_layers, "pool_bytes_total": n_layers * NE * stride,
-                   "meta_dtype": args.meta, "launches_per_layer": 3, "hip_graph": True},
-        "hbm_peak_frac_on_expert_bytes": round(value / HBM_PEAK_GBPS, 4),
-        "expert_bytes_per_step": expert_bytes, "total_bytes_per_step": total_bytes,
-        "kernel_us_per_layer": {k: round(v, 3) for k, v in parts.items()},
-        "roofline": {"bound": "hbm", "kernel": "k_phase1<4,1,4,false,0> (routed gate/up matvec + SiLU-multiply)",
-                     "achieved": round(p1_bytes / (p1_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(p1_bytes / (p1_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-                     "bytes_per_launch": p1_bytes, "us_per_launch": round(p1_us, 3), "traffic": PHASE1_TRAFFIC_BYTES,
-                     "floors_us": {"empty_launch": round(parts["empty launch of phase 1's grid"], 3),
-                                   "read_only_same_bytes": round(parts["read-only kernel over phase 1's bytes"], 3)}},
-        "setup_seconds": round(gen_s, 1),
-    }
-    if args.cpu_sample > 0:
-        out["cpu_baseline"] = cpu_baseline(S, keep[4], args.cpu_sample, meta)
+        return print(json.dumps(kimi_workload(args, rt, capi, S, meta)))
+    out = decode_workload(args, rt, capi, S, meta)
+    if not args.no_secondary:
+        # the other workloads of the benchmark definition, measured by this same run with sizes of their own
+        side = argparse.Namespace(**vars(args))
+        side.steps, side.warmup, side.layers = 4000, 400, 40
+        secondary = {}
+        for name, run in (("config3_ragged_prefill_512_tokens", lambda: prefill_workload(side, rt, capi, S, meta)),
+                          ("config4_gpt_oss_shape_4_tokens_int4", lambda: gptoss_workload(side, rt, capi, S, meta, 4)),
+                          ("config4_gpt_oss_shape_4_tokens_int8", lambda: gptoss_workload(side, rt, capi, S, meta, 8)),
+                          ("config5_kimi_shape_16_sequences_64_of_256_cells", lambda: kimi_workload(side, rt, capi, S, meta))):
+            gc.collect()
+            r = run()
+            secondary[name] = {k: r[k] for k in r if k in ("metric", "value", "unit", "ms_per_step", "us_per_layer", "config",
+                                                           "kernel_us_per_chunk", "roofline", "GBps_on_pair_bytes",
+                                                           "hbm_peak_frac_on_expert_bytes", "miss_rate", "host_to_device_GBps",
+                                                           "bytes_copied_per_step", "experts_requested_per_step", "steps", "dtype")}
+        out["secondary"] = secondary
     print(json.dumps(out))
 
 

@@ -305,6 +305,15 @@ typedef struct {
 } shrike_decode_layer_args;
 int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
                                 const shrike_decode_layer_args *args);
+/* The same layer one launch (or any subset) at a time, for a host that encodes other work between them, as
+ * the reference's runner does between the shared-expert work, phase 1 and phase 2
+ * (RealForwardRunner.swift:5436-5560): `launches` is a mask, bit 0 = router logit rows, route entries and
+ * the shared expert's gate/up rows; bit 1 = select + classify, the routed gate/up rows and the shared
+ * expert's down rows; bit 2 = the routed down rows, the weighted combine and hidden += y. 7 is
+ * shrike_hip_moe_decode_layer. Launches of one layer must run in this order on one stream with the same
+ * handle and args, and no other layer call on the handle between them (the route entries live in it). */
+int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream,
+                                         const shrike_decode_layer_args *args, uint32_t launches);
 
 /* The decode layer for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc). NO COUNTERPART IN THE REFERENCE. Same kernels and same
@@ -321,16 +330,6 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
  * GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
 int shrike_hip_moe_decode_layer_noalloc(const shrike_moe_desc *desc, void *stream,
                                         const shrike_decode_layer_args *args);
-
-/* ------------------------------------------------------- measurement aids
- * No counterpart in the reference. An empty launch of `workgroups` x 256 threads, and a
- * kernel that only reads bytes [byte_offset, byte_offset + bytes_per_cell) of each pool cell
- * in d_cells (u32[cell_count], as resolvedSlots holds them): the two floors a decode kernel
- * on the same cells is measured against. d_sink: u32[1], never written in practice. */
-int shrike_hip_probe_empty_launch(void *stream, uint32_t workgroups, uint32_t *d_sink);
-int shrike_hip_probe_read(void *stream, const shrike_pool_bases *pool, uint64_t pool_slot_stride,
-                          const uint32_t *d_cells, uint32_t cell_count, uint64_t byte_offset,
-                          uint64_t bytes_per_cell, uint32_t *d_sink);
 
 /* ------------------------------------------------------- prefill operators */
 

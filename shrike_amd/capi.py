@@ -290,9 +290,8 @@ SIGNATURES = {
     "shrike_hip_shared_expert": (C.c_int, [_VP, _VP, C.POINTER(Projection), C.POINTER(Projection),
                                            C.POINTER(Projection), _U32, _VP, _VP, _VP, _VP, _U32, _U32]),
     "shrike_hip_moe_decode_layer": (C.c_int, [_VP, _VP, C.POINTER(DecodeLayerArgs)]),
+    "shrike_hip_moe_decode_layer_launches": (C.c_int, [_VP, _VP, C.POINTER(DecodeLayerArgs), _U32]),
     "shrike_hip_moe_decode_layer_noalloc": (C.c_int, [C.POINTER(MoEDesc), _VP, C.POINTER(DecodeLayerArgs)]),
-    "shrike_hip_probe_empty_launch": (C.c_int, [_VP, C.c_uint32, _VP]),
-    "shrike_hip_probe_read": (C.c_int, [_VP, C.POINTER(PoolBases), _U64, _VP, C.c_uint32, _U64, _U64, _VP]),
     "shrike_hip_residual_add_rmsnorm_bf16w": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _U32, C.c_float, _U32]),
     "shrike_hip_malloc": (_VP, [_U64]),
     "shrike_hip_free": (C.c_int, [_VP]),

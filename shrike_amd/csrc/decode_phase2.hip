@@ -334,7 +334,13 @@ int shrike_hip_shared_expert(shrike_hip_moe *moe, void *stream, const shrike_pro
 // prologue of every phase-1 workgroup, the routed gate/up rows, and the shared down rows;
 // (3) phase 2 with the shared expert's output as the residual.
 int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *g) {
+    return shrike_hip_moe_decode_layer_launches(moe, stream, g, 7u);
+}
+
+int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *g,
+                                         uint32_t launches) {
     SHRIKE_REQUIRE(moe != nullptr && g != nullptr, "moe handle or args is NULL");
+    SHRIKE_REQUIRE(launches != 0 && launches <= 7u, "decodeLayer: launches=%u is not a mask of the three launches", launches);
     const shrike_moe_desc &m = moe->desc;
     if (int rc = check_router(moe, m.num_experts, m.d, m.top_k)) return rc;
     if (int rc = check_offsets(&g->offsets, m.d, m.f, m.routed_weight_bits)) return rc;
@@ -403,7 +409,8 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
     if (shared) {
         GemvArgs gu = {};
         fill_gemv_gate_up(gu, &g->shared_gate, &g->shared_up, gate_out, up_out, g->shared_f, m.d, m.meta_dtype, g->x);
-        if (int rc = launch_head(r, m.router_weight_bits, gu, sbits, normed ? &norm : nullptr, s)) return rc;
+        if (launches & 1u)
+            if (int rc = launch_head(r, m.router_weight_bits, gu, sbits, normed ? &norm : nullptr, s)) return rc;
         fill_gemv_down(p1.shared_down, &g->shared_down, gate_out, up_out, g->h1, m.d, g->shared_f, m.meta_dtype,
                        m.activation, g->shared_scalar_gate);
         down_fused = nch_for(g->shared_f, sbits) == 1;
@@ -411,12 +418,16 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_
     } else {  // the head launch with router rows only
         GemvArgs none = {};
         none.n = m.d;
-        if (int rc = launch_head(r, m.router_weight_bits, none, sbits, normed ? &norm : nullptr, s)) return rc;
+        if (launches & 1u)
+            if (int rc = launch_head(r, m.router_weight_bits, none, sbits, normed ? &norm : nullptr, s)) return rc;
     }
-    if (int rc = launch_phase1(p1, m.routed_weight_bits, true, down_fused ? sbits : 0u, s)) return rc;
-    if (shared && !down_fused) {
-        if (int rc = launch_gemv(p1.shared_down, sbits, s)) return rc;
+    if (launches & 2u) {
+        if (int rc = launch_phase1(p1, m.routed_weight_bits, true, down_fused ? sbits : 0u, s)) return rc;
+        if (shared && !down_fused) {
+            if (int rc = launch_gemv(p1.shared_down, sbits, s)) return rc;
+        }
     }
+    if (!(launches & 4u)) return 0;
 
     Phase2Args p = {};
     fill_pool(p.pool, g->pool);

@@ -1,10 +1,26 @@
-// Measurement aids, not operators: an empty launch and a kernel that only reads a byte range
-// of each listed pool cell. Timed beside a real kernel on the same cells they give the two
-// floors that bound it on this part: what a launch costs with nothing to do, and what
-// moving the same bytes costs with no arithmetic and no dependent loads behind it.
+// Measurement aids, not operators, and not part of libshrikehip: this file is built into a small library of its
+// own (libshrikeprobe.so) that only the benchmark and its test load. An empty launch and a kernel that only
+// reads a byte range of each listed pool cell: timed beside a real kernel on the same cells they give the two
+// floors that bound it on this part, what a launch costs with nothing to do, and what moving the same bytes
+// costs with no arithmetic and no dependent loads behind it.
 #include "gemv_common.h"
 
 namespace shrike {
+
+// this library's own error text (libshrikehip's is not linked in)
+static std::string g_probe_error;
+void set_error(const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_probe_error = buf;
+}
+int hip_failed(hipError_t err, const char *what) {
+    set_error("%s: %s", what, hipGetErrorString(err));
+    return EIO;
+}
 
 __global__ __launch_bounds__(256) void k_probe_empty(uint32_t *sink) {
     if (sink == nullptr && threadIdx.x == 0xffffffffu) *sink = 0u;  // never true; keeps the argument live
@@ -40,14 +56,16 @@ using namespace shrike;
 
 extern "C" {
 
-int shrike_hip_probe_empty_launch(void *stream, uint32_t workgroups, uint32_t *d_sink) {
+const char *shrike_probe_last_error(void) { return g_probe_error.c_str(); }
+
+int shrike_probe_empty_launch(void *stream, uint32_t workgroups, uint32_t *d_sink) {
     SHRIKE_REQUIRE(workgroups >= 1 && d_sink != nullptr, "probe: workgroups must be positive and the sink bound");
     hipLaunchKernelGGL(k_probe_empty, dim3(workgroups), dim3(256), 0, as_stream(stream), d_sink);
     SHRIKE_HIP(hipGetLastError());
     return 0;
 }
 
-int shrike_hip_probe_read(void *stream, const shrike_pool_bases *pool, uint64_t pool_slot_stride, const uint32_t *d_cells,
+int shrike_probe_read(void *stream, const shrike_pool_bases *pool, uint64_t pool_slot_stride, const uint32_t *d_cells,
                           uint32_t cell_count, uint64_t byte_offset, uint64_t bytes_per_cell, uint32_t *d_sink) {
     SHRIKE_REQUIRE(pool != nullptr && d_cells != nullptr && d_sink != nullptr, "probe: pool, cells and sink must be bound");
     SHRIKE_REQUIRE(cell_count >= 1 && bytes_per_cell >= 1024u, "probe: nothing to read");

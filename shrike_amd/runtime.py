@@ -359,6 +359,11 @@ class MoE:
         check(capi.load().shrike_hip_moe_decode_layer(self.handle, self._s(), C.byref(args)),
               "shrike_hip_moe_decode_layer")
 
+    def encode_decode_layer_launches(self, args: DecodeLayerArgs, launches: int):
+        """A subset of the layer's three launches (bit 0 head, bit 1 phase 1, bit 2 phase 2)."""
+        check(capi.load().shrike_hip_moe_decode_layer_launches(self.handle, self._s(), C.byref(args), launches),
+              "shrike_hip_moe_decode_layer_launches")
+
 
 class GroupedRoutesDevice:
     """Device buffers of shrike_hip_grouped_routes for up to `pairs` pairs over `num_experts`."""

@@ -445,6 +445,29 @@ def test_decode_layer_is_deterministic(gpu):
         assert all(np.array_equal(a, b) for a, b in zip(o, outs[0]))
 
 
+def test_decode_layer_one_launch_at_a_time(gpu):
+    """The layer's three launches encoded one by one (with other work on the stream between them) give the bytes
+    of the one call; a mask outside 1...7 is refused."""
+    L = Layer(0x5EED0002, 2048, 512, 64, 8, shared_f=512)
+    dl = DeviceLayer(gpu, L)
+    dl.moe.encode_decode_layer(dl.layer_args())
+    want = (dl.y.download(np.uint16, 2048), dl.hidden.download(np.uint16, 2048), dl.out_idx.download(np.uint32, 8),
+            dl.acts.download(np.uint16, 8 * 512))
+    dl.hidden.upload(L.hidden)
+    for b in (dl.y, dl.out_idx, dl.acts):
+        b.fill(0x5A)
+    other = gpu.empty(4096)
+    for launches in (1, 2, 4):
+        dl.moe.encode_decode_layer_launches(dl.layer_args(), launches)
+        other.fill(launches)  # unrelated work on the same stream
+    got = (dl.y.download(np.uint16, 2048), dl.hidden.download(np.uint16, 2048), dl.out_idx.download(np.uint32, 8),
+           dl.acts.download(np.uint16, 8 * 512))
+    assert all(np.array_equal(a, b) for a, b in zip(got, want))
+    for bad in (0, 8):
+        with pytest.raises(capi.ShrikeError, match="mask"):
+            dl.moe.encode_decode_layer_launches(dl.layer_args(), bad)
+
+
 def test_multi_chunk_pool_addressing(gpu):
     """The same cells through a pool split into several chunks (ExpertCellArena chunking)."""
     d, f, k, ne = 256, 128, 4, 12
@@ -461,24 +484,24 @@ def test_multi_chunk_pool_addressing(gpu):
 
 
 def test_measurement_probes_run_and_check_their_arguments(gpu):
-    """The empty launch and the read-only kernel that bench.py times beside phase 1."""
+    """The empty launch and the read-only kernel that bench.py times beside phase 1 (a library of their own)."""
+    from shrike_amd import probes
     L = Layer(33, 256, 128, 12, 4)
     dl = DeviceLayer(gpu, L)
-    lib = capi.load()
+    lib = probes.load()
     sink = gpu.empty(4).fill(0)
     cells = gpu.empty(4 * 4)
     cells.upload(np.array([dl.cell_of[e] for e in (0, 5, 7, 11)], np.uint32))
     nbytes = (dl.off.down_w_off - dl.off.gate_w_off) // 1024 * 1024
-    capi.check(lib.shrike_hip_probe_empty_launch(None, 64, sink.ptr), "probe_empty_launch")
-    capi.check(lib.shrike_hip_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, dl.off.gate_w_off, nbytes,
-                                         sink.ptr), "probe_read")
+    probes.check(lib.shrike_probe_empty_launch(None, 64, sink.ptr), "probe_empty_launch")
+    probes.check(lib.shrike_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, dl.off.gate_w_off, nbytes,
+                                       sink.ptr), "probe_read")
     gpu.synchronize()
     assert sink.download(np.uint32, 1)[0] == 0
-    assert lib.shrike_hip_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 0, dl.pool.stride + 1024,
-                                     sink.ptr) != 0
-    assert "leaves the cell" in capi.last_error()
-    assert lib.shrike_hip_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 8, 1024, sink.ptr) != 0
-    assert lib.shrike_hip_probe_empty_launch(None, 0, sink.ptr) != 0
+    assert lib.shrike_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 0, dl.pool.stride + 1024, sink.ptr) != 0
+    assert "leaves the cell" in probes.last_error()
+    assert lib.shrike_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 8, 1024, sink.ptr) != 0
+    assert lib.shrike_probe_empty_launch(None, 0, sink.ptr) != 0
 
 
 def test_argument_errors_are_reported_not_trapped(gpu):
