@@ -13,7 +13,9 @@ constexpr int kPhase1RowPairs = 4;  // (gate, up) row pairs per wave
 // A wave owns RP consecutive f of one routed position: RP gate rows and RP up rows, each a
 // run of 16-byte chunks across the lanes. The lane's slice of x comes straight from global
 // memory (L2-resident) ahead of the row loads, so in-order load return never holds it back.
-template <int BITS, int NCH, int RP, bool ROUTE, int SBITS>
+// STREAM: one token, so every routed row is read exactly once: the row loads are non-temporal (a batch of tokens
+// reads an expert's rows once per token routed to it, and there the caches are what makes the second read cheap).
+template <int BITS, int NCH, int RP, bool ROUTE, int SBITS, bool STREAM>
 __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
@@ -71,7 +73,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
         const uint8_t *w = base + (up ? a.off.up_w_off : a.off.gate_w_off) + size_t(f) * row_bytes;
         const uint16_t *s = reinterpret_cast<const uint16_t *>(base + (up ? a.off.up_s_off : a.off.gate_s_off)) + size_t(f) * groups;
         const uint16_t *b = reinterpret_cast<const uint16_t *>(base + (up ? a.off.up_b_off : a.off.gate_b_off)) + size_t(f) * groups;
-        load_row<BITS, NCH>(rows[r], w, s, b, cpr, lane, true);
+        load_row<BITS, NCH, STREAM>(rows[r], w, s, b, cpr, lane, true);
     }
     float gab = 0.0f, uab = 0.0f;
     if (a.ebias && lane < uint32_t(RP)) {  // moe.metal:261-269
@@ -101,15 +103,15 @@ uint32_t phase1_blocks(uint32_t top_k, uint32_t f) {
     return (waves + 3) / 4;
 }
 
-template <int BITS, bool ROUTE, int SBITS>
+template <int BITS, bool ROUTE, int SBITS, bool STREAM>
 static void launch_phase1_nch(const Phase1Args &a, dim3 grid, hipStream_t s) {
     constexpr int RP = kPhase1RowPairs;
     const dim3 block(256);
     switch (nch_for(a.d, BITS)) {
-        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, RP, ROUTE, SBITS>), grid, block, 0, s, a); break;
-        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, RP, ROUTE, SBITS>), grid, block, 0, s, a); break;
-        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RP, ROUTE, SBITS>), grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RP, ROUTE, SBITS>), grid, block, 0, s, a); break;
+        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
+        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
     }
 }
 
@@ -124,16 +126,17 @@ int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t sha
     Phase1Args b = a;
     b.lists_block = routing ? a.routed_blocks + extra : 0xffffffffu;
     const dim3 grid(a.routed_blocks + extra + (routing ? 1u : 0u), a.tokens ? a.tokens : 1u);
+    const bool one_token = a.tokens <= 1u;
     if (bits == 4) {
-        if (!routing) launch_phase1_nch<4, false, 0>(b, grid, s);
-        else if (shared_down_bits == 0) launch_phase1_nch<4, true, 0>(b, grid, s);
-        else if (shared_down_bits == 4) launch_phase1_nch<4, true, 4>(b, grid, s);
-        else launch_phase1_nch<4, true, 8>(b, grid, s);
+        if (!routing) { if (one_token) launch_phase1_nch<4, false, 0, true>(b, grid, s); else launch_phase1_nch<4, false, 0, false>(b, grid, s); }
+        else if (shared_down_bits == 0) launch_phase1_nch<4, true, 0, true>(b, grid, s);
+        else if (shared_down_bits == 4) launch_phase1_nch<4, true, 4, true>(b, grid, s);
+        else launch_phase1_nch<4, true, 8, true>(b, grid, s);
     } else {
-        if (!routing) launch_phase1_nch<8, false, 0>(b, grid, s);
-        else if (shared_down_bits == 0) launch_phase1_nch<8, true, 0>(b, grid, s);
-        else if (shared_down_bits == 4) launch_phase1_nch<8, true, 4>(b, grid, s);
-        else launch_phase1_nch<8, true, 8>(b, grid, s);
+        if (!routing) { if (one_token) launch_phase1_nch<8, false, 0, true>(b, grid, s); else launch_phase1_nch<8, false, 0, false>(b, grid, s); }
+        else if (shared_down_bits == 0) launch_phase1_nch<8, true, 0, true>(b, grid, s);
+        else if (shared_down_bits == 4) launch_phase1_nch<8, true, 4, true>(b, grid, s);
+        else launch_phase1_nch<8, true, 8, true>(b, grid, s);
     }
     SHRIKE_HIP(hipGetLastError());
     return 0;

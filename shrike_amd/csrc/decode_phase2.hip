@@ -19,7 +19,8 @@ __device__ __forceinline__ void phase2_finish(uint16_t *y, uint16_t *hidden, uin
 // One wave per routed position (blockDim = 64 * top_k); a workgroup owns kPhase2Rows output
 // rows. When a down row is shorter than a wave's 1 KiB load, the wave covers 64/cpr rows per
 // load and reduces over lane segments. BATCH row groups are in flight per wave.
-template <int BITS, int NCH, int BATCH>
+// STREAM: one token, every down row is read once: non-temporal row loads (see k_phase1).
+template <int BITS, int NCH, int BATCH, bool STREAM>
 __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
@@ -80,7 +81,7 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
                 row[j] = d0 + (g0 + j) * rpl + sub;
                 on[j] = lane_on && (g0 + j) < n_groups && row[j] < a.d;
                 const uint32_t rr = on[j] ? row[j] : 0u;
-                load_row<BITS, NCH>(rows[j], base + a.off.down_w_off + size_t(rr) * row_bytes,
+                load_row<BITS, NCH, STREAM>(rows[j], base + a.off.down_w_off + size_t(rr) * row_bytes,
                                     s_all + size_t(rr) * groups, b_all + size_t(rr) * groups, cpr, col, on[j]);
             }
             if (g0 == 0) unpack_slices<BITS, NCH>(xr, x, xs);
@@ -116,9 +117,15 @@ static void launch_phase2_batch(const Phase2Args &a, dim3 grid, dim3 block, hipS
     const uint32_t cpr = a.f * BITS / 128u;
     const uint32_t rpl = (cpr < 64u && 64u % cpr == 0u) ? (64u / cpr < kPhase2Rows ? 64u / cpr : kPhase2Rows) : 1u;
     const uint32_t n_groups = kPhase2Rows / rpl;  // row groups per wave; up to 4 in flight
-    if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4>), grid, block, 0, s, a);
-    else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1>), grid, block, 0, s, a);
+    if (a.tokens <= 1u) {
+        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, true>), grid, block, 0, s, a);
+        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, true>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, true>), grid, block, 0, s, a);
+    } else {
+        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, false>), grid, block, 0, s, a);
+        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, false>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, false>), grid, block, 0, s, a);
+    }
 }
 
 template <int BITS>

@@ -132,7 +132,12 @@ struct RowRegs {
     uint16_t s[NCH], b[NCH];
 };
 
-template <int BITS, int NCH>
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// STREAM: the row is read once and by nobody else (a routed expert's rows in decode): the loads are marked
+// non-temporal, so that what they bring in does not displace the small tensors every layer call reads again
+// (router rows, shared expert, route tables) from the caches behind the compute units.
+template <int BITS, int NCH, bool STREAM = false>
 __device__ __forceinline__ void load_row(RowRegs<BITS, NCH> &r, const uint8_t *w_row, const uint16_t *s_row,
                                          const uint16_t *b_row, uint32_t cpr, uint32_t col, bool lane_on) {
     typedef Chunk<BITS> C;
@@ -142,9 +147,16 @@ __device__ __forceinline__ void load_row(RowRegs<BITS, NCH> &r, const uint8_t *w
         const bool on = lane_on && c < cpr;
         const uint32_t cc = on ? c : 0u;
         const uint32_t g = cc * C::E / kGroup;
-        r.w[i] = *reinterpret_cast<const uint4 *>(w_row + 16u * cc);
-        r.s[i] = s_row[g];
-        r.b[i] = b_row[g];
+        if (STREAM) {
+            const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(w_row + 16u * cc));
+            r.w[i] = make_uint4(v.x, v.y, v.z, v.w);
+            r.s[i] = __builtin_nontemporal_load(s_row + g);
+            r.b[i] = __builtin_nontemporal_load(b_row + g);
+        } else {
+            r.w[i] = *reinterpret_cast<const uint4 *>(w_row + 16u * cc);
+            r.s[i] = s_row[g];
+            r.b[i] = b_row[g];
+        }
     }
 }
 

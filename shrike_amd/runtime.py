@@ -844,6 +844,11 @@ class AgreedDecodeLayer:
         self.acts = empty(2 * k * moe.desc.f)
         self.tag = 0
         self.fixups = self.overflows = self.landed_hits = self.demand_reads = 0
+        # the demand batch's status word on the device and the three values it takes, in pinned memory
+        self.status = empty(4).fill(0)
+        self.status_values = PinnedBuffer(12)
+        self.agreed_row = PinnedBuffer(32)
+        self.status_values.array.view(np.uint32)[:] = (0, 1, 2)
 
     def drop_landing(self, layer: int, expert: int, cell: int) -> None:
         """The ring's reclaim of a landing no plan wanted (called with the ring locked)."""
@@ -851,13 +856,22 @@ class AgreedDecodeLayer:
             self.cache.drop_landing(expert, cell)
 
     def _copy(self, experts, cells):
-        """The reads: each expert's blob from the pinned store into its cell; returns when the bytes are in HBM."""
+        """The reads: each expert's blob from the pinned store into its cell, enqueued on the upload stream. Returns
+        the event recorded behind them; the bytes are in HBM once it has completed."""
         L = capi.load()
         for expert, cell in zip(experts, cells):
             check(L.shrike_hip_pool_upload_async(self.pool.handle, cell, self.store.ptr + expert * self.store_stride,
                                                  self.expert_bytes, self.upload_stream.handle),
                   "shrike_hip_pool_upload_async")
-        self.upload_stream.synchronize()
+        landed = Event()
+        landed.record(self.upload_stream)
+        return landed
+
+    def _store_status(self, value: int):
+        """The batch's status word (ExpertIOCompletionToken.status: 0 loading, 1 complete, 2 failed), stored on the
+        upload stream behind whatever was enqueued there."""
+        check(capi.load().shrike_hip_memcpy_h2d_async(self.status.ptr, self.status_values.ptr + 4 * value, 4,
+                                                      self.upload_stream.handle), "shrike_hip_memcpy_h2d_async")
 
     def _publish(self):
         """The cache's changed residency words into the device table, in order, ahead of the next launch."""
@@ -875,7 +889,7 @@ class AgreedDecodeLayer:
             def work():
                 operation.mark_in_flight()
                 try:
-                    self._copy(experts, cells)
+                    self._copy(experts, cells).synchronize()
                     for expert, cell in zip(experts, cells):
                         self.cache.complete_landing(expert, cell)
                     operation.finish(0)
@@ -959,19 +973,35 @@ class AgreedDecodeLayer:
         self.overflows += len(overflow)
 
         # submitAgreedReads, :5319-5340 (beginAgreedReads, PreadExpertStreamer.swift:903-964)
+        # The storage thread enqueues the copies, the status word and an event on the upload stream and finishes the
+        # operation once they are enqueued; the compute stream then waits for that event ahead of the fixup
+        # launches, which read the status word (moe.metal:36-39). What the host waits for is the enqueue, not the
+        # bytes: the wait for them is the GPU's, as with the reference's encodeWaitForEvent
+        # (RealForwardRunner.swift:5124, ExpertIOEventCoordinator.swift:76-89).
         operation = _host.ExpertLoadOperation()
+        uploaded = []
         if read_experts:
             started = _host.monotonic_nanos()
+            self._store_status(0)
 
             def work():
                 operation.mark_in_flight()
                 fetch_started = _host.monotonic_nanos()
                 try:
-                    self._copy(read_experts, read_cells)
-                    landed = _host.monotonic_nanos()
-                    self.cache.finish_agreed_reads(read_experts, read_cells, True, landed - started, landed - fetch_started)
+                    copies = self._copy(read_experts, read_cells)
+                    self._store_status(1)
+                    landed = Event()
+                    landed.record(self.upload_stream)
+                    uploaded.append(landed)
+                    del copies
+                    enqueued = _host.monotonic_nanos()
+                    self.cache.finish_agreed_reads(read_experts, read_cells, True, enqueued - started, enqueued - fetch_started)
                     operation.finish(0)
                 except Exception:
+                    try:
+                        self._store_status(2)
+                    except Exception:
+                        pass
                     self.cache.finish_agreed_reads(read_experts, read_cells, False)
                     operation.finish(5)
             self.scheduler.submit(work, _host.ExpertIOScheduler.DEMAND)
@@ -984,15 +1014,28 @@ class AgreedDecodeLayer:
         held = list(set(leased) | set(claimed))
         if misses:
             try:
-                operation.wait()  # the reference's fixup waits on the batch's event value instead of the host
+                operation.wait()  # until the batch is enqueued on the upload stream (or has failed)
             except Exception:
                 self.ring.consume(self.layer, held, {})  # abandonPendingAgreedLayer, :5351-5355
                 raise ShrikeError(f"layer {self.layer}: an agreed read failed")
-            self.agreed.upload(row)
+            if compute:  # the agreed row goes out on the compute stream: a blocking copy would wait for the upload stream too
+                self.agreed_row.array.view(np.uint32)[:] = row
+                check(capi.load().shrike_hip_memcpy_h2d_async(self.agreed.ptr, self.agreed_row.ptr, 32, compute.handle),
+                      "shrike_hip_memcpy_h2d_async")
+            else:
+                self.agreed.upload(row)
             self._publish()
-            m.encode_spec_phase1(self.pool, self.agreed, self.off, x, self.acts, d, f, k, indirect=spec + 24)
+            io_status = None
+            if uploaded:
+                if compute:
+                    compute.wait_event(uploaded[0])  # the GPU waits for the bytes; the host goes on encoding
+                else:
+                    uploaded[0].synchronize()        # the null stream has no handle to wait on
+                io_status = self.status
+            m.encode_spec_phase1(self.pool, self.agreed, self.off, x, self.acts, d, f, k, indirect=spec + 24,
+                                 io_status=io_status)
             m.encode_spec_phase2(self.pool, self.resolved, self.off, self.acts, self.w, residual, y, hidden, d, f, k,
-                                 fallback_cells=self.agreed, indirect=spec + 36)
+                                 fallback_cells=self.agreed, indirect=spec + 36, io_status=io_status)
             self.fixups += 1
 
         # planAgreedLayer, :5380-5411
