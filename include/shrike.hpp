@@ -400,6 +400,23 @@ public:
         check(shrike_hip_moe_phase2_pool(h_, s, pool.bases(), pool.stride(), resolvedSlots, fallbackCells, &offsets, acts, routingWeights,
                                          residual, y, hidden, d, f, topK, indirect, ioStatus));
     }
+    // MoE.swift:651-665 and, with activeSlots, :694-712: the route's blobs named by a device array of pointers
+    void encodeRoutedPersistentPhase1U16Load(Stream s, const void *const *routedArgBuffer, const shrike_expert_offsets &offsets,
+                                             const void *x, void *acts, uint32_t d, uint32_t f, uint32_t topK,
+                                             const uint32_t *ioStatus = nullptr) {
+        check(shrike_hip_moe_phase1_blobs(h_, s, routedArgBuffer, &offsets, x, acts, d, f, topK, nullptr, 0, ioStatus));
+    }
+    void encodeRoutedPersistentPhase1SubsetU16Load(Stream s, const void *const *routedArgBuffer, const shrike_expert_offsets &offsets,
+                                                   const void *x, void *acts, const uint32_t *activeSlots, uint32_t activeCount,
+                                                   uint32_t d, uint32_t f, uint32_t topK, const uint32_t *ioStatus = nullptr) {
+        if (activeCount == 0) return;  // MoE.swift:710
+        check(shrike_hip_moe_phase1_blobs(h_, s, routedArgBuffer, &offsets, x, acts, d, f, topK, activeSlots, activeCount, ioStatus));
+    }
+    void encodeRoutedPersistentPhase2Reduce(Stream s, const void *const *routedArgBuffer, const shrike_expert_offsets &offsets,
+                                            const void *acts, const void *routingWeights, const void *residual, void *y, void *hidden,
+                                            uint32_t d, uint32_t f, uint32_t topK, const uint32_t *ioStatus = nullptr) {  // MoE.swift:816-836
+        check(shrike_hip_moe_phase2_blobs(h_, s, routedArgBuffer, &offsets, acts, routingWeights, residual, y, hidden, d, f, topK, ioStatus));
+    }
     void encodeSharedExpert(Stream s, const shrike_projection &gate, const shrike_projection &up, const shrike_projection &down,
                             uint32_t bits, const void *x, void *scratch, void *h1, const void *scalarGate, uint32_t d, uint32_t fShared) {
         check(shrike_hip_shared_expert(h_, s, &gate, &up, &down, bits, x, scratch, h1, scalarGate, d, fShared));

@@ -219,6 +219,28 @@ int shrike_hip_moe_phase1_pool(shrike_hip_moe *moe, void *stream, const shrike_p
                                void *d_acts, uint32_t d, uint32_t f, uint32_t top_k,
                                const uint32_t *d_indirect, const uint32_t *d_io_status);
 
+/* Argument-buffer addressing: MoE.makeReusedRoutedArgumentBuffer (MoE.swift:612-620) gives position k of the route the
+ * blob routedBlobs[k] instead of a pool cell. Here the argument buffer is a device array of top_k pointers
+ * (d_routed_blobs[k] = the 16-byte aligned blob of position k; a NULL entry skips the position), which the host
+ * fills with an ordinary copy.
+ *
+ * MoE.encodeRoutedPersistentPhase1U16Load, MoE.swift:651-692 (moe_phase1_gate_up_act_u16load, moe.metal:779-830), and,
+ * with d_active_slots bound, MoE.encodeRoutedPersistentPhase1SubsetU16Load, MoE.swift:694-776
+ * (moe_phase1_gate_up_act_subset_u16load, moe.metal:832-884): only the positions d_active_slots[0 .. active_count) are
+ * computed (an entry >= top_k is skipped), the other positions' acts stay as they are; active_count == 0 with a list
+ * bound does nothing. acts: fp16[top_k * f]. */
+int shrike_hip_moe_phase1_blobs(shrike_hip_moe *moe, void *stream, const void *const *d_routed_blobs,
+                                const shrike_expert_offsets *offsets, const void *d_x, void *d_acts,
+                                uint32_t d, uint32_t f, uint32_t top_k, const uint32_t *d_active_slots,
+                                uint32_t active_count, const uint32_t *d_io_status);
+/* MoE.encodeRoutedPersistentPhase2Reduce, MoE.swift:778-864 (moe_phase2_down_reduce_k8, moe.metal:897-941):
+ * shrike_hip_moe_phase2_pool's arithmetic over the argument buffer's blobs. */
+int shrike_hip_moe_phase2_blobs(shrike_hip_moe *moe, void *stream, const void *const *d_routed_blobs,
+                                const shrike_expert_offsets *offsets, const void *d_acts,
+                                const void *d_routing_weights, const void *d_residual, void *d_y,
+                                void *d_hidden, uint32_t d, uint32_t f, uint32_t top_k,
+                                const uint32_t *d_io_status);
+
 /* MoE.encodeSpecPhase2Reduce, MoE.swift:992-1047 (moe_phase2_down_reduce_spec_k8,
  * moe.metal:1008-1057): y = half(residual + sum_k half_w[k] * down_k . acts_k),
  * hidden = half(hidden + y). A sentinel position takes d_fallback_cells[k] when that

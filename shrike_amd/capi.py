@@ -287,6 +287,8 @@ SIGNATURES = {
     "shrike_hip_moe_phase2_pool": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, _VP, _VP,
                                              C.POINTER(ExpertOffsets), _VP, _VP, _VP, _VP, _VP,
                                              _U32, _U32, _U32, _VP, _VP]),
+    "shrike_hip_moe_phase1_blobs": (C.c_int, [_VP, _VP, _VP, C.POINTER(ExpertOffsets), _VP, _VP, _U32, _U32, _U32, _VP, _U32, _VP]),
+    "shrike_hip_moe_phase2_blobs": (C.c_int, [_VP, _VP, _VP, C.POINTER(ExpertOffsets), _VP, _VP, _VP, _VP, _VP, _U32, _U32, _U32, _VP]),
     "shrike_hip_shared_expert": (C.c_int, [_VP, _VP, C.POINTER(Projection), C.POINTER(Projection),
                                            C.POINTER(Projection), _U32, _VP, _VP, _VP, _VP, _U32, _U32]),
     "shrike_hip_moe_decode_layer": (C.c_int, [_VP, _VP, C.POINTER(DecodeLayerArgs)]),

@@ -31,6 +31,11 @@ struct Phase1Args {
     uint32_t d, f, top_k, meta, act, ebias;
     const uint32_t *indirect, *io_status;
     uint32_t tokens, x_stride;  // tokens > 1: grid.y walks tokens; x rows x_stride elements apart
+    // argument-buffer addressing (moe.metal:779-884): position k's blob is blobs[k] in place of a pool cell; with
+    // `active` bound only the positions active[0 .. active_count) are computed, the grid covering active_count * f rows
+    const uint8_t *const *blobs;
+    const uint32_t *active;
+    uint32_t active_count;
     // fused layer only: every wave selects from the route table the previous launch left, the shared expert's down
     // projection runs in workgroups past `routed_blocks`, and one more workgroup behind those writes the route lists
     SelectArgs sel;
@@ -51,6 +56,7 @@ struct Phase2Args {
     uint32_t d, f, top_k, meta, ebias;
     const uint32_t *indirect, *io_status;
     uint32_t tokens;  // tokens > 1: grid.y walks tokens; residual, y and hidden rows are d apart
+    const uint8_t *const *blobs;  // argument-buffer addressing (moe.metal:897-941): position k's blob, in place of a pool cell
     const uint16_t *delta;  // fp16[d] or null: hidden = half(half(hidden + delta) + y), the residual add of a norm fused ahead
 };
 

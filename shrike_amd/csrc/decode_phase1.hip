@@ -45,9 +45,14 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t cpr = a.d * BITS / 128u, groups = a.d / kGroup, row_bytes = cpr * 16u;
     const uint32_t pair0 = (blockIdx.x * 4u + wave) * RP;
-    const bool in_range = pair0 < a.top_k * a.f;
-    const uint32_t k = in_range ? pair0 / a.f : 0u;
+    bool in_range = pair0 < (a.active ? a.active_count : a.top_k) * a.f;
+    uint32_t k = in_range ? pair0 / a.f : 0u;
     const uint32_t f0 = pair0 - k * a.f;
+    if (!ROUTE && a.active) {  // moe.metal:873-876: the wave's position comes from the list; one past top_k is skipped
+        k = in_range ? a.active[k] : 0u;
+        in_range = in_range && k < a.top_k;
+        k = in_range ? k : 0u;
+    }
 
     uint32_t cell = kSentinel;
     SliceRegs<BITS, NCH> xr;
@@ -60,10 +65,16 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
         if (in_range) cell = uint32_t(__builtin_amdgcn_readlane(int(t.my_cell), int(k)));
     } else {
         load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
-        if (in_range) cell = resolved_tok[k];
+        if (in_range && !a.blobs) cell = resolved_tok[k];
     }
-    if (cell == kSentinel) return;  // moe.metal:986, and waves past the last row
-    const uint8_t *base = cell_base_uniform(a.pool, cell, a.stride);
+    const uint8_t *base;
+    if (!ROUTE && a.blobs) {  // moe.metal:821: the blob the argument buffer names for this position
+        base = in_range ? a.blobs[k] : nullptr;
+        if (base == nullptr) return;
+    } else {
+        if (cell == kSentinel) return;  // moe.metal:986, and waves past the last row
+        base = cell_base_uniform(a.pool, cell, a.stride);
+    }
 
     RowRegs<BITS, NCH> rows[2 * RP];
 #pragma unroll
@@ -98,6 +109,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     if (lane < uint32_t(RP)) acts_tok[size_t(k) * a.f + f0 + lane] = act;
 }
 
+// positions: top_k, or the length of the active list
 uint32_t phase1_blocks(uint32_t top_k, uint32_t f) {
     const uint32_t waves = (top_k * f + kPhase1RowPairs - 1) / kPhase1RowPairs;
     return (waves + 3) / 4;
@@ -182,6 +194,31 @@ int shrike_hip_moe_phase1_pool(shrike_hip_moe *moe, void *stream, const shrike_p
     a.ebias = moe->desc.expert_additive_biases;
     a.indirect = d_indirect; a.io_status = moe->desc.event_gated_io ? d_io_status : nullptr;
     a.routed_blocks = phase1_blocks(top_k, f);
+    return launch_phase1(a, bits, false, 0, as_stream(stream));
+}
+
+int shrike_hip_moe_phase1_blobs(shrike_hip_moe *moe, void *stream, const void *const *d_routed_blobs,
+                                const shrike_expert_offsets *offsets, const void *d_x, void *d_acts, uint32_t d, uint32_t f,
+                                uint32_t top_k, const uint32_t *d_active_slots, uint32_t active_count,
+                                const uint32_t *d_io_status) {
+    SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
+    SHRIKE_REQUIRE(top_k >= 1 && top_k <= SHRIKE_MAX_TOP_K, "phase1: topK=%u not in 1...8", top_k);  // MoE.validate(routedBlobs:topK:)
+    const uint32_t bits = moe->desc.routed_weight_bits;
+    if (int rc = check_offsets(offsets, d, f, bits)) return rc;
+    SHRIKE_REQUIRE(d_routed_blobs && d_x && d_acts, "phase1: the argument buffer, x and acts must be bound");
+    if (d_active_slots != nullptr && active_count == 0) return 0;  // MoE.swift:710: nothing to do is not an error
+    SHRIKE_REQUIRE(d_active_slots != nullptr || active_count == 0, "phase1: activeCount=%u without an active list", active_count);
+    SHRIKE_REQUIRE(active_count <= SHRIKE_MAX_TOP_K, "phase1: activeCount=%u exceeds %u", active_count, SHRIKE_MAX_TOP_K);
+    Phase1Args a = {};
+    a.blobs = reinterpret_cast<const uint8_t *const *>(d_routed_blobs);
+    a.active = d_active_slots; a.active_count = active_count;
+    a.off = *offsets;
+    a.x = static_cast<const uint16_t *>(d_x); a.acts = static_cast<uint16_t *>(d_acts);
+    a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.act = moe->desc.activation;
+    a.ebias = moe->desc.expert_additive_biases;
+    a.io_status = moe->desc.event_gated_io ? d_io_status : nullptr;
+    a.resolved = nullptr;
+    a.routed_blocks = phase1_blocks(d_active_slots ? active_count : top_k, f);
     return launch_phase1(a, bits, false, 0, as_stream(stream));
 }
 

@@ -60,11 +60,18 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
 
     SliceRegs<BITS, NCH> xr;
     load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(acts_tok + size_t(k) * a.f), cpr, col, lane_on);
-    uint32_t cell = resolved_tok[k];
     const float wk = f16_to_f32(routing_tok[k]);
-    if (cell == kSentinel && fallback_tok) cell = fallback_tok[k];  // moe.metal:1037-1038
-    const bool live = cell != kSentinel;
-    const uint8_t *base = cell_base_uniform(a.pool, live ? cell : 0u, a.stride);
+    bool live;
+    const uint8_t *base;
+    if (a.blobs) {  // moe.metal:924: the blob the argument buffer names for this position
+        base = a.blobs[k];
+        live = base != nullptr;
+    } else {
+        uint32_t cell = resolved_tok[k];
+        if (cell == kSentinel && fallback_tok) cell = fallback_tok[k];  // moe.metal:1037-1038
+        live = cell != kSentinel;
+        base = cell_base_uniform(a.pool, live ? cell : 0u, a.stride);
+    }
     const uint16_t *s_all = reinterpret_cast<const uint16_t *>(base + a.off.down_s_off);
     const uint16_t *b_all = reinterpret_cast<const uint16_t *>(base + a.off.down_b_off);
 
@@ -266,6 +273,27 @@ int shrike_hip_moe_phase2_pool(shrike_hip_moe *moe, void *stream, const shrike_p
     a.y = static_cast<uint16_t *>(d_y); a.hidden = static_cast<uint16_t *>(d_hidden);
     a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.ebias = moe->desc.expert_additive_biases;
     a.indirect = d_indirect; a.io_status = moe->desc.event_gated_io ? d_io_status : nullptr;
+    return launch_phase2(a, bits, as_stream(stream));
+}
+
+int shrike_hip_moe_phase2_blobs(shrike_hip_moe *moe, void *stream, const void *const *d_routed_blobs,
+                                const shrike_expert_offsets *offsets, const void *d_acts, const void *d_routing_weights,
+                                const void *d_residual, void *d_y, void *d_hidden, uint32_t d, uint32_t f, uint32_t top_k,
+                                const uint32_t *d_io_status) {
+    SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
+    SHRIKE_REQUIRE(top_k >= 1 && top_k <= SHRIKE_MAX_TOP_K, "phase2: topK=%u not in 1...8", top_k);
+    const uint32_t bits = moe->desc.routed_weight_bits;
+    if (int rc = check_offsets(offsets, d, f, bits)) return rc;
+    SHRIKE_REQUIRE(d_routed_blobs && d_acts && d_routing_weights && d_residual && d_y,
+                   "phase2: the argument buffer, acts, routingWeights, residual and y must be bound");
+    Phase2Args a = {};
+    a.blobs = reinterpret_cast<const uint8_t *const *>(d_routed_blobs);
+    a.off = *offsets;
+    a.acts = static_cast<const uint16_t *>(d_acts); a.routing_w = static_cast<const uint16_t *>(d_routing_weights);
+    a.residual = static_cast<const uint16_t *>(d_residual);
+    a.y = static_cast<uint16_t *>(d_y); a.hidden = static_cast<uint16_t *>(d_hidden);
+    a.d = d; a.f = f; a.top_k = top_k; a.meta = moe->desc.meta_dtype; a.ebias = moe->desc.expert_additive_biases;
+    a.io_status = moe->desc.event_gated_io ? d_io_status : nullptr;
     return launch_phase2(a, bits, as_stream(stream));
 }
 

@@ -332,6 +332,27 @@ class MoE:
             C.byref(offsets), ptr(acts), ptr(routing_weights), ptr(residual), ptr(y), ptr(hidden),
             d, f, top_k, ptr(indirect), ptr(io_status)), "shrike_hip_moe_phase2_pool")
 
+    def make_routed_argument_buffer(self, blob_ptrs, buffer: "DeviceBuffer | None" = None) -> "DeviceBuffer":
+        """MoE.makeReusedRoutedArgumentBuffer (MoE.swift:612-620): the device array of the route's blob pointers."""
+        words = np.asarray(list(blob_ptrs), np.uint64)
+        buffer = buffer or empty(8 * capi.MAX_TOP_K).fill(0)
+        buffer.upload(words)
+        return buffer
+
+    def encode_routed_persistent_phase1(self, routed_arg_buffer, offsets, x, acts, d, f, top_k, active_slots=None,
+                                        active_count=0, io_status=None):
+        """encodeRoutedPersistentPhase1U16Load, and with active_slots encodeRoutedPersistentPhase1SubsetU16Load."""
+        check(capi.load().shrike_hip_moe_phase1_blobs(
+            self.handle, self._s(), ptr(routed_arg_buffer), C.byref(offsets), ptr(x), ptr(acts), d, f, top_k,
+            ptr(active_slots), active_count, ptr(io_status)), "shrike_hip_moe_phase1_blobs")
+
+    def encode_routed_persistent_phase2(self, routed_arg_buffer, offsets, acts, routing_weights, residual, y, hidden,
+                                        d, f, top_k, io_status=None):
+        """encodeRoutedPersistentPhase2Reduce."""
+        check(capi.load().shrike_hip_moe_phase2_blobs(
+            self.handle, self._s(), ptr(routed_arg_buffer), C.byref(offsets), ptr(acts), ptr(routing_weights),
+            ptr(residual), ptr(y), ptr(hidden), d, f, top_k, ptr(io_status)), "shrike_hip_moe_phase2_blobs")
+
     def encode_resolve_batch(self, topk, residency, resolved_slots, count, num_experts, miss_count=None):
         check(capi.load().shrike_hip_moe_resolve_batch(self._s(), ptr(topk), ptr(residency), ptr(resolved_slots), count,
                                                        num_experts, ptr(miss_count)), "shrike_hip_moe_resolve_batch")

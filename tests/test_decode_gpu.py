@@ -247,6 +247,57 @@ def test_phase1_phase2_against_oracle(gpu, bits, meta, d, f):
     assert np.array_equal(got_hidden, expect_hidden)
 
 
+@pytest.mark.parametrize("bits,d,f,k", [(4, 2048, 512, 8), (8, 256, 128, 4), (4, 2880, 384, 3)])
+def test_argument_buffer_operators(gpu, bits, d, f, k):
+    """encodeRoutedPersistentPhase1U16Load / ...SubsetU16Load / ...Phase2Reduce: the route's blobs named by a device
+    array of pointers. Against the oracle, and byte for byte the pool operators' results over the same blobs."""
+    L = Layer(0x5EED0A00 + d + bits, d, f, k + 2, k, bits=bits)
+    dl = DeviceLayer(gpu, L)
+    order = [(3 * p + 1) % (k + 2) for p in range(k)]  # position p's expert
+    cells = np.array([dl.cell_of[e] for e in order], np.uint32)
+    arg = dl.moe.make_routed_argument_buffer([dl.pool.cell_ptr(int(c)) for c in cells])
+    blobs = [dl.pool_blobs()[int(c)] for c in cells]
+    acts0 = S.f32_to_f16_bits(np.full(k * f, 0.25, np.float32))
+    # all positions
+    dl.acts.upload(acts0)
+    dl.moe.encode_routed_persistent_phase1(arg, dl.off, dl.x, dl.acts, d, f, k)
+    acts = dl.acts.download(np.uint16, k * f)
+    ref_acts = O.moe_phase1(blobs, L.oracle_offsets(), L.x, d, f, bits=bits, acts=acts0.copy())
+    assert_ffn_close(acts, ref_acts, "argument-buffer phase-1 acts")
+    dl.acts.upload(acts0)
+    dl.moe.encode_spec_phase1(dl.pool, gpu.dev(cells), dl.off, dl.x, dl.acts, d, f, k)
+    assert np.array_equal(acts, dl.acts.download(np.uint16, k * f))
+    # a subset: listed positions only, in list order, an entry past top_k skipped
+    active = np.array([k - 1, 0, k + 5], np.uint32)
+    dl.acts.upload(acts0)
+    dl.moe.encode_routed_persistent_phase1(arg, dl.off, dl.x, dl.acts, d, f, k, active_slots=gpu.dev(active), active_count=3)
+    sub = dl.acts.download(np.uint16, k * f)
+    for p in range(k):
+        want = acts if p in (0, k - 1) else acts0
+        assert np.array_equal(sub[p * f:(p + 1) * f], want[p * f:(p + 1) * f]), p
+    dl.acts.upload(acts0)
+    dl.moe.encode_routed_persistent_phase1(arg, dl.off, dl.x, dl.acts, d, f, k, active_slots=gpu.dev(active), active_count=0)
+    assert np.array_equal(dl.acts.download(np.uint16, k * f), acts0)
+    # phase 2 over the argument buffer
+    w = S.f32_to_f16_bits(L.tree.key("w").uniform(0.05, 0.3, k))
+    residual = S.activations_f16(L.tree, "residual", d)
+    dl.acts.upload(ref_acts)
+    dw, dr = gpu.dev(w), gpu.dev(residual)
+    dl.moe.encode_routed_persistent_phase2(arg, dl.off, dl.acts, dw, dr, dl.y, dl.hidden, d, f, k)
+    y, hidden = dl.y.download(np.uint16, d), dl.hidden.download(np.uint16, d)
+    ref_y = O.moe_phase2(blobs, L.oracle_offsets(), ref_acts, w, residual, d, f, bits=bits, hidden_f16=L.hidden.copy())
+    assert_ffn_close(y, ref_y, "argument-buffer phase-2 y")
+    assert np.array_equal(hidden, O.residual_add_f16(L.hidden.copy(), y))
+    dl.hidden.upload(L.hidden)
+    dl.moe.encode_spec_phase2(dl.pool, gpu.dev(cells), dl.off, dl.acts, dw, dr, dl.y, dl.hidden, d, f, k)
+    assert np.array_equal(y, dl.y.download(np.uint16, d)) and np.array_equal(hidden, dl.hidden.download(np.uint16, d))
+    # an unbound argument buffer is an error, not a fault
+    with pytest.raises(capi.ShrikeError, match="argument buffer"):
+        dl.moe.encode_routed_persistent_phase1(None, dl.off, dl.x, dl.acts, d, f, k)
+    with pytest.raises(capi.ShrikeError, match="activeCount"):
+        dl.moe.encode_routed_persistent_phase1(arg, dl.off, dl.x, dl.acts, d, f, k, active_slots=gpu.dev(active), active_count=9)
+
+
 def test_phase2_fallback_cells_and_indirect_zero_grid(gpu):
     d, f, k = 256, 128, 4
     L = Layer(11, d, f, k, k)
