@@ -861,6 +861,8 @@ class AgreedDecodeLayer:
         self.hit_pos, self.miss_pos, self.miss_exp = empty(32), empty(32), empty(32)
         self.spec_args = empty(48)
         self.predicted = empty(4 * 8).fill(0)
+        self.predicted_w = empty(2 * 8)
+        self.predicted_next = []
         self.readback = PinnedBuffer(4 * (2 + 5 * k))
         self.acts = empty(2 * k * moe.desc.f)
         self.tag = 0
@@ -926,15 +928,26 @@ class AgreedDecodeLayer:
         except Exception:
             self.ring.note_hook_failure()
 
-    def run(self, router, x, residual, y, hidden):
+    def run(self, router, x, residual, y, hidden, probe=None):
         """router: dict(weights, scales, biases, eff_scale, expert_scale, bias). x: fp16[d], residual: fp16[d],
-        y: fp16[d] out, hidden: fp16[d] updated in place. Returns the route's plan."""
+        y: fp16[d] out, hidden: fp16[d] updated in place. Returns the route's plan.
+        probe: the following layer's router (same dict), or None. With it the router runs as the reference's pair
+        (MoE.encodeRouterPair, RealForwardRunner.swift:2861): the second router over this layer's x names the experts
+        the following layer is likely to want; they come back with the classifier's tagged readback and are left in
+        `self.predicted_next` for the caller to hand to that layer's prefetch."""
         m = self.moe
         d, f, ne, k = m.desc.d, m.desc.f, m.desc.num_experts, m.desc.top_k
         compute = m.stream
         self._publish()
-        m.encode_router(router["weights"], router.get("scales"), router.get("biases"), x, router["eff_scale"],
-                        router["expert_scale"], router["bias"], self.idx, self.w, ne, d, k)
+        if probe is None:
+            m.encode_router(router["weights"], router.get("scales"), router.get("biases"), x, router["eff_scale"],
+                            router["expert_scale"], router["bias"], self.idx, self.w, ne, d, k)
+        else:
+            def operands(r, out_indices, out_weights):
+                return dict(weights=r["weights"], scales=r.get("scales"), biases=r.get("biases"),
+                            effective_scale=r["eff_scale"], logit_bias=r["bias"], out_indices=out_indices, out_weights=out_weights)
+            m.encode_router_pair(operands(router, self.idx, self.w), operands(probe, self.predicted, self.predicted_w), x,
+                                 router["expert_scale"], ne, d, k)
         self.tag = self.tag % 0xFFFF + 1
         m.encode_residency_classification(self.idx, self.pool.table, self.hit_count, self.hit_pos, self.miss_count,
                                           self.miss_pos, self.miss_exp, self.resolved, k, ne, full_grids=[1] * 12,
@@ -952,6 +965,7 @@ class AgreedDecodeLayer:
         misses = int(rb[1])
         experts = rb[2:2 + k].tolist()
         miss_positions = rb[2 + 3 * k: 2 + 3 * k + misses].tolist()
+        self.predicted_next = rb[2 + 4 * k: 2 + 5 * k].tolist() if probe is not None else []
 
         # joinAgreedLandings, :5262-5267
         leased = self.ring.ready_cells(self.layer, experts, self.JOIN_NANOS)

@@ -120,6 +120,9 @@ def test_two_layers_share_one_arena_and_one_ring(gpu):
     cells = sum(slots) + ring_cells
     layers = [Layer(0x5EED00A1, d, f, ne, k, bits=4), Layer(0x5EED00A2, d, f, ne, k, bits=4)]
     inputs = [token_inputs(L, tokens) for L in layers]
+    # the second layer routes on what the first one routed on (what is between two MoE layers is left out): the
+    # first layer's router pair, whose second router is the second layer's, then foresees the second layer's experts
+    inputs[1] = [(inputs[0][t][0], inputs[1][t][1]) for t in range(tokens)]
     want = []
     for L, ins in zip(layers, inputs):
         full, rows = DeviceLayer(gpu, L), []
@@ -154,12 +157,7 @@ def test_two_layers_share_one_arena_and_one_ring(gpu):
         devs.append(dev)
         stores.append(store)
     residual = gpu.dev(np.zeros(d, np.uint16))
-    rng = np.random.default_rng(7)
-
-    def predictions(layer_index, token):
-        coming = want[layer_index][token][0]
-        right = [e for e in coming if rng.random() < 0.6]
-        return right + [int(e) for e in rng.choice(ne, 2, replace=False) if e not in coming]
+    foreseen = []
 
     try:
         for t in range(tokens):
@@ -168,7 +166,8 @@ def test_two_layers_share_one_arena_and_one_ring(gpu):
                 x, hidden = inputs[index][t]
                 dev.x.upload(x)
                 dev.hidden.upload(hidden)
-                agreed[index].run(routers[index], dev.x, residual, dev.y, dev.hidden)
+                # MoE.encodeRouterPair: this layer's router and, as the probe, the following layer's over the same x
+                agreed[index].run(routers[index], dev.x, residual, dev.y, dev.hidden, probe=routers[1 - index])
                 stream.synchronize()
                 idx, y, hid = want[index][t]
                 assert agreed[index].idx.download(np.uint32, k).tolist() == idx, f"token {t} layer {index}: routes"
@@ -178,7 +177,12 @@ def test_two_layers_share_one_arena_and_one_ring(gpu):
                 # the runner schedules the next layer's predictions while this layer's reads are behind it
                 following, at = (1, t) if index == 0 else (0, t + 1)
                 if at < tokens:
-                    agreed[following].prefetch(predictions(following, at))
+                    predicted = agreed[index].predicted_next
+                    assert len(predicted) == k and all(0 <= e < ne for e in predicted)
+                    if index == 0:  # the probe saw the very row the second layer routes on: it names its experts exactly
+                        assert sorted(predicted) == sorted(want[1][t][0])
+                    foreseen.append(len(set(predicted) & set(want[following][at][0])))
+                    agreed[following].prefetch(predicted)
                     wait_for_the_ring(ring)
             owned = [caches[i].slot_cell(s) for i in (0, 1) for s in range(slots[i])]
             assert len(set(owned)) == sum(slots), "two slots name one cell"
@@ -189,7 +193,7 @@ def test_two_layers_share_one_arena_and_one_ring(gpu):
     moved = [sum(1 for s in range(slots[i]) if not (i * slots[0] <= caches[i].slot_cell(s) < slots[0] + i * slots[1]))
              for i in (0, 1)]
     hits = [a.landed_hits for a in agreed]
-    print(f"\ntwo layers: landed hits {hits}, slots now on cells outside their first range {moved}, "
+    print(f"\ntwo layers: experts foreseen by the router pair per step {foreseen}, landed hits {hits}, slots now on cells outside their first range {moved}, "
           f"overflow {[a.overflows for a in agreed]}, ring {ring.statistics}")
     assert sum(hits) > 0 and sum(moved) > 0
     for cache in caches:
