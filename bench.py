@@ -579,7 +579,7 @@ def decode_workload(args, rt, capi, S, meta):
     launch2_us = parts["launch 2: select + routed gate/up rows + shared down rows (k_phase1, routing)"]
     alone_us = parts["operator: phase 1 alone (no routing, no shared rows)"]
     value = expert_bytes / (ms_per_step * 1e-3) / 1e9
-    kernel = "k_phase1<4,1,4,true,4>"
+    kernel = "k_phase1<4,1,4,true,4,true>"
     out = {
         "metric": "MoE-layer decode: HBM GB/s on expert bytes (us per layer in ms_per_step), 35B-A3B int4 shape",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warm,
