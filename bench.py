@@ -231,6 +231,25 @@ def cpu_baseline(S, blobs, sample_layers, meta):
                         "sample": f"{singles} experts drawn from the pool, one thread"}}
 
 
+def cpu_pairs(S, blobs, d, f, bits, meta, pairs, evaluations, label):
+    """The oracle's fp32 port of one step's expert FFNs on this host's cores: `pairs` (token, expert) FFN evaluations,
+    one task each (sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:102-140 with the generic-bit body), every one over the
+    same activation row (the cost of an evaluation does not depend on the row)."""
+    from oracle import oracle as O
+    off, _ = O.expert_offsets(d, f, bits)
+    cores = min(pairs, len(os.sched_getaffinity(0)))
+    x = S.SeedTree(0xC0FFEE).key("x").normal(d)
+    rng = np.random.default_rng(1)
+    weights = np.full(pairs, 1.0 / pairs, np.float32)
+    t0 = time.perf_counter()
+    for _ in range(evaluations):
+        picks = rng.choice(len(blobs), pairs, replace=pairs > len(blobs))
+        O.cpu_layer_fp32([blobs[int(e)] for e in picks], weights, off, x, d, f, cores, bits=bits, meta=meta)
+    per_step = (time.perf_counter() - t0) / evaluations
+    return {"us_per_step": round(per_step * 1e6, 1), "cores": cores, "kind": "port",
+            "sample": f"{evaluations} evaluations of {label}, fp32 scalar C port, {cores} threads, gcc -O2"}
+
+
 def prefill_workload(args, rt, capi, S, meta):
     """Config 3: one ragged prefill chunk of T tokens through router -> grouping -> grouped expert FFN
     -> reduce, top-8 of 256 int4 experts with a Zipf skew injected through the router's logit-bias
@@ -297,7 +316,12 @@ def prefill_workload(args, rt, capi, S, meta):
     flops = T * K * 6 * D * F
     ffn_us = parts["grouped FFN (4 launches)"]
     traffic = profile_figure("prefill_chunk_q35b_int4_t512.txt", "hbm_bytes_per_chunk_grouped_ffn") if T == 512 else None
+    cpu = None
+    if getattr(args, "cpu_sample", 0) > 0:  # the chunk's T * K pair FFNs on the host's cores
+        cpu = cpu_pairs(S, keep[4], D, F, BITS, meta, T * K, 1, f"one chunk's {T * K} pair FFNs at the 35B-A3B shape, int4")
+        cpu["us_per_chunk"] = cpu.pop("us_per_step")
     return {
+        **({"cpu_baseline": cpu} if cpu else {}),
         "metric": "ragged prefill chunk through the routed experts: tokens/s (ms per chunk in ms_per_step), 35B-A3B int4 shape",
         "value": round(T / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 x u4 -> f32",
@@ -337,6 +361,10 @@ def gptoss_workload(args, rt, capi, S, meta, bits):
             pool.publish(e, e, capi.RESIDENT)
         pools.append(pool)
         routers.append(rt.dev(S.router_f16(tree, f"layer.{l}.router.w", ne, d)))
+    cpu = None
+    if getattr(args, "cpu_sample", 0) > 0:  # one layer's 16 (token, expert) FFNs on the host's cores
+        cpu = cpu_pairs(S, blobs, d, f, bits, meta, t * k, 3, f"one layer's {t * k} expert FFNs at the gpt-oss shape, int{bits}")
+        cpu["us_per_layer"] = cpu.pop("us_per_step")
     del blobs
     moe = rt.MoE(d, f, ne, k, routed_bits=bits, router_bits=0, meta=meta)
     stream = rt.Stream()
@@ -389,7 +417,8 @@ def gptoss_workload(args, rt, capi, S, meta, bits):
                    "distinct_experts_per_layer": distinct, "expert_bytes_per_stack": expert_bytes,
                    "pair_bytes_per_stack": n_layers * t * k * stride, "meta_dtype": args.meta},
         "GBps_on_pair_bytes": round(n_layers * t * k * stride / (ms * 1e-3) / 1e9, 2),
-        "hbm_peak_frac_on_expert_bytes": round(expert_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+        "hbm_peak_frac_on_expert_bytes": round(expert_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        **({"cpu_baseline": cpu} if cpu else {})}
 
 
 def kimi_workload(args, rt, capi, S, meta):
@@ -435,6 +464,10 @@ def kimi_workload(args, rt, capi, S, meta):
     dt = time.perf_counter() - t0
     st = cache.statistics(stride)
     req, miss, read, plans = st.requested_experts - base[0], st.misses - base[1], st.bytes_read - base[2], st.plans - base[3]
+    cpu = None
+    if getattr(args, "cpu_sample", 0) > 0:  # one step's 128 routed + 16 shared-expert FFNs on the host's cores
+        views = [store.array[e * stride:e * stride + stride] for e in range(0, ne, 4)]
+        cpu = cpu_pairs(S, views, d, f, bits, meta, t * k + t, 2, f"one step's {t * k} routed and {t} shared-expert FFNs at the Kimi shape, int8")
     return {
         "metric": "Kimi-Linear-48B-shape MoE decode, 16 sequences through a 64-of-256 slot pool: ms per step (wall clock, misses included)",
         "value": round(t / (dt / steps), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
@@ -444,7 +477,8 @@ def kimi_workload(args, rt, capi, S, meta):
                                f"pool of {slots} cells, misses from pinned host memory on a side stream",
                    "passes_per_step": round(plans / steps, 2)},
         "miss_rate": round(miss / max(1, req), 4), "experts_requested_per_step": round(req / steps, 1),
-        "host_to_device_GBps": round(read / dt / 1e9, 2), "bytes_copied_per_step": int(read / steps)}
+        "host_to_device_GBps": round(read / dt / 1e9, 2), "bytes_copied_per_step": int(read / steps),
+        **({"cpu_baseline": cpu} if cpu else {})}
 
 
 def decode_workload(args, rt, capi, S, meta):
@@ -665,7 +699,7 @@ def main():
             secondary[name] = {k: r[k] for k in r if k in ("metric", "value", "unit", "ms_per_step", "us_per_layer", "config",
                                                            "kernel_us_per_chunk", "roofline", "GBps_on_pair_bytes",
                                                            "hbm_peak_frac_on_expert_bytes", "miss_rate", "host_to_device_GBps",
-                                                           "bytes_copied_per_step", "experts_requested_per_step", "steps", "dtype")}
+                                                           "bytes_copied_per_step", "experts_requested_per_step", "steps", "dtype", "cpu_baseline")}
         out["secondary"] = secondary
     print(json.dumps(out))
 
