@@ -223,16 +223,18 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
     const uint32_t scale_misalign = uint32_t((reinterpret_cast<uintptr_t>(bs[0]) | reinterpret_cast<uintptr_t>(bs[1])) & 7u);
     const bool wide_scales = (G & 3u) == 0u && __builtin_amdgcn_readfirstlane(int(scale_misalign)) == 0;
     uint2 scales_cur[2] = {make_uint2(0u, 0u), make_uint2(0u, 0u)}, scales_nxt[2] = {make_uint2(0u, 0u), make_uint2(0u, 0u)};
-    BRegs<BITS> cur[2], nxt[2];
+    // the codes of one group (8-bit) or two (4-bit, where the registers allow it) are on their way while a group is multiplied
+    constexpr uint32_t kAhead = BITS == 4 ? 2u : 1u;
+    BRegs<BITS> cur[2], nxt[2], nx2[2];
     const uint32_t chunks = (K + kChunkK - 1u) / kChunkK;
 
-    // One group of 64 k: the next group's codes are put in flight, this group's are unpacked and
+    // One group of 64 k: the codes of the group kAhead further on are put in flight, this group's are unpacked and
     // multiplied, and the products are scaled into the totals.
     auto group_step = [&](uint32_t c, uint32_t buf, uint32_t gi, auto wide_tag) {
         constexpr bool WIDE = decltype(wide_tag)::value;
-        const uint32_t gn = min(kGroupsPerChunk * c + gi + 1u, G - 1u);
+        const uint32_t gn = min(kGroupsPerChunk * c + gi + kAhead, G - 1u);
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) load_b<BITS>(nxt[nt], bw[nt], WIDE ? nullptr : bs[nt], gn, kb);
+        for (int nt = 0; nt < 2; ++nt) load_b<BITS>(kAhead == 2u ? nx2[nt] : nxt[nt], bw[nt], WIDE ? nullptr : bs[nt], gn, kb);
         half8 af[MT][4];
 #pragma unroll
         for (uint32_t mt = 0; mt < MT; ++mt)
@@ -258,6 +260,10 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
         }
         cur[0] = nxt[0];
         cur[1] = nxt[1];
+        if (kAhead == 2u) {
+            nxt[0] = nx2[0];
+            nxt[1] = nx2[1];
+        }
     };
     auto main_loop = [&](auto wide_tag) {
         constexpr bool WIDE = decltype(wide_tag)::value;
@@ -265,6 +271,7 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt) {
                 load_b<BITS>(cur[nt], bw[nt], WIDE ? nullptr : bs[nt], 0, kb);
+                if (kAhead == 2u) load_b<BITS>(nxt[nt], bw[nt], WIDE ? nullptr : bs[nt], min(1u, G - 1u), kb);
                 if (WIDE) scales_cur[nt] = *reinterpret_cast<const uint2 *>(bs[nt]);
             }
         }
