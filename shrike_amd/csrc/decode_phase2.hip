@@ -7,7 +7,8 @@
 
 namespace shrike {
 
-constexpr uint32_t kPhase2Rows = 8;  // output rows per workgroup
+constexpr uint32_t kPhase2Rows = 8;       // output rows per workgroup
+constexpr uint32_t kPhase2RowsBatch = 16;  // the same for a batch of tokens over rows of more than one wave load
 
 // moe.metal:889-893
 __device__ __forceinline__ void phase2_finish(uint16_t *y, uint16_t *hidden, uint32_t d, uint16_t value,
@@ -20,10 +21,13 @@ __device__ __forceinline__ void phase2_finish(uint16_t *y, uint16_t *hidden, uin
 // rows. When a down row is shorter than a wave's 1 KiB load, the wave covers 64/cpr rows per
 // load and reduces over lane segments. BATCH row groups are in flight per wave.
 // STREAM: one token, every down row is read once: non-temporal row loads (see k_phase1).
-template <int BITS, int NCH, int BATCH, bool STREAM>
+// ROWS: output rows a workgroup owns. One token takes 8 (at d = 2048 that is one workgroup a compute unit); a batch of
+// tokens over long rows takes 16, so that a wave's slice of the activations, fetched once, serves twice the rows.
+template <int BITS, int NCH, int BATCH, bool STREAM, uint32_t ROWS>
 __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
+    constexpr uint32_t kPhase2Rows = ROWS;
     __shared__ float partial[SHRIKE_MAX_TOP_K][kPhase2Rows];
     if (a.indirect && a.indirect[0] == 0u) return;
     // a batch of tokens: grid.y is this workgroup's token (the argument block itself stays untouched)
@@ -119,30 +123,37 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
     gemv_job<BITS, NCH>(a, blockIdx.x);
 }
 
-template <int BITS, int NCH>
-static void launch_phase2_batch(const Phase2Args &a, dim3 grid, dim3 block, hipStream_t s) {
+template <int BITS, int NCH, uint32_t ROWS>
+static void launch_phase2_rows(const Phase2Args &a, dim3 block, hipStream_t s) {
+    const dim3 grid((a.d + ROWS - 1) / ROWS, a.tokens ? a.tokens : 1u);
     const uint32_t cpr = a.f * BITS / 128u;
-    const uint32_t rpl = (cpr < 64u && 64u % cpr == 0u) ? (64u / cpr < kPhase2Rows ? 64u / cpr : kPhase2Rows) : 1u;
-    const uint32_t n_groups = kPhase2Rows / rpl;  // row groups per wave; up to 4 in flight
+    const uint32_t rpl = (cpr < 64u && 64u % cpr == 0u) ? (64u / cpr < ROWS ? 64u / cpr : ROWS) : 1u;
+    const uint32_t n_groups = ROWS / rpl;  // row groups per wave; up to 4 in flight
     if (a.tokens <= 1u) {
-        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, true>), grid, block, 0, s, a);
-        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, true>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, true>), grid, block, 0, s, a);
+        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, true, ROWS>), grid, block, 0, s, a);
+        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, true, ROWS>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, true, ROWS>), grid, block, 0, s, a);
     } else {
-        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, false>), grid, block, 0, s, a);
-        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, false>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, false>), grid, block, 0, s, a);
+        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, false, ROWS>), grid, block, 0, s, a);
+        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, false, ROWS>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, false, ROWS>), grid, block, 0, s, a);
     }
+}
+
+template <int BITS, int NCH>
+static void launch_phase2_batch(const Phase2Args &a, dim3 block, hipStream_t s) {
+    if (NCH >= 2 && a.tokens > 1u) launch_phase2_rows<BITS, NCH, kPhase2RowsBatch>(a, block, s);
+    else launch_phase2_rows<BITS, NCH, kPhase2Rows>(a, block, s);
 }
 
 template <int BITS>
 static void launch_phase2_bits(const Phase2Args &a, hipStream_t s) {
-    const dim3 grid((a.d + kPhase2Rows - 1) / kPhase2Rows, a.tokens ? a.tokens : 1u), block(64 * a.top_k);
+    const dim3 block(64 * a.top_k);
     switch (nch_for(a.f, BITS)) {
-        case 1: launch_phase2_batch<BITS, 1>(a, grid, block, s); break;
-        case 2: launch_phase2_batch<BITS, 2>(a, grid, block, s); break;
-        case 3: launch_phase2_batch<BITS, 3>(a, grid, block, s); break;
-        default: launch_phase2_batch<BITS, 4>(a, grid, block, s); break;
+        case 1: launch_phase2_batch<BITS, 1>(a, block, s); break;
+        case 2: launch_phase2_batch<BITS, 2>(a, block, s); break;
+        case 3: launch_phase2_batch<BITS, 3>(a, block, s); break;
+        default: launch_phase2_batch<BITS, 4>(a, block, s); break;
     }
 }
 
