@@ -152,6 +152,18 @@ class Event:
         check(capi.load().shrike_hip_event_elapsed_ms(self.handle, later.handle, C.byref(ms)), "event_elapsed")
         return ms.value
 
+    def close(self):
+        """Destroys the event (work already enqueued that waits for it is not affected)."""
+        if self.handle:
+            capi.load().shrike_hip_event_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
 
 def expert_offsets(d: int, f: int, bits: int = 4, additive_biases: bool = False):
     off = ExpertOffsets()
