@@ -305,7 +305,7 @@ def prefill_workload(args, rt, capi, S, meta):
     timed(step, warm)
     ms = timed(step, steps, regions=5)
     parts = {name: timed(fn, max(6, steps // 2), regions=3) * 1e3 for name, fn in
-             (("router (2 launches)", router), ("grouping (1 launch)", group), ("grouped FFN (4 launches)", ffn), ("reduce", reduce))}
+             (("router (2 launches)", router), ("grouping (1 launch)", group), ("grouped FFN (3 launches)", ffn), ("reduce", reduce))}
     rt.synchronize()
     counts = routes.counts.download(np.uint32, NE)
     tiles = int(routes.row_tile_count.download(np.uint32, 1)[0])
@@ -314,7 +314,7 @@ def prefill_workload(args, rt, capi, S, meta):
     expert_bytes = used * stride
     algorithmic = expert_bytes + 2 * T * D * 2 + T * K * 16
     flops = T * K * 6 * D * F
-    ffn_us = parts["grouped FFN (4 launches)"]
+    ffn_us = parts["grouped FFN (3 launches)"]
     traffic = profile_figure("prefill_chunk_q35b_int4_t512.txt", "hbm_bytes_per_chunk_grouped_ffn") if T == 512 else None
     cpu = None
     if getattr(args, "cpu_sample", 0) > 0:  # the chunk's T * K pair FFNs on the host's cores

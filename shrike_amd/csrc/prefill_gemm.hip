@@ -114,6 +114,10 @@ __device__ __forceinline__ half8 b_step(const BRegs<BITS> &r, int s) {
 // One row tile against one block of weight rows. MT = the tile's 32-row MFMA tiles, a template
 // parameter so that the main loop is straight-line code: the compiler is then free to put one
 // chain's matrix instructions beside another chain's vector work.
+// MODE 0 leaves its activations through LDS: whole 16-byte pieces of a row go out together, and the group sums of the
+// tile's rows that the down product's bias term needs are formed here, in k_row_group_sums' order of additions (eight
+// lanes a group, a lane adds its eight values in order, the partial sums fold pairwise), instead of by a launch of
+// their own between the two products. Every wave of the workgroup stays to the end for the barriers.
 template <int BITS, int MODE, bool DENSE, uint32_t MT>
 __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile &tile, uint32_t tile_index, uint32_t col_block,
                                          uint16_t (&s_a)[2][kRowTile][kLdsRow]) {
@@ -302,11 +306,11 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
     };
     if (wide_scales) main_loop(std::true_type{});
     else main_loop(std::false_type{});
-    if (!active) return;
+    if (MODE != 0 && !active) return;
 
     // ---- bias term: (group sums of the rows) x (group biases), sixteen k' = eight groups an MFMA.
     // The operands of four steps are fetched together, four values a load where the rows allow it.
-    {
+    if (active) {
         // a lane's four groups are one aligned 8- or 16-byte run when G is a multiple of 4 and the bias rows start aligned
         const bool wide = (G & 3u) == 0u && ((reinterpret_cast<uintptr_t>(bb[0]) | reinterpret_cast<uintptr_t>(bb[1])) & 7u) == 0u;
         for (uint32_t gbase = 0; gbase < G; gbase += 32u) {
@@ -357,26 +361,52 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
     // ---- epilogue: lane holds (m = 32 mt + 8 (i / 4) + 4 kb + i % 4, n = n0 + col)
     const uint32_t n = n0 + col;
     if (MODE == 0) {
-        float gab = 0.0f, uab = 0.0f;
-        if (!DENSE && a.ebias) {  // moe.metal:261-269
-            gab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.gate_ab_off)[n]);
-            uab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.up_ab_off)[n]);
-        }
+        // the main loop ended on a barrier: nobody reads the staged rows any more, and the first buffer takes the
+        // tile's fp16 activations, [row][column of this block of 128]
+        if (active) {
+            float gab = 0.0f, uab = 0.0f;
+            if (!DENSE && a.ebias) {  // moe.metal:261-269
+                gab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.gate_ab_off)[n]);
+                uab = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.up_ab_off)[n]);
+            }
 #pragma unroll
-        for (uint32_t mt = 0; mt < MT; ++mt) {
+            for (uint32_t mt = 0; mt < MT; ++mt) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
-                if (m < tile.rows) {
+                for (int i = 0; i < 16; ++i) {
+                    const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
                     float g = total[0][mt][i] + gab, u = total[1][mt][i] + uab;
                     if (DENSE && a.round_gate_up) {
                         g = f16_to_f32(f32_to_f16(g));
                         u = f16_to_f32(f32_to_f16(u));
                     }
-                    const float act = glu_rt(g, u, a.act_kind);
-                    a.act[(size_t(tile_index) * kRowTile + m) * a.f + n] = f32_to_f16(act);
+                    s_a[0][m][wave * 32u + col] = f32_to_f16(glu_rt(g, u, a.act_kind));
                 }
             }
+        }
+        __syncthreads();
+        const uint32_t c0 = col_block * 128u, columns = min(128u, N - c0);  // N is a multiple of 64
+        for (uint32_t idx = threadIdx.x; idx < tile.rows * 16u; idx += 256u) {
+            const uint32_t m = idx >> 4, pc = idx & 15u;
+            if (pc * 8u < columns)
+                *reinterpret_cast<uint4 *>(a.act + (size_t(tile_index) * kRowTile + m) * a.f + c0 + pc * 8u) =
+                    *reinterpret_cast<const uint4 *>(&s_a[0][m][pc * 8u]);
+        }
+        uint32_t *sums_out = const_cast<uint32_t *>(a.act_sums);
+        for (uint32_t slot = threadIdx.x; slot < kRowTile * 16u; slot += 256u) {  // (row, group of the block, eighth)
+            const uint32_t m = slot >> 4, gl = (slot >> 3) & 1u, eighth = slot & 7u;
+            const uint4 v = *reinterpret_cast<const uint4 *>(&s_a[0][m][gl * 64u + eighth * 8u]);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            float sum = 0.0f;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                sum = __fadd_rn(sum, f16_to_f32(uint16_t(w[t])));
+                sum = __fadd_rn(sum, f16_to_f32(uint16_t(w[t] >> 16)));
+            }
+            sum = __fadd_rn(sum, __shfl_xor(sum, 1));
+            sum = __fadd_rn(sum, __shfl_xor(sum, 2));
+            sum = __fadd_rn(sum, __shfl_xor(sum, 4));
+            if (eighth == 0u && m < tile.rows && gl * 64u < columns)
+                sums_out[(size_t(tile_index) * kRowTile + m) * (a.f / kGroup) + c0 / kGroup + gl] = split_hi_lo(sum);
         }
     } else {
         // a call over a range of the sorted pairs writes the rows of its pairs only
@@ -461,7 +491,7 @@ static int launch_ffn(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
     const uint32_t grid_tiles = (max_tiles + 7u) & ~7u;  // whole runs for the kernel's XCD mapping
     hipLaunchKernelGGL((k_grouped_ffn<BITS, 0, DENSE>), dim3(grid_tiles, (a.f + 127u) / 128u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
-    if (int rc = launch_row_group_sums(a.act, a.f, max_tiles * kRowTile, a.f, const_cast<uint32_t *>(a.act_sums), a.tile_count, s)) return rc;
+    // (the activations' group sums were written by the gate/up launch itself)
     hipLaunchKernelGGL((k_grouped_ffn<BITS, 1, DENSE>), dim3(grid_tiles, (a.d + 255u) / 256u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     return 0;
