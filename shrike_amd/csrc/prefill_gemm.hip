@@ -306,7 +306,7 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
     };
     if (wide_scales) main_loop(std::true_type{});
     else main_loop(std::false_type{});
-    if (MODE != 0 && !active) return;
+    // (no wave leaves here: the epilogue's barrier needs them all)
 
     // ---- bias term: (group sums of the rows) x (group biases), sixteen k' = eight groups an MFMA.
     // The operands of four steps are fetched together, four values a load where the rows allow it.
@@ -409,37 +409,54 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
                 sums_out[(size_t(tile_index) * kRowTile + m) * (a.f / kGroup) + c0 / kGroup + gl] = split_hi_lo(sum);
         }
     } else {
-        // a call over a range of the sorted pairs writes the rows of its pairs only
+        // the down product's rows leave through the first staging buffer too, [row][column of this block of 256], and go
+        // to their (token, rank) rows as whole 16-byte pieces; a call over a range of the sorted pairs writes the rows of
+        // its pairs only
         const uint32_t row_lo = DENSE ? 0u : max(a.pair_lo, tile.pair_start) - tile.pair_start;
         const uint32_t row_hi = DENSE ? tile.rows : min(a.pair_hi, tile.pair_start + tile.rows) - tile.pair_start;
-        float dab[2] = {0.0f, 0.0f};
-        if (!DENSE && a.ebias) {
-            dab[0] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n]);
-            dab[1] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n + 32u]);
-        }
+        if (active) {
+            float dab[2] = {0.0f, 0.0f};
+            if (!DENSE && a.ebias) {
+                dab[0] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n]);
+                dab[1] = bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[n + 32u]);
+            }
 #pragma unroll
-        for (uint32_t mt = 0; mt < MT; ++mt) {
+            for (uint32_t mt = 0; mt < MT; ++mt) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
-                if (m >= row_lo && m < row_hi) {
-                    uint16_t *dst;
-                    if (DENSE) {
-                        dst = a.partials + size_t(tile.pair_start + m) * a.d + n;
-                    } else {
-                        const shrike_token_expert_pair p = a.pairs[tile.pair_start + m];
-                        dst = a.partials + (size_t(p.token) * a.top_k + p.rank) * a.d + n;
-                    }
+                for (int i = 0; i < 16; ++i) {
+                    const uint32_t m = mt * 32u + 8u * (i / 4) + 4u * kb + (i % 4);
                     uint16_t y0 = f32_to_f16(total[0][mt][i] + dab[0]), y1 = f32_to_f16(total[1][mt][i] + dab[1]);
-                    if (DENSE && a.scalar_gate) {  // one gate a token row (moe.metal:1195-1207)
+                    if (DENSE && a.scalar_gate && m < tile.rows) {  // one gate a token row (moe.metal:1195-1207)
                         const float gate_mul = 1.0f + expf(-f16_to_f32(a.scalar_gate[tile.pair_start + m]));
                         y0 = f32_to_f16(f16_to_f32(y0) / gate_mul);
                         y1 = f32_to_f16(f16_to_f32(y1) / gate_mul);
                     }
-                    dst[0] = y0;
-                    dst[32] = y1;
+                    s_a[0][m][wave * 64u + col] = y0;
+                    s_a[0][m][wave * 64u + col + 32u] = y1;
                 }
             }
+        }
+        __syncthreads();
+        const uint32_t c0 = col_block * 256u, columns = min(256u, N - c0);  // N is a multiple of 64
+        constexpr uint32_t kPasses = MT * 32u * 32u / 256u;  // 32 pieces a row, 256 threads
+        const uint16_t *dst_row[kPasses];
+        const uint32_t pc = threadIdx.x & 31u;
+#pragma unroll
+        for (uint32_t pass = 0; pass < kPasses; ++pass) {
+            const uint32_t m = pass * 8u + (threadIdx.x >> 5);
+            const uint32_t mm = min(m, tile.rows - 1u);
+            if (DENSE) {
+                dst_row[pass] = a.partials + size_t(tile.pair_start + mm) * a.d;
+            } else {
+                const shrike_token_expert_pair p = a.pairs[tile.pair_start + mm];
+                dst_row[pass] = a.partials + (size_t(p.token) * a.top_k + p.rank) * a.d;
+            }
+        }
+#pragma unroll
+        for (uint32_t pass = 0; pass < kPasses; ++pass) {
+            const uint32_t m = pass * 8u + (threadIdx.x >> 5);
+            if (m >= row_lo && m < row_hi && pc * 8u < columns)
+                *reinterpret_cast<uint4 *>(const_cast<uint16_t *>(dst_row[pass]) + c0 + pc * 8u) = *reinterpret_cast<const uint4 *>(&s_a[0][m][pc * 8u]);
         }
     }
 }
