@@ -220,6 +220,36 @@ def cpu_baseline(S, blobs, sample_layers, meta):
     for e in picks:
         O.cpu_expert_ffn_accumulate(blobs[int(e)], off, x, D, F, 0.125, out, bits=BITS, meta=meta)
     per_expert = (time.perf_counter() - t0) / singles
+    # the same with the reference's own shrike_int4_affine_gemv, compiled from its source by oracle/Makefile where the
+    # reference checkout was present at build time (three calls and the fp32 SiLU-multiply between them, as
+    # CPUExpertFFN.accumulate composes them); its metadata is bf16, so it runs over blobs generated with bf16 metadata
+    reference = None
+    if O.ref_lib_path() is not None:
+        tree_r = S.SeedTree(0x5EED0001)
+        blobs_r = [S.expert_blob(tree_r, f"expert.{e}", D, F, BITS, S.META_BF16) for e in range(8)]
+        codes, metas = F * D // 2, F * (D // 64) * 2
+        down_codes, down_metas = D * F // 2, D * (F // 64) * 2
+
+        def parts(blob):
+            at, out = 0, []
+            for c, m in ((codes, metas), (codes, metas), (down_codes, down_metas)):
+                out.append((blob[at:at + c], blob[at + c:at + c + m].view(np.uint16), blob[at + c + m:at + c + 2 * m].view(np.uint16)))
+                at += c + 2 * m
+            return out
+        split = [parts(b) for b in blobs_r]
+        xr = np.ascontiguousarray(x, np.float32)
+        acc = np.zeros(D, np.float32)
+        t0 = time.perf_counter()
+        for i in range(singles):
+            (gw, gs, gb), (uw, us, ub), (dw, ds, db) = split[i % len(split)]
+            g = O.ref_int4_affine_gemv(gw, gs, gb, xr, F, D)
+            u = O.ref_int4_affine_gemv(uw, us, ub, xr, F, D)
+            act = (g / (1.0 + np.exp(-g)) * u).astype(np.float32)
+            acc += 0.125 * O.ref_int4_affine_gemv(dw, ds, db, act, D, F)
+        per_ref = (time.perf_counter() - t0) / singles
+        reference = {"kind": "reference", "cores": 1, "us_per_expert": round(per_ref * 1e6, 1),
+                     "value": round(1_769_472 / per_ref / 1e9, 3), "unit": "GB/s",
+                     "sample": f"{singles} experts, the reference's int4_affine_gemv.c (gcc -std=c99 -O2, portable branch), one thread"}
     return {"value": round(expert_bytes / per_layer / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
             "us_per_layer": round(per_layer * 1e6, 1),
             "sample": f"{sample_layers} layer evaluations of 9 experts (8 routed + 1 shared-sized) drawn from the "
@@ -228,7 +258,8 @@ def cpu_baseline(S, blobs, sample_layers, meta):
             "config1": {"workload": "config 1: one routed expert SwiGLU FFN for one token (hidden 2048, intermediate 512, int4)",
                         "cores": 1, "us_per_expert": round(per_expert * 1e6, 1),
                         "value": round(1_769_472 / per_expert / 1e9, 3), "unit": "GB/s", "bytes_per_expert": 1_769_472,
-                        "sample": f"{singles} experts drawn from the pool, one thread"}}
+                        "sample": f"{singles} experts drawn from the pool, one thread",
+                        **({"reference_c": reference} if reference else {})}}
 
 
 def cpu_pairs(S, blobs, d, f, bits, meta, pairs, evaluations, label):
