@@ -9,6 +9,10 @@
 namespace shrike {
 
 constexpr int kPhase1RowPairs = 4;  // (gate, up) row pairs per wave
+// ... and in a launch that does not route, for one token or for rows of three or more 16-byte chunks a lane: twice the
+// waves with half the rows in flight each measured faster there (one token 5.06 -> 4.68 us at hidden 2048, a batch of
+// four tokens at hidden 2880 with 8-bit codes 84 -> 79 us a layer; the same batch with 4-bit codes is slower with them)
+constexpr int kPhase1RowPairsNarrow = 2;
 
 // A wave owns RP consecutive f of one routed position: RP gate rows and RP up rows, each a
 // run of 16-byte chunks across the lanes. The lane's slice of x comes straight from global
@@ -110,20 +114,25 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
 }
 
 // positions: top_k, or the length of the active list
-uint32_t phase1_blocks(uint32_t top_k, uint32_t f) {
-    const uint32_t waves = (top_k * f + kPhase1RowPairs - 1) / kPhase1RowPairs;
+static uint32_t phase1_blocks_of(uint32_t positions, uint32_t f, uint32_t row_pairs) {
+    const uint32_t waves = (positions * f + row_pairs - 1) / row_pairs;
     return (waves + 3) / 4;
+}
+uint32_t phase1_blocks(uint32_t top_k, uint32_t f) { return phase1_blocks_of(top_k, f, kPhase1RowPairs); }
+
+static bool phase1_narrow(bool routing, bool one_token, uint32_t d, uint32_t bits) {
+    return !routing && (one_token || nch_for(d, bits) >= 3);
 }
 
 template <int BITS, bool ROUTE, int SBITS, bool STREAM>
 static void launch_phase1_nch(const Phase1Args &a, dim3 grid, hipStream_t s) {
-    constexpr int RP = kPhase1RowPairs;
+    constexpr int RP = kPhase1RowPairs, RN = ROUTE ? kPhase1RowPairs : kPhase1RowPairsNarrow;
     const dim3 block(256);
     switch (nch_for(a.d, BITS)) {
-        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
-        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
-        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
+        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, STREAM ? RN : RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
+        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RN, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RN, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
     }
 }
 
@@ -136,9 +145,11 @@ int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t sha
         extra = gemv_blocks(a.shared_down.rows, a.shared_down.n, shared_down_bits);
     }
     Phase1Args b = a;
-    b.lists_block = routing ? a.routed_blocks + extra : 0xffffffffu;
-    const dim3 grid(a.routed_blocks + extra + (routing ? 1u : 0u), a.tokens ? a.tokens : 1u);
     const bool one_token = a.tokens <= 1u;
+    if (phase1_narrow(routing, one_token, a.d, bits))
+        b.routed_blocks = phase1_blocks_of(a.active ? a.active_count : a.top_k, a.f, kPhase1RowPairsNarrow);
+    b.lists_block = routing ? b.routed_blocks + extra : 0xffffffffu;
+    const dim3 grid(b.routed_blocks + extra + (routing ? 1u : 0u), a.tokens ? a.tokens : 1u);
     if (bits == 4) {
         if (!routing) { if (one_token) launch_phase1_nch<4, false, 0, true>(b, grid, s); else launch_phase1_nch<4, false, 0, false>(b, grid, s); }
         else if (shared_down_bits == 0) launch_phase1_nch<4, true, 0, true>(b, grid, s);
