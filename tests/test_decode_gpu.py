@@ -216,7 +216,28 @@ def test_phase1_phase2_against_oracle(gpu, bits, meta, d, f):
     k, ne = 8, 8
     if d * f > 4_000_000:
         k, ne = 4, 4
-    L = Layer(0x5EED0000 + d + f + bits, d, f, ne, k, bits=bits, meta=meta)
+    check_phase1_phase2(gpu, bits, meta, d, f, k, ne, 0x5EED0000 + d + f + bits)
+
+
+def _swept_shapes():
+    """Sixteen shapes drawn once from a fixed seed: hidden and intermediate sizes any multiple of 64 up to 2,560
+    (rows of 1 to 160 sixteen-byte chunks: every chunks-per-lane count, whole and ragged waves, rows shorter than
+    a wave load), 1 to 8 routed positions, both code widths and both metadata types."""
+    rng = np.random.default_rng(0x5EED5EED)
+    out = []
+    for _ in range(16):
+        d, f = (int(64 * rng.integers(1, 41)) for _ in range(2))
+        out.append((d, f, int(rng.integers(1, 9)), int(rng.choice([4, 8])), int(rng.choice([S.META_BF16, S.META_F16]))))
+    return out
+
+
+@pytest.mark.parametrize("d,f,k,bits,meta", _swept_shapes())
+def test_phase1_phase2_shape_sweep(gpu, d, f, k, bits, meta):
+    check_phase1_phase2(gpu, bits, meta, d, f, k, k, 0x5EED1000 + d * 41 + f + k)
+
+
+def check_phase1_phase2(gpu, bits, meta, d, f, k, ne, seed):
+    L = Layer(seed, d, f, ne, k, bits=bits, meta=meta)
     dl = DeviceLayer(gpu, L)
     resolved = np.array([dl.cell_of[e] for e in range(k)], np.uint32)
     resolved[k - 1] = SENT  # one sentinel position: its acts must stay untouched, its partial must be zero
