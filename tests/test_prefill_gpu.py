@@ -196,6 +196,35 @@ def test_grouped_ffn_against_oracle(gpu, case):
     assert not np.any(np.all(got == 0xD4D0, axis=-1)), "a pair's partial row was left unwritten"
 
 
+def _swept_ffn_cases():
+    """Ten chunks drawn once from a fixed seed: hidden and intermediate sizes any multiple of 64 up to 1,536 (column blocks
+    that end inside a workgroup's 128 or 256 columns, k that ends inside a staged chunk of 256, group counts that are not
+    multiples of four), 1 to 150 tokens over 2 to 20 experts (row tiles of one row, of 32, of 33, of 64 and more)."""
+    rng = np.random.default_rng(0x5EEDFF)
+    out = []
+    for i in range(10):
+        d, f = (int(64 * rng.integers(1, 25)) for _ in range(2))
+        ne = int(rng.integers(2, 21))
+        k = int(rng.integers(1, min(ne, 8) + 1))
+        out.append((f"sweep-{i}-d{d}-f{f}", d, f, ne, k, int(rng.integers(1, 151)), int(rng.choice([4, 8])),
+                    int(rng.choice([S.META_BF16, S.META_F16])), int(rng.choice([0, 8, 24]))))
+    return out
+
+
+@pytest.mark.parametrize("case", _swept_ffn_cases(), ids=[c[0] for c in _swept_ffn_cases()])
+def test_grouped_ffn_shape_sweep(gpu, case):
+    name, d, f, ne, k, t, bits, meta, pad = case
+    L = Layer(0x5EED0300 + d + f, d, f, ne, k, bits=bits, meta=meta)
+    pc = PrefillCase(gpu, L, t, stride_pad=pad)
+    got = pc.run()
+    rng = np.random.default_rng(5)
+    sample = [(int(a), int(b)) for a, b in zip(rng.integers(0, t, 24), rng.integers(0, k, 24))] if t * k > 24 else \
+        [(a, b) for a in range(t) for b in range(k)]
+    for tok, rank in sample:
+        pc.check_pair(got, tok, rank, f"{name} token {tok} rank {rank}")
+    assert not np.any(np.all(got == 0xD4D0, axis=-1)), "a pair's partial row was left unwritten"
+
+
 def test_grouped_ffn_gpt_oss_epilogues(gpu):
     # additive biases + clamped SwiGLU at the gpt-oss shape (moe.metal:257-288), 45 groups per row
     d = f = 2880
