@@ -125,6 +125,10 @@ uint64_t shrike_hip_pool_table_entry(const shrike_hip_pool *pool, uint32_t exper
  * host_store + e * store_expert_stride (pinned memory for an asynchronous copy) into its
  * reserved cell on `stream`; the misses become resident in the cache and every residency
  * word that changed is stored to the device table on the same stream, behind the copies.
+ * With two misses or more every other copy runs on a stream of the pool's own, which starts
+ * behind everything `stream` holds at the call and which `stream` waits for before the table
+ * stores: to the caller the copies are ordered as if all were on `stream` (a stream under
+ * capture gets them all itself).
  * The caller orders `stream` against the kernels that still read an evicted cell. */
 int shrike_hip_pool_execute_plan(shrike_hip_pool *pool, shrike_slot_cache *cache,
                                  const shrike_expert_cache_plan *plan, const void *host_store, uint64_t store_expert_stride,

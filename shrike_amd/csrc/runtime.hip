@@ -54,6 +54,10 @@ struct shrike_hip_pool {
     uint64_t *d_table;
     std::vector<uint64_t> shadow;  // host copy of the table, updated at publish
     bool owns_cells = true;        // false for a layer's table over another pool's cells
+    // execute_plan's second copy queue: two host-to-device copies in flight fill the link better than one
+    // (57 against 53 GB/s for 7 MB blobs from pinned memory); made at the first plan with two misses or more
+    hipStream_t side_stream = nullptr;
+    hipEvent_t side_fork = nullptr, side_join = nullptr;
 };
 
 namespace shrike {
@@ -263,6 +267,9 @@ void shrike_hip_pool_destroy(shrike_hip_pool *pool) {
     for (void *c : pool->chunks)
         if (c && pool->owns_cells) (void)hipFree(c);
     if (pool->d_table) (void)hipFree(pool->d_table);
+    if (pool->side_stream) (void)hipStreamDestroy(pool->side_stream);
+    if (pool->side_fork) (void)hipEventDestroy(pool->side_fork);
+    if (pool->side_join) (void)hipEventDestroy(pool->side_join);
     delete pool;
 }
 
@@ -359,7 +366,28 @@ int shrike_hip_pool_execute_plan(shrike_hip_pool *pool, shrike_slot_cache *cache
     SHRIKE_REQUIRE(pool && cache && plan, "execute plan: NULL argument");
     SHRIKE_REQUIRE(plan->miss_count == 0 || host_store, "execute plan: the plan has misses and no host store to read them from");
     SHRIKE_REQUIRE(expert_bytes <= pool->stride && expert_bytes <= store_expert_stride, "execute plan: expert bytes exceed a cell or the store's stride");
-    // the reads (PreadExpertStreamer.swift:610-621): one host-to-device copy per miss into the cell the plan reserved
+    // the reads (PreadExpertStreamer.swift:610-621): one host-to-device copy per miss into the cell the plan reserved.
+    // With two misses or more every other copy goes to a second queue that starts behind what `stream` holds so far
+    // and that `stream` waits for before anything else is put on it, so the caller sees one ordered stream.
+    hipStream_t main_stream = as_stream(stream);
+    bool two_queues = plan->miss_count >= 2;
+    if (two_queues) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(main_stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            two_queues = false;  // a stream under capture keeps its copies to itself
+        }
+    }
+    if (two_queues && pool->side_stream == nullptr) {
+        if (hipStreamCreateWithFlags(&pool->side_stream, hipStreamNonBlocking) != hipSuccess
+            || hipEventCreateWithFlags(&pool->side_fork, hipEventDisableTiming) != hipSuccess
+            || hipEventCreateWithFlags(&pool->side_join, hipEventDisableTiming) != hipSuccess)
+            return hip_failed(hipGetLastError(), "execute plan: second copy queue");
+    }
+    if (two_queues) {
+        SHRIKE_HIP(hipEventRecord(pool->side_fork, main_stream));
+        SHRIKE_HIP(hipStreamWaitEvent(pool->side_stream, pool->side_fork, 0));
+    }
     for (uint32_t m = 0; m < plan->miss_count; ++m) {
         const uint32_t i = plan->misses[m];
         const int32_t expert = plan->experts[i];
@@ -369,7 +397,11 @@ int shrike_hip_pool_execute_plan(shrike_hip_pool *pool, shrike_slot_cache *cache
         const uint32_t cell = uint32_t(word);
         SHRIKE_REQUIRE(cell < pool->cells, "execute plan: cell %u out of range", cell);
         SHRIKE_HIP(hipMemcpyAsync(shrike_hip_pool_cell_ptr(pool, cell), static_cast<const uint8_t *>(host_store) + uint64_t(expert) * store_expert_stride,
-                                  expert_bytes, hipMemcpyHostToDevice, as_stream(stream)));
+                                  expert_bytes, hipMemcpyHostToDevice, two_queues && (m & 1u) ? pool->side_stream : main_stream));
+    }
+    if (two_queues) {
+        SHRIKE_HIP(hipEventRecord(pool->side_join, pool->side_stream));
+        SHRIKE_HIP(hipStreamWaitEvent(main_stream, pool->side_join, 0));
     }
     // markPlanMissesResident, then every residency word that changed since the last drain goes to
     // the device table behind the copies on the same stream
