@@ -477,7 +477,8 @@ def kimi_workload(args, rt, capi, S, meta):
     cache = HL.SlotCache(slots, ne)
     moe = rt.MoE(d, f, ne, k, routed_bits=bits, router_bits=0, meta=meta)
     moe.stream = rt.Stream()
-    layer = rt.BatchedDecodeLayer(moe, pool, cache, off, store, stride, stride, t)
+    from harness import runners
+    layer = runners.BatchedDecodeLayer(moe, pool, cache, off, store, stride, stride, t)
     router = dict(weights=rt.dev(S.router_f16(tree, "router.w", ne, d)), eff_scale=rt.dev(S.f32_to_bf16_bits(np.ones(d, np.float32))),
                   expert_scale=rt.dev(S.f32_to_bf16_bits(np.ones(ne, np.float32))), bias=rt.dev(np.zeros(ne, np.uint16)))
     shared = {n: tuple(rt.dev(a) for a in S.affine_matrix(tree.key(f"shared.{n}"), r, c, bits, meta))
@@ -523,7 +524,7 @@ def kimi_workload(args, rt, capi, S, meta):
 
 
 def decode_workload(args, rt, capi, S, meta):
-    from shrike_amd import probes
+    from harness import probes
     n_layers = args.layers
     layers, off, stride, keep, gen_s = build_layers(rt, capi, S, n_layers, meta, shared=not args.no_shared)
     moe = rt.MoE(D, F, NE, K, routed_bits=BITS, router_bits=0, meta=meta)

@@ -6,7 +6,7 @@ from __future__ import annotations
 import ctypes as C
 import os
 
-from .capi import PoolBases, ShrikeError
+from shrike_amd.capi import PoolBases, ShrikeError
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _lib = None
@@ -17,7 +17,7 @@ def load() -> C.CDLL:
     if _lib is None:
         path = os.path.join(_HERE, "libshrikeprobe.so")
         if not os.path.exists(path):
-            raise ShrikeError(f"{path} is not built (make -C shrike_amd/csrc)")
+            raise ShrikeError(f"{path} is not built (make -C harness)")
         _lib = C.CDLL(path)
         _lib.shrike_probe_last_error.restype = C.c_char_p
         _lib.shrike_probe_empty_launch.restype = C.c_int

@@ -15,6 +15,9 @@
 //   PackedExpertsLayout(Reader) (Infrastructure/ModelIO) shrike::PackedExpertsLayout
 //   PrefillRoutedTileScheduler / ...Sequencer / ...Driver shrike::PrefillRoutedTileScheduler, ...Sequencer, ...Driver
 //   ExpertLoadOperation, ExpertPrefetchRing           shrike::ExpertLoadOperation, shrike::ExpertPrefetchRing
+//   ExpertIOScheduler, ExpertIOEventCoordinator       shrike::ExpertIOScheduler, shrike::ExpertIOEventCoordinator
+//   RouterHostReadback (Runtime/Inference)            shrike::RouterHostReadback
+//   CPUExpertFFN (Kernels/CPU)                        shrike::CPUExpertFFN
 #pragma once
 
 #include <cerrno>
@@ -24,6 +27,7 @@
 #include <exception>
 #include <functional>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <optional>
 #include <stdexcept>
@@ -709,55 +713,114 @@ private:
     shrike_load_operation *h_;
 };
 
-// ExpertIOScheduler (Infrastructure/Streaming/ExpertLoadOperation.swift:166-219): a fixed set of submission
-// threads; a queued demand batch runs before any queued speculative one. The destructor runs what is
-// queued, then joins the threads.
+// ExpertIOScheduler (Infrastructure/Streaming/ExpertLoadOperation.swift:166-219) over the library's submission
+// threads: a queued demand batch runs before any queued speculative one. The destructor runs what is queued,
+// then joins the threads.
 class ExpertIOScheduler {
 public:
-    enum class Priority { demand, speculative };
+    enum class Priority { demand = SHRIKE_IO_DEMAND, speculative = SHRIKE_IO_SPECULATIVE };
     explicit ExpertIOScheduler(int workerCount = 4) {
-        if (workerCount <= 0) throw Error(EINVAL, "workerCount must be positive");
-        for (int i = 0; i < workerCount; ++i) workers_.emplace_back([this] { run(); });
+        int err = 0;
+        h_ = shrike_io_scheduler_create(workerCount, &err);
+        if (!h_) throw Error(err, shrike_hip_last_error());
     }
-    ~ExpertIOScheduler() {
-        {
-            std::lock_guard<std::mutex> held(lock_);
-            closed_ = true;
-        }
-        wake_.notify_all();
-        for (std::thread &worker : workers_) worker.join();
-    }
+    ~ExpertIOScheduler() { shrike_io_scheduler_destroy(h_); }
     ExpertIOScheduler(const ExpertIOScheduler &) = delete;
     ExpertIOScheduler &operator=(const ExpertIOScheduler &) = delete;
     void submit(std::function<void()> work, Priority priority = Priority::demand) {
-        {
-            std::lock_guard<std::mutex> held(lock_);
-            if (closed_) throw Error(EINVAL, "the expert I/O scheduler is closed");
-            (priority == Priority::demand ? demand_ : speculative_).push_back(std::move(work));
+        auto *boxed = new std::function<void()>(std::move(work));
+        const int rc = shrike_io_scheduler_submit(h_, int(priority), &ExpertIOScheduler::run, boxed);
+        if (rc != 0) {
+            delete boxed;
+            throw Error(rc, shrike_hip_last_error());
         }
-        wake_.notify_one();
+    }
+    void close() { shrike_io_scheduler_close(h_); }
+
+private:
+    static void run(void *context) {
+        std::unique_ptr<std::function<void()>> work(static_cast<std::function<void()> *>(context));
+        (*work)();
+    }
+    shrike_io_scheduler *h_;
+};
+
+// ExpertIOEventCoordinator + ExpertIOCompletionToken (Infrastructure/Streaming/ExpertIOEventCoordinator.swift:7-90)
+using ExpertIOCompletionToken = shrike_io_completion_token;
+class ExpertIOEventCoordinator {
+public:
+    static constexpr uint32_t statusWordCount = SHRIKE_IO_STATUS_WORDS;
+    // statusWords: memory the GPU can read (pinned host memory) for the ring, or nullptr for words of its own
+    explicit ExpertIOEventCoordinator(uint32_t *statusWords = nullptr, uint32_t wordCount = statusWordCount) {
+        int err = 0;
+        h_ = shrike_io_timeline_create(statusWords, wordCount, &err);
+        if (!h_) throw Error(err, shrike_hip_last_error());
+    }
+    ~ExpertIOEventCoordinator() { shrike_io_timeline_destroy(h_); }
+    ExpertIOEventCoordinator(const ExpertIOEventCoordinator &) = delete;
+    ExpertIOEventCoordinator &operator=(const ExpertIOEventCoordinator &) = delete;
+    ExpertIOCompletionToken reserve() {
+        ExpertIOCompletionToken token;
+        check(shrike_io_timeline_reserve(h_, &token));
+        return token;
+    }
+    uint64_t publish(const ExpertIOCompletionToken &token, bool succeeded) { return shrike_io_timeline_publish(h_, &token, succeeded); }
+    uint64_t signaledValue() { return shrike_io_timeline_published(h_); }
+
+private:
+    shrike_io_timeline *h_;
+};
+
+// RouterHostReadback (Runtime/Inference/RouterHostReadback.swift:8-63)
+struct RouterHostReadback {
+    static constexpr uint32_t tagBits = 16, valueMask = 0xffff, fixedWords = 2;
+    int hitCount = 0, missCount = 0;
+    std::vector<uint32_t> expertIDs;
+    std::vector<uint16_t> weightBits;
+    std::vector<uint32_t> hitPositions, missPositions, predictedIDs;
+    static int wordCount(int topK) { return int(shrike_router_readback_word_count(uint32_t(topK))); }
+    static uint32_t word(uint32_t tag, uint32_t value) { return shrike_router_readback_word(tag, value); }
+    static uint32_t nextTag(uint32_t after) { return shrike_router_readback_next_tag(after); }
+    static bool isComplete(const uint32_t *words, int topK, uint32_t tag) {
+        return shrike_router_readback_is_complete(words, uint32_t(topK), tag) != 0;
+    }
+    static std::optional<RouterHostReadback> decode(const uint32_t *words, int topK, uint32_t tag) {
+        shrike_router_readback r;
+        if (!shrike_router_readback_decode(words, uint32_t(topK), tag, &r)) return std::nullopt;
+        return from(r, topK);
+    }
+    // the runner's wait while the command still runs (RealForwardRunner.swift:3294-3310)
+    static std::optional<RouterHostReadback> poll(const uint32_t *words, int topK, uint32_t tag, uint64_t timeoutNanos) {
+        shrike_router_readback r;
+        if (!shrike_router_readback_poll(words, uint32_t(topK), tag, shrike_monotonic_nanos() + timeoutNanos, &r)) return std::nullopt;
+        return from(r, topK);
     }
 
 private:
-    void run() {
-        for (;;) {
-            std::function<void()> work;
-            {
-                std::unique_lock<std::mutex> held(lock_);
-                wake_.wait(held, [this] { return closed_ || !demand_.empty() || !speculative_.empty(); });
-                std::deque<std::function<void()>> &queue = demand_.empty() ? speculative_ : demand_;
-                if (queue.empty()) return;  // closed and drained
-                work = std::move(queue.front());
-                queue.pop_front();
-            }
-            work();
-        }
+    static RouterHostReadback from(const shrike_router_readback &r, int topK) {
+        RouterHostReadback out;
+        out.hitCount = int(r.hit_count);
+        out.missCount = int(r.miss_count);
+        out.expertIDs.assign(r.expert_ids, r.expert_ids + topK);
+        out.weightBits.assign(r.weight_bits, r.weight_bits + topK);
+        out.hitPositions.assign(r.hit_positions, r.hit_positions + r.hit_count);
+        out.missPositions.assign(r.miss_positions, r.miss_positions + r.miss_count);
+        out.predictedIDs.assign(r.predicted_ids, r.predicted_ids + topK);
+        return out;
     }
-    std::mutex lock_;
-    std::condition_variable wake_;
-    std::deque<std::function<void()>> demand_, speculative_;
-    std::vector<std::thread> workers_;
-    bool closed_ = false;
+};
+
+// CPUExpertFFN (Kernels/CPU/CPUExpertFFN.swift:10-140): the CPU expert kernel over host memory
+struct CPUExpertFFN {
+    static void gemv(const uint8_t *weights, const uint16_t *scales, const uint16_t *biases, const float *x, size_t rows, size_t n,
+                     float *out) {
+        shrike_int4_affine_gemv(weights, scales, biases, x, rows, n, out);
+    }
+    static size_t scratchFloats(uint32_t d, uint32_t f) { return shrike_cpu_expert_ffn_scratch_floats(d, f); }
+    static void accumulate(const void *expert, const shrike_expert_offsets &offsets, const float *x, uint32_t d, uint32_t f,
+                           float routeWeight, float *scratch, float *out) {
+        check(shrike_cpu_expert_ffn_accumulate(expert, &offsets, x, d, f, routeWeight, scratch, out));
+    }
 };
 
 // ExpertPrefetchRing (Runtime/Inference/ExpertPrefetchRing.swift:42-352)

@@ -545,6 +545,90 @@ void shrike_prefetch_ring_statistics(shrike_prefetch_ring *ring, shrike_prefetch
 int shrike_prefetch_ring_in_flight_count(shrike_prefetch_ring *ring);
 int shrike_prefetch_ring_leased_count(shrike_prefetch_ring *ring);
 
+/* ------------------------------------------------------- the CPU expert kernel */
+
+/* shrike_int4_affine_gemv, sources/ShrikeKernelsC/include/shrike_kernels.h:9-29 (implementation
+ * sources/ShrikeKernelsC/int4_affine_gemv.c:28-135), same name, arguments and meaning:
+ * out[r] = sum_i (q[r][i] * scale[r][g(i)] + bias[r][g(i)]) * x[i] over a rows-by-n matrix of 4-bit codes, low nibble
+ * first, one bf16 scale and one bf16 bias per group of 64; n a multiple of 64; out is written, not accumulated. The sum
+ * is factored per group as scale * sum(q x) + bias * sum(x) and its additions run in the order of the reference's
+ * portable branch (:114-134), whose bits the results are. Host memory only; thread-safe. */
+void shrike_int4_affine_gemv(const uint8_t *weights, const uint16_t *scales, const uint16_t *biases, const float *x,
+                             size_t rows, size_t n, float *out);
+/* CPUExpertFFN.accumulate, sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:102-140 (called at :82-90 by the CPU expert
+ * workers): out[0..d) += route_weight * down(silu(gate . x) * (up . x)) for the expert blob at `expert` (bf16 metadata,
+ * 4-bit codes), all in fp32. scratch: shrike_cpu_expert_ffn_scratch_floats(d, f) = 2 f + d floats, caller-owned. */
+size_t shrike_cpu_expert_ffn_scratch_floats(uint32_t d, uint32_t f);
+int shrike_cpu_expert_ffn_accumulate(const void *expert, const shrike_expert_offsets *offsets, const float *x, uint32_t d,
+                                     uint32_t f, float route_weight, float *scratch, float *out);
+
+/* ------------------------------------------------------- shared words between the host and the GPU */
+
+/* sources/ShrikeKernelsC/include/shrike_atomics.h:7-14: an acquire load of a word a kernel writes while the host polls
+ * it, a release store of a word the host publishes for a kernel to read. */
+uint32_t shrike_load_acquire_u32(const uint32_t *word);
+void shrike_store_release_u64(uint64_t *word, uint64_t value);
+
+/* RouterHostReadback (sources/Shrike/Runtime/Inference/RouterHostReadback.swift:8-63): the host's half of the
+ * classifier's tagged copy (the device's half is shrike_hip_moe_classify's host_readback operand). Every word carries
+ * the launch's tag in its high 16 bits and a value in its low 16: the two counts, then five runs of top_k words (ids,
+ * weight bits, hit positions, miss positions, predicted ids). The host polls the words while the command still runs
+ * (RealForwardRunner.swift:3294) and trusts them only once every word carries the tag. */
+typedef struct {
+    uint32_t hit_count, miss_count;        /* clamped to top_k */
+    uint32_t expert_ids[8];
+    uint16_t weight_bits[8];
+    uint32_t hit_positions[8];             /* the first hit_count are meaningful */
+    uint32_t miss_positions[8];            /* the first miss_count are meaningful */
+    uint32_t predicted_ids[8];
+} shrike_router_readback;
+uint32_t shrike_router_readback_word_count(uint32_t top_k);            /* wordCount(topK:), :24 */
+uint32_t shrike_router_readback_word(uint32_t tag, uint32_t value);     /* word(tag:value:), :26-28 */
+uint32_t shrike_router_readback_next_tag(uint32_t tag);                 /* nextTag(after:), :31-33: never 0, wraps at 16 bits */
+int shrike_router_readback_is_complete(const uint32_t *words, uint32_t top_k, uint32_t tag);   /* isComplete, :35-41 */
+/* decode, :43-62: 1 and *out filled when every word carries the tag, 0 (out untouched) otherwise. */
+int shrike_router_readback_decode(const uint32_t *words, uint32_t top_k, uint32_t tag, shrike_router_readback *out);
+/* The runner's wait (RealForwardRunner.swift:3294-3310): decode until it succeeds or shrike_monotonic_nanos() reaches
+ * the deadline; 1 on success, 0 at the deadline. */
+int shrike_router_readback_poll(const uint32_t *words, uint32_t top_k, uint32_t tag, uint64_t deadline_nanos,
+                                shrike_router_readback *out);
+
+/* ------------------------------------------------------- the storage submission service and its completion timeline */
+
+/* ExpertIOScheduler (sources/Shrike/Infrastructure/Streaming/ExpertLoadOperation.swift:166-219): a fixed set of
+ * submission threads over two queues; a queued demand batch runs before any queued speculative one. close runs what is
+ * queued and ends the threads (submit then returns ESHUTDOWN); destroy closes first. work(context) runs on a worker. */
+enum { SHRIKE_IO_DEMAND = 0, SHRIKE_IO_SPECULATIVE = 1 };  /* ExpertIOPriority, :166-169 */
+typedef struct shrike_io_scheduler shrike_io_scheduler;
+typedef void (*shrike_io_work)(void *context);
+shrike_io_scheduler *shrike_io_scheduler_create(int worker_count, int *out_errno);   /* the reference's shared one has 4 */
+int shrike_io_scheduler_submit(shrike_io_scheduler *scheduler, int priority, shrike_io_work work, void *context);
+void shrike_io_scheduler_close(shrike_io_scheduler *scheduler);
+void shrike_io_scheduler_destroy(shrike_io_scheduler *scheduler);
+int shrike_io_scheduler_workers(const shrike_io_scheduler *scheduler);
+
+/* ExpertIOEventCoordinator (sources/Shrike/Infrastructure/Streaming/ExpertIOEventCoordinator.swift:23-90): one timeline
+ * for all expert reads of a model. reserve hands out the next value (never 0, never reused) and its status word, set to
+ * 0 = loading; publish stores 1 = complete or 2 = failed and returns the timeline's published value, which moves only
+ * over values whose predecessors are all terminal (an out-of-order completion is held). The status words are a ring of
+ * word_count (0: SHRIKE_IO_STATUS_WORDS), a value's word at (value - 1) % word_count. status_words: caller-owned memory
+ * the GPU can read (pinned host memory), or NULL for words of the timeline's own. A consumer on the GPU waits for value v
+ * by waiting (hipStreamWaitEvent) for the event recorded behind v's copies and status store once published >= v says
+ * that event and every earlier one is recorded, then reads the status word as the reference's kernels do. */
+#define SHRIKE_IO_STATUS_WORDS 4096u  /* ExpertIOEventCoordinator.statusWordCount, :36 */
+enum { SHRIKE_IO_STATUS_LOADING = 0, SHRIKE_IO_STATUS_COMPLETE = 1, SHRIKE_IO_STATUS_FAILED = 2 };
+typedef struct shrike_io_timeline shrike_io_timeline;
+typedef struct {
+    uint64_t value;
+    uint32_t status_index;     /* (value - 1) % word_count */
+    uint32_t *status;          /* the word itself */
+} shrike_io_completion_token;  /* ExpertIOCompletionToken, :7-15 */
+shrike_io_timeline *shrike_io_timeline_create(uint32_t *status_words, uint32_t word_count, int *out_errno);
+void shrike_io_timeline_destroy(shrike_io_timeline *timeline);
+int shrike_io_timeline_reserve(shrike_io_timeline *timeline, shrike_io_completion_token *out);             /* reserve, :48-78 */
+uint64_t shrike_io_timeline_publish(shrike_io_timeline *timeline, const shrike_io_completion_token *token, int succeeded); /* publish, :80-89 */
+uint64_t shrike_io_timeline_published(shrike_io_timeline *timeline);  /* event.signaledValue */
+
 #ifdef __cplusplus
 }
 #endif

@@ -182,8 +182,42 @@ PREFETCH_DROP = C.CFUNCTYPE(None, C.c_void_p, C.c_int, C.c_int, C.c_int)
 PREFETCH_ISSUE = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_size_t, C.POINTER(C.c_void_p))
 
 
+class RouterReadback(C.Structure):
+    _fields_ = [("hit_count", C.c_uint32), ("miss_count", C.c_uint32), ("expert_ids", C.c_uint32 * 8),
+                ("weight_bits", C.c_uint16 * 8), ("hit_positions", C.c_uint32 * 8), ("miss_positions", C.c_uint32 * 8),
+                ("predicted_ids", C.c_uint32 * 8)]
+
+
+class IOCompletionToken(C.Structure):
+    _fields_ = [("value", C.c_uint64), ("status_index", C.c_uint32), ("status", C.POINTER(C.c_uint32))]
+
+
+IO_WORK = C.CFUNCTYPE(None, C.c_void_p)
+
 SIGNATURES = {
     "shrike_hip_last_error": (C.c_char_p, []),
+    "shrike_int4_affine_gemv": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]),
+    "shrike_cpu_expert_ffn_scratch_floats": (C.c_size_t, [C.c_uint32, C.c_uint32]),
+    "shrike_cpu_expert_ffn_accumulate": (C.c_int, [C.c_void_p, C.POINTER(ExpertOffsets), C.c_void_p, C.c_uint32, C.c_uint32,
+                                                   C.c_float, C.c_void_p, C.c_void_p]),
+    "shrike_load_acquire_u32": (C.c_uint32, [C.c_void_p]),
+    "shrike_store_release_u64": (None, [C.c_void_p, C.c_uint64]),
+    "shrike_router_readback_word_count": (C.c_uint32, [C.c_uint32]),
+    "shrike_router_readback_word": (C.c_uint32, [C.c_uint32, C.c_uint32]),
+    "shrike_router_readback_next_tag": (C.c_uint32, [C.c_uint32]),
+    "shrike_router_readback_is_complete": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32]),
+    "shrike_router_readback_decode": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(RouterReadback)]),
+    "shrike_router_readback_poll": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint64, C.POINTER(RouterReadback)]),
+    "shrike_io_scheduler_create": (C.c_void_p, [C.c_int, C.POINTER(C.c_int)]),
+    "shrike_io_scheduler_submit": (C.c_int, [C.c_void_p, C.c_int, IO_WORK, C.c_void_p]),
+    "shrike_io_scheduler_close": (None, [C.c_void_p]),
+    "shrike_io_scheduler_destroy": (None, [C.c_void_p]),
+    "shrike_io_scheduler_workers": (C.c_int, [C.c_void_p]),
+    "shrike_io_timeline_create": (C.c_void_p, [C.c_void_p, C.c_uint32, C.POINTER(C.c_int)]),
+    "shrike_io_timeline_destroy": (None, [C.c_void_p]),
+    "shrike_io_timeline_reserve": (C.c_int, [C.c_void_p, C.POINTER(IOCompletionToken)]),
+    "shrike_io_timeline_publish": (C.c_uint64, [C.c_void_p, C.POINTER(IOCompletionToken), C.c_int]),
+    "shrike_io_timeline_published": (C.c_uint64, [C.c_void_p]),
     "shrike_tile_scheduler_config_make": (None, [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(TileSchedulerConfig)]),
     "shrike_tile_scheduler_fits_slot_budget": (C.c_int, [C.POINTER(TileSchedulerConfig), C.c_int, C.c_int]),
     "shrike_tile_scheduler_fitting": (C.c_int, [C.POINTER(TileSchedulerConfig), C.c_int, C.c_int, C.POINTER(TileSchedulerConfig)]),

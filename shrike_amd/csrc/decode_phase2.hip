@@ -495,6 +495,15 @@ int shrike_hip_moe_decode_layer_noalloc(const shrike_moe_desc *desc, void *strea
     SHRIKE_REQUIRE(desc->f <= kNoAllocMaxF, "decodeLayerNoAlloc: f=%u exceeds the static scratch's %u", desc->f, kNoAllocMaxF);
     SHRIKE_REQUIRE(g->shared_gate.weights == nullptr || g->shared_f <= kNoAllocMaxSharedF,
                    "decodeLayerNoAlloc: sharedF=%u exceeds the static scratch's %u", g->shared_f, kNoAllocMaxSharedF);
+    if (stream != nullptr) {
+        // every GPU holds its own copy of the array: the one used must be the one of the GPU the launches go to
+        int current = -1;
+        hipDevice_t of_stream = -1;
+        SHRIKE_HIP(hipGetDevice(&current));
+        SHRIKE_HIP(hipStreamGetDevice(as_stream(stream), &of_stream));
+        SHRIKE_REQUIRE(int(of_stream) == current, "decodeLayerNoAlloc: the stream belongs to device %d, the current device is %d",
+                       int(of_stream), current);
+    }
     unsigned char *base = nullptr;
     if (int rc = layer_scratch(&base)) return rc;
     shrike_hip_moe moe = {};

@@ -379,30 +379,67 @@ int shrike_hip_pool_execute_plan(shrike_hip_pool *pool, shrike_slot_cache *cache
         }
     }
     if (two_queues && pool->side_stream == nullptr) {
-        if (hipStreamCreateWithFlags(&pool->side_stream, hipStreamNonBlocking) != hipSuccess
-            || hipEventCreateWithFlags(&pool->side_fork, hipEventDisableTiming) != hipSuccess
-            || hipEventCreateWithFlags(&pool->side_join, hipEventDisableTiming) != hipSuccess)
-            return hip_failed(hipGetLastError(), "execute plan: second copy queue");
+        // the queue and its two events are made together or not at all: on any failure the plan goes over one queue
+        hipStream_t side = nullptr;
+        hipEvent_t fork = nullptr, join = nullptr;
+        // (another stream of this thread may be under a global-mode capture, which a stream creation would break:
+        // the thread's capture mode is relaxed for the three calls)
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        (void)hipThreadExchangeStreamCaptureMode(&mode);
+        const bool made = hipStreamCreateWithFlags(&side, hipStreamNonBlocking) == hipSuccess
+                          && hipEventCreateWithFlags(&fork, hipEventDisableTiming) == hipSuccess
+                          && hipEventCreateWithFlags(&join, hipEventDisableTiming) == hipSuccess;
+        (void)hipThreadExchangeStreamCaptureMode(&mode);
+        if (made) {
+            pool->side_stream = side; pool->side_fork = fork; pool->side_join = join;
+        } else {
+            (void)hipGetLastError();
+            if (join) (void)hipEventDestroy(join);
+            if (fork) (void)hipEventDestroy(fork);
+            if (side) (void)hipStreamDestroy(side);
+            two_queues = false;
+        }
     }
     if (two_queues) {
         SHRIKE_HIP(hipEventRecord(pool->side_fork, main_stream));
         SHRIKE_HIP(hipStreamWaitEvent(pool->side_stream, pool->side_fork, 0));
     }
-    for (uint32_t m = 0; m < plan->miss_count; ++m) {
+    // From here on the second queue may hold work: whatever ends the loop, `stream` waits for it before this call
+    // returns, so that the caller's later work on `stream` is ordered behind every copy that was enqueued.
+    int rc = 0;
+    for (uint32_t m = 0; m < plan->miss_count && rc == 0; ++m) {
         const uint32_t i = plan->misses[m];
         const int32_t expert = plan->experts[i];
-        SHRIKE_REQUIRE(expert >= 0 && uint32_t(expert) < pool->num_experts, "execute plan: expert %d out of range", expert);
+        if (expert < 0 || uint32_t(expert) >= pool->num_experts) {
+            set_error("execute plan: expert %d out of range", expert);
+            rc = EINVAL;
+            break;
+        }
         const uint64_t word = shrike_slot_cache_entry(cache, uint32_t(expert));
-        SHRIKE_REQUIRE(uint32_t(word >> 32) == SHRIKE_RESIDENCY_LOADING, "execute plan: expert %d is not loading (stale plan)", expert);
         const uint32_t cell = uint32_t(word);
-        SHRIKE_REQUIRE(cell < pool->cells, "execute plan: cell %u out of range", cell);
-        SHRIKE_HIP(hipMemcpyAsync(shrike_hip_pool_cell_ptr(pool, cell), static_cast<const uint8_t *>(host_store) + uint64_t(expert) * store_expert_stride,
-                                  expert_bytes, hipMemcpyHostToDevice, two_queues && (m & 1u) ? pool->side_stream : main_stream));
+        if (uint32_t(word >> 32) != SHRIKE_RESIDENCY_LOADING) {
+            set_error("execute plan: expert %d is not loading (stale plan)", expert);
+            rc = EINVAL;
+        } else if (cell >= pool->cells) {
+            set_error("execute plan: cell %u out of range", cell);
+            rc = EINVAL;
+        } else {
+            const hipError_t err = hipMemcpyAsync(shrike_hip_pool_cell_ptr(pool, cell),
+                                                  static_cast<const uint8_t *>(host_store) + uint64_t(expert) * store_expert_stride,
+                                                  expert_bytes, hipMemcpyHostToDevice, two_queues && (m & 1u) ? pool->side_stream : main_stream);
+            if (err != hipSuccess) rc = hip_failed(err, "execute plan: hipMemcpyAsync");
+        }
     }
     if (two_queues) {
-        SHRIKE_HIP(hipEventRecord(pool->side_join, pool->side_stream));
-        SHRIKE_HIP(hipStreamWaitEvent(main_stream, pool->side_join, 0));
+        hipError_t err = hipEventRecord(pool->side_join, pool->side_stream);
+        if (err == hipSuccess) err = hipStreamWaitEvent(main_stream, pool->side_join, 0);
+        if (err != hipSuccess) {
+            // the join could not be enqueued: wait the second queue out on the host rather than leave it unordered
+            (void)hipStreamSynchronize(pool->side_stream);
+            if (rc == 0) rc = hip_failed(err, "execute plan: joining the second copy queue");
+        }
     }
+    if (rc != 0) return rc;
     // markPlanMissesResident, then every residency word that changed since the last drain goes to
     // the device table behind the copies on the same stream
     if (int rc = shrike_slot_cache_complete(cache, plan, elapsed_nanos, elapsed_nanos)) return rc;

@@ -777,48 +777,149 @@ class PrefetchClaimRefused(Exception):
 
 
 class ExpertIOScheduler:
-    """ExpertIOScheduler (sources/Shrike/Infrastructure/Streaming/ExpertLoadOperation.swift:166-219): a fixed
-    set of submission threads; a queued demand batch runs before any queued speculative one."""
+    """ExpertIOScheduler (sources/Shrike/Infrastructure/Streaming/ExpertLoadOperation.swift:166-219): the library's
+    submission threads (shrike_io_scheduler_*); a queued demand batch runs before any queued speculative one. A
+    submitted callable is kept alive until it has run."""
 
     DEMAND, SPECULATIVE = 0, 1
 
     def __init__(self, worker_count: int = 4):
-        import collections
         import threading
         if worker_count <= 0:
             raise ValueError("workerCount must be positive")
-        self._condition = threading.Condition()
-        self._queues = (collections.deque(), collections.deque())
-        self._closed = False
-        self._workers = [threading.Thread(target=self._run, name=f"Shrike.expert-io.{i}", daemon=True)
-                         for i in range(worker_count)]
-        for worker in self._workers:
-            worker.start()
+        err = C.c_int(0)
+        self._h = capi.load().shrike_io_scheduler_create(worker_count, C.byref(err))
+        if not self._h:
+            raise ShrikeError(capi.last_error())
+        self._lock = threading.Lock()
+        self._pending = {}
+        self._next = 1
+
+        def run(context):
+            with self._lock:
+                work = self._pending.pop(context)
+            work()
+        self._trampoline = capi.IO_WORK(run)  # one C callback for every submission; the context word names the work
 
     def submit(self, work, priority: int = 0) -> None:
-        with self._condition:
-            if self._closed:
-                raise ShrikeError("the expert I/O scheduler is closed")
-            self._queues[priority].append(work)
-            self._condition.notify()
-
-    def _run(self):
-        while True:
-            with self._condition:
-                while not self._closed and not self._queues[0] and not self._queues[1]:
-                    self._condition.wait()
-                if not self._queues[0] and not self._queues[1]:
-                    return  # closed and drained
-                work = (self._queues[0] or self._queues[1]).popleft()
-            work()
+        with self._lock:
+            key, self._next = self._next, self._next + 1
+            self._pending[key] = work
+        rc = capi.load().shrike_io_scheduler_submit(self._h, priority, self._trampoline, key)
+        if rc != 0:
+            with self._lock:
+                self._pending.pop(key, None)
+            raise ShrikeError(capi.last_error())
 
     def close(self) -> None:
         """Runs what is queued, then ends the threads."""
-        with self._condition:
-            self._closed = True
-            self._condition.notify_all()
-        for worker in self._workers:
-            worker.join()
+        if self._h:
+            capi.load().shrike_io_scheduler_close(self._h)
+
+    def __del__(self):
+        try:
+            if self._h:
+                capi.load().shrike_io_scheduler_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class ExpertIOTimeline:
+    """ExpertIOEventCoordinator (sources/Shrike/Infrastructure/Streaming/ExpertIOEventCoordinator.swift:23-90):
+    values never reused, status words in a ring, the published value held behind an out-of-order completion."""
+
+    def __init__(self, status_words: int | None = None, word_count: int = 0):
+        err = C.c_int(0)
+        self._h = capi.load().shrike_io_timeline_create(status_words, word_count, C.byref(err))
+        if not self._h:
+            raise ShrikeError(capi.last_error())
+
+    def reserve(self) -> "capi.IOCompletionToken":
+        token = capi.IOCompletionToken()
+        if capi.load().shrike_io_timeline_reserve(self._h, C.byref(token)) != 0:
+            raise ShrikeError(capi.last_error())
+        return token
+
+    def publish(self, token, succeeded: bool) -> int:
+        return int(capi.load().shrike_io_timeline_publish(self._h, C.byref(token), int(bool(succeeded))))
+
+    @property
+    def published(self) -> int:
+        return int(capi.load().shrike_io_timeline_published(self._h))
+
+    def __del__(self):
+        try:
+            if self._h:
+                capi.load().shrike_io_timeline_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class RouterHostReadback:
+    """RouterHostReadback (sources/Shrike/Runtime/Inference/RouterHostReadback.swift:8-63) over the library's
+    shrike_router_readback_*: `words` is the address of the tagged words (pinned host memory a kernel writes)."""
+
+    @staticmethod
+    def word_count(top_k: int) -> int:
+        return int(capi.load().shrike_router_readback_word_count(top_k))
+
+    @staticmethod
+    def word(tag: int, value: int) -> int:
+        return int(capi.load().shrike_router_readback_word(tag, value))
+
+    @staticmethod
+    def next_tag(tag: int) -> int:
+        return int(capi.load().shrike_router_readback_next_tag(tag))
+
+    @staticmethod
+    def is_complete(words: int, top_k: int, tag: int) -> bool:
+        return bool(capi.load().shrike_router_readback_is_complete(words, top_k, tag))
+
+    @staticmethod
+    def _fields(r, top_k):
+        return dict(hit_count=int(r.hit_count), miss_count=int(r.miss_count), expert_ids=list(r.expert_ids[:top_k]),
+                    weight_bits=list(r.weight_bits[:top_k]), hit_positions=list(r.hit_positions[:r.hit_count]),
+                    miss_positions=list(r.miss_positions[:r.miss_count]), predicted_ids=list(r.predicted_ids[:top_k]))
+
+    @classmethod
+    def decode(cls, words: int, top_k: int, tag: int):
+        r = capi.RouterReadback()
+        if not capi.load().shrike_router_readback_decode(words, top_k, tag, C.byref(r)):
+            return None
+        return cls._fields(r, top_k)
+
+    @classmethod
+    def poll(cls, words: int, top_k: int, tag: int, timeout_nanos: int):
+        """Polls the words until every one carries the tag (the command may still be running); None at the deadline."""
+        r = capi.RouterReadback()
+        if not capi.load().shrike_router_readback_poll(words, top_k, tag, monotonic_nanos() + timeout_nanos, C.byref(r)):
+            return None
+        return cls._fields(r, top_k)
+
+
+def int4_affine_gemv(weights: np.ndarray, scales: np.ndarray, biases: np.ndarray, x: np.ndarray, rows: int, n: int) -> np.ndarray:
+    """shrike_int4_affine_gemv (sources/ShrikeKernelsC/include/shrike_kernels.h:23-29) on host arrays."""
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty(rows, np.float32)
+    capi.load().shrike_int4_affine_gemv(weights.ctypes.data, scales.ctypes.data, biases.ctypes.data, x.ctypes.data, rows, n,
+                                        out.ctypes.data)
+    return out
+
+
+def cpu_expert_ffn_accumulate(blob: np.ndarray, offsets, x: np.ndarray, d: int, f: int, route_weight: float, out: np.ndarray,
+                              scratch: np.ndarray | None = None) -> np.ndarray:
+    """CPUExpertFFN.accumulate (sources/Shrike/Kernels/CPU/CPUExpertFFN.swift:102-140): out += w * FFN(x), fp32."""
+    L = capi.load()
+    if scratch is None:
+        scratch = np.empty(L.shrike_cpu_expert_ffn_scratch_floats(d, f), np.float32)
+    x = np.ascontiguousarray(x, np.float32)
+    rc = L.shrike_cpu_expert_ffn_accumulate(blob.ctypes.data, C.byref(offsets), x.ctypes.data, d, f, route_weight,
+                                            scratch.ctypes.data, out.ctypes.data)
+    if rc != 0:
+        raise ShrikeError(capi.last_error())
+    return out
 
 
 def _ints(values):

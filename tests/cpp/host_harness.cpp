@@ -2,6 +2,7 @@
 // reference writes them against its Swift classes. No GPU call is made: budget ladder,
 // grouping, sweep order, wave planner, slot cache, the packed-experts layout and the parallel reader run on the host. Exit code 0 = all passed.
 #include <array>
+#include <cmath>
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -178,6 +179,85 @@ static void ioScheduler() {
         gate.unlock();
     }  // the destructor drains the queues
     EXPECT(order == (std::vector<int>{0, 1, 2, 10, 11, 12}));
+}
+
+// ExpertLoadOperationTests.swift:95-150: the timeline holds an out-of-order completion, a failure is terminal,
+// status words recycle after one ring
+static void ioCoordinator() {
+    {
+        ExpertIOEventCoordinator coordinator;
+        auto first = coordinator.reserve(), second = coordinator.reserve();
+        coordinator.publish(second, true);
+        EXPECT(*second.status == 1 && coordinator.signaledValue() == 0);
+        coordinator.publish(first, true);
+        EXPECT(coordinator.signaledValue() == second.value && first.value != second.value);
+    }
+    {
+        ExpertIOEventCoordinator coordinator;
+        auto token = coordinator.reserve();
+        coordinator.publish(token, false);
+        EXPECT(*token.status == 2 && coordinator.signaledValue() == token.value);
+    }
+    {
+        ExpertIOEventCoordinator coordinator;
+        auto first = coordinator.reserve();
+        for (uint32_t i = 1; i < ExpertIOEventCoordinator::statusWordCount; ++i) coordinator.publish(coordinator.reserve(), true);
+        coordinator.publish(first, false);
+        auto recycled = coordinator.reserve();
+        EXPECT(recycled.value == first.value + ExpertIOEventCoordinator::statusWordCount);
+        EXPECT(recycled.status == first.status && *recycled.status == 0);
+        coordinator.publish(recycled, true);
+        EXPECT(coordinator.signaledValue() == recycled.value);
+    }
+}
+
+// RouterHostReadbackTests.swift:18-91
+static void routerReadback() {
+    const int topK = 4;
+    auto words = [&](uint32_t tag, uint32_t hits = 3, uint32_t misses = 1) {
+        const uint32_t values[] = {hits, misses, 5, 9, 200, 3, 0x3c00, 0x3800, 0x3400, 0x3000, 0, 2, 3, 0, 1, 0, 0, 0, 1, 2, 3, 4};
+        std::vector<uint32_t> out;
+        for (uint32_t v : values) out.push_back(RouterHostReadback::word(tag, v));
+        return out;
+    };
+    EXPECT(RouterHostReadback::wordCount(4) == 22 && RouterHostReadback::wordCount(8) == 42);
+    auto w = words(7);
+    auto r = RouterHostReadback::decode(w.data(), topK, 7);
+    EXPECT(r && r->hitCount == 3 && r->missCount == 1 && (r->expertIDs == std::vector<uint32_t>{5, 9, 200, 3}));
+    EXPECT(r && (r->weightBits == std::vector<uint16_t>{0x3c00, 0x3800, 0x3400, 0x3000}) && (r->hitPositions == std::vector<uint32_t>{0, 2, 3}));
+    EXPECT(r && (r->missPositions == std::vector<uint32_t>{1}) && (r->predictedIDs == std::vector<uint32_t>{1, 2, 3, 4}));
+    w.back() = RouterHostReadback::word(6, 4);
+    EXPECT(!RouterHostReadback::isComplete(w.data(), topK, 7) && !RouterHostReadback::decode(w.data(), topK, 7));
+    std::vector<uint32_t> zeroed(22, 0u);
+    EXPECT(!RouterHostReadback::isComplete(zeroed.data(), topK, 1));
+    auto clamped = words(3, 9, 9);
+    auto c = RouterHostReadback::decode(clamped.data(), topK, 3);
+    EXPECT(c && c->hitCount == 4 && c->missCount == 4 && c->hitPositions.size() == 4);
+    EXPECT(RouterHostReadback::nextTag(0) == 1 && RouterHostReadback::nextTag(5) == 6 && RouterHostReadback::nextTag(0xffff) == 1);
+    EXPECT(!RouterHostReadback::poll(zeroed.data(), topK, 1, 1000000));
+}
+
+// CPUExpertFFNTests.swift:56-67 (the blob's size) and the closed form of MoEFusedFFNTests: codes 1, scale 1, bias 0
+// make every projection a plain sum
+static void cpuExpertFFN() {
+    const uint32_t d = 128, f = 64;
+    ExpertOffsets off(d, f, 4);
+    std::vector<uint8_t> blob(off.strideBytes, 0);
+    auto fill = [&](uint32_t w_off, uint32_t s_off, uint32_t rows, uint32_t n) {
+        for (uint32_t i = 0; i < rows * n / 2; ++i) blob[w_off + i] = 0x11;
+        for (uint32_t i = 0; i < rows * n / 64; ++i) {
+            blob[s_off + 2 * i] = 0x80;  // bf16 1.0 = 0x3f80
+            blob[s_off + 2 * i + 1] = 0x3f;
+        }
+    };
+    fill(off.gate_w_off, off.gate_s_off, f, d);
+    fill(off.up_w_off, off.up_s_off, f, d);
+    fill(off.down_w_off, off.down_s_off, d, f);
+    std::vector<float> x(d, 1.0f / d), out(d, 1.0f), scratch(CPUExpertFFN::scratchFloats(d, f));
+    CPUExpertFFN::accumulate(blob.data(), off, x.data(), d, f, 0.5f, scratch.data(), out.data());
+    // gate = up = 1, act = silu(1) = 1 / (1 + e^-1), down = f * act, out = 1 + 0.5 * that
+    const float want = 1.0f + 0.5f * float(f) * (1.0f / (1.0f + std::exp(-1.0f)));
+    for (float v : out) EXPECT(std::fabs(v - want) < 1e-4f);
 }
 
 static void slotCache() {
@@ -388,6 +468,9 @@ int main() {
     slotCache();
     landings();
     ioScheduler();
+    ioCoordinator();
+    routerReadback();
+    cpuExpertFFN();
     std::printf(failures ? "%d checks failed\n" : "all host checks passed\n", failures);
     return failures ? 1 : 0;
 }

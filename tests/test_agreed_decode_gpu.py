@@ -9,6 +9,7 @@ import pytest
 
 from shrike_amd import capi, host
 from shrike_amd import synth as S
+from harness import runners
 from tests.helpers import Layer
 from tests.test_decode_gpu import DeviceLayer
 
@@ -58,7 +59,7 @@ def test_agreed_layer_with_a_prefetch_ring_equals_the_resident_layer(gpu, bits, 
     holder = {}
     ring = host.ExpertPrefetchRing(list(range(slots, slots + ring_cells)),
                                    drop=lambda layer, expert, cell: holder["layer"].drop_landing(layer, expert, cell))
-    layer = gpu.AgreedDecodeLayer(small.moe, small.pool, cache, ring, small.off, store, L.stride, L.stride, scheduler,
+    layer = runners.AgreedDecodeLayer(small.moe, small.pool, cache, ring, small.off, store, L.stride, L.stride, scheduler,
                                   layer=3)
     holder["layer"] = layer
     router = dict(weights=small.router_w, eff_scale=small.eff_scale, expert_scale=small.expert_scale, bias=small.logit_bias)
@@ -151,7 +152,7 @@ def test_two_layers_share_one_arena_and_one_ring(gpu):
         store = gpu.PinnedBuffer(ne * L.stride)
         for e in range(ne):
             store.array[e * L.stride:(e + 1) * L.stride] = L.blobs[e]
-        agreed.append(gpu.AgreedDecodeLayer(dev.moe, pools[index], caches[index], ring, dev.off, store, L.stride, L.stride,
+        agreed.append(runners.AgreedDecodeLayer(dev.moe, pools[index], caches[index], ring, dev.off, store, L.stride, L.stride,
                                             scheduler, layer=index))
         routers.append(dict(weights=dev.router_w, eff_scale=dev.eff_scale, expert_scale=dev.expert_scale, bias=dev.logit_bias))
         devs.append(dev)
@@ -221,7 +222,7 @@ def test_a_failed_agreed_read_leaves_the_cache_and_the_ring_clean(gpu):
     holder = {}
     ring = host.ExpertPrefetchRing(list(range(slots, slots + ring_cells)),
                                    drop=lambda layer, expert, cell: holder["layer"].drop_landing(layer, expert, cell))
-    layer = gpu.AgreedDecodeLayer(small.moe, small.pool, cache, ring, small.off, store, L.stride, L.stride, scheduler)
+    layer = runners.AgreedDecodeLayer(small.moe, small.pool, cache, ring, small.off, store, L.stride, L.stride, scheduler)
     holder["layer"] = layer
     router = dict(weights=small.router_w, eff_scale=small.eff_scale, expert_scale=small.expert_scale, bias=small.logit_bias)
     residual = gpu.dev(np.zeros(d, np.uint16))

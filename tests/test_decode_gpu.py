@@ -10,6 +10,7 @@ from oracle import oracle as O
 from shrike_amd import capi
 from shrike_amd import host as HL
 from shrike_amd import synth as S
+from harness import runners
 from tests.helpers import Layer, assert_ffn_close, assert_rel_close, f16
 
 pytestmark = pytest.mark.gpu
@@ -555,27 +556,6 @@ def test_multi_chunk_pool_addressing(gpu):
     assert np.array_equal(outs[0], outs[1])
 
 
-def test_measurement_probes_run_and_check_their_arguments(gpu):
-    """The empty launch and the read-only kernel that bench.py times beside phase 1 (a library of their own)."""
-    from shrike_amd import probes
-    L = Layer(33, 256, 128, 12, 4)
-    dl = DeviceLayer(gpu, L)
-    lib = probes.load()
-    sink = gpu.empty(4).fill(0)
-    cells = gpu.empty(4 * 4)
-    cells.upload(np.array([dl.cell_of[e] for e in (0, 5, 7, 11)], np.uint32))
-    nbytes = (dl.off.down_w_off - dl.off.gate_w_off) // 1024 * 1024
-    probes.check(lib.shrike_probe_empty_launch(None, 64, sink.ptr), "probe_empty_launch")
-    probes.check(lib.shrike_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, dl.off.gate_w_off, nbytes,
-                                       sink.ptr), "probe_read")
-    gpu.synchronize()
-    assert sink.download(np.uint32, 1)[0] == 0
-    assert lib.shrike_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 0, dl.pool.stride + 1024, sink.ptr) != 0
-    assert "leaves the cell" in probes.last_error()
-    assert lib.shrike_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 8, 1024, sink.ptr) != 0
-    assert lib.shrike_probe_empty_launch(None, 0, sink.ptr) != 0
-
-
 def test_argument_errors_are_reported_not_trapped(gpu):
     moe = gpu.MoE(128, 64, 16, 8)
     with pytest.raises(capi.ShrikeError, match="topK"):
@@ -671,7 +651,7 @@ def test_decode_with_misses_equals_the_resident_layer(gpu, bits, resident_of_sel
     warm = cache.plan(resident)
     small.pool.execute_plan(cache, warm, store, L.stride, L.stride)
     gpu.synchronize()
-    layer = gpu.DecodeLayerWithMisses(small.moe, small.pool, cache, small.off, store, L.stride, L.stride)
+    layer = runners.DecodeLayerWithMisses(small.moe, small.pool, cache, small.off, store, L.stride, L.stride)
     router = dict(weights=small.router_w, eff_scale=small.eff_scale, expert_scale=small.expert_scale, bias=small.logit_bias)
     d_res = gpu.dev(residual)
     layer.run(router, small.x, d_res, small.y, small.hidden)

@@ -10,6 +10,7 @@ from oracle import oracle as O
 from shrike_amd import capi
 from shrike_amd import host as HL
 from shrike_amd import synth as S
+from harness import runners
 from tests.helpers import Layer, assert_ffn_close, assert_rel_close, f16
 from tests.test_decode_gpu import DeviceLayer
 
@@ -109,6 +110,39 @@ def test_device_grouping_equals_host_grouping(gpu, t, k, ne, mode):
     assert got["row_tile_count"] <= routes.max_row_tiles
 
 
+def check_pair_stagewise(L: Layer, blob, x_row, dev_act, got_row, what, act=O.ACT_SILU):
+    """Stage by stage, so that each comparison holds one rounding: the activations against the
+    oracle's, the partial row against the oracle's down projection of the device's own
+    activations; then the whole chain in the reference's relative-error metric."""
+    off = L.oracle_offsets()
+    dev_act = np.ascontiguousarray(dev_act)
+    assert_ffn_close(dev_act, O.moe_phase1([blob], off, x_row, L.d, L.f, L.bits, L.meta, act, L.additive), f"{what}: activations")
+    one, zero = np.array([0x3C00], np.uint16), np.zeros(L.d, np.uint16)
+    assert_ffn_close(got_row, O.moe_phase2([blob], off, dev_act, one, zero, L.d, L.f, L.bits, L.meta, L.additive),
+                     f"{what}: partial row from the device's activations")
+    whole = O.prefill_pair_partial(blob, off, x_row, L.d, L.f, L.bits, L.meta, act, L.additive)
+    assert_rel_close(got_row, whole, f"{what}: whole chain")
+
+
+class WorkspaceActs:
+    """The pairs' fp16 activation rows as the grouped FFN left them in its workspace: row tile j keeps rows
+    [64 j, 64 j + 64), a pair sits at its place in the sorted pairs."""
+
+    def __init__(self, routes, ws, t, d, f):
+        self.tables = routes.download()
+        act_off = (t * (d // 64) * 4 + 255) & ~255
+        rows = routes.max_row_tiles * 64
+        self.act = ws.download(np.uint16, rows * f, offset=act_off).reshape(rows, f)
+        self.pos = {(int(r[0]), int(r[2])): i for i, r in enumerate(self.tables["sorted_pairs"])}
+
+    def row(self, tok, rank):
+        at = self.pos[(tok, rank)]
+        for j, (cell, start, rows, expert) in enumerate(self.tables["row_tiles"].tolist()):
+            if start <= at < start + rows:
+                return self.act[j * 64 + at - start]
+        raise AssertionError("pair not covered by a row tile")
+
+
 class PrefillCase:
     def __init__(self, gpu, L: Layer, t, stride_pad=0, idx=None, moe_kwargs=None, resident=None):
         self.gpu, self.L, self.t = gpu, L, t
@@ -134,40 +168,15 @@ class PrefillCase:
         self.gpu.synchronize()
         return self.partials.download(np.uint16, self.t * self.L.k * self.L.d).reshape(self.t, self.L.k, self.L.d)
 
-    def oracle_row(self, tok, rank, act=O.ACT_SILU):
-        L = self.L
-        x = np.ascontiguousarray(self.x[tok * self.stride:tok * self.stride + L.d])
-        return O.prefill_pair_partial(L.blobs[int(self.idx[tok * L.k + rank])], L.oracle_offsets(), x, L.d, L.f, L.bits, L.meta,
-                                      act, L.additive)
-
     def device_act(self, tok, rank):
-        """The pair's fp16 activation row in the workspace: row tile j keeps rows [64 j, 64 j + 64)."""
-        L = self.L
-        if not hasattr(self, "_tables"):
-            self._tables = self.routes.download()
-            act_off = (self.t * (L.d // 64) * 4 + 255) & ~255
-            rows = self.routes.max_row_tiles * 64
-            self._act = self.ws.download(np.uint16, rows * L.f, offset=act_off).reshape(rows, L.f)
-            self._pos = {(int(r[0]), int(r[2])): i for i, r in enumerate(self._tables["sorted_pairs"])}
-        at = self._pos[(tok, rank)]
-        for j, (cell, start, rows, expert) in enumerate(self._tables["row_tiles"].tolist()):
-            if start <= at < start + rows:
-                return self._act[j * 64 + at - start]
-        raise AssertionError("pair not covered by a row tile")
+        if not hasattr(self, "_acts"):
+            self._acts = WorkspaceActs(self.routes, self.ws, self.t, self.L.d, self.L.f)
+        return self._acts.row(tok, rank)
 
     def check_pair(self, got, tok, rank, what, act=O.ACT_SILU):
-        """Stage by stage, so that each comparison holds one rounding: the activations against the
-        oracle's, the partial row against the oracle's down projection of the device's own
-        activations; then the whole chain in the reference's relative-error metric."""
         L = self.L
-        blob, off = L.blobs[int(self.idx[tok * L.k + rank])], L.oracle_offsets()
         x = np.ascontiguousarray(self.x[tok * self.stride:tok * self.stride + L.d])
-        dev_act = np.ascontiguousarray(self.device_act(tok, rank))
-        assert_ffn_close(dev_act, O.moe_phase1([blob], off, x, L.d, L.f, L.bits, L.meta, act, L.additive), f"{what}: activations")
-        one, zero = np.array([0x3C00], np.uint16), np.zeros(L.d, np.uint16)
-        assert_ffn_close(got[tok, rank], O.moe_phase2([blob], off, dev_act, one, zero, L.d, L.f, L.bits, L.meta, L.additive),
-                         f"{what}: partial row from the device's activations")
-        assert_rel_close(got[tok, rank], self.oracle_row(tok, rank, act), f"{what}: whole chain")
+        check_pair_stagewise(L, L.blobs[int(self.idx[tok * L.k + rank])], x, self.device_act(tok, rank), got[tok, rank], what, act)
 
 
 FFN_CASES = [
@@ -234,6 +243,21 @@ def test_grouped_ffn_gpt_oss_epilogues(gpu):
     for tok in range(5):
         for rank in range(2):
             pc.check_pair(got, tok, rank, f"gpt-oss token {tok} rank {rank}", O.ACT_CLAMPED_SWIGLU)
+
+
+@pytest.mark.parametrize("d,f,ne,k,t,bits", [(512, 256, 6, 2, 70, 4), (320, 192, 5, 3, 21, 8)])
+def test_grouped_ffn_gelu_tanh(gpu, d, f, ne, k, t, bits):
+    # the GELU-tanh GLU of moe.metal:98-105 through the grouped kernels (prefill.metal:318-363): one- and two-tile
+    # row tiles, both code widths
+    L = Layer(0x5EED0009, d, f, ne, k, bits=bits, meta=S.META_F16)
+    pc = PrefillCase(gpu, L, t, moe_kwargs=dict(activation=capi.ACT_GELU_TANH))
+    got = pc.run()
+    rng = np.random.default_rng(8)
+    for tok, rank in {(int(a), int(b)) for a, b in zip(rng.integers(0, t, 30), rng.integers(0, k, 30))}:
+        pc.check_pair(got, tok, rank, f"gelu token {tok} rank {rank}", O.ACT_GELU_TANH)
+    # and it is not the SiLU result: the activation switch reached the kernel
+    silu = PrefillCase(gpu, L, t).run()
+    assert not np.array_equal(silu, got)
 
 
 def test_grouped_ffn_skips_absent_experts(gpu):
@@ -332,11 +356,11 @@ def test_reduce_and_residual_bit_exact(gpu):
 
 
 def test_prefill_layer_at_full_size_agrees_with_the_decode_kernels(gpu):
-    """T = 512 tokens, 256 experts, top 8 at the 35B-A3B int4 shape: too large for the CPU oracle,
-    so the whole chain (router -> grouping -> grouped FFN -> reduce) is checked by what does not
-    depend on size: the grouping is a permutation with the host function's tables, and every
-    sampled token's h2 equals the decode kernels' y for that token alone (no shared expert,
-    residual 0), which the decode tests hold to the oracle."""
+    """T = 512 tokens, 256 experts, top 8 at the 35B-A3B int4 shape with the Zipf(1.1) skew: the routes of all
+    512 tokens equal the oracle's router bit for bit (logits, indices), the grouping is a permutation with the
+    host function's tables, 24 sampled pairs' activation and partial rows are held to the oracle stage by stage,
+    the reduced rows equal the oracle's reduce of the device's partial rows, and sampled tokens' h2 agree with
+    the decode kernels' y for that token alone (no shared expert, residual 0)."""
     d, f, ne, k, t = 2048, 512, 256, 8, 512
     L = Layer(0x5EED0003, d, f, ne, k, bits=4, meta=S.META_F16)
     # Zipf skew through the logit bias operand, over a seeded permutation
@@ -357,13 +381,36 @@ def test_prefill_layer_at_full_size_agrees_with_the_decode_kernels(gpu):
     pf.encode_reduce_token_major(partials, w, h2, t, k, d)
     gpu.synchronize()
     h_idx, h_w = idx.download(np.uint32, t * k), w.download(np.uint16, t * k)
+    # every token's routes against the oracle's router, bit for bit
+    ref_idx, ref_w, ref_logits = O.prefill_router(L.router_dict(), x, t, d, k)
+    assert np.array_equal(ws.download(np.float32, t * ne).view(np.uint32), ref_logits.reshape(-1).view(np.uint32))
+    assert np.array_equal(h_idx, ref_idx), "a token's routing indices differ from the oracle's"
+    assert np.max(np.abs(f16(h_w) - f16(ref_w))) <= 1e-3
+    counts = np.bincount(h_idx, minlength=ne)
+    assert counts.max() > 64 and np.count_nonzero(counts) < ne, "the skew should give long experts and leave some without a pair"
     got = routes.download()
     host = HL.group_token_expert_pairs(HL.make_token_expert_pairs(h_idx, h_w, t, k), t, k, ne)
     assert got["counts"].tolist() == host.per_expert_counts.tolist() and int(got["counts"].sum()) == t * k
     assert got["offsets"].tolist() == host.per_expert_offsets.tolist()
     assert np.array_equal(got["sorted_pairs"], host.sorted_pairs.view(np.uint32).reshape(-1, 4))
     out = h2.download(np.uint16, t * d).reshape(t, d)
-    assert not np.any(np.all(partials.download(np.uint16, t * k * d).reshape(t * k, d) == 0xD4D0, axis=-1))
+    rows = partials.download(np.uint16, t * k * d).reshape(t, k, d)
+    assert not np.any(np.all(rows.reshape(t * k, d) == 0xD4D0, axis=-1))
+    # sampled pairs against the oracle, stage by stage: pairs of the longest expert (two MFMA row tiles, several row
+    # tiles), of an expert with a single pair if the routes have one, and 20 drawn over the chunk
+    acts = WorkspaceActs(routes, work, t, d, f)
+    rng = np.random.default_rng(6)
+    sample = {(int(a), int(b)) for a, b in zip(rng.integers(0, t, 20), rng.integers(0, k, 20))}
+    by_expert = {}
+    for i, e in enumerate(h_idx.tolist()):
+        by_expert.setdefault(e, []).append((i // k, i % k))
+    longest = by_expert[int(np.argmax(counts))]
+    sample.update([longest[0], longest[len(longest) // 2], longest[-1]])
+    sample.add(by_expert[min(by_expert, key=lambda e: len(by_expert[e]))][0])
+    for tok, rank in sorted(sample):
+        check_pair_stagewise(L, L.blobs[int(h_idx[tok * k + rank])], np.ascontiguousarray(x[tok * d:(tok + 1) * d]),
+                             acts.row(tok, rank), rows[tok, rank], f"full-size chunk token {tok} rank {rank}")
+    assert np.array_equal(out.reshape(-1), O.prefill_reduce(rows.reshape(-1), h_w, t, k, d)), "reduce differs from the oracle's"
     zero = gpu.dev(np.zeros(d, np.uint16))
     for tok in (0, 1, 77, 255, 256, 511):
         one = gpu.dev(np.ascontiguousarray(x[tok * d:(tok + 1) * d]))
@@ -450,7 +497,7 @@ def test_batched_decode_through_a_pool_smaller_than_the_expert_set(gpu, d, f, ne
     store = gpu.PinnedBuffer(ne * L.stride)
     for e in range(ne):
         store.array[e * L.stride:(e + 1) * L.stride] = L.blobs[e]
-    layer = gpu.BatchedDecodeLayer(dl.moe, dl.pool, cache, dl.off, store, L.stride, L.stride, t)
+    layer = runners.BatchedDecodeLayer(dl.moe, dl.pool, cache, dl.off, store, L.stride, L.stride, t)
     x = token_rows(L, t, d)
     hidden = gpu.dev(x)
     router = dict(weights=dl.router_w, eff_scale=dl.eff_scale, expert_scale=dl.expert_scale, bias=dl.logit_bias)
@@ -462,12 +509,14 @@ def test_batched_decode_through_a_pool_smaller_than_the_expert_set(gpu, d, f, ne
     used = len(set(idx.tolist()))
     assert layer.passes == -(-used // slots) and layer.passes >= 2
     partials = layer.partials.download(np.uint16, t * k * d).reshape(t, k, d)
-    off = L.oracle_offsets()
+    # every pair stage by stage (the passes share one grouping, so a pair's activation row stays where the pass that
+    # served its expert left it)
+    acts = WorkspaceActs(layer.routes, layer.ffn_ws, t, d, f)
     for tok in range(t):
         xt = np.ascontiguousarray(x[tok * d:(tok + 1) * d])
         for rank in range(k):
-            ref = O.prefill_pair_partial(L.blobs[int(idx[tok * k + rank])], off, xt, d, f, bits, L.meta)
-            assert_rel_close(partials[tok, rank], ref, f"token {tok} rank {rank}")
+            check_pair_stagewise(L, L.blobs[int(idx[tok * k + rank])], xt, acts.row(tok, rank), partials[tok, rank],
+                                 f"token {tok} rank {rank}")
     assert np.array_equal(h2.download(np.uint16, t * d), O.prefill_reduce(partials.reshape(-1), w, t, k, d))
     st = cache.statistics(L.stride)
     assert (st.plans, st.requested_experts, st.misses, st.hits) == (layer.passes, used, used, 0)

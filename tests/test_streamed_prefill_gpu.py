@@ -7,6 +7,7 @@ import pytest
 from oracle import oracle as O
 from shrike_amd import capi, host
 from shrike_amd import synth as S
+from harness import runners
 from tests.helpers import Layer, assert_rel_close
 from tests.test_decode_gpu import DeviceLayer
 from tests.test_prefill_gpu import token_rows
@@ -50,7 +51,7 @@ def test_streamed_chunk_equals_the_resident_chunk(gpu, tmp_path, slots, depth, w
     cache = host.SlotCache(slots, ne)
     config = host.TileSchedulerConfig(max_pending_depth=depth, tile_experts=8, tiles_per_command_buffer=width,
                                       fetch_lookahead=lookahead)
-    layer = gpu.StreamedPrefillLayer(small.moe, small.pool, cache, layout.expert_offsets(0, False), reader,
+    layer = runners.StreamedPrefillLayer(small.moe, small.pool, cache, layout.expert_offsets(0, False), reader,
                                      [layout.expert(0, e)["offset"] for e in range(ne)], stride, gpu.PinnedBuffer(4 * stride), t, config)
     assert layer.config.fits_slot_budget(slots)
     router = dict(weights=small.router_w, eff_scale=small.eff_scale, expert_scale=small.expert_scale, bias=small.logit_bias)
@@ -111,7 +112,7 @@ def test_a_failed_read_ends_the_chunk_and_leaves_no_slot_loading(gpu, tmp_path):
     ids, _, _ = O.prefill_router(L.router_dict(), x, t, d, k)
     victim = sorted(set(ids.tolist()))[-1]       # in the chunk's last tile
     offsets[victim] = ne * stride                 # past the end of the file
-    layer = gpu.StreamedPrefillLayer(small.moe, small.pool, cache, layout.expert_offsets(0, False), reader, offsets, stride,
+    layer = runners.StreamedPrefillLayer(small.moe, small.pool, cache, layout.expert_offsets(0, False), reader, offsets, stride,
                                      gpu.PinnedBuffer(4 * stride), t, host.TileSchedulerConfig(2, 8, 1, 1))
     router = dict(weights=small.router_w, eff_scale=small.eff_scale, expert_scale=small.expert_scale, bias=small.logit_bias)
     with pytest.raises(capi.ShrikeError, match="expert read failed"):

@@ -16,7 +16,7 @@ SCRATCH_FIELDS = ("resolved_slots", "hit_count", "hit_positions", "miss_count", 
                   "acts", "shared_scratch", "h1")
 
 
-def run_both(gpu, L, resident=None, bind_lists=False):
+def run_both(gpu, L, resident=None, bind_lists=False, stream=None):
     d, k = L.d, L.k
     dl = DeviceLayer(gpu, L, resident=resident)
     dl.moe.encode_decode_layer(dl.layer_args())
@@ -32,8 +32,16 @@ def run_both(gpu, L, resident=None, bind_lists=False):
     for name in SCRATCH_FIELDS:
         if not (bind_lists and name in ("resolved_slots", "miss_count")):
             setattr(args, name, None)
-    capi.check(capi.load().shrike_hip_moe_decode_layer_noalloc(C.byref(dl.moe.desc), None, C.byref(args)),
+    # what the entry point exists for: device memory is not allocated (or freed) by the call. The first call of the
+    # process has looked the scratch's address up already (shrike_hip_init does), so every call is held to it.
+    lib = capi.load()
+    free_before, free_after = C.c_uint64(0), C.c_uint64(0)
+    gpu.synchronize()
+    capi.check(lib.shrike_hip_mem_info(C.byref(free_before), None), "shrike_hip_mem_info")
+    capi.check(lib.shrike_hip_moe_decode_layer_noalloc(C.byref(dl.moe.desc), stream.handle if stream else None, C.byref(args)),
                "shrike_hip_moe_decode_layer_noalloc")
+    capi.check(lib.shrike_hip_mem_info(C.byref(free_after), None), "shrike_hip_mem_info")
+    assert free_after.value == free_before.value, "the allocation-free entry point changed the device's free memory"
     gpu.synchronize()
     assert np.array_equal(dl.out_idx.download(np.uint32, k), want["idx"])
     assert np.array_equal(dl.out_w.download(np.uint16, k), want["w"])
@@ -55,6 +63,7 @@ def test_the_allocation_free_layer_equals_the_layer_entry_point(gpu):
     assert 0 < want["misses"] < 8
     no_shared = Layer(0x5EED0703, 2880, 192, 32, 4, router_bits=8)
     run_both(gpu, no_shared)
+    run_both(gpu, small, stream=gpu.Stream())  # on a stream of the caller's: the scratch is the stream's device's
 
 
 def test_the_allocation_free_layer_rejects_what_its_scratch_cannot_hold(gpu):
