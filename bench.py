@@ -43,8 +43,21 @@ if ROOT not in sys.path:
 D, F, NE, K, FS, BITS = 2048, 512, 256, 8, 512, 4
 HBM_PEAK_GBPS = 8000.0
 REGIONS = 15          # timed regions; the median is reported
+CHASE_HOPS = 64       # dependent loads in the round-trip probe
 X_VARIANTS = 4        # activation vectors in rotation
 PROFILES = os.path.join(ROOT, "profiles")
+
+
+# Under rocprofv3 a run of --steps 2000 once ended in an abort inside hipGraphLaunch (an earlier form of this file: one
+# executable graph of 120 kernel nodes launched fifty times back to back). Its cause was never shown, so a profiled run
+# is held to what has run clean under the profiler: at most this many steps a region.
+PROFILED_MAX_STEPS = 400
+
+
+def profiler_attached() -> bool:
+    env = os.environ
+    named = " ".join(env.get(k, "") for k in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB", "ROCPROFILER_LIBRARY_PATH"))
+    return "rocprof" in named.lower() or any(k.startswith(("ROCPROF_", "ROCPROFILER_")) for k in env)
 
 
 def profile_figure(filename: str, key: str):
@@ -120,7 +133,13 @@ def build_layers(rt, capi, S, n_layers, meta, shared=True):
 
 def capture(rt, capi, stream, body):
     capi.check(capi.load().shrike_hip_graph_begin_capture(stream.handle), "graph_begin_capture")
-    body()
+    try:
+        body()
+    except Exception:
+        broken = capi.load().shrike_hip_graph_end_capture(stream.handle)  # the stream must leave capture mode
+        if broken:
+            capi.load().shrike_hip_graph_destroy(broken)
+        raise
     g = capi.load().shrike_hip_graph_end_capture(stream.handle)
     if not g:
         raise capi.ShrikeError(capi.last_error())
@@ -183,6 +202,18 @@ class LayerWalk:
             self.variant = (self.variant + 1) % X_VARIANTS
             steps -= count
 
+    def encode(self, steps):
+        """Encodes exactly `steps` layers on the stream (for a capture that holds several regions), continuing where
+        the last call stopped, the activation variant moving on at every wrap of the stack as in enqueue."""
+        n = len(self.layers)
+        while steps > 0:
+            count = min(steps, n - self.at)
+            for lay in self.layers[self.at:self.at + count]:
+                self.moe.encode_decode_layer(lay["args_x"][self.variant])
+            self.at = (self.at + count) % n
+            self.variant = (self.variant + 1) % X_VARIANTS
+            steps -= count
+
     def plan(self, steps, regions):
         """Captures what `regions` regions of `steps` steps will launch, so that no capture falls into a timed region."""
         at, variant = self.at, self.variant
@@ -220,6 +251,21 @@ def cpu_baseline(S, blobs, sample_layers, meta):
     for e in picks:
         O.cpu_expert_ffn_accumulate(blobs[int(e)], off, x, D, F, 0.125, out, bits=BITS, meta=meta)
     per_expert = (time.perf_counter() - t0) / singles
+    # the library's own host export of the same kernel (shrike_cpu_expert_ffn_accumulate: what a host that keeps experts
+    # in CPU memory would call), over blobs with the bf16 metadata the reference's CPU kernel takes
+    from shrike_amd import host as HL
+    from shrike_amd import capi as _capi
+    tree_p = S.SeedTree(0x5EED0001)
+    blobs_p = [S.expert_blob(tree_p, f"expert.{e}", D, F, BITS, S.META_BF16) for e in range(8)]
+    p_off = _capi.ExpertOffsets()
+    _capi.load().shrike_expert_offsets_make(D, F, BITS, 0, p_off)
+    p_scratch = np.empty(2 * F + D, np.float32)
+    p_out = np.zeros(D, np.float32)
+    xp = np.ascontiguousarray(x, np.float32)
+    t0 = time.perf_counter()
+    for i in range(singles):
+        HL.cpu_expert_ffn_accumulate(blobs_p[i % len(blobs_p)], p_off, xp, D, F, 0.125, p_out, p_scratch)
+    per_product = (time.perf_counter() - t0) / singles
     # the same with the reference's own shrike_int4_affine_gemv, compiled from its source by oracle/Makefile where the
     # reference checkout was present at build time (three calls and the fp32 SiLU-multiply between them, as
     # CPUExpertFFN.accumulate composes them); its metadata is bf16, so it runs over blobs generated with bf16 metadata
@@ -256,9 +302,11 @@ def cpu_baseline(S, blobs, sample_layers, meta):
                       f"256-expert pool, fp32 scalar C port of shrike_int4_affine_gemv + CPUExpertFFN.accumulate, "
                       f"{cores} threads, gcc -O2",
             "config1": {"workload": "config 1: one routed expert SwiGLU FFN for one token (hidden 2048, intermediate 512, int4)",
-                        "cores": 1, "us_per_expert": round(per_expert * 1e6, 1),
-                        "value": round(1_769_472 / per_expert / 1e9, 3), "unit": "GB/s", "bytes_per_expert": 1_769_472,
-                        "sample": f"{singles} experts drawn from the pool, one thread",
+                        "cores": 1, "kind": "port", "us_per_expert": round(per_product * 1e6, 1),
+                        "value": round(1_769_472 / per_product / 1e9, 3), "unit": "GB/s", "bytes_per_expert": 1_769_472,
+                        "sample": f"{singles} calls of the library's host export shrike_cpu_expert_ffn_accumulate over 8 seeded experts, one thread",
+                        "oracle_port": {"us_per_expert": round(per_expert * 1e6, 1), "value": round(1_769_472 / per_expert / 1e9, 3),
+                                        "unit": "GB/s", "sample": f"{singles} experts drawn from the pool through the oracle's scalar C, one thread"},
                         **({"reference_c": reference} if reference else {})}}
 
 
@@ -465,7 +513,10 @@ def gptoss_workload(args, rt, capi, S, meta, bits):
 def kimi_workload(args, rt, capi, S, meta):
     """Config 5: 16 sequences, one token each, Kimi-Linear-48B shape (hidden 2304, 256 int8 experts of
     intermediate 1024, top-8, shared expert 1024); the pool holds 64 of the 256 experts and misses are copied
-    from pinned host memory on a side stream. Reports the miss rate, the wall time per step and the host->device rate."""
+    from pinned host memory on a side stream. Reports the miss rate, the wall time per step and the host->device
+    rate; beside them the step with every expert resident (what the kernels alone take), the step's time on each
+    stream (how much of the copies runs beside kernels), and the miss rate under the other eviction policy."""
+    from harness import runners
     from shrike_amd import host as HL
     d, f, ne, k, t, bits, slots = 2304, 1024, 256, 8, 16, 8, 64
     tree = S.SeedTree(0x5EED0005)
@@ -473,12 +524,8 @@ def kimi_workload(args, rt, capi, S, meta):
     store = rt.PinnedBuffer(ne * stride)
     for e in range(ne):
         store.array[e * stride:(e + 1) * stride] = S.expert_blob(tree, f"layer.0.expert.{e}", d, f, bits, meta)
-    pool = rt.ExpertPool(slots, stride, ne)
-    cache = HL.SlotCache(slots, ne)
     moe = rt.MoE(d, f, ne, k, routed_bits=bits, router_bits=0, meta=meta)
     moe.stream = rt.Stream()
-    from harness import runners
-    layer = runners.BatchedDecodeLayer(moe, pool, cache, off, store, stride, stride, t)
     router = dict(weights=rt.dev(S.router_f16(tree, "router.w", ne, d)), eff_scale=rt.dev(S.f32_to_bf16_bits(np.ones(d, np.float32))),
                   expert_scale=rt.dev(S.f32_to_bf16_bits(np.ones(ne, np.float32))), bias=rt.dev(np.zeros(ne, np.uint16)))
     shared = {n: tuple(rt.dev(a) for a in S.affine_matrix(tree.key(f"shared.{n}"), r, c, bits, meta))
@@ -486,26 +533,60 @@ def kimi_workload(args, rt, capi, S, meta):
     h1 = rt.empty(2 * t * d)
     batches = [rt.dev(S.activations_f16(tree, f"x.{i}", t * d)) for i in range(8)]
     steps, warm = max(8, args.steps // 100), 8
-    sws = None
 
-    def step(i):
-        nonlocal sws
-        x = batches[i % len(batches)]
-        layer.run(router, x, t, d)
-        sws = layer.pf.encode_shared_expert(shared["gate"], shared["up"], shared["down"], bits, x, d, h1, t, f, workspace=sws)
-        layer.pf.residual_add(layer.h2, h1, t * d)
-        moe.stream.synchronize()
+    def run(cells, slru_share, steps, trace=False):
+        """`steps` steps through a pool of `cells` cells under one eviction policy, after 8 warm-up steps."""
+        pool = rt.ExpertPool(cells, stride, ne)
+        cache = HL.SlotCache(cells, ne, slru_share=slru_share)
+        layer = runners.BatchedDecodeLayer(moe, pool, cache, off, store, stride, stride, t)
+        sws = [None]
 
-    for i in range(warm):
-        step(i)
-    base = cache.statistics(stride)
-    base = (base.requested_experts, base.misses, base.bytes_read, base.plans)
-    t0 = time.perf_counter()
-    for i in range(steps):
-        step(warm + i)
-    dt = time.perf_counter() - t0
-    st = cache.statistics(stride)
-    req, miss, read, plans = st.requested_experts - base[0], st.misses - base[1], st.bytes_read - base[2], st.plans - base[3]
+        def step(i):
+            x = batches[i % len(batches)]
+            layer.run(router, x, t, d)
+
+            def tail():
+                sws[0] = layer.pf.encode_shared_expert(shared["gate"], shared["up"], shared["down"], bits, x, d, h1, t, f, workspace=sws[0])
+                layer.pf.residual_add(layer.h2, h1, t * d)
+            if layer.trace is None:
+                tail()
+            else:
+                start, stop = rt.Event(), rt.Event()
+                start.record(moe.stream)
+                tail()
+                stop.record(moe.stream)
+                layer.trace.append(("compute", start, stop))
+            moe.stream.synchronize()
+
+        for i in range(warm):
+            step(i)
+        base = cache.statistics(stride)
+        base = (base.requested_experts, base.misses, base.bytes_read, base.plans)
+        if trace:
+            layer.trace = []
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(warm + i)
+        dt = time.perf_counter() - t0
+        st = cache.statistics(stride)
+        out = dict(dt=dt, steps=steps, requested=st.requested_experts - base[0], misses=st.misses - base[1],
+                   read=st.bytes_read - base[2], plans=st.plans - base[3], on_stream={})
+        if trace:
+            for name, start, stop in layer.trace:
+                out["on_stream"][name] = out["on_stream"].get(name, 0.0) + start.elapsed_ms(stop)
+        pool.close()
+        return out
+
+    main = run(slots, None, steps)
+    dt, req, miss, read, plans = main["dt"], main["requested"], main["misses"], main["read"], main["plans"]
+    # the same steps with every expert resident (256 cells): what the kernels alone take, every route a hit
+    resident = run(ne, None, steps)
+    # the step's time on each stream (events round everything enqueued), a shorter run of its own: kernels and copies
+    # summed apart against the wall clock say how much of one runs beside the other
+    traced = run(slots, None, max(4, steps // 4), trace=True)
+    n_tr = traced["steps"]
+    copy_ms, kernel_ms, wall_ms = traced["on_stream"].get("upload", 0.0) / n_tr, traced["on_stream"].get("compute", 0.0) / n_tr, traced["dt"] / n_tr * 1e3
+    slru = run(slots, 0.5, max(8, steps // 2))
     cpu = None
     if getattr(args, "cpu_sample", 0) > 0:  # one step's 128 routed + 16 shared-expert FFNs on the host's cores
         views = [store.array[e * stride:e * stride + stride] for e in range(0, ne, 4)]
@@ -517,9 +598,19 @@ def kimi_workload(args, rt, capi, S, meta):
         "dtype": "f16 x u8 -> f32", "data": "synthetic (seeded SplitMix64), 8 token batches in rotation",
         "config": {"workload": f"config 5: {t} sequences, top-{k} of {ne} int8 experts, hidden {d}, intermediate {f}, shared expert {f}, "
                                f"pool of {slots} cells, misses from pinned host memory on a side stream",
-                   "passes_per_step": round(plans / steps, 2)},
+                   "passes_per_step": round(plans / steps, 2), "eviction": "aging LFU (the reference's default)"},
         "miss_rate": round(miss / max(1, req), 4), "experts_requested_per_step": round(req / steps, 1),
         "host_to_device_GBps": round(read / dt / 1e9, 2), "bytes_copied_per_step": int(read / steps),
+        "hit_only_kernel_ms": round(resident["dt"] / resident["steps"] * 1e3, 4),
+        "hit_only": {"cells": ne, "miss_rate": round(resident["misses"] / max(1, resident["requested"]), 4),
+                     "note": "the same steps through a pool that holds all 256 experts: router, grouping, grouped FFN, reduce, shared "
+                             "expert, wall clock with the step's host synchronisations"},
+        "timeline_ms_per_step": {"copies_on_the_upload_stream": round(copy_ms, 4), "kernels_on_the_compute_stream": round(kernel_ms, 4),
+                                 "wall_clock": round(wall_ms, 4)},
+        "copy_ms_hidden_behind_compute": round(max(0.0, copy_ms + kernel_ms - wall_ms), 4),
+        "miss_rate_by_policy": {"aging_lfu": round(miss / max(1, req), 4),
+                                "slru_protected_share_0.5": round(slru["misses"] / max(1, slru["requested"]), 4)},
+        "miss_rate_floor": round(max(0.0, req / steps - slots) / max(1e-9, req / steps), 4),
         **({"cpu_baseline": cpu} if cpu else {})}
 
 
@@ -543,17 +634,50 @@ def decode_workload(args, rt, capi, S, meta):
     walk = LayerWalk(rt, capi, moe, stream, layers)
     walk.plan(warm, 1)
     walk.enqueue(warm)
-    walk.plan(steps, REGIONS)
-    events = [rt.Event() for _ in range(REGIONS + 1)]
-    stream.synchronize()
-    rt.synchronize()
-    events[0].record(stream)
-    for r in range(REGIONS):
-        walk.enqueue(steps)
-        events[r + 1].record(stream)
-    events[-1].synchronize()
-    rt.synchronize()
-    region_ms = [events[r].elapsed_ms(events[r + 1]) for r in range(REGIONS)]
+    region_ms, timing_method, whole_graph_us = None, None, None
+    from harness import probes as _probes
+    clock_khz = _probes.load().shrike_probe_wall_clock_khz()
+    if args.timing == "graph" and clock_khz > 0:
+        # All REGIONS regions are ONE captured graph with a time-stamp kernel between regions (one thread stores the
+        # device's constant-rate clock, in graph order): a region is then K layers and one 64-thread launch, where a
+        # graph launch per region bills every region a launch boundary of its own (about 19 us on this part, which a
+        # 20-layer region feels). HIP events cannot do this: an event recorded by a captured graph cannot be timed
+        # (hipEventElapsedTime: invalid resource handle). Events still bracket the whole graph as the cross-check.
+        stamps = rt.empty(8 * (REGIONS + 1)).fill(0)
+
+        def regions_body():
+            _probes.check(_probes.load().shrike_probe_timestamp(stream.handle, stamps.ptr), "probe_timestamp")
+            for r in range(REGIONS):
+                walk.encode(steps)
+                _probes.check(_probes.load().shrike_probe_timestamp(stream.handle, stamps.ptr + 8 * (r + 1)), "probe_timestamp")
+        timed = capture(rt, capi, stream, regions_body)
+        first, last = rt.Event(), rt.Event()
+        stream.synchronize()
+        rt.synchronize()
+        first.record(stream)
+        capi.check(capi.load().shrike_hip_graph_launch(timed, stream.handle), "graph_launch")
+        last.record(stream)
+        last.synchronize()
+        rt.synchronize()
+        ticks = stamps.download(np.uint64, REGIONS + 1).astype(np.int64)
+        region_ms = [float(ticks[r + 1] - ticks[r]) / clock_khz for r in range(REGIONS)]
+        whole_graph_us = first.elapsed_ms(last) * 1e3 / (REGIONS * steps)
+        capi.check(capi.load().shrike_hip_graph_destroy(timed), "graph_destroy")
+        timing_method = (f"one captured graph of {REGIONS} regions of K layers, the device clock ({clock_khz} kHz) stored by a "
+                         "one-thread kernel between regions; HIP events round the whole graph as the cross-check")
+    if region_ms is None:
+        events = [rt.Event() for _ in range(REGIONS + 1)]
+        walk.plan(steps, REGIONS)
+        stream.synchronize()
+        rt.synchronize()
+        events[0].record(stream)
+        for r in range(REGIONS):
+            walk.enqueue(steps)
+            events[r + 1].record(stream)
+        events[-1].synchronize()
+        rt.synchronize()
+        region_ms = [events[r].elapsed_ms(events[r + 1]) for r in range(REGIONS)]
+        timing_method = "graph launches of up to 40 layers, a HIP event record between regions"
     ms_per_step = statistics.median(region_ms) / steps
     # the experts a pass over the stack touches, per activation variant (routes differ from variant to variant)
     distinct = set()
@@ -605,6 +729,20 @@ def decode_workload(args, rt, capi, S, meta):
             probes.check(probes.load().shrike_probe_read(stream.handle, lay["pool"].bases, lay["pool"].stride, lay["res"].ptr,
                                                          K, off.gate_w_off, p1_bytes_per_cell, sink.ptr), "probe_read")
 
+    # a memory round trip as a kernel sees it: one wave walks CHASE_HOPS dependent loads through a 128 MB table, 4 MB and
+    # a line apart (every hop a miss of the caches on the compute units' side); each launch starts elsewhere
+    chase_words, chase_stride = 32 << 20, (1 << 20) + 16
+    chase = rt.dev(((np.arange(chase_words, dtype=np.uint64) + chase_stride) % chase_words).astype(np.uint32))
+
+    def empty_one():
+        for lay in layers:
+            probes.check(probes.load().shrike_probe_empty_launch(stream.handle, 1, sink.ptr), "probe_empty_launch")
+
+    def chase_only():
+        for l, lay in enumerate(layers):
+            probes.check(probes.load().shrike_probe_dependent_loads(stream.handle, chase.ptr, chase_words, CHASE_HOPS, 4099 * l + 64,
+                                                                    sink.ptr), "probe_dependent_loads")
+
     # the step ahead of the layer (residual add + RMS norm producing x): as a launch of its own, and in the
     # prologue of the layer's first launch; both on a residual stream and an x buffer of their own
     tree_n = S.SeedTree(0x5EED0003)
@@ -640,6 +778,8 @@ def decode_workload(args, rt, capi, S, meta):
                        ("operator: shared expert (2 launches)", shared_only),
                        ("floor: empty launch of phase 1's grid", empty_only),
                        ("floor: read-only kernel over phase 1's routed bytes", read_only),
+                       ("floor: empty launch of one workgroup", empty_one),
+                       (f"floor: one wave, {CHASE_HOPS} dependent loads", chase_only),
                        ("norm launch + layer (4 launches)", norm_apart),
                        ("layer with the norm in its first launch", norm_fused)):
         g = capture(rt, capi, stream, body)
@@ -656,6 +796,15 @@ def decode_workload(args, rt, capi, S, meta):
     alone_us = parts["operator: phase 1 alone (no routing, no shared rows)"]
     value = expert_bytes / (ms_per_step * 1e-3) / 1e9
     kernel = "k_phase1<4,1,4,true,4,true>"
+    # The floor of the layer AS IT IS BUILT (three launches in a row, five dependent memory round trips: x and rows in
+    # the first; the route table, then rows in the second; cells and activations, then rows in the third), from this
+    # run's own probes: launches x an empty launch + round trips x one dependent load + the layer's bytes at the rate
+    # the read-only kernel streams at once it has started.
+    empty_us = parts["floor: empty launch of phase 1's grid"]
+    read_us = parts["floor: read-only kernel over phase 1's routed bytes"]
+    hop_us = max(0.0, parts[f"floor: one wave, {CHASE_HOPS} dependent loads"] - parts["floor: empty launch of one workgroup"]) / CHASE_HOPS
+    stream_gbps = routed_gate_up / max(1e-9, (read_us - empty_us) * 1e-6) / 1e9
+    floor_us = 3 * empty_us + 5 * hop_us + total_bytes / (stream_gbps * 1e9) * 1e6
     out = {
         "metric": "MoE-layer decode: HBM GB/s on expert bytes (us per layer in ms_per_step), 35B-A3B int4 shape",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warm,
@@ -665,12 +814,15 @@ def decode_workload(args, rt, capi, S, meta):
         "config": {"workload": "config 2: full MoE layer decode, 1 token, hidden 2048, top-8 of 256 int4 experts "
                                "(intermediate 512, group 64) + 1 shared expert, fp16 router, all slots resident",
                    "stacked_layers": n_layers, "pool_bytes_total": n_layers * NE * stride,
+                   "pools": "layer 0's experts come from the seeded generator; layers 1.. hold byte copies of layer 0's pool at "
+                            "addresses of their own (routers, shared experts and activations are distinct per layer)",
                    "activation_variants": X_VARIANTS,
                    "expert_bytes_touched_by_a_pass_over_every_variant": len(distinct) * stride,
                    "meta_dtype": args.meta, "launches_per_layer": 3, "hip_graph": True},
-        "timing": {"regions": REGIONS, "steps_per_region": steps, "statistic": "median",
+        "timing": {"regions": REGIONS, "steps_per_region": steps, "statistic": "median", "method": timing_method,
                    "us_per_layer_min": round(min(region_ms) / steps * 1e3, 3),
-                   "us_per_layer_max": round(max(region_ms) / steps * 1e3, 3)},
+                   "us_per_layer_max": round(max(region_ms) / steps * 1e3, 3),
+                   **({"us_per_layer_by_hip_events_round_all_regions": round(whole_graph_us, 3)} if whole_graph_us else {})},
         "hbm_peak_frac_on_expert_bytes": round(value / HBM_PEAK_GBPS, 4),
         "expert_bytes_per_step": expert_bytes, "total_bytes_per_step": total_bytes,
         "kernel_us_per_layer": {k: round(v, 3) for k, v in parts.items()},
@@ -680,11 +832,18 @@ def decode_workload(args, rt, capi, S, meta):
                      "frac": round(launch2_bytes / (launch2_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                      "bytes_per_launch": launch2_bytes, "us_per_launch": round(launch2_us, 3),
                      "traffic": profile_figure("decode_phase1_q35b_int4_hbm_traffic.txt", "hbm_bytes_per_launch"),
-                     "standalone_operator": {"kernel": "k_phase1<4,1,4,false,0> (gate/up rows alone)", "bytes_per_launch": routed_gate_up,
+                     "standalone_operator": {"kernel": "k_phase1<4,1,2,false,0,true> (gate/up rows alone: no routing, two row pairs a wave)", "bytes_per_launch": routed_gate_up,
                                              "us_per_launch": round(alone_us, 3),
                                              "frac": round(routed_gate_up / (alone_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
-                     "floors_us": {"empty_launch": round(parts["floor: empty launch of phase 1's grid"], 3),
-                                   "read_only_same_bytes": round(parts["floor: read-only kernel over phase 1's routed bytes"], 3)}},
+                     "traffic_source": "profiles/decode_phase1_q35b_int4_hbm_traffic.txt (FETCH_SIZE + WRITE_SIZE of a profiled run "
+                                       "of this kernel, scaled by a copy's; not measured by this run)",
+                     "floors_us": {"empty_launch": round(empty_us, 3), "read_only_same_bytes": round(read_us, 3)},
+                     "design_floor_us": round(floor_us, 2),
+                     "design_floor": {"launches": 3, "empty_launch_us": round(empty_us, 3), "dependent_round_trips": 5,
+                                      "round_trip_us": round(hop_us, 3), "bytes": total_bytes,
+                                      "streamed_GBps": round(stream_gbps, 1),
+                                      "frac_of_peak_at_the_floor": round(expert_bytes / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                                      "measured_over_floor": round(ms_per_step * 1e3 / floor_us, 3)}},
         "setup_seconds": round(gen_s, 1),
     }
     if args.cpu_sample > 0:
@@ -702,6 +861,9 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=60, help="layer evaluations timed on the CPU (0 = skip)")
     ap.add_argument("--no-shared", action="store_true", help="diagnostic: leave the shared expert out of the layer")
     ap.add_argument("--no-secondary", action="store_true", help="the headline workload alone")
+    ap.add_argument("--timing", choices=["graph", "launches"], default="graph",
+                    help="decode: the timed regions in one captured graph with a time-stamp kernel between them (default), or a "
+                         "graph launch of up to 40 layers at a time with HIP event records between regions")
     ap.add_argument("--workload", choices=["decode", "prefill", "gptoss", "kimi"], default="decode",
                     help="decode: the headline metric (config 2) with the other workloads in its `secondary` block; "
                          "prefill: the ragged 512-token chunk (config 3) alone; gptoss: 4 tokens through 24 gpt-oss-shape "
@@ -713,6 +875,12 @@ def main():
     if args.gpus != 1:
         print("bench.py measures one GPU: this path is built and measured on a single MI355X "
               "(--gpus N with N > 1 is not supported)", file=sys.stderr)
+        sys.exit(2)
+
+    if profiler_attached() and args.steps > PROFILED_MAX_STEPS:
+        print(f"bench.py: a profiler is attached and --steps {args.steps} exceeds {PROFILED_MAX_STEPS}, the largest region that has "
+              "run clean under rocprofv3 (a profiled run at --steps 2000 once aborted inside hipGraphLaunch and its cause was "
+              "never shown); profile at --steps <= 400", file=sys.stderr)
         sys.exit(2)
 
     from shrike_amd import capi, runtime as rt
@@ -740,7 +908,8 @@ def main():
             r = run()
             secondary[name] = {k: r[k] for k in r if k in ("metric", "value", "unit", "ms_per_step", "us_per_layer", "config",
                                                            "kernel_us_per_chunk", "roofline", "GBps_on_pair_bytes",
-                                                           "hbm_peak_frac_on_expert_bytes", "miss_rate", "host_to_device_GBps",
+                                                           "hbm_peak_frac_on_expert_bytes", "miss_rate", "host_to_device_GBps", "hit_only_kernel_ms", "hit_only",
+                                                           "timeline_ms_per_step", "copy_ms_hidden_behind_compute", "miss_rate_by_policy", "miss_rate_floor",
                                                            "bytes_copied_per_step", "experts_requested_per_step", "steps", "dtype", "cpu_baseline")}
         out["secondary"] = secondary
     print(json.dumps(out))

@@ -50,6 +50,20 @@ __global__ __launch_bounds__(256) void k_probe_read(PoolArg pool, uint64_t strid
     if (acc == 0x9E3779B9u) sink[0] = wave;
 }
 
+// One wave walks a chain of dependent loads: word i of the table holds the index of the next word. What a launch of
+// `hops` hops costs beyond an empty launch, divided by hops, is one memory round trip as a kernel sees it.
+__global__ __launch_bounds__(64) void k_probe_chase(const uint32_t *table, uint32_t hops, uint32_t start, uint32_t *sink) {
+    uint32_t at = start;
+    asm volatile("" : "+v"(at));  // a vector register: the hops are vector loads, as the kernels' row loads are
+    for (uint32_t i = 0; i < hops; ++i) at = __builtin_nontemporal_load(table + at);
+    if (at == 0xffffffffu) sink[0] = at;  // never true for a table of indices; keeps the chain live
+}
+
+// The device's constant-rate clock into a slot: a time stamp that sits in stream (or graph) order between other kernels.
+__global__ void k_probe_timestamp(uint64_t *slot) {
+    if (threadIdx.x == 0) *slot = wall_clock64();
+}
+
 }  // namespace shrike
 
 using namespace shrike;
@@ -81,6 +95,30 @@ int shrike_probe_read(void *stream, const shrike_pool_bases *pool, uint64_t pool
                        cell_count, byte_offset, waves_per_cell, loads, d_sink);
     SHRIKE_HIP(hipGetLastError());
     return 0;
+}
+
+// d_table: `words` 32-bit indices below `words` (the caller fills them; a stride of many cache lines between
+// consecutive hops keeps every hop a miss). The chain starts at `start`.
+int shrike_probe_dependent_loads(void *stream, const uint32_t *d_table, uint32_t words, uint32_t hops, uint32_t start, uint32_t *d_sink) {
+    SHRIKE_REQUIRE(d_table != nullptr && d_sink != nullptr && words >= 1 && start < words, "probe: table, sink and a start inside the table");
+    SHRIKE_REQUIRE(hops >= 1 && hops <= 4096u, "probe: 1...4096 hops");
+    hipLaunchKernelGGL(k_probe_chase, dim3(1), dim3(64), 0, as_stream(stream), d_table, hops, start, d_sink);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+
+// One thread stores wall_clock64() to *d_slot behind whatever the stream holds. The clock's rate in kHz comes from
+// shrike_probe_wall_clock_khz (hipDeviceAttributeWallClockRate of the current device; 0 on failure).
+int shrike_probe_timestamp(void *stream, uint64_t *d_slot) {
+    SHRIKE_REQUIRE(d_slot != nullptr && reinterpret_cast<uintptr_t>(d_slot) % 8u == 0, "probe: the slot must be bound and 8-byte aligned");
+    hipLaunchKernelGGL(k_probe_timestamp, dim3(1), dim3(64), 0, as_stream(stream), d_slot);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+int shrike_probe_wall_clock_khz(void) {
+    int device = 0, khz = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) != hipSuccess) return 0;
+    return khz;
 }
 
 }  // extern "C"

@@ -1,5 +1,5 @@
-"""ctypes face of libshrikeprobe.so: the benchmark's two measurement aids (an empty launch, and a kernel that
-only reads a byte range of listed pool cells). Not part of the product's ABI: nothing in libshrikehip or in the
+"""ctypes face of libshrikeprobe.so: the benchmark's measurement aids (an empty launch, a kernel that only reads
+a byte range of listed pool cells, a chain of dependent loads). Not part of the product's ABI: nothing in libshrikehip or in the
 operator mirror depends on it."""
 from __future__ import annotations
 
@@ -25,6 +25,12 @@ def load() -> C.CDLL:
         _lib.shrike_probe_read.restype = C.c_int
         _lib.shrike_probe_read.argtypes = [C.c_void_p, C.POINTER(PoolBases), C.c_uint64, C.c_void_p, C.c_uint32,
                                            C.c_uint64, C.c_uint64, C.c_void_p]
+        _lib.shrike_probe_dependent_loads.restype = C.c_int
+        _lib.shrike_probe_dependent_loads.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]
+        _lib.shrike_probe_timestamp.restype = C.c_int
+        _lib.shrike_probe_timestamp.argtypes = [C.c_void_p, C.c_void_p]
+        _lib.shrike_probe_wall_clock_khz.restype = C.c_int
+        _lib.shrike_probe_wall_clock_khz.argtypes = []
     return _lib
 
 

@@ -53,6 +53,7 @@ class BatchedDecodeLayer:
         self.pass_table = empty(8 * ne)
         self.passes = 0
         self.plan_log = []  # every batch of experts handed to the cache, in order
+        self.trace = None   # a list: run() then appends (stream name, start event, stop event) around what it enqueues
 
     def run(self, router, hidden, t: int, stride: int):
         """router: dict(weights, scales, biases, eff_scale, expert_scale, bias) of device buffers.
@@ -60,8 +61,19 @@ class BatchedDecodeLayer:
         m, pf = self.moe, self.pf
         d, ne, k = m.desc.d, m.desc.num_experts, m.desc.top_k
         compute = m.stream
-        pf.encode_block(router["weights"], router.get("scales"), router.get("biases"), hidden, router["eff_scale"],
-                        router["expert_scale"], router["bias"], self.idx, self.w, self.router_ws, t, ne, d, k, stride)
+
+        def span(name, stream, body):
+            if self.trace is None:
+                return body()
+            start, stop = Event(), Event()
+            start.record(stream)
+            out = body()
+            stop.record(stream)
+            self.trace.append((name, start, stop))
+            return out
+        span("compute", compute, lambda: pf.encode_block(
+            router["weights"], router.get("scales"), router.get("biases"), hidden, router["eff_scale"],
+            router["expert_scale"], router["bias"], self.idx, self.w, self.router_ws, t, ne, d, k, stride))
         (compute.synchronize() if compute else synchronize())
         ids = self.idx.download(np.uint32, t * k)  # the router's host readback
         # experts the pool already holds go first (PrefillSweepOrder.residentFirstBalanced), so a
@@ -83,7 +95,8 @@ class BatchedDecodeLayer:
             self.plan_log.append(list(batch))
             if self.passes:
                 self.upload_stream.wait_event(served)  # the cells about to be overwritten were still being read
-            self.pool.execute_plan(self.cache, plan, self.store, self.store_stride, self.expert_bytes, self.upload_stream)
+            span("upload", self.upload_stream, lambda: self.pool.execute_plan(
+                self.cache, plan, self.store, self.store_stride, self.expert_bytes, self.upload_stream))
             # this pass's residency view: only its experts count as resident for the grouping
             table = np.full(ne, (capi.EMPTY << 32) | SENTINEL, np.uint64)
             for e in batch:
@@ -93,13 +106,15 @@ class BatchedDecodeLayer:
             uploaded.record(self.upload_stream)
             if compute:
                 compute.wait_event(uploaded)
-            pf.group_pairs(self.idx, self.w, t, k, ne, self.routes, residency=self.pass_table)
-            pf.encode_grouped_expert_gemms(self.pool, self.off, self.routes, hidden, stride, self.partials, self.ffn_ws, t, k)
+            def pass_kernels():
+                pf.group_pairs(self.idx, self.w, t, k, ne, self.routes, residency=self.pass_table)
+                pf.encode_grouped_expert_gemms(self.pool, self.off, self.routes, hidden, stride, self.partials, self.ffn_ws, t, k)
+            span("compute", compute, pass_kernels)
             served.record(compute)
             (compute.synchronize() if compute else synchronize())
             todo = todo[len(batch):]
             self.passes += 1
-        pf.encode_reduce_token_major(self.partials, self.w, self.h2, t, k, d)
+        span("compute", compute, lambda: pf.encode_reduce_token_major(self.partials, self.w, self.h2, t, k, d))
         return self.h2
 
 
