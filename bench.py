@@ -468,10 +468,23 @@ def gptoss_workload(args, rt, capi, S, meta, bits):
     work = rt.empty(pf.ffn_workspace_bytes(t, routes.max_row_tiles))
 
     resolved, acts, y = rt.empty(4 * t * k), rt.empty(2 * t * k * f), rt.empty(2 * t * d)
-    grouped = os.environ.get("SHRIKE_BENCH_GROUPED") == "1"  # diagnostic: the prefill operators instead of the decode ones
+    # diagnostics: the prefill operators instead of the decode ones; the decode operators one by one (router, resolve,
+    # phase 1, phase 2: four launches) instead of the fused layer for a batch (three)
+    grouped = os.environ.get("SHRIKE_BENCH_GROUPED") == "1"
+    split = os.environ.get("SHRIKE_BENCH_SPLIT") == "1"
+    layer_args = []
+    for l in range(n_layers):
+        a = capi.DecodeLayerArgs()
+        a.router_weights, a.effective_scale, a.per_expert_scale, a.logit_bias = routers[l].ptr, ones_d.ptr, ones_e.ptr, zeros_e.ptr
+        a.pool, a.pool_slot_stride, a.residency, a.offsets = pools[l].bases, pools[l].stride, pools[l].table, off
+        a.x, a.y, a.out_indices, a.out_weights, a.resolved_slots, a.acts = hidden.ptr, y.ptr, idx.ptr, w.ptr, resolved.ptr, acts.ptr
+        layer_args.append(a)
 
     def all_layers():
         for l in range(n_layers):
+            if not grouped and not split:
+                moe.encode_decode_layer_batch(layer_args[l], t, d)
+                continue
             pf.encode_block(routers[l], None, None, hidden, ones_d, ones_e, zeros_e, idx, w, rws, t, ne, d, k, d)
             if grouped:
                 pf.group_pairs(idx, w, t, k, ne, routes, residency=pools[l].table)
@@ -502,7 +515,9 @@ def gptoss_workload(args, rt, capi, S, meta, bits):
         "ms_per_step": round(ms, 5), "us_per_layer": round(ms * 1e3 / n_layers, 2), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16 x u%d -> f32" % bits, "data": "synthetic (seeded SplitMix64)",
         "config": {"workload": f"config 4: {t} tokens, top-{k} of {ne} int{bits} experts, hidden {d}, intermediate {f}, {n_layers} stacked layers "
-                               "in one HIP graph, all slots resident", "operators": "grouped (prefill)" if grouped else "batched decode",
+                               "in one HIP graph, all slots resident",
+                   "operators": "grouped (prefill)" if grouped else "batched decode, four operators a layer" if split else
+                                "the fused layer for a batch (three launches a layer)",
                    "distinct_experts_per_layer": distinct, "expert_bytes_per_stack": expert_bytes,
                    "pair_bytes_per_stack": n_layers * t * k * stride, "meta_dtype": args.meta},
         "GBps_on_pair_bytes": round(n_layers * t * k * stride / (ms * 1e-3) / 1e9, 2),

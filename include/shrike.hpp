@@ -426,6 +426,10 @@ public:
         check(shrike_hip_shared_expert(h_, s, &gate, &up, &down, bits, x, scratch, h1, scalarGate, d, fShared));
     }
     void encodeDecodeLayer(Stream s, const shrike_decode_layer_args &args) { check(shrike_hip_moe_decode_layer(h_, s, &args)); }
+    // the same for several sequences, one token each (rows of x xStrideElements apart)
+    void encodeDecodeLayerBatch(Stream s, const shrike_decode_layer_args &args, uint32_t tokens, uint32_t xStrideElements) {
+        check(shrike_hip_moe_decode_layer_batch(h_, s, &args, tokens, xStrideElements));
+    }
 
 private:
     shrike_hip_moe *h_;

@@ -340,6 +340,15 @@ int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream,
  * handle and args, and no other layer call on the handle between them (the route entries live in it). */
 int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream,
                                          const shrike_decode_layer_args *args, uint32_t launches);
+/* The same three launches for several sequences that decode one token each (1...16): the runner's layer
+ * (RealForwardRunner.swift:2834-2901, :5520-5560) once per sequence, with the token on the grid instead of one call a
+ * sequence, so that a batch costs three launches and an expert two sequences route to is found in the caches by the
+ * second. Token t reads x + t * x_stride_elements and writes row t of y and hidden (d apart), of out_indices,
+ * out_weights and resolved_slots (top_k apart) and of acts (top_k * f apart); per token the bytes are those of
+ * shrike_hip_moe_decode_layer. The shared expert and the fused norm must not be bound (they take one token: run
+ * shrike_hip_prefill_shared_expert beside this call); the hit and miss lists are not written and may be NULL. */
+int shrike_hip_moe_decode_layer_batch(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *args,
+                                      uint32_t tokens, uint32_t x_stride_elements);
 
 /* The decode layer for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc). NO COUNTERPART IN THE REFERENCE. Same kernels and same

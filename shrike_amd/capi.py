@@ -196,6 +196,7 @@ IO_WORK = C.CFUNCTYPE(None, C.c_void_p)
 
 SIGNATURES = {
     "shrike_hip_last_error": (C.c_char_p, []),
+    "shrike_hip_moe_decode_layer_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(DecodeLayerArgs), C.c_uint32, C.c_uint32]),
     "shrike_int4_affine_gemv": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]),
     "shrike_cpu_expert_ffn_scratch_floats": (C.c_size_t, [C.c_uint32, C.c_uint32]),
     "shrike_cpu_expert_ffn_accumulate": (C.c_int, [C.c_void_p, C.POINTER(ExpertOffsets), C.c_void_p, C.c_uint32, C.c_uint32,

@@ -75,7 +75,10 @@ constexpr uint32_t kRouterLaunchTokens = 16;  // up to here the one-launch route
 int launch_router_tokens(const RouterArgs &a, uint32_t router_bits, uint32_t tokens, hipStream_t s);
 // router logit rows + the shared expert's gate/up rows in one grid
 // norm: null, or the norm to run in every workgroup's prologue (r.hidden and g.x are then not read)
-int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, const NormArgs *norm, hipStream_t s);
+// tokens > 1 (router rows only): grid.y walks tokens, token t reading r.hidden + t * r.token_stride and writing the t-th
+// logit row and route table (SHRIKE_MAX_ROUTER_EXPERTS entries apart)
+int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, const NormArgs *norm, hipStream_t s,
+                uint32_t tokens = 1);
 uint32_t phase1_blocks(uint32_t top_k, uint32_t f);
 // shared_down_bits: 0 = none, else the shared down rows ride in the same grid (one chunk
 // column per lane only: nch_for(shared_f, bits) == 1)

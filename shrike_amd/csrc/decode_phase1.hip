@@ -25,11 +25,18 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     typedef Chunk<BITS> C;
     if (ROUTE && blockIdx.x == a.lists_block) {
         // the workgroup behind all others: one wave selects once more and writes what the host and phase 2 read
-        // (indices, weights, hit and miss lists, resolved cells); nobody in this launch waits for it
+        // (indices, weights, hit and miss lists, resolved cells); nobody in this launch waits for it. With a batch of
+        // tokens (grid.y) each token has one, writing its own top_k indices, weights and cells.
         if (threadIdx.x < 64u) {
-            const TableSelect t = select_from_table(a.route_table, a.sel.num_experts, a.sel.top_k, threadIdx.x, a.sel.top_k);
+            const size_t t_ = blockIdx.y;
+            const TableSelect t = select_from_table(a.route_table + t_ * SHRIKE_MAX_ROUTER_EXPERTS, a.sel.num_experts, a.sel.top_k,
+                                                    threadIdx.x, a.sel.top_k);
+            RouteLists lists = a.lists;
+            lists.out_indices = a.lists.out_indices + t_ * a.top_k;
+            lists.out_weights = a.lists.out_weights + t_ * a.top_k;
+            lists.resolved_slots = a.lists.resolved_slots + t_ * a.top_k;
             uint32_t my_cell;
-            finish_routes(a.sel, a.lists, threadIdx.x, true, t.mine, t.my_key, t.my_raw, bf16_to_f32(uint16_t(t.my_gain)),
+            finish_routes(a.sel, lists, threadIdx.x, true, t.mine, t.my_key, t.my_raw, bf16_to_f32(uint16_t(t.my_gain)),
                           t.my_cell, my_cell);
         }
         return;
@@ -42,7 +49,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     if (!io_ready(a.io_status)) return;
     // a batch of tokens: grid.y is this workgroup's token (the argument block itself stays untouched:
     // writing to it would move it to private memory)
-    const size_t tok = ROUTE ? 0u : blockIdx.y;
+    const size_t tok = blockIdx.y;
     const uint16_t *x_tok = a.x + tok * a.x_stride;
     const uint32_t *resolved_tok = a.resolved + tok * a.top_k;
     uint16_t *acts_tok = a.acts + tok * a.top_k * a.f;
@@ -64,7 +71,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
         // every wave selects for itself, in registers, from the table the previous launch left: no barrier, and the
         // table's loads go out ahead of the activation slice's (loads return in order)
         // (a wave stops at the round that names its own position's expert)
-        const TableSelect t = select_from_table(a.route_table, a.sel.num_experts, a.sel.top_k, lane, k);
+        const TableSelect t = select_from_table(a.route_table + tok * SHRIKE_MAX_ROUTER_EXPERTS, a.sel.num_experts, a.sel.top_k, lane, k);
         load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
         if (in_range) cell = uint32_t(__builtin_amdgcn_readlane(int(t.my_cell), int(k)));
     } else {
@@ -121,12 +128,13 @@ static uint32_t phase1_blocks_of(uint32_t positions, uint32_t f, uint32_t row_pa
 uint32_t phase1_blocks(uint32_t top_k, uint32_t f) { return phase1_blocks_of(top_k, f, kPhase1RowPairs); }
 
 static bool phase1_narrow(bool routing, bool one_token, uint32_t d, uint32_t bits) {
-    return !routing && (one_token || nch_for(d, bits) >= 3);
+    return one_token ? !routing : nch_for(d, bits) >= 3;
 }
 
 template <int BITS, bool ROUTE, int SBITS, bool STREAM>
 static void launch_phase1_nch(const Phase1Args &a, dim3 grid, hipStream_t s) {
-    constexpr int RP = kPhase1RowPairs, RN = ROUTE ? kPhase1RowPairs : kPhase1RowPairsNarrow;
+    // (the one-token routing launch keeps four pairs; a batch takes the narrow form for long rows whether it routes or not)
+    constexpr int RP = kPhase1RowPairs, RN = (ROUTE && STREAM) ? kPhase1RowPairs : kPhase1RowPairsNarrow;
     const dim3 block(256);
     switch (nch_for(a.d, BITS)) {
         case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
@@ -139,6 +147,7 @@ static void launch_phase1_nch(const Phase1Args &a, dim3 grid, hipStream_t s) {
 int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t shared_down_bits, hipStream_t s) {
     SHRIKE_REQUIRE(a.f % kPhase1RowPairs == 0, "phase1: f=%u must be a multiple of %d", a.f, kPhase1RowPairs);
     uint32_t extra = 0;
+    SHRIKE_REQUIRE(a.tokens <= 1u || shared_down_bits == 0, "phase1: the shared down rows ride along with one token only");
     if (shared_down_bits) {
         SHRIKE_REQUIRE(routing && nch_for(a.shared_down.n, shared_down_bits) == 1,
                        "phase1: the shared down rows ride along only in the routed launch and with one chunk column per lane");
@@ -152,12 +161,12 @@ int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t sha
     const dim3 grid(b.routed_blocks + extra + (routing ? 1u : 0u), a.tokens ? a.tokens : 1u);
     if (bits == 4) {
         if (!routing) { if (one_token) launch_phase1_nch<4, false, 0, true>(b, grid, s); else launch_phase1_nch<4, false, 0, false>(b, grid, s); }
-        else if (shared_down_bits == 0) launch_phase1_nch<4, true, 0, true>(b, grid, s);
+        else if (shared_down_bits == 0) { if (one_token) launch_phase1_nch<4, true, 0, true>(b, grid, s); else launch_phase1_nch<4, true, 0, false>(b, grid, s); }
         else if (shared_down_bits == 4) launch_phase1_nch<4, true, 4, true>(b, grid, s);
         else launch_phase1_nch<4, true, 8, true>(b, grid, s);
     } else {
         if (!routing) { if (one_token) launch_phase1_nch<8, false, 0, true>(b, grid, s); else launch_phase1_nch<8, false, 0, false>(b, grid, s); }
-        else if (shared_down_bits == 0) launch_phase1_nch<8, true, 0, true>(b, grid, s);
+        else if (shared_down_bits == 0) { if (one_token) launch_phase1_nch<8, true, 0, true>(b, grid, s); else launch_phase1_nch<8, true, 0, false>(b, grid, s); }
         else if (shared_down_bits == 4) launch_phase1_nch<8, true, 4, true>(b, grid, s);
         else launch_phase1_nch<8, true, 8, true>(b, grid, s);
     }

@@ -379,13 +379,36 @@ int shrike_hip_shared_expert(shrike_hip_moe *moe, void *stream, const shrike_pro
 // Three launches: (1) router logit rows + shared gate/up rows; (2) select + classify in the
 // prologue of every phase-1 workgroup, the routed gate/up rows, and the shared down rows;
 // (3) phase 2 with the shared expert's output as the residual.
+static int decode_layer(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *g, uint32_t launches, uint32_t tokens,
+                        uint32_t x_stride);
+
 int shrike_hip_moe_decode_layer(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *g) {
-    return shrike_hip_moe_decode_layer_launches(moe, stream, g, 7u);
+    return decode_layer(moe, stream, g, 7u, 1u, 0u);
 }
 
 int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *g,
                                          uint32_t launches) {
+    return decode_layer(moe, stream, g, launches, 1u, 0u);
+}
+
+// The same three launches for a batch of sequences, one token each: grid.y walks the tokens in every launch. Token t
+// reads x + t * x_stride, selects from its own logit row and route table, and writes row t of y, hidden, out_indices,
+// out_weights, resolved_slots and acts. No shared expert and no fused norm (those take one token); hit and miss lists are
+// not written.
+int shrike_hip_moe_decode_layer_batch(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *g, uint32_t tokens,
+                                      uint32_t x_stride_elements) {
     SHRIKE_REQUIRE(moe != nullptr && g != nullptr, "moe handle or args is NULL");
+    SHRIKE_REQUIRE(tokens >= 1 && tokens <= kLayerBatchTokens, "decodeLayerBatch: %u tokens not in 1...%u", tokens, kLayerBatchTokens);
+    SHRIKE_REQUIRE(x_stride_elements >= moe->desc.d && x_stride_elements % 8u == 0, "decodeLayerBatch: x stride is too small or leaves rows unaligned");
+    SHRIKE_REQUIRE(g->shared_gate.weights == nullptr && g->norm_weight == nullptr,
+                   "decodeLayerBatch: the shared expert and the fused norm take one token; run them as operators of their own");
+    return decode_layer(moe, stream, g, 7u, tokens, x_stride_elements);
+}
+
+static int decode_layer(shrike_hip_moe *moe, void *stream, const shrike_decode_layer_args *g, uint32_t launches, uint32_t tokens,
+                        uint32_t x_stride) {
+    SHRIKE_REQUIRE(moe != nullptr && g != nullptr, "moe handle or args is NULL");
+    const bool batch = tokens > 1u || x_stride != 0u;
     SHRIKE_REQUIRE(launches != 0 && launches <= 7u, "decodeLayer: launches=%u is not a mask of the three launches", launches);
     const shrike_moe_desc &m = moe->desc;
     if (int rc = check_router(moe, m.num_experts, m.d, m.top_k)) return rc;
@@ -394,9 +417,10 @@ int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream, cons
                    "decodeLayer: router operands must be bound");
     SHRIKE_REQUIRE(m.router_weight_bits == 0 || (g->router_scales && g->router_biases),
                    "decodeLayer: affine router needs scales and biases");
-    SHRIKE_REQUIRE(g->pool && g->residency && g->x && g->y && g->out_indices && g->out_weights && g->resolved_slots
-                   && g->hit_count && g->hit_positions && g->miss_count && g->miss_positions && g->miss_experts
-                   && g->acts, "decodeLayer: pool, residency, x, y and the scratch buffers must be bound");
+    SHRIKE_REQUIRE(g->pool && g->residency && g->x && g->y && g->out_indices && g->out_weights && g->resolved_slots && g->acts,
+                   "decodeLayer: pool, residency, x, y and the scratch buffers must be bound");
+    SHRIKE_REQUIRE(batch || (g->hit_count && g->hit_positions && g->miss_count && g->miss_positions && g->miss_experts),
+                   "decodeLayer: pool, residency, x, y and the scratch buffers must be bound");
     SHRIKE_REQUIRE(g->pool_slot_stride % 16u == 0, "decodeLayer: pool slot stride must be a multiple of 16");
     const bool normed = g->norm_weight != nullptr;
     NormArgs norm = {};
@@ -435,6 +459,7 @@ int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream, cons
     // launch 1 writes the logits and, beside each, the expert's route entry; no list yet
     r.lists.residency = g->residency;
     r.route_table = moe->d_route;
+    r.token_stride = x_stride;
 
     Phase1Args p1 = {};
     fill_pool(p1.pool, g->pool);
@@ -444,9 +469,13 @@ int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream, cons
     p1.ebias = m.expert_additive_biases;
     p1.sel = r.sel;
     p1.lists.out_indices = g->out_indices; p1.lists.out_weights = static_cast<uint16_t *>(g->out_weights);
-    p1.lists.residency = g->residency; p1.lists.hit_count = g->hit_count; p1.lists.hit_positions = g->hit_positions;
-    p1.lists.miss_count = g->miss_count; p1.lists.miss_positions = g->miss_positions;
-    p1.lists.miss_experts = g->miss_experts; p1.lists.resolved_slots = g->resolved_slots;
+    p1.lists.residency = g->residency; p1.lists.resolved_slots = g->resolved_slots;
+    if (!batch) {  // a batch writes the cells alone
+        p1.lists.hit_count = g->hit_count; p1.lists.hit_positions = g->hit_positions;
+        p1.lists.miss_count = g->miss_count; p1.lists.miss_positions = g->miss_positions;
+        p1.lists.miss_experts = g->miss_experts;
+    }
+    p1.tokens = tokens; p1.x_stride = x_stride;
     p1.route_table = moe->d_route;
     p1.routed_blocks = phase1_blocks(m.top_k, m.f);
 
@@ -465,7 +494,7 @@ int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream, cons
         GemvArgs none = {};
         none.n = m.d;
         if (launches & 1u)
-            if (int rc = launch_head(r, m.router_weight_bits, none, sbits, normed ? &norm : nullptr, s)) return rc;
+            if (int rc = launch_head(r, m.router_weight_bits, none, sbits, normed ? &norm : nullptr, s, tokens)) return rc;
     }
     if (launches & 2u) {
         if (int rc = launch_phase1(p1, m.routed_weight_bits, true, down_fused ? sbits : 0u, s)) return rc;
@@ -483,6 +512,7 @@ int shrike_hip_moe_decode_layer_launches(shrike_hip_moe *moe, void *stream, cons
     p.y = static_cast<uint16_t *>(g->y); p.hidden = static_cast<uint16_t *>(g->hidden);
     p.d = m.d; p.f = m.f; p.top_k = m.top_k; p.meta = m.meta_dtype; p.ebias = m.expert_additive_biases;
     p.delta = normed ? norm.delta : nullptr;
+    p.tokens = tokens;
     return launch_phase2(p, m.routed_weight_bits, s);
 }
 

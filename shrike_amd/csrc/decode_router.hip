@@ -79,14 +79,18 @@ __global__ __launch_bounds__(256) void k_head(RouterArgs r, GemvArgs g, uint32_t
     };
     if (blockIdx.x < router_blocks) {
         const uint32_t e = blockIdx.x * 4u + wave_index();
+        // a batch of tokens (no norm, no shared rows): grid.y is the token, with an activation row, a logit row and a
+        // route table of its own
+        const size_t tok = NORM ? 0u : blockIdx.y;
         if (e < r.sel.num_experts) {
             // what the expert's route entry needs beside the logit: fetched beside the row, used behind it
             const uint16_t bias_bits = r.sel.logit_bias[e], gain_bits = r.sel.per_expert_scale[e];
             const uint64_t word = r.lists.residency ? r.lists.residency[e] : 0;
             float logit;
             if (NORM) logit = router_row<RK>(r, [&] { return reinterpret_cast<const uint16_t *>(normed_row()); }, r.logits_out, e, threadIdx.x & 63u, false);
-            else logit = router_row<RK>(r, e, threadIdx.x & 63u);
-            if (r.route_table && (threadIdx.x & 63u) == 0) write_route_entry(r.route_table, e, logit, bias_bits, gain_bits, word, r.sel.sigmoid);
+            else logit = router_row<RK>(r, r.hidden + tok * r.token_stride, r.logits_out + tok * SHRIKE_MAX_ROUTER_EXPERTS, e, threadIdx.x & 63u, false);
+            if (r.route_table && (threadIdx.x & 63u) == 0)
+                write_route_entry(r.route_table + tok * SHRIKE_MAX_ROUTER_EXPERTS, e, logit, bias_bits, gain_bits, word, r.sel.sigmoid);
         } else if (NORM) {
             normed_row();  // the workgroup's barriers need every wave
         }
@@ -212,10 +216,11 @@ static void launch_head_nch(const RouterArgs &r, const GemvArgs &g, uint32_t rou
 
 // g.rows + g.rows_b == 0: router rows only (g.n must still be a valid row length)
 int launch_head(const RouterArgs &r, uint32_t router_bits, const GemvArgs &g, uint32_t shared_bits, const NormArgs *norm,
-                hipStream_t s) {
+                hipStream_t s, uint32_t tokens) {
     const uint32_t router_blocks = (r.sel.num_experts + 3) / 4;
     const uint32_t shared_rows = g.rows + g.rows_b;
-    const dim3 grid(router_blocks + (shared_rows ? gemv_blocks(shared_rows, g.n, shared_bits) : 0u));
+    SHRIKE_REQUIRE(tokens >= 1 && (tokens == 1 || (shared_rows == 0 && norm == nullptr)), "head launch: a batch of tokens takes router rows only");
+    const dim3 grid(router_blocks + (shared_rows ? gemv_blocks(shared_rows, g.n, shared_bits) : 0u), tokens);
     if (shared_bits == 4) {
         if (router_bits == 0) launch_head_nch<0, 4>(r, g, router_blocks, grid, norm, s);
         else if (router_bits == 8) launch_head_nch<8, 4>(r, g, router_blocks, grid, norm, s);

@@ -489,6 +489,10 @@ __device__ __forceinline__ void finish_routes(const SelectArgs &a, const RouteLi
     const bool hit = on && cell_of_mine != kSentinel;
     if (hit) my_cell = cell_of_mine;
     if (!write_lists) return;
+    if (out.hit_count == nullptr) {  // a batch of tokens: the cells alone, no hit and miss lists
+        if (on) out.resolved_slots[lane] = hit ? cell_of_mine : kSentinel;
+        return;
+    }
     const uint64_t hit_mask = __ballot(hit), miss_mask = __ballot(on && !hit);
     const uint64_t below = (uint64_t(1) << lane) - 1u;
     if (hit) {

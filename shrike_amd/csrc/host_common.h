@@ -43,14 +43,16 @@ namespace shrike { struct RouteEntry; }
 
 // MoE.swift:41-216: the handle keeps the shape it was made for, the router's fp32
 // logits (routerLogits, MoE.swift:74) and the router's arrival counter.
+constexpr unsigned kLayerBatchTokens = 16;  // tokens the fused layer takes in one call (a logit row and a route table each)
 constexpr unsigned kCounterWords = 256;
 constexpr unsigned kRouterTokenCounters = 128;  // first of the per-token arrival counters
 
 struct shrike_hip_moe {
     shrike_moe_desc desc;
     int device;
-    float *d_logits;        // fp32[2][SHRIKE_MAX_ROUTER_EXPERTS]: this layer's logits, then the paired router's
-    shrike::RouteEntry *d_route;  // [SHRIKE_MAX_ROUTER_EXPERTS]: the fused layer's route table, in d_logits' allocation
+    float *d_logits;        // fp32[kLayerBatchTokens][SHRIKE_MAX_ROUTER_EXPERTS]: this layer's logits (one row a token of a batch), the
+                            // paired router's in the second row
+    shrike::RouteEntry *d_route;  // [kLayerBatchTokens][SHRIKE_MAX_ROUTER_EXPERTS]: the fused layer's route tables, in d_logits' allocation
     uint32_t *d_counter;    // u32[kCounterWords], zero between launches: [0] the router's arrivals ([1] the paired router's), from
                             // [kRouterTokenCounters] one word a token of the several-token router
 };

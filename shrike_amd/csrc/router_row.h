@@ -14,12 +14,14 @@ namespace shrike {
 // x_source(): called once the row's own loads are in flight; returns the activation row to read (it may
 // first have to produce it, e.g. a norm into LDS behind a barrier — then every wave of the workgroup
 // must come through here or call it by itself). Returns the logit (in every lane).
-template <int RK, class XSource>
-__device__ __forceinline__ float router_row(const RouterArgs &a, XSource &&x_source, float *logits, uint32_t e, uint32_t lane,
-                                            bool publish) {
+// MAXI: 16-byte chunks a lane takes at most (chunks lane + 64 i, i < MAXI, past the row's end skipped); a row of up
+// to 64 MAXI chunks gives the same sums under any larger MAXI, so a short row can run the narrower instance and
+// leave out the loads of chunks it does not have.
+template <int RK, int MAXI, class XSource>
+__device__ __forceinline__ float router_row_n(const RouterArgs &a, XSource &&x_source, float *logits, uint32_t e, uint32_t lane,
+                                              bool publish) {
     constexpr int E = RK == 0 ? 8 : RK == 8 ? 16 : 32;  // elements per 16-byte weight chunk
     constexpr int PIECES = E / 8;
-    constexpr int MAXI = RK == 0 ? 8 : 4;
     const uint32_t chunks = a.d / E;
     const uint32_t groups = a.d / kGroup;
     const uint32_t row_bytes = chunks * 16u;
@@ -92,6 +94,14 @@ __device__ __forceinline__ float router_row(const RouterArgs &a, XSource &&x_sou
         else logits[e] = acc;
     }
     return acc;  // every lane holds the sum
+}
+
+template <int RK, class XSource>
+__device__ __forceinline__ float router_row(const RouterArgs &a, XSource &&x_source, float *logits, uint32_t e, uint32_t lane,
+                                            bool publish) {
+    // fp16 rows: eight chunks a lane reach the activation ceiling (4,096); four cover hidden sizes up to 2,048
+    if (RK == 0 && a.d <= 2048u) return router_row_n<RK, 4>(a, x_source, logits, e, lane, publish);
+    return router_row_n<RK, RK == 0 ? 8 : 4>(a, x_source, logits, e, lane, publish);
 }
 
 template <int RK>

@@ -472,8 +472,10 @@ uint64_t shrike_hip_pool_table_entry(const shrike_hip_pool *pool, uint32_t exper
 
 // --------------------------------------------------------------------- moe
 
-constexpr size_t kLogitsBytes = sizeof(float) * 2u * SHRIKE_MAX_ROUTER_EXPERTS;  // this layer's logits and the paired router's
-constexpr size_t kRouteBytes = 16u * SHRIKE_MAX_ROUTER_EXPERTS;                   // the fused layer's route table
+// this layer's logits and the paired router's; the fused layer for a batch of tokens keeps a logit row and a route
+// table per token
+constexpr size_t kLogitsBytes = sizeof(float) * kLayerBatchTokens * SHRIKE_MAX_ROUTER_EXPERTS;
+constexpr size_t kRouteBytes = 16u * kLayerBatchTokens * SHRIKE_MAX_ROUTER_EXPERTS;
 
 shrike_hip_moe *shrike_hip_moe_create(const shrike_moe_desc *desc, int *out_errno) {
     auto fail = [&](int code) -> shrike_hip_moe * { if (out_errno) *out_errno = code; return nullptr; };

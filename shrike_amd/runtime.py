@@ -392,6 +392,11 @@ class MoE:
         check(capi.load().shrike_hip_moe_decode_layer(self.handle, self._s(), C.byref(args)),
               "shrike_hip_moe_decode_layer")
 
+    def encode_decode_layer_batch(self, args: DecodeLayerArgs, tokens: int, x_stride: int):
+        """The fused layer for `tokens` sequences, one token each (shrike_hip_moe_decode_layer_batch)."""
+        check(capi.load().shrike_hip_moe_decode_layer_batch(self.handle, self._s(), C.byref(args), tokens, x_stride),
+              "shrike_hip_moe_decode_layer_batch")
+
     def encode_decode_layer_launches(self, args: DecodeLayerArgs, launches: int):
         """A subset of the layer's three launches (bit 0 head, bit 1 phase 1, bit 2 phase 2)."""
         check(capi.load().shrike_hip_moe_decode_layer_launches(self.handle, self._s(), C.byref(args), launches),

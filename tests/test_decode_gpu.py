@@ -627,6 +627,55 @@ def test_batched_decode_operators_equal_the_single_token_ones(gpu, d, f, ne, k, 
     assert_ffn_close(all_y[:d], ref_y, "token 0 y from the device's activations")
 
 
+@pytest.mark.parametrize("d,f,ne,k,t,bits,router_bits", [(2880, 2880, 32, 4, 4, 4, 0), (2880, 2880, 32, 4, 4, 8, 0), (512, 256, 40, 8, 16, 4, 8),
+                                                          (2304, 1024, 256, 8, 5, 8, 0), (256, 128, 8, 3, 1, 4, 4)])
+def test_decode_layer_for_a_batch_equals_the_layer_token_by_token(gpu, d, f, ne, k, t, bits, router_bits):
+    """shrike_hip_moe_decode_layer_batch: the three launches with the token on the grid give, for every token, the
+    routes, cells, y and hidden bytes of shrike_hip_moe_decode_layer on that token alone (which the tests above hold
+    to the oracle); routes also against the oracle bit for bit. Some experts are missing from the pool."""
+    L = Layer(0x5EED0044 + bits, d, f, ne, k, bits=bits, router_bits=router_bits)
+    L.logit_bias = S.f32_to_bf16_bits(L.tree.key("bias").normal(ne, std=0.01))
+    resident = [e for e in range(ne) if e % 7 != 2]
+    dl = DeviceLayer(gpu, L, resident=resident)
+    stride = d + 24
+    x = S.activations_f16(L.tree, "batch.x", t * stride)
+    hidden0 = S.activations_f16(L.tree, "batch.hidden", t * d)
+    a = dl.layer_args()
+    dx, dhid, dy = gpu.dev(x), gpu.dev(hidden0), gpu.dev(np.full(t * d, 0xD4D0, np.uint16))
+    idx, w, res = gpu.empty(4 * t * k).fill(0xA5), gpu.empty(2 * t * k).fill(0xA5), gpu.empty(4 * t * k).fill(0xA5)
+    acts = gpu.empty(2 * t * k * f)
+    a.x, a.hidden, a.y, a.out_indices, a.out_weights, a.resolved_slots, a.acts = dx.ptr, dhid.ptr, dy.ptr, idx.ptr, w.ptr, res.ptr, acts.ptr
+    for name in ("hit_count", "hit_positions", "miss_count", "miss_positions", "miss_experts"):
+        setattr(a, name, None)  # a batch writes no lists
+    dl.moe.encode_decode_layer_batch(a, t, stride)
+    gpu.synchronize()
+    h_idx, h_w, h_res = idx.download(np.uint32, t * k), w.download(np.uint16, t * k), res.download(np.uint32, t * k)
+    ref_idx, ref_w, _ = O.prefill_router(L.router_dict(), x, t, d, k, stride=stride)
+    assert np.array_equal(h_idx, ref_idx)
+    assert h_res.tolist() == [dl.cell_of.get(int(e), SENT) for e in h_idx]
+    assert SENT in h_res.tolist() or t * k < 8
+    all_y, all_hid = dy.download(np.uint16, t * d), dhid.download(np.uint16, t * d)
+    for tok in range(t):
+        b = dl.layer_args()
+        one_x, one_hid = gpu.dev(np.ascontiguousarray(x[tok * stride:tok * stride + d])), gpu.dev(hidden0[tok * d:(tok + 1) * d].copy())
+        b.x, b.hidden = one_x.ptr, one_hid.ptr
+        dl.moe.encode_decode_layer(b)
+        gpu.synchronize()
+        assert np.array_equal(dl.out_idx.download(np.uint32, k), h_idx[tok * k:(tok + 1) * k])
+        assert np.array_equal(dl.out_w.download(np.uint16, k), h_w[tok * k:(tok + 1) * k])
+        assert np.array_equal(dl.resolved.download(np.uint32, k), h_res[tok * k:(tok + 1) * k])
+        assert np.array_equal(dl.y.download(np.uint16, d), all_y[tok * d:(tok + 1) * d]), f"token {tok}: y differs from the one-token layer"
+        assert np.array_equal(one_hid.download(np.uint16, d), all_hid[tok * d:(tok + 1) * d])
+    # what the entry point refuses
+    lib = capi.load()
+    assert lib.shrike_hip_moe_decode_layer_batch(dl.moe.handle, None, C.byref(a), 17, stride) != 0 and "tokens" in capi.last_error()
+    assert lib.shrike_hip_moe_decode_layer_batch(dl.moe.handle, None, C.byref(a), t, d - 8) != 0
+    shared = Layer(0x5EED0045, 256, 128, 8, 2, shared_f=128)
+    sdl = DeviceLayer(gpu, shared)
+    assert lib.shrike_hip_moe_decode_layer_batch(sdl.moe.handle, None, C.byref(sdl.layer_args()), 2, 256) != 0
+    assert "shared expert" in capi.last_error()
+
+
 @pytest.mark.parametrize("bits,resident_of_selection", [(4, 5), (8, 0), (4, 8)])
 def test_decode_with_misses_equals_the_resident_layer(gpu, bits, resident_of_selection):
     """The speculative pass and the agreed fixup: a token whose selection is partly (or wholly) absent from a
