@@ -676,6 +676,72 @@ def test_decode_layer_for_a_batch_equals_the_layer_token_by_token(gpu, d, f, ne,
     assert "shared expert" in capi.last_error()
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_config4_stack_of_24_layers_for_four_tokens(gpu, bits):
+    """Config 4 as it is stated: 4 independent tokens through 24 stacked gpt-oss-shape layers (hidden = intermediate =
+    2880, 32 experts, top-4), every layer with a pool and a router of its own, the residual stream (`hidden`) carried
+    from layer to layer and each layer's x a fresh seeded row block. Every layer's routes for every token equal the
+    oracle's router bit for bit; three layers' y rows are held to the oracle stage by stage for two tokens; and the
+    residual stream after the last layer equals the fp16 sum, layer by layer, of the y rows the device produced."""
+    d = f = 2880
+    ne, k, t, n_layers = 32, 4, 4, 24
+    L = Layer(0x5EED0004, d, f, ne, k, bits=bits, meta=S.META_F16)
+    base = DeviceLayer(gpu, L)
+    routers = [S.router_f16(L.tree, f"layer.{l}.router.w", ne, d) for l in range(n_layers)]
+    xs = [S.activations_f16(L.tree, f"layer.{l}.x", t * d) for l in range(n_layers)]
+    hidden0 = S.activations_f16(L.tree, "stack.hidden", t * d)
+    d_hidden = gpu.dev(hidden0)
+    # layers share layer 0's blobs but each has a pool of its own with its own expert -> cell map
+    pools, cell_of = [base.pool], [base.cell_of]
+    for l in range(1, n_layers):
+        pool = gpu.ExpertPool(ne, L.stride, ne)
+        cells = {}
+        for e in range(ne):
+            cell = (e * 5 + l) % ne
+            capi.check(capi.load().shrike_hip_memcpy_d2d(pool.cell_ptr(cell), base.pool.cell_ptr(base.cell_of[e]), L.stride), "d2d")
+            pool.publish(e, cell, capi.RESIDENT)
+            cells[e] = cell
+        pools.append(pool)
+        cell_of.append(cells)
+    idx, w, res = gpu.empty(4 * t * k), gpu.empty(2 * t * k), gpu.empty(4 * t * k)
+    acts, y = gpu.empty(2 * t * k * f), gpu.empty(2 * t * d)
+    ys, routes, all_acts = [], [], []
+    for l in range(n_layers):
+        a = base.layer_args()
+        rw, dx = gpu.dev(routers[l]), gpu.dev(xs[l])
+        a.router_weights = rw.ptr
+        a.pool, a.pool_slot_stride, a.residency = pools[l].bases, pools[l].stride, pools[l].table
+        a.x, a.hidden, a.y, a.out_indices, a.out_weights, a.resolved_slots, a.acts = dx.ptr, d_hidden.ptr, y.ptr, idx.ptr, w.ptr, res.ptr, acts.ptr
+        base.moe.encode_decode_layer_batch(a, t, d)
+        gpu.synchronize()
+        ys.append(y.download(np.uint16, t * d))
+        routes.append((idx.download(np.uint32, t * k), w.download(np.uint16, t * k), res.download(np.uint32, t * k)))
+        all_acts.append(acts.download(np.uint16, t * k * f) if l in (0, 11, 23) else None)
+    off = L.oracle_offsets()
+    router = L.router_dict()
+    for l in range(n_layers):
+        router["weights"] = routers[l]
+        ref_idx, ref_w, _ = O.prefill_router(router, xs[l], t, d, k)
+        got_idx, got_w, got_res = routes[l]
+        assert np.array_equal(got_idx, ref_idx), f"layer {l}: routes differ from the oracle's"
+        assert np.max(np.abs(f16(got_w) - f16(ref_w))) <= 1e-3
+        assert got_res.tolist() == [cell_of[l][int(e)] for e in got_idx]
+    for l in (0, 11, 23):
+        for tok in (0, 3):
+            experts = routes[l][0][tok * k:(tok + 1) * k]
+            blobs = [L.blobs[int(e)] for e in experts]
+            x_row = np.ascontiguousarray(xs[l][tok * d:(tok + 1) * d])
+            dev_acts = np.ascontiguousarray(all_acts[l][tok * k * f:(tok + 1) * k * f])
+            assert_ffn_close(dev_acts, O.moe_phase1(blobs, off, x_row, d, f, bits, L.meta), f"layer {l} token {tok}: activations")
+            ref_y = O.moe_phase2(blobs, off, dev_acts, routes[l][1][tok * k:(tok + 1) * k].copy(), np.zeros(d, np.uint16), d, f, bits, L.meta)
+            assert_ffn_close(ys[l][tok * d:(tok + 1) * d], ref_y, f"layer {l} token {tok}: y from the device's activations")
+    want = hidden0.copy()
+    for l in range(n_layers):
+        want = O.residual_add_f16(want, ys[l])
+    assert np.array_equal(d_hidden.download(np.uint16, t * d), want), "the residual stream after 24 layers"
+    assert len({tuple(r[0].tolist()) for r in routes}) == n_layers, "every layer routes on its own"
+
+
 @pytest.mark.parametrize("bits,resident_of_selection", [(4, 5), (8, 0), (4, 8)])
 def test_decode_with_misses_equals_the_resident_layer(gpu, bits, resident_of_selection):
     """The speculative pass and the agreed fixup: a token whose selection is partly (or wholly) absent from a
