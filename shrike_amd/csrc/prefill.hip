@@ -130,18 +130,41 @@ __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weig
                 }
             }
         }
+        // The butterfly of router_row (xor 32, 16, ..., 1) over the step's TPS * ROWS sums at once. While more than one
+        // sum is left, a step's two partner lanes split them: each keeps half and adds the partner's copy of that half,
+        // so a step costs half the exchanges of the one before; what a lane adds is what the plain butterfly adds in that
+        // lane (the same two operands, and addition commutes), so every sum is router_row's bit for bit. Sum j ends in the
+        // lanes whose upper bits spell j.
+        constexpr uint32_t kSums = TPS * uint32_t(ROWS);
+        static_assert(kSums == 1u || kSums == 2u || kSums == 4u || kSums == 8u, "the split butterfly takes 1, 2, 4 or 8 sums");
+        float v[kSums];
 #pragma unroll
-        for (int o = 32; o >= 1; o >>= 1)
+        for (uint32_t u = 0; u < TPS; ++u)
 #pragma unroll
-            for (uint32_t u = 0; u < TPS; ++u)
+            for (int r = 0; r < ROWS; ++r) v[u * ROWS + r] = acc[u][r];
+        uint32_t live = kSums;  // sums this lane still carries: v[0 .. live)
 #pragma unroll
-                for (int r = 0; r < ROWS; ++r) acc[u][r] = __fadd_rn(acc[u][r], __shfl_xor(acc[u][r], o));
-        if (lane == 0) {
+        for (int o = 32; o >= 1; o >>= 1) {
+            if (live > 1u) {
+                const bool upper = (lane & uint32_t(o)) != 0u;  // the upper partner keeps the upper half of the sums
+                live >>= 1;
 #pragma unroll
-            for (uint32_t u = 0; u < TPS; ++u)
-#pragma unroll
-                for (int r = 0; r < ROWS; ++r)
-                    if (t + u < t1 && e0 + uint32_t(r) < num_experts) logits[size_t(t + u) * num_experts + e0 + r] = acc[u][r];
+                for (uint32_t j = 0; j < kSums / 2u; ++j) {
+                    if (j < live) {
+                        const float keep = upper ? v[j + live] : v[j], send = upper ? v[j] : v[j + live];
+                        v[j] = __fadd_rn(keep, __shfl_xor(send, o));
+                    }
+                }
+            } else {
+                v[0] = __fadd_rn(v[0], __shfl_xor(v[0], o));
+            }
+        }
+        // which sum this lane holds: one bit a split, from the first split (xor 32) down
+        constexpr uint32_t kSplits = kSums == 8u ? 3u : kSums == 4u ? 2u : kSums == 2u ? 1u : 0u;
+        const uint32_t mine = kSplits ? lane >> (6u - kSplits) : 0u;
+        if ((lane & ((64u >> kSplits) - 1u)) == 0u) {
+            const uint32_t u = mine / uint32_t(ROWS), r = mine % uint32_t(ROWS);
+            if (t + u < t1 && e0 + r < num_experts) logits[size_t(t + u) * num_experts + e0 + r] = v[0];
         }
     };
     uint4 staged[TPS][kStage];  // live across a step's arithmetic; handed to the lambdas as a parameter so it stays in registers
