@@ -404,6 +404,24 @@ def prefill_workload(args, rt, capi, S, meta):
     flops = T * K * 6 * D * F
     ffn_us = parts["grouped FFN (3 launches)"]
     traffic = profile_figure("prefill_chunk_q35b_int4_t512.txt", "hbm_bytes_per_chunk_grouped_ffn") if T == 512 else None
+    # What a SIMD makes of matrix and vector instructions side by side, at the FFN kernels' two waves a SIMD: a slot of
+    # four 32x32x16 matrix instructions, a slot of thirty-two fused multiply-adds, and both (the FFN's main loop issues
+    # about as many cycles of each). Where `both` is near the sum and not near the longer one, the kernel's floor is
+    # the sum of its matrix and vector cycles, not the larger.
+    from harness import probes
+    one, sink = rt.dev(np.ones(1, np.float32)), rt.empty(64)
+    slots = 2048
+
+    def issue_us(what, waves):
+        def fn(_):
+            probes.check(probes.load().shrike_probe_issue(stream.handle, what, waves, slots, one.ptr, sink.ptr), "probe_issue")
+        return timed(fn, 4, regions=3) * 1e3
+    issue = {"slots": slots, "slot": "4 x v_mfma_f32_32x32x16_f16 | 32 x v_fma_f32", "by_waves_per_simd": {}}
+    for waves in (2, 4):
+        m_us, v_us, b_us = issue_us(1, waves), issue_us(2, waves), issue_us(3, waves)
+        issue["by_waves_per_simd"][str(waves)] = {"matrix_us": round(m_us, 1), "vector_us": round(v_us, 1), "both_us": round(b_us, 1),
+                                                 "both_over_longer": round(b_us / max(m_us, v_us), 3),
+                                                 "both_over_sum": round(b_us / (m_us + v_us), 3)}
     cpu = None
     if getattr(args, "cpu_sample", 0) > 0:  # the chunk's T * K pair FFNs on the host's cores
         cpu = cpu_pairs(S, keep[4], D, F, BITS, meta, T * K, 1, f"one chunk's {T * K} pair FFNs at the 35B-A3B shape, int4")
@@ -424,7 +442,8 @@ def prefill_workload(args, rt, capi, S, meta):
                      "achieved": round(expert_bytes / (ffn_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(expert_bytes / (ffn_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "bytes_per_launch": expert_bytes,
                      "us_per_launch": round(ffn_us, 2), "traffic": traffic,
-                     "mfma_tflops_on_pair_flops": round(flops / (ffn_us * 1e-6) / 1e12, 2)},
+                     "mfma_tflops_on_pair_flops": round(flops / (ffn_us * 1e-6) / 1e12, 2),
+                     "matrix_and_vector_issue": issue},
         "algorithmic_bytes_per_chunk": algorithmic, "pair_flops_per_chunk": flops,
     }
 

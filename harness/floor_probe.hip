@@ -64,6 +64,44 @@ __global__ void k_probe_timestamp(uint64_t *slot) {
     if (threadIdx.x == 0) *slot = wall_clock64();
 }
 
+// What a SIMD does with matrix and vector instructions side by side. Every wave runs `slots` slots; a slot is four
+// v_mfma_f32_32x32x16_f16 (WHAT & 1) and thirty-two fp32 fused multiply-adds on eight independent chains (WHAT & 2),
+// a matrix instruction followed by eight of the vector ones. One workgroup of 4 x waves_per_simd waves a compute unit.
+typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+template <int WHAT>
+__global__ __launch_bounds__(1024) void k_probe_issue(uint32_t slots, const float *one, float *sink) {
+    probe_half8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        a[i] = _Float16(float(threadIdx.x & 7u) + float(i));
+        b[i] = _Float16(0.5f * float(i));
+    }
+    probe_f32x16 c[4] = {{0}, {0}, {0}, {0}};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = float(threadIdx.x + i);
+    const float m = one[0];
+    for (uint32_t it = 0; it < slots; ++it) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (WHAT & 1) c[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c[q], 0, 0, 0);
+            if (WHAT & 2) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = fmaf(v[i], m, 1.0f);
+            }
+        }
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum += c[q][i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum += v[i];
+    if (sum == -1.0f) sink[0] = sum;  // sums of non-negative terms: never true; keeps the work live
+}
+
 }  // namespace shrike
 
 using namespace shrike;
@@ -112,6 +150,21 @@ int shrike_probe_dependent_loads(void *stream, const uint32_t *d_table, uint32_t
 int shrike_probe_timestamp(void *stream, uint64_t *d_slot) {
     SHRIKE_REQUIRE(d_slot != nullptr && reinterpret_cast<uintptr_t>(d_slot) % 8u == 0, "probe: the slot must be bound and 8-byte aligned");
     hipLaunchKernelGGL(k_probe_timestamp, dim3(1), dim3(64), 0, as_stream(stream), d_slot);
+    SHRIKE_HIP(hipGetLastError());
+    return 0;
+}
+// what: 1 matrix instructions only, 2 vector only, 3 both. d_one: a float holding 1.0f (the multiplier, unknown to the
+// compiler). One workgroup per compute unit of the current device.
+int shrike_probe_issue(void *stream, uint32_t what, uint32_t waves_per_simd, uint32_t slots, const float *d_one, float *d_sink) {
+    SHRIKE_REQUIRE(what >= 1 && what <= 3 && (waves_per_simd == 1 || waves_per_simd == 2 || waves_per_simd == 4), "probe: what 1...3, 1, 2 or 4 waves a SIMD");
+    SHRIKE_REQUIRE(slots >= 1 && slots <= (1u << 20) && d_one != nullptr && d_sink != nullptr, "probe: 1...2^20 slots, multiplier and sink bound");
+    int device = 0, units = 0;
+    SHRIKE_HIP(hipGetDevice(&device));
+    SHRIKE_HIP(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
+    const dim3 grid = dim3(static_cast<uint32_t>(units)), block = dim3(256u * waves_per_simd);
+    if (what == 1) hipLaunchKernelGGL(k_probe_issue<1>, grid, block, 0, as_stream(stream), slots, d_one, d_sink);
+    else if (what == 2) hipLaunchKernelGGL(k_probe_issue<2>, grid, block, 0, as_stream(stream), slots, d_one, d_sink);
+    else hipLaunchKernelGGL(k_probe_issue<3>, grid, block, 0, as_stream(stream), slots, d_one, d_sink);
     SHRIKE_HIP(hipGetLastError());
     return 0;
 }

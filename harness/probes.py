@@ -1,5 +1,5 @@
 """ctypes face of libshrikeprobe.so: the benchmark's measurement aids (an empty launch, a kernel that only reads
-a byte range of listed pool cells, a chain of dependent loads). Not part of the product's ABI: nothing in libshrikehip or in the
+a byte range of listed pool cells, a chain of dependent loads, matrix and vector instructions side by side). Not part of the product's ABI: nothing in libshrikehip or in the
 operator mirror depends on it."""
 from __future__ import annotations
 
@@ -29,6 +29,8 @@ def load() -> C.CDLL:
         _lib.shrike_probe_dependent_loads.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]
         _lib.shrike_probe_timestamp.restype = C.c_int
         _lib.shrike_probe_timestamp.argtypes = [C.c_void_p, C.c_void_p]
+        _lib.shrike_probe_issue.restype = C.c_int
+        _lib.shrike_probe_issue.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         _lib.shrike_probe_wall_clock_khz.restype = C.c_int
         _lib.shrike_probe_wall_clock_khz.argtypes = []
     return _lib

@@ -31,3 +31,22 @@ def test_measurement_probes_run_and_check_their_arguments():
     assert "leaves the cell" in probes.last_error()
     assert lib.shrike_probe_read(None, dl.pool.bases, dl.pool.stride, cells.ptr, 4, 8, 1024, sink.ptr) != 0
     assert lib.shrike_probe_empty_launch(None, 0, sink.ptr) != 0
+
+
+def test_issue_probe_runs_and_checks_its_arguments():
+    """Matrix and vector instructions side by side: the three forms launch, drain, and leave the sink alone."""
+    gpu = runtime
+    gpu.init(0)
+    lib = probes.load()
+    one = gpu.empty(4)
+    one.upload(np.ones(1, np.float32))
+    sink = gpu.empty(64).fill(0)
+    for what in (1, 2, 3):
+        for waves in (1, 2, 4):
+            probes.check(lib.shrike_probe_issue(None, what, waves, 64, one.ptr, sink.ptr), "probe_issue")
+    gpu.synchronize()
+    assert not sink.download(np.uint32, 16).any()
+    assert lib.shrike_probe_issue(None, 0, 2, 64, one.ptr, sink.ptr) != 0
+    assert lib.shrike_probe_issue(None, 3, 3, 64, one.ptr, sink.ptr) != 0
+    assert lib.shrike_probe_issue(None, 3, 2, 0, one.ptr, sink.ptr) != 0
+    assert lib.shrike_probe_issue(None, 3, 2, 64, None, sink.ptr) != 0

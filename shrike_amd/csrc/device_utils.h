@@ -218,6 +218,26 @@ __device__ __forceinline__ float gelu_tanh(float v) {
     inner = fminf(fmaxf(inner, -20.0f), 20.0f);
     return 0.5f * v * (1.0f + tanhf(inner));
 }
+// The same three activations through the hardware's exp2 and reciprocal (each within 1 ulp of fp32; a sigmoid
+// a few ulp): for results that are rounded to fp16 next, where a correctly rounded division and expf buy nothing.
+// gelu_tanh(v) = v * sigmoid(2 * inner), since 0.5 * (1 + tanh(t)) = 1 / (1 + exp(-2 t)).
+__device__ __forceinline__ float sigmoid_fast(float v) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
+}
+template <int ACT>
+__device__ __forceinline__ float glu_fast(float gate, float up) {
+    if (ACT == 2) {
+        const float g = fminf(gate, 7.0f);
+        const float u = fminf(fmaxf(up, -7.0f), 7.0f);
+        return (g * sigmoid_fast(1.702f * g)) * (u + 1.0f);
+    }
+    if (ACT == 1) return (gate * sigmoid_fast(gate)) * up;
+    const float cube = gate * gate * gate;
+    float inner = 0.7978845608028654f * (gate + 0.044715f * cube);
+    inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+    return (gate * sigmoid_fast(2.0f * inner)) * up;
+}
+
 // moe.metal:280-288
 template <int ACT>
 __device__ __forceinline__ float glu(float gate, float up) {

@@ -43,6 +43,12 @@ __device__ __forceinline__ float glu_rt(float g, float u, uint32_t act) {
     return glu<0>(g, u);
 }
 
+__device__ __forceinline__ float glu_rt_fast(float g, float u, uint32_t act) {
+    if (act == SHRIKE_ACT_SILU) return glu_fast<1>(g, u);
+    if (act == SHRIKE_ACT_CLAMPED_SWIGLU) return glu_fast<2>(g, u);
+    return glu_fast<0>(g, u);
+}
+
 // moe.metal:36-39
 __device__ __forceinline__ bool io_ready(const uint32_t *io_status) {
     if (!io_status) return true;

@@ -379,7 +379,7 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
                         g = f16_to_f32(f32_to_f16(g));
                         u = f16_to_f32(f32_to_f16(u));
                     }
-                    s_a[0][m][wave * 32u + col] = f32_to_f16(glu_rt(g, u, a.act_kind));
+                    s_a[0][m][wave * 32u + col] = f32_to_f16(glu_rt_fast(g, u, a.act_kind));
                 }
             }
         }
