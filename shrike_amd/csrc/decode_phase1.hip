@@ -19,7 +19,8 @@ constexpr int kPhase1RowPairsNarrow = 2;
 // memory (L2-resident) ahead of the row loads, so in-order load return never holds it back.
 // STREAM: one token, so every routed row is read exactly once: the row loads are non-temporal (a batch of tokens
 // reads an expert's rows once per token routed to it, and there the caches are what makes the second read cheap).
-template <int BITS, int NCH, int RP, bool ROUTE, int SBITS, bool STREAM>
+// TAIL: the rows end in a step of half chunks (load_slice_regs); NCH then counts the whole steps ahead of it.
+template <int BITS, int NCH, int RP, bool ROUTE, int SBITS, bool STREAM, bool TAIL>
 __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
@@ -66,16 +67,16 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     }
 
     uint32_t cell = kSentinel;
-    SliceRegs<BITS, NCH> xr;
+    SliceRegs<BITS, NCH, TAIL> xr;
     if (ROUTE) {
         // every wave selects for itself, in registers, from the table the previous launch left: no barrier, and the
         // table's loads go out ahead of the activation slice's (loads return in order)
         // (a wave stops at the round that names its own position's expert)
         const TableSelect t = select_from_table(a.route_table + tok * SHRIKE_MAX_ROUTER_EXPERTS, a.sel.num_experts, a.sel.top_k, lane, k);
-        load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
+        load_slice_regs<BITS, NCH, TAIL>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
         if (in_range) cell = uint32_t(__builtin_amdgcn_readlane(int(t.my_cell), int(k)));
     } else {
-        load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
+        load_slice_regs<BITS, NCH, TAIL>(xr, reinterpret_cast<const uint4 *>(x_tok), cpr, lane, true);
         if (in_range && !a.blobs) cell = resolved_tok[k];
     }
     const uint8_t *base;
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
         base = cell_base_uniform(a.pool, cell, a.stride);
     }
 
-    RowRegs<BITS, NCH> rows[2 * RP];
+    RowRegs<BITS, NCH, TAIL> rows[2 * RP];
 #pragma unroll
     for (int r = 0; r < 2 * RP; ++r) {
         const bool up = r >= RP;
@@ -95,7 +96,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
         const uint8_t *w = base + (up ? a.off.up_w_off : a.off.gate_w_off) + size_t(f) * row_bytes;
         const uint16_t *s = reinterpret_cast<const uint16_t *>(base + (up ? a.off.up_s_off : a.off.gate_s_off)) + size_t(f) * groups;
         const uint16_t *b = reinterpret_cast<const uint16_t *>(base + (up ? a.off.up_b_off : a.off.gate_b_off)) + size_t(f) * groups;
-        load_row<BITS, NCH, STREAM>(rows[r], w, s, b, cpr, lane, true);
+        load_row<BITS, NCH, STREAM, TAIL>(rows[r], w, s, b, cpr, lane, true);
     }
     float gab = 0.0f, uab = 0.0f;
     if (a.ebias && lane < uint32_t(RP)) {  // moe.metal:261-269
@@ -105,10 +106,11 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
 
     typename C::X x[NCH];
     float xs[NCH];
-    unpack_slices<BITS, NCH>(xr, x, xs);
+    TailX xt;
+    unpack_slices<BITS, NCH, TAIL>(xr, x, xs, xt);
     float res[2 * RP];
 #pragma unroll
-    for (int r = 0; r < 2 * RP; ++r) res[r] = wave_sum(row_partial<BITS, NCH>(rows[r], x, xs, a.meta));
+    for (int r = 0; r < 2 * RP; ++r) res[r] = wave_sum(row_partial<BITS, NCH, TAIL>(rows[r], x, xs, xt, a.meta));
     // lane p < RP finishes row pair p
     float g = res[0], u = res[RP];
 #pragma unroll
@@ -127,6 +129,7 @@ static uint32_t phase1_blocks_of(uint32_t positions, uint32_t f, uint32_t row_pa
 }
 uint32_t phase1_blocks(uint32_t top_k, uint32_t f) { return phase1_blocks_of(top_k, f, kPhase1RowPairs); }
 
+// (a row that ends in half chunks counts the steps it would take without them: the choice stays what it was measured as)
 static bool phase1_narrow(bool routing, bool one_token, uint32_t d, uint32_t bits) {
     return one_token ? !routing : nch_for(d, bits) >= 3;
 }
@@ -136,11 +139,16 @@ static void launch_phase1_nch(const Phase1Args &a, dim3 grid, hipStream_t s) {
     // (the one-token routing launch keeps four pairs; a batch takes the narrow form for long rows whether it routes or not)
     constexpr int RP = kPhase1RowPairs, RN = (ROUTE && STREAM) ? kPhase1RowPairs : kPhase1RowPairsNarrow;
     const dim3 block(256);
+    if (BITS == 4 && half_chunk_tail(a.d * BITS / 128u, BITS)) {
+        // d <= SHRIKE_MAX_HIDDEN: one whole step and the half chunks (65...96 chunks a row)
+        hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM, BITS == 4>), grid, block, 0, s, a);
+        return;
+    }
     switch (nch_for(a.d, BITS)) {
-        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
-        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, STREAM ? RN : RP, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
-        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RN, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RN, ROUTE, SBITS, STREAM>), grid, block, 0, s, a); break;
+        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM, false>), grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, STREAM ? RN : RP, ROUTE, SBITS, STREAM, false>), grid, block, 0, s, a); break;
+        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RN, ROUTE, SBITS, STREAM, false>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RN, ROUTE, SBITS, STREAM, false>), grid, block, 0, s, a); break;
     }
 }
 

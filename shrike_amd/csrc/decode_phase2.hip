@@ -23,7 +23,8 @@ __device__ __forceinline__ void phase2_finish(uint16_t *y, uint16_t *hidden, uin
 // STREAM: one token, every down row is read once: non-temporal row loads (see k_phase1).
 // ROWS: output rows a workgroup owns. One token takes 8 (at d = 2048 that is one workgroup a compute unit); a batch of
 // tokens over long rows takes 16, so that a wave's slice of the activations, fetched once, serves twice the rows.
-template <int BITS, int NCH, int BATCH, bool STREAM, uint32_t ROWS>
+// TAIL: the rows end in a step of half chunks (load_slice_regs); NCH then counts the whole steps ahead of it.
+template <int BITS, int NCH, int BATCH, bool STREAM, uint32_t ROWS, bool TAIL>
 __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
@@ -62,8 +63,8 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     const uint32_t sub = packed ? lane / cpr : 0u, col = packed ? lane % cpr : lane;
     const bool lane_on = sub < rpl;
 
-    SliceRegs<BITS, NCH> xr;
-    load_slice_regs<BITS, NCH>(xr, reinterpret_cast<const uint4 *>(acts_tok + size_t(k) * a.f), cpr, col, lane_on);
+    SliceRegs<BITS, NCH, TAIL> xr;
+    load_slice_regs<BITS, NCH, TAIL>(xr, reinterpret_cast<const uint4 *>(acts_tok + size_t(k) * a.f), cpr, col, lane_on);
     const float wk = f16_to_f32(routing_tok[k]);
     bool live;
     const uint8_t *base;
@@ -83,8 +84,9 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
         const uint32_t n_groups = kPhase2Rows / rpl;
         typename C::X x[NCH];
         float xs[NCH];
+        TailX xt;
         for (uint32_t g0 = 0; g0 < n_groups; g0 += BATCH) {
-            RowRegs<BITS, NCH> rows[BATCH];
+            RowRegs<BITS, NCH, TAIL> rows[BATCH];
             uint32_t row[BATCH];
             bool on[BATCH];
 #pragma unroll
@@ -92,13 +94,13 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
                 row[j] = d0 + (g0 + j) * rpl + sub;
                 on[j] = lane_on && (g0 + j) < n_groups && row[j] < a.d;
                 const uint32_t rr = on[j] ? row[j] : 0u;
-                load_row<BITS, NCH, STREAM>(rows[j], base + a.off.down_w_off + size_t(rr) * row_bytes,
+                load_row<BITS, NCH, STREAM, TAIL>(rows[j], base + a.off.down_w_off + size_t(rr) * row_bytes,
                                     s_all + size_t(rr) * groups, b_all + size_t(rr) * groups, cpr, col, on[j]);
             }
-            if (g0 == 0) unpack_slices<BITS, NCH>(xr, x, xs);
+            if (g0 == 0) unpack_slices<BITS, NCH, TAIL>(xr, x, xs, xt);
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
-                float v = seg_sum(row_partial<BITS, NCH>(rows[j], x, xs, a.meta), seg);
+                float v = seg_sum(row_partial<BITS, NCH, TAIL>(rows[j], x, xs, xt, a.meta), seg);
                 const bool writer = on[j] && (lane % seg) == seg - 1u;
                 if (writer) {
                     if (a.ebias) v += bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[row[j]]);
@@ -123,37 +125,47 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
     gemv_job<BITS, NCH>(a, blockIdx.x);
 }
 
-template <int BITS, int NCH, uint32_t ROWS>
+template <int BITS, int NCH, uint32_t ROWS, bool TAIL>
 static void launch_phase2_rows(const Phase2Args &a, dim3 block, hipStream_t s) {
     const dim3 grid((a.d + ROWS - 1) / ROWS, a.tokens ? a.tokens : 1u);
     const uint32_t cpr = a.f * BITS / 128u;
     const uint32_t rpl = (cpr < 64u && 64u % cpr == 0u) ? (64u / cpr < ROWS ? 64u / cpr : ROWS) : 1u;
     const uint32_t n_groups = ROWS / rpl;  // row groups per wave; up to 4 in flight
     if (a.tokens <= 1u) {
-        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, true, ROWS>), grid, block, 0, s, a);
-        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, true, ROWS>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, true, ROWS>), grid, block, 0, s, a);
+        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, true, ROWS, TAIL>), grid, block, 0, s, a);
+        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, true, ROWS, TAIL>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, true, ROWS, TAIL>), grid, block, 0, s, a);
     } else {
-        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, false, ROWS>), grid, block, 0, s, a);
-        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, false, ROWS>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, false, ROWS>), grid, block, 0, s, a);
+        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, false, ROWS, TAIL>), grid, block, 0, s, a);
+        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, false, ROWS, TAIL>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, false, ROWS, TAIL>), grid, block, 0, s, a);
     }
 }
 
-template <int BITS, int NCH>
+// (rows of more than one step a lane, whole or half)
+template <int BITS, int NCH, bool TAIL>
 static void launch_phase2_batch(const Phase2Args &a, dim3 block, hipStream_t s) {
-    if (NCH >= 2 && a.tokens > 1u) launch_phase2_rows<BITS, NCH, kPhase2RowsBatch>(a, block, s);
-    else launch_phase2_rows<BITS, NCH, kPhase2Rows>(a, block, s);
+    if ((NCH >= 2 || TAIL) && a.tokens > 1u) launch_phase2_rows<BITS, NCH, kPhase2RowsBatch, TAIL>(a, block, s);
+    else launch_phase2_rows<BITS, NCH, kPhase2Rows, TAIL>(a, block, s);
 }
 
 template <int BITS>
 static void launch_phase2_bits(const Phase2Args &a, hipStream_t s) {
     const dim3 block(64 * a.top_k);
+    const uint32_t cpr = a.f * BITS / 128u;
+    if (BITS == 4 && half_chunk_tail(cpr, BITS)) {  // whole steps, then the half chunks
+        switch (cpr / 64u) {
+            case 1: launch_phase2_batch<BITS, 1, BITS == 4>(a, block, s); break;
+            case 2: launch_phase2_batch<BITS, 2, BITS == 4>(a, block, s); break;
+            default: launch_phase2_batch<BITS, 3, BITS == 4>(a, block, s); break;
+        }
+        return;
+    }
     switch (nch_for(a.f, BITS)) {
-        case 1: launch_phase2_batch<BITS, 1>(a, block, s); break;
-        case 2: launch_phase2_batch<BITS, 2>(a, block, s); break;
-        case 3: launch_phase2_batch<BITS, 3>(a, block, s); break;
-        default: launch_phase2_batch<BITS, 4>(a, block, s); break;
+        case 1: launch_phase2_batch<BITS, 1, false>(a, block, s); break;
+        case 2: launch_phase2_batch<BITS, 2, false>(a, block, s); break;
+        case 3: launch_phase2_batch<BITS, 3, false>(a, block, s); break;
+        default: launch_phase2_batch<BITS, 4, false>(a, block, s); break;
     }
 }
 

@@ -81,16 +81,25 @@ __device__ __forceinline__ uint4 zero4() { return make_uint4(0u, 0u, 0u, 0u); }
 // `off` has bit i set when slice i is not this lane's to use: the load then went to a valid
 // stand-in address and unpack_slices zeroes the slice. (Zeroing right behind the load would
 // make the wave wait for that load there and then, one load at a time.)
-template <int BITS, int NCH>
+//
+// TAIL (4-bit codes): a row of 64 NCH + r chunks with 1 <= r <= 32 ends in a step of half chunks (8 bytes of codes,
+// 16 activations) spread over 2 r lanes, in place of a whole step that r lanes would work through and the others
+// idle: half chunk 128 NCH + col of the row, for col < 2 r. Bit NCH of `off` marks a lane without one.
+template <int BITS, int NCH, bool TAIL = false>
 struct SliceRegs {
     uint4 v[NCH][Chunk<BITS>::PIECES];
+    uint4 t[2];
     uint32_t off;
 };
 
-template <int BITS, int NCH>
-__device__ __forceinline__ void load_slice_regs(SliceRegs<BITS, NCH> &r, const uint4 *vec, uint32_t cpr,
+// whether a row of `cpr` 16-byte chunks is walked as cpr / 64 whole steps and a step of half chunks
+inline bool half_chunk_tail(uint32_t cpr, uint32_t bits) { return bits == 4u && cpr > 64u && (cpr % 64u) >= 1u && (cpr % 64u) <= 32u; }
+
+template <int BITS, int NCH, bool TAIL = false>
+__device__ __forceinline__ void load_slice_regs(SliceRegs<BITS, NCH, TAIL> &r, const uint4 *vec, uint32_t cpr,
                                                 uint32_t col, bool lane_on) {
     typedef Chunk<BITS> C;
+    static_assert(!TAIL || BITS == 4, "half chunks are for 4-bit codes");
     r.off = 0u;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -101,12 +110,26 @@ __device__ __forceinline__ void load_slice_regs(SliceRegs<BITS, NCH> &r, const u
 #pragma unroll
         for (int j = 0; j < C::PIECES; ++j) r.v[i][j] = vec[cc * C::PIECES + j];
     }
+    if (TAIL) {
+        const uint32_t h = 128u * NCH + col;
+        const bool on = lane_on && h < 2u * cpr;
+        const uint32_t hh = on ? h : 0u;
+        r.off |= on ? 0u : 1u << NCH;
+        r.t[0] = vec[hh * 2u];
+        r.t[1] = vec[hh * 2u + 1u];
+    }
 }
 
+// the activations of a half chunk in the dot's pair layout, and their fp32 sum
+struct TailX {
+    h2_t p[8];
+    float sum;
+};
+
 // Pieces -> the dot's pair layout plus the fp32 sum of each slice (for the bias term).
-template <int BITS, int NCH>
-__device__ __forceinline__ void unpack_slices(const SliceRegs<BITS, NCH> &r, typename Chunk<BITS>::X (&x)[NCH],
-                                              float (&xs)[NCH]) {
+template <int BITS, int NCH, bool TAIL>
+__device__ __forceinline__ void unpack_slices(const SliceRegs<BITS, NCH, TAIL> &r, typename Chunk<BITS>::X (&x)[NCH],
+                                              float (&xs)[NCH], TailX &xt) {
     typedef Chunk<BITS> C;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -119,6 +142,19 @@ __device__ __forceinline__ void unpack_slices(const SliceRegs<BITS, NCH> &r, typ
         }
         xs[i] = s;
     }
+    if (TAIL) {
+        const bool off = (r.off >> NCH) & 1u;
+        const uint4 v0 = off ? zero4() : r.t[0], v1 = off ? zero4() : r.t[1];
+        pairs_from_x8(v0, xt.p);
+        pairs_from_x8(v1, xt.p + 4);
+        xt.sum = sum_x8(v0) + sum_x8(v1);
+    }
+}
+template <int BITS, int NCH>
+__device__ __forceinline__ void unpack_slices(const SliceRegs<BITS, NCH, false> &r, typename Chunk<BITS>::X (&x)[NCH],
+                                              float (&xs)[NCH]) {
+    TailX none;
+    unpack_slices<BITS, NCH, false>(r, x, xs, none);
 }
 
 template <int BITS, int NCH>
@@ -132,10 +168,12 @@ __device__ __forceinline__ void load_slices(const uint4 *vec, uint32_t cpr, uint
 // One row's codes and metadata for the lane's column chunks. A chunk that is not this lane's
 // is loaded from a valid stand-in address (chunk 0 of the same row) and left as it is: the
 // lane's activation slice for it is zero, and so is its term (the row's data being finite).
-template <int BITS, int NCH>
+template <int BITS, int NCH, bool TAIL = false>
 struct RowRegs {
     uint4 w[NCH];
     uint16_t s[NCH], b[NCH];
+    uint2 tw;  // TAIL: the lane's half chunk of the row, and its group's scale and bias
+    uint16_t ts, tb;
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -143,8 +181,10 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 // STREAM: the row is read once and by nobody else (a routed expert's rows in decode): the loads are marked
 // non-temporal, so that what they bring in does not displace the small tensors every layer call reads again
 // (router rows, shared expert, route tables) from the caches behind the compute units.
-template <int BITS, int NCH, bool STREAM = false>
-__device__ __forceinline__ void load_row(RowRegs<BITS, NCH> &r, const uint8_t *w_row, const uint16_t *s_row,
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+template <int BITS, int NCH, bool STREAM = false, bool TAIL = false>
+__device__ __forceinline__ void load_row(RowRegs<BITS, NCH, TAIL> &r, const uint8_t *w_row, const uint16_t *s_row,
                                          const uint16_t *b_row, uint32_t cpr, uint32_t col, bool lane_on) {
     typedef Chunk<BITS> C;
 #pragma unroll
@@ -164,18 +204,47 @@ __device__ __forceinline__ void load_row(RowRegs<BITS, NCH> &r, const uint8_t *w
             r.b[i] = b_row[g];
         }
     }
+    if (TAIL) {
+        const uint32_t h = 128u * NCH + col;
+        const bool on = lane_on && h < 2u * cpr;
+        const uint32_t hh = on ? h : 0u;
+        const uint32_t g = hh / 4u;  // sixteen codes a half chunk, 64 a group
+        if (STREAM) {
+            const u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(w_row + 8u * hh));
+            r.tw = make_uint2(v.x, v.y);
+            r.ts = __builtin_nontemporal_load(s_row + g);
+            r.tb = __builtin_nontemporal_load(b_row + g);
+        } else {
+            r.tw = *reinterpret_cast<const uint2 *>(w_row + 8u * hh);
+            r.ts = s_row[g];
+            r.tb = b_row[g];
+        }
+    }
 }
 
-template <int BITS, int NCH>
-__device__ __forceinline__ float row_partial(const RowRegs<BITS, NCH> &r, const typename Chunk<BITS>::X (&x)[NCH],
-                                             const float (&xs)[NCH], uint32_t meta) {
+template <int BITS, int NCH, bool TAIL>
+__device__ __forceinline__ float row_partial(const RowRegs<BITS, NCH, TAIL> &r, const typename Chunk<BITS>::X (&x)[NCH],
+                                             const float (&xs)[NCH], const TailX &xt, uint32_t meta) {
     float acc = 0.0f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
         acc = fmaf(meta_f32(r.s[i], meta), Chunk<BITS>::dot(r.w[i], x[i]), acc);
         acc = fmaf(meta_f32(r.b[i], meta), xs[i], acc);
     }
+    if (TAIL) {
+        float lo = 0.0f, hi = 0.0f;
+        dot_word4(r.tw.x, xt.p, lo, hi);
+        dot_word4(r.tw.y, xt.p + 4, lo, hi);
+        acc = fmaf(meta_f32(r.ts, meta), fmaf(lo, 16.0f, hi) * 1048576.0f, acc);
+        acc = fmaf(meta_f32(r.tb, meta), xt.sum, acc);
+    }
     return acc;
+}
+template <int BITS, int NCH>
+__device__ __forceinline__ float row_partial(const RowRegs<BITS, NCH, false> &r, const typename Chunk<BITS>::X (&x)[NCH],
+                                             const float (&xs)[NCH], uint32_t meta) {
+    TailX none;
+    return row_partial<BITS, NCH, false>(r, x, xs, none, meta);
 }
 
 // ------------------------------------------------- dense group-affine GEMV

@@ -205,14 +205,16 @@ def test_classify_truth_table_and_spec_args(gpu):
 # --------------------------------------------------------------------- phase 1 / 2
 
 SHAPES = [  # d, f
-    (2048, 512), (128, 64), (192, 320), (704, 192), (2880, 2880), (2304, 1024), (4096, 256)]
+    (2048, 512), (128, 64), (192, 320), (704, 192), (2880, 2880), (2304, 1024), (4096, 256),
+    # 4-bit rows that end in a step of half chunks behind one, two and three whole steps (and the 8-bit rows of the same sizes)
+    (2304, 4352), (128, 6400), (3072, 2112)]
 
 
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("meta", [S.META_BF16, S.META_F16])
 @pytest.mark.parametrize("d,f", SHAPES)
 def test_phase1_phase2_against_oracle(gpu, bits, meta, d, f):
-    if d * bits // 128 > 256:
+    if max(d, f) * bits // 128 > 256:
         pytest.skip("row longer than four wave loads")
     k, ne = 8, 8
     if d * f > 4_000_000:
