@@ -62,6 +62,7 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     const uint32_t seg = packed ? cpr : 64u;
     const uint32_t sub = packed ? lane / cpr : 0u, col = packed ? lane % cpr : lane;
     const bool lane_on = sub < rpl;
+    const bool writer_lane = (lane & (seg - 1u)) == seg - 1u;  // a segment is a power of two lanes: 64, or a divisor of it
 
     SliceRegs<BITS, NCH, TAIL> xr;
     load_slice_regs<BITS, NCH, TAIL>(xr, reinterpret_cast<const uint4 *>(acts_tok + size_t(k) * a.f), cpr, col, lane_on);
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
                 float v = seg_sum(row_partial<BITS, NCH, TAIL>(rows[j], x, xs, xt, a.meta), seg);
-                const bool writer = on[j] && (lane % seg) == seg - 1u;
+                const bool writer = on[j] && writer_lane;
                 if (writer) {
                     if (a.ebias) v += bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[row[j]]);
                     partial[k][row[j] - d0] = wk * v;  // moe.metal:1049

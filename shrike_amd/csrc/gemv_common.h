@@ -621,8 +621,39 @@ struct TableSelect {
 // full 32-bit key is compared, so the order is exact. Positions that find nothing left take expert 0 with score
 // -inf, as the reference's initial slots do.
 // last_round (uniform): the last position the caller needs; later rounds are skipped.
+// Up to 64 experts: lane l holds expert l alone, so there is nothing to sort and a round pops by clearing one key.
+__device__ __forceinline__ TableSelect select_from_small_table(const RouteEntry *table, uint32_t num_experts, uint32_t K,
+                                                               uint32_t lane, uint32_t last_round) {
+    const uint4 v = reinterpret_cast<const uint4 *>(table)[lane];
+    uint32_t key = lane < num_experts ? v.x : 0u;
+    TableSelect r;
+    r.mine = 0; r.my_key = 0;
+    r.my_cell = uint32_t(__builtin_amdgcn_readfirstlane(int(v.y)));
+    r.my_gain = uint32_t(__builtin_amdgcn_readfirstlane(int(v.w)));
+    r.my_raw = __uint_as_float(uint32_t(__builtin_amdgcn_readfirstlane(int(v.z))));
+#pragma unroll
+    for (int round = 0; round < 8; ++round) {
+        if (uint32_t(round) < K && uint32_t(round) <= last_round) {
+            const uint32_t top = wave_max_u32(key);
+            if (top != 0u) {  // uniform
+                const int win = __ffsll((long long)__ballot(key == top)) - 1;
+                const uint32_t wcell = uint32_t(__builtin_amdgcn_readlane(int(v.y), win));
+                const uint32_t wraw = uint32_t(__builtin_amdgcn_readlane(int(v.z), win));
+                const uint32_t wgain = uint32_t(__builtin_amdgcn_readlane(int(v.w), win));
+                key = lane == uint32_t(win) ? 0u : key;
+                if (lane == uint32_t(round)) {
+                    r.mine = uint32_t(win); r.my_key = top; r.my_cell = wcell; r.my_gain = wgain;
+                    r.my_raw = __uint_as_float(wraw);
+                }
+            }
+        }
+    }
+    return r;
+}
+
 __device__ __forceinline__ TableSelect select_from_table(const RouteEntry *table, uint32_t num_experts, uint32_t K,
                                                          uint32_t lane, uint32_t last_round) {
+    if (num_experts <= 64u) return select_from_small_table(table, num_experts, K, lane, last_round);
     uint32_t key[4], cellv[4], rawv[4], gainv[4], idx[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
