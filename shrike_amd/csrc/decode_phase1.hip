@@ -20,7 +20,8 @@ constexpr int kPhase1RowPairsNarrow = 2;
 // STREAM: one token, so every routed row is read exactly once: the row loads are non-temporal (a batch of tokens
 // reads an expert's rows once per token routed to it, and there the caches are what makes the second read cheap).
 // TAIL: the rows end in a step of half chunks (load_slice_regs); NCH then counts the whole steps ahead of it.
-template <int BITS, int NCH, int RP, bool ROUTE, int SBITS, bool STREAM, bool TAIL>
+// META: the type of the routed experts' scales and biases (SHRIKE_META_*), known to the instance so that a row converts them one way.
+template <int BITS, int NCH, int RP, bool ROUTE, int SBITS, bool STREAM, bool TAIL, int META>
 __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(256) void k_phase1(Phase1Args a) {
     unpack_slices<BITS, NCH, TAIL>(xr, x, xs, xt);
     float res[2 * RP];
 #pragma unroll
-    for (int r = 0; r < 2 * RP; ++r) res[r] = wave_sum(row_partial<BITS, NCH, TAIL>(rows[r], x, xs, xt, a.meta));
+    for (int r = 0; r < 2 * RP; ++r) res[r] = wave_sum(row_partial<BITS, NCH, TAIL>(rows[r], x, xs, xt, uint32_t(META)));
     // lane p < RP finishes row pair p
     float g = res[0], u = res[RP];
 #pragma unroll
@@ -134,22 +135,28 @@ static bool phase1_narrow(bool routing, bool one_token, uint32_t d, uint32_t bit
     return one_token ? !routing : nch_for(d, bits) >= 3;
 }
 
-template <int BITS, bool ROUTE, int SBITS, bool STREAM>
-static void launch_phase1_nch(const Phase1Args &a, dim3 grid, hipStream_t s) {
+template <int BITS, bool ROUTE, int SBITS, bool STREAM, int META>
+static void launch_phase1_meta(const Phase1Args &a, dim3 grid, hipStream_t s) {
     // (the one-token routing launch keeps four pairs; a batch takes the narrow form for long rows whether it routes or not)
     constexpr int RP = kPhase1RowPairs, RN = (ROUTE && STREAM) ? kPhase1RowPairs : kPhase1RowPairsNarrow;
     const dim3 block(256);
     if (BITS == 4 && half_chunk_tail(a.d * BITS / 128u, BITS)) {
         // d <= SHRIKE_MAX_HIDDEN: one whole step and the half chunks (65...96 chunks a row)
-        hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM, BITS == 4>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM, BITS == 4, META>), grid, block, 0, s, a);
         return;
     }
     switch (nch_for(a.d, BITS)) {
-        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM, false>), grid, block, 0, s, a); break;
-        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, STREAM ? RN : RP, ROUTE, SBITS, STREAM, false>), grid, block, 0, s, a); break;
-        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RN, ROUTE, SBITS, STREAM, false>), grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RN, ROUTE, SBITS, STREAM, false>), grid, block, 0, s, a); break;
+        case 1: hipLaunchKernelGGL((k_phase1<BITS, 1, STREAM ? RN : RP, ROUTE, SBITS, STREAM, false, META>), grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL((k_phase1<BITS, 2, STREAM ? RN : RP, ROUTE, SBITS, STREAM, false, META>), grid, block, 0, s, a); break;
+        case 3: hipLaunchKernelGGL((k_phase1<BITS, 3, RN, ROUTE, SBITS, STREAM, false, META>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((k_phase1<BITS, 4, RN, ROUTE, SBITS, STREAM, false, META>), grid, block, 0, s, a); break;
     }
+}
+
+template <int BITS, bool ROUTE, int SBITS, bool STREAM>
+static void launch_phase1_nch(const Phase1Args &a, dim3 grid, hipStream_t s) {
+    if (a.meta == SHRIKE_META_F16) launch_phase1_meta<BITS, ROUTE, SBITS, STREAM, SHRIKE_META_F16>(a, grid, s);
+    else launch_phase1_meta<BITS, ROUTE, SBITS, STREAM, SHRIKE_META_BF16>(a, grid, s);
 }
 
 int launch_phase1(const Phase1Args &a, uint32_t bits, bool routing, uint32_t shared_down_bits, hipStream_t s) {

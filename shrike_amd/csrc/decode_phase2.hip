@@ -24,7 +24,8 @@ __device__ __forceinline__ void phase2_finish(uint16_t *y, uint16_t *hidden, uin
 // ROWS: output rows a workgroup owns. One token takes 8 (at d = 2048 that is one workgroup a compute unit); a batch of
 // tokens over long rows takes 16, so that a wave's slice of the activations, fetched once, serves twice the rows.
 // TAIL: the rows end in a step of half chunks (load_slice_regs); NCH then counts the whole steps ahead of it.
-template <int BITS, int NCH, int BATCH, bool STREAM, uint32_t ROWS, bool TAIL>
+// META: the type of the scales and biases (SHRIKE_META_*), known to the instance so that a row converts them one way.
+template <int BITS, int NCH, int BATCH, bool STREAM, uint32_t ROWS, bool TAIL, int META>
 __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
     warm_kernel_arguments(a);
     typedef Chunk<BITS> C;
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
             if (g0 == 0) unpack_slices<BITS, NCH, TAIL>(xr, x, xs, xt);
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
-                float v = seg_sum(row_partial<BITS, NCH, TAIL>(rows[j], x, xs, xt, a.meta), seg);
+                float v = seg_sum(row_partial<BITS, NCH, TAIL>(rows[j], x, xs, xt, uint32_t(META)), seg);
                 const bool writer = on[j] && writer_lane;
                 if (writer) {
                     if (a.ebias) v += bf16_to_f32(reinterpret_cast<const uint16_t *>(base + a.off.down_ab_off)[row[j]]);
@@ -126,21 +127,27 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
     gemv_job<BITS, NCH>(a, blockIdx.x);
 }
 
-template <int BITS, int NCH, uint32_t ROWS, bool TAIL>
-static void launch_phase2_rows(const Phase2Args &a, dim3 block, hipStream_t s) {
+template <int BITS, int NCH, uint32_t ROWS, bool TAIL, int META>
+static void launch_phase2_meta(const Phase2Args &a, dim3 block, hipStream_t s) {
     const dim3 grid((a.d + ROWS - 1) / ROWS, a.tokens ? a.tokens : 1u);
     const uint32_t cpr = a.f * BITS / 128u;
     const uint32_t rpl = (cpr < 64u && 64u % cpr == 0u) ? (64u / cpr < ROWS ? 64u / cpr : ROWS) : 1u;
     const uint32_t n_groups = ROWS / rpl;  // row groups per wave; up to 4 in flight
     if (a.tokens <= 1u) {
-        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, true, ROWS, TAIL>), grid, block, 0, s, a);
-        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, true, ROWS, TAIL>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, true, ROWS, TAIL>), grid, block, 0, s, a);
+        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, true, ROWS, TAIL, META>), grid, block, 0, s, a);
+        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, true, ROWS, TAIL, META>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, true, ROWS, TAIL, META>), grid, block, 0, s, a);
     } else {
-        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, false, ROWS, TAIL>), grid, block, 0, s, a);
-        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, false, ROWS, TAIL>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, false, ROWS, TAIL>), grid, block, 0, s, a);
+        if (n_groups >= 4) hipLaunchKernelGGL((k_phase2<BITS, NCH, 4, false, ROWS, TAIL, META>), grid, block, 0, s, a);
+        else if (n_groups == 2) hipLaunchKernelGGL((k_phase2<BITS, NCH, 2, false, ROWS, TAIL, META>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((k_phase2<BITS, NCH, 1, false, ROWS, TAIL, META>), grid, block, 0, s, a);
     }
+}
+
+template <int BITS, int NCH, uint32_t ROWS, bool TAIL>
+static void launch_phase2_rows(const Phase2Args &a, dim3 block, hipStream_t s) {
+    if (a.meta == SHRIKE_META_F16) launch_phase2_meta<BITS, NCH, ROWS, TAIL, SHRIKE_META_F16>(a, block, s);
+    else launch_phase2_meta<BITS, NCH, ROWS, TAIL, SHRIKE_META_BF16>(a, block, s);
 }
 
 // (rows of more than one step a lane, whole or half)

@@ -167,10 +167,18 @@ __device__ __forceinline__ void pairs_from_x8(const uint4 v, h2_t *p) {
     p[3] = as_h2(__builtin_amdgcn_perm(v.w, v.y, 0x07060302u));  // (e3,e7)
 }
 
+// The first dot of a chain, against a zero accumulator. The compiler only forms the two-operand dot (the accumulator is
+// the destination) and would clear a register for every chain first; the three-operand form takes the zero as a constant.
+__device__ __forceinline__ float dot2_from_zero(h2_t a, h2_t b) {
+    float r;
+    asm("v_dot2_f32_f16 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 // fp32 sum of 8 fp16 activations: four 2-way dots against (1, 1).
 __device__ __forceinline__ float sum_x8(const uint4 v) {
     const h2_t one = {(_Float16)1.0f, (_Float16)1.0f};
-    float s = __builtin_amdgcn_fdot2(as_h2(v.x), one, 0.0f, false);
+    float s = dot2_from_zero(as_h2(v.x), one);
     s = __builtin_amdgcn_fdot2(as_h2(v.y), one, s, false);
     s = __builtin_amdgcn_fdot2(as_h2(v.z), one, s, false);
     s = __builtin_amdgcn_fdot2(as_h2(v.w), one, s, false);
@@ -185,9 +193,18 @@ __device__ __forceinline__ void dot_word4(uint32_t w, const h2_t *p, float &lo, 
     hi = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), p[3], hi, false);
 }
 
+// the same for the first word of a chunk: its first two dots start the two accumulators
+__device__ __forceinline__ void dot_word4_first(uint32_t w, const h2_t *p, float &lo, float &hi) {
+    const uint32_t w8 = w >> 8;
+    lo = dot2_from_zero(as_h2(w & 0x000F000Fu), p[0]);
+    hi = dot2_from_zero(as_h2(w & 0x00F000F0u), p[1]);
+    lo = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), p[2], lo, false);
+    hi = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), p[3], hi, false);
+}
+
 __device__ __forceinline__ float dot_chunk4(const uint4 w, const XChunk4 &x) {
-    float lo = 0.0f, hi = 0.0f;
-    dot_word4(w.x, x.p + 0, lo, hi);
+    float lo, hi;
+    dot_word4_first(w.x, x.p + 0, lo, hi);
     dot_word4(w.y, x.p + 4, lo, hi);
     dot_word4(w.z, x.p + 8, lo, hi);
     dot_word4(w.w, x.p + 12, lo, hi);
@@ -203,8 +220,8 @@ __device__ __forceinline__ float dot_word8(uint32_t w, const h2_t *p, float acc)
 }
 
 __device__ __forceinline__ float dot_chunk8(const uint4 w, const XChunk8 &x) {
-    float acc = 0.0f;
-    acc = dot_word8(w.x, x.p + 0, acc);
+    float acc = dot2_from_zero(as_h2(__builtin_amdgcn_perm(0u, w.x, 0x0c010c00u)), x.p[0]);
+    acc = __builtin_amdgcn_fdot2(as_h2(__builtin_amdgcn_perm(0u, w.x, 0x0c030c02u)), x.p[1], acc, false);
     acc = dot_word8(w.y, x.p + 2, acc);
     acc = dot_word8(w.z, x.p + 4, acc);
     acc = dot_word8(w.w, x.p + 6, acc);

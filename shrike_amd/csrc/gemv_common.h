@@ -232,8 +232,8 @@ __device__ __forceinline__ float row_partial(const RowRegs<BITS, NCH, TAIL> &r, 
         acc = fmaf(meta_f32(r.b[i], meta), xs[i], acc);
     }
     if (TAIL) {
-        float lo = 0.0f, hi = 0.0f;
-        dot_word4(r.tw.x, xt.p, lo, hi);
+        float lo, hi;
+        dot_word4_first(r.tw.x, xt.p, lo, hi);
         dot_word4(r.tw.y, xt.p + 4, lo, hi);
         acc = fmaf(meta_f32(r.ts, meta), fmaf(lo, 16.0f, hi) * 1048576.0f, acc);
         acc = fmaf(meta_f32(r.tb, meta), xt.sum, acc);
