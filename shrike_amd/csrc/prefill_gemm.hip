@@ -474,9 +474,11 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     const uint32_t tile_total = DENSE ? (a.dense_rows + kRowTile - 1u) / kRowTile : *a.tile_count;
     const uint32_t w = blockIdx.y * gridDim.x + blockIdx.x;
     const uint32_t xcd = w & 7u, item = w >> 3;
-    const uint32_t run = (tile_total + 7u) / 8u;  // tiles an XCD takes
-    if (item / column_blocks >= run) return;
-    const uint32_t tile_index = xcd * run + item / column_blocks, col_block = item % column_blocks;
+    // tiles an XCD takes: an eighth of them, the first (total mod 8) XCDs one more
+    const uint32_t run = tile_total / 8u + (xcd < tile_total % 8u ? 1u : 0u), first = xcd * (tile_total / 8u) + min(xcd, tile_total % 8u);
+    const uint32_t place = item / column_blocks, col_block = item % column_blocks;  // the workgroup's place in its XCD's run
+    if (place >= run) return;
+    uint32_t tile_index = first + place;
     shrike_row_tile tile;
     if (DENSE) {
         if (tile_index >= tile_total) return;
@@ -486,7 +488,27 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
         tile.expert = 0;
     } else {
         if (tile_index >= tile_total) return;
-        tile = a.tiles[tile_index];
+        const uint32_t count = run;
+        if (count <= 64u) {
+            // Within the run, the tiles of more than 32 rows go first (each kind in table order): where a run holds more
+            // workgroups than its XCD has room for at once, the ones that start late are then the short ones. A lane reads one
+            // record of the run; the chosen one is read across.
+            const uint32_t lane = threadIdx.x & 63u;
+            const uint4 rec = lane < count ? reinterpret_cast<const uint4 *>(a.tiles)[first + lane] : zero4();
+            const uint64_t heavy = __ballot(lane < count && rec.z > 32u), light = __ballot(lane < count && rec.z <= 32u);
+            const uint32_t heavies = uint32_t(__popcll(heavy));
+            const uint64_t set = place < heavies ? heavy : light;
+            const uint32_t want = place < heavies ? place : place - heavies;
+            const bool mine = ((set >> lane) & 1ull) != 0ull && uint32_t(__popcll(set & ((1ull << lane) - 1ull))) == want;
+            const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)__ballot(mine)) - 1);
+            tile.cell = uint32_t(__builtin_amdgcn_readlane(int(rec.x), src));
+            tile.pair_start = uint32_t(__builtin_amdgcn_readlane(int(rec.y), src));
+            tile.rows = uint32_t(__builtin_amdgcn_readlane(int(rec.z), src));
+            tile.expert = uint32_t(__builtin_amdgcn_readlane(int(rec.w), src));
+            tile_index = first + uint32_t(src);
+        } else {
+            tile = a.tiles[tile_index];
+        }
         if (a.residency) {  // moe.metal:136-146: a hit names its cell, anything else is the sentinel
             const uint64_t word = a.residency[tile.expert];
             tile.cell = uint32_t(word >> 32) == SHRIKE_RESIDENCY_RESIDENT ? uint32_t(word) : kSentinel;
