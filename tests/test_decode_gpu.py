@@ -507,6 +507,25 @@ def test_decode_layer_matches_oracle_and_split_calls(gpu, cfg):
     assert np.array_equal(dl.y.download(np.uint16, d), y_fused)
 
 
+@pytest.mark.parametrize("ne,k,same", [(32, 4, 32), (64, 8, 64), (64, 8, 5), (256, 8, 256), (256, 8, 11), (40, 8, 40)])
+def test_decode_layer_ties_go_to_the_lower_index(gpu, ne, k, same):
+    """The fused layer's own select (every phase-1 wave and the workgroup that writes the lists select from the route table:
+    one entry a lane up to 64 experts, four sorted entries a lane above): `same` identical router rows give `same` equal
+    keys, and equal keys must come out in index order wherever they rank."""
+    L = Layer(0x71E5 + ne + same, 128, 64, ne, k)
+    L.router_w[:same] = L.router_w[0]
+    dl = DeviceLayer(gpu, L)
+    dl.moe.encode_decode_layer(dl.layer_args())
+    ref = oracle_layer(L, dl)
+    idx = dl.out_idx.download(np.uint32, k)
+    assert np.array_equal(idx, ref["indices"]), (idx, ref["indices"])
+    tied = [int(i) for i in idx if i < same]
+    assert tied == list(range(len(tied))), tied  # the lowest indices of the tied group, in order
+    assert np.array_equal(dl.resolved.download(np.uint32, k), ref["classify"]["resolved_slots"])
+    # the waves of phase 1 selected the same experts: their activations are the oracle's
+    assert_ffn_close(dl.acts.download(np.uint16, k * 64), ref["acts"], "acts")
+
+
 def test_decode_layer_is_deterministic(gpu):
     L = Layer(0x5EED0002, 2048, 512, 256, 8, shared_f=512)
     dl = DeviceLayer(gpu, L)
