@@ -118,7 +118,8 @@ __device__ __forceinline__ half8 b_step(const BRegs<BITS> &r, int s) {
 // tile's rows that the down product's bias term needs are formed here, in k_row_group_sums' order of additions (eight
 // lanes a group, a lane adds its eight values in order, the partial sums fold pairwise), instead of by a launch of
 // their own between the two products. Every wave of the workgroup stays to the end for the barriers.
-template <int BITS, int MODE, bool DENSE, uint32_t MT>
+// META: the type of the scales and biases (SHRIKE_META_*), known to the instance so that a scale converts one way.
+template <int BITS, int MODE, bool DENSE, uint32_t MT, int META>
 __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile &tile, uint32_t tile_index, uint32_t col_block,
                                          uint16_t (&s_a)[2][kRowTile][kLdsRow]) {
     const uint32_t K = MODE == 0 ? a.d : a.f, N = MODE == 0 ? a.f : a.d;
@@ -252,7 +253,7 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
             for (int s = 0; s < 4; ++s) bf[s] = b_step<BITS>(cur[nt], s);
             const uint32_t pair = gi < 2u ? scales_cur[nt].x : scales_cur[nt].y;
             const uint16_t scale_bits = WIDE ? uint16_t(pair >> (16u * (gi & 1u))) : cur[nt].scale;
-            const float sc = meta_f32(scale_bits, a.meta) * kTwo24;
+            const float sc = meta_f32(scale_bits, uint32_t(META)) * kTwo24;
 #pragma unroll
             for (uint32_t mt = 0; mt < MT; ++mt) {
                 f32x16 p = {0};
@@ -348,7 +349,7 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
 #pragma unroll
                     for (int jj = 0; jj < 4; ++jj) {  // the bias as fp16, doubled against (hi, lo)
                         uint16_t bits = uint16_t(bfr[step][nt].u[jj]);
-                        if (a.meta == SHRIKE_META_BF16) bits = f32_to_f16(bf16_to_f32(bits));
+                        if (META == SHRIKE_META_BF16) bits = f32_to_f16(bf16_to_f32(bits));
                         bfr[step][nt].u[jj] = uint32_t(bits) * 0x00010001u;
                     }
 #pragma unroll
@@ -461,7 +462,7 @@ __device__ __forceinline__ void ffn_tile(const FfnArgs &a, const shrike_row_tile
     }
 }
 
-template <int BITS, int MODE, bool DENSE>
+template <int BITS, int MODE, bool DENSE, int META>
 __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
     warm_kernel_arguments(a);
     __shared__ __align__(16) uint16_t s_a[2][kRowTile][kLdsRow];
@@ -517,23 +518,28 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
         if (tile.pair_start + tile.rows <= a.pair_lo || tile.pair_start >= a.pair_hi) return;
     }
 
-    if (tile.rows > 32u) ffn_tile<BITS, MODE, DENSE, 2>(a, tile, tile_index, col_block, s_a);
-    else ffn_tile<BITS, MODE, DENSE, 1>(a, tile, tile_index, col_block, s_a);
+    if (tile.rows > 32u) ffn_tile<BITS, MODE, DENSE, 2, META>(a, tile, tile_index, col_block, s_a);
+    else ffn_tile<BITS, MODE, DENSE, 1, META>(a, tile, tile_index, col_block, s_a);
 }
 
 int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uint32_t n, uint32_t *out,
                           const uint32_t *row_limit_tiles, hipStream_t s);
 
-template <int BITS, bool DENSE>
-static int launch_ffn(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
+template <int BITS, bool DENSE, int META>
+static int launch_ffn_meta(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
     const dim3 block(256);
     const uint32_t grid_tiles = (max_tiles + 7u) & ~7u;  // whole runs for the kernel's XCD mapping
-    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0, DENSE>), dim3(grid_tiles, (a.f + 127u) / 128u), block, 0, s, a);
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 0, DENSE, META>), dim3(grid_tiles, (a.f + 127u) / 128u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     // (the activations' group sums were written by the gate/up launch itself)
-    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1, DENSE>), dim3(grid_tiles, (a.d + 255u) / 256u), block, 0, s, a);
+    hipLaunchKernelGGL((k_grouped_ffn<BITS, 1, DENSE, META>), dim3(grid_tiles, (a.d + 255u) / 256u), block, 0, s, a);
     SHRIKE_HIP(hipGetLastError());
     return 0;
+}
+template <int BITS, bool DENSE>
+static int launch_ffn(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
+    return a.meta == SHRIKE_META_F16 ? launch_ffn_meta<BITS, DENSE, SHRIKE_META_F16>(a, max_tiles, s)
+                                     : launch_ffn_meta<BITS, DENSE, SHRIKE_META_BF16>(a, max_tiles, s);
 }
 
 struct Workspace {
