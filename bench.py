@@ -829,7 +829,8 @@ def decode_workload(args, rt, capi, S, meta):
     launch2_us = parts["launch 2: select + routed gate/up rows + shared down rows (k_phase1, routing)"]
     alone_us = parts["operator: phase 1 alone (no routing, no shared rows)"]
     value = expert_bytes / (ms_per_step * 1e-3) / 1e9
-    kernel = "k_phase1<4,1,4,true,4,true,false,1>"
+    meta_param = 1 if args.meta == "f16" else 0  # the kernels' last template parameter: SHRIKE_META_F16 = 1, SHRIKE_META_BF16 = 0
+    kernel = f"k_phase1<4,1,4,true,4,true,false,{meta_param}>"
     # The floor of the layer AS IT IS BUILT (three launches in a row, five dependent memory round trips: x and rows in
     # the first; the route table, then rows in the second; cells and activations, then rows in the third), from this
     # run's own probes: launches x an empty launch + round trips x one dependent load + the layer's bytes at the rate
@@ -866,7 +867,7 @@ def decode_workload(args, rt, capi, S, meta):
                      "frac": round(launch2_bytes / (launch2_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                      "bytes_per_launch": launch2_bytes, "us_per_launch": round(launch2_us, 3),
                      "traffic": profile_figure("decode_phase1_q35b_int4_hbm_traffic.txt", "hbm_bytes_per_launch"),
-                     "standalone_operator": {"kernel": "k_phase1<4,1,2,false,0,true,false,1> (gate/up rows alone: no routing, two row pairs a wave)", "bytes_per_launch": routed_gate_up,
+                     "standalone_operator": {"kernel": f"k_phase1<4,1,2,false,0,true,false,{meta_param}> (gate/up rows alone: no routing, two row pairs a wave)", "bytes_per_launch": routed_gate_up,
                                              "us_per_launch": round(alone_us, 3),
                                              "frac": round(routed_gate_up / (alone_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
                      "traffic_source": "profiles/decode_phase1_q35b_int4_hbm_traffic.txt (FETCH_SIZE + WRITE_SIZE of a profiled run "
