@@ -113,10 +113,10 @@ __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weig
                 uint32_t ww[ROWS][4];
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
+                    // the widening belongs to the multiply-add: keep it from being hoisted out of the token loop. The row's own
+                    // registers are named as changed (they are not), so that nothing is copied for it.
+                    asm volatile("" : "+v"(w[r][i].x), "+v"(w[r][i].y), "+v"(w[r][i].z), "+v"(w[r][i].w));
                     ww[r][0] = w[r][i].x; ww[r][1] = w[r][i].y; ww[r][2] = w[r][i].z; ww[r][3] = w[r][i].w;
-                    // the widening belongs to the multiply-add: keep it from being hoisted out of the token loop
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(ww[r][q]));
                 }
 #pragma unroll
                 for (uint32_t u = 0; u < TPS; ++u) {
