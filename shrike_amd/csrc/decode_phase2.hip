@@ -58,7 +58,10 @@ __global__ __launch_bounds__(512) void k_phase2(Phase2Args a) {
         return;
     }
     const uint32_t cpr = a.f * BITS / 128u, groups = a.f / kGroup, row_bytes = cpr * 16u;
-    const bool packed = cpr < 64u && (64u % cpr) == 0u;
+    // (an instance for rows of more than one step a lane never packs rows: its segment is the wave, and the segment sums'
+    // selects fold away)
+    constexpr bool kWholeWave = NCH >= 2 || TAIL;
+    const bool packed = !kWholeWave && cpr < 64u && (64u % cpr) == 0u;
     const uint32_t rpl = packed ? min(64u / cpr, kPhase2Rows) : 1u;  // rows per wave load
     const uint32_t seg = packed ? cpr : 64u;
     const uint32_t sub = packed ? lane / cpr : 0u, col = packed ? lane % cpr : lane;

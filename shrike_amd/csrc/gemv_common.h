@@ -277,7 +277,7 @@ __device__ __forceinline__ void gemv_job(const GemvArgs &a, uint32_t block, XSou
     typedef Chunk<BITS> C;
     const uint32_t lane = threadIdx.x & 63u, wave = wave_index();
     const uint32_t cpr = a.n * BITS / 128u, groups = a.n / kGroup, row_bytes = cpr * 16u;
-    const bool packed = cpr < 64u && (64u % cpr) == 0u;
+    const bool packed = NCH == 1 && cpr < 64u && (64u % cpr) == 0u;  // (NCH >= 2: more than 64 chunks a row, known to the instance)
     const uint32_t rpl = packed ? 64u / cpr : 1u;
     const uint32_t seg = packed ? cpr : 64u;
     const uint32_t sub = packed ? lane / cpr : 0u, col = packed ? lane % cpr : lane;
