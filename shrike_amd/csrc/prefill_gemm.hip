@@ -54,6 +54,7 @@ struct FfnArgs {
     uint32_t dense_rows;
     uint32_t round_gate_up;        // gate and up pass through fp16 before the GLU (dequant_int4.metal:206-287)
     const uint16_t *scalar_gate;   // fp16[rows] or null: row m's output * sigmoid(gate[m]) (moe.metal:1195-1207)
+    uint32_t resident_workgroups;  // workgroups of these kernels the device holds at once (two a compute unit)
 };
 
 union Frag {
@@ -489,12 +490,60 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
         tile.expert = 0;
     } else {
         if (tile_index >= tile_total) return;
+        // Which tile of the table the workgroup takes. A compute unit holds two of these workgroups, whose waves share its
+        // SIMDs' issue, and an XCD's workgroups reach its compute units in launch order, one each before any gets a second
+        // (read from the hardware: item i and item i + 32 of an XCD share a unit). A tile of more than 32 rows is twice a
+        // smaller one's matrix work, and the launch ends with the units that hold two of those.
+        //  - Where the gate/up launch fits the chip at once: every XCD takes the same number of the larger tiles (a block of
+        //    them in table order, so an expert's stay together) and fills its eighth with a block of the smaller ones; the
+        //    larger go first, so each gets a smaller neighbour.
+        //  - Otherwise the XCD's eighth is a contiguous run of the table, its larger tiles first: the workgroups that start
+        //    late are then the short ones, on the XCDs with the least work.
+        // A lane reads one record; the chosen one is read across (no second load).
+        const uint32_t lane = threadIdx.x & 63u;
+        const uint32_t gate_up_blocks = (a.f + 127u) / 128u;
+        bool chosen = false;
+        if (tile_total <= 256u && tile_total * gate_up_blocks <= a.resident_workgroups) {
+            uint4 rec[4];
+            uint64_t larger[4], smaller[4];
+            uint32_t larger_total = 0;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                const uint32_t idx = lane + 64u * j;
+                rec[j] = idx < tile_total ? reinterpret_cast<const uint4 *>(a.tiles)[idx] : zero4();
+                larger[j] = __ballot(idx < tile_total && rec[j].z > 32u);
+                smaller[j] = __ballot(idx < tile_total && rec[j].z <= 32u);
+                larger_total += uint32_t(__popcll(larger[j]));
+            }
+            const uint32_t lq = larger_total / 8u, lr = larger_total % 8u;
+            if (lq + 1u <= tile_total / 8u) {  // every XCD's share of the larger tiles fits its eighth
+                const uint32_t mine_larger = lq + (xcd < lr ? 1u : 0u), larger_first = xcd * lq + min(xcd, lr);
+                const bool take_larger = place < mine_larger;
+                uint32_t want = take_larger ? larger_first + place : (first - larger_first) + (place - mine_larger);
+                uint64_t set = 0;
+                uint32_t block = 0;
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) {
+                    const uint64_t m = take_larger ? larger[j] : smaller[j];
+                    const uint32_t c = uint32_t(__popcll(m));
+                    if (!chosen && want < c) { set = m; block = j; chosen = true; }
+                    else if (!chosen) want -= c;
+                }
+                if (chosen) {
+                    const bool me = ((set >> lane) & 1ull) != 0ull && uint32_t(__popcll(set & ((1ull << lane) - 1ull))) == want;
+                    const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)__ballot(me)) - 1);
+                    const uint4 pick = block == 0 ? rec[0] : block == 1 ? rec[1] : block == 2 ? rec[2] : rec[3];
+                    tile.cell = uint32_t(__builtin_amdgcn_readlane(int(pick.x), src));
+                    tile.pair_start = uint32_t(__builtin_amdgcn_readlane(int(pick.y), src));
+                    tile.rows = uint32_t(__builtin_amdgcn_readlane(int(pick.z), src));
+                    tile.expert = uint32_t(__builtin_amdgcn_readlane(int(pick.w), src));
+                    tile_index = 64u * block + uint32_t(src);
+                }
+            }
+        }
         const uint32_t count = run;
-        if (count <= 64u) {
-            // Within the run, the tiles of more than 32 rows go first (each kind in table order): where a run holds more
-            // workgroups than its XCD has room for at once, the ones that start late are then the short ones. A lane reads one
-            // record of the run; the chosen one is read across.
-            const uint32_t lane = threadIdx.x & 63u;
+        if (chosen) {
+        } else if (count <= 64u) {
             const uint4 rec = lane < count ? reinterpret_cast<const uint4 *>(a.tiles)[first + lane] : zero4();
             const uint64_t heavy = __ballot(lane < count && rec.z > 32u), light = __ballot(lane < count && rec.z <= 32u);
             const uint32_t heavies = uint32_t(__popcll(heavy));
@@ -540,6 +589,14 @@ template <int BITS, bool DENSE>
 static int launch_ffn(const FfnArgs &a, uint32_t max_tiles, hipStream_t s) {
     return a.meta == SHRIKE_META_F16 ? launch_ffn_meta<BITS, DENSE, SHRIKE_META_F16>(a, max_tiles, s)
                                      : launch_ffn_meta<BITS, DENSE, SHRIKE_META_BF16>(a, max_tiles, s);
+}
+
+// Two workgroups of the FFN kernels a compute unit (their registers and LDS allow no more).
+static uint32_t resident_ffn_workgroups() {
+    int device = 0, units = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
+        return 0;
+    return 2u * uint32_t(units);
 }
 
 struct Workspace {
@@ -603,6 +660,7 @@ static int grouped_ffn(shrike_hip_moe *moe, void *stream, const shrike_pool_base
     a.meta = moe->desc.meta_dtype;
     a.act_kind = moe->desc.activation;
     a.ebias = moe->desc.expert_additive_biases;
+    a.resident_workgroups = resident_ffn_workgroups();
     hipStream_t s = as_stream(stream);
     if (int rc = launch_row_group_sums(a.hidden, hidden_stride_elements, query_count, d, const_cast<uint32_t *>(a.hidden_sums), nullptr, s)) return rc;
     return moe->desc.routed_weight_bits == 8 ? launch_ffn<8, false>(a, max_row_tiles, s) : launch_ffn<4, false>(a, max_row_tiles, s);
