@@ -392,13 +392,14 @@ def prefill_workload(args, rt, capi, S, meta):
         router(lay); group(lay)
         us = timed(lambda _, lay=lay: ffn(lay), max(6, steps // 2), regions=3) * 1e3
         counts = routes.counts.download(np.uint32, NE)
-        # how the kernels deal the tiles: XCD x takes an eighth of them in table order (the first tiles mod 8 XCDs one more)
+        # the table's eighths (the first tiles mod 8 of them one tile longer): what an XCD takes where the launch does not fit the
+        # chip at once; where it does, the kernels even out the tiles of more than 32 rows over the XCDs
         tile_rows = routes.download()["row_tiles"][:, 2]
         q, r = divmod(len(tile_rows), 8)
         starts = [x * q + min(x, r) for x in range(9)]
         by_layer.append({"us": round(us, 2), "row_tiles": int(routes.row_tile_count.download(np.uint32, 1)[0]),
-                         "tiles_by_xcd": [starts[x + 1] - starts[x] for x in range(8)],
-                         "tiles_over_32_rows_by_xcd": [int(np.count_nonzero(tile_rows[starts[x]:starts[x + 1]] > 32)) for x in range(8)],
+                         "tiles_by_table_eighth": [starts[x + 1] - starts[x] for x in range(8)],
+                         "tiles_over_32_rows_by_table_eighth": [int(np.count_nonzero(tile_rows[starts[x]:starts[x + 1]] > 32)) for x in range(8)],
                          "experts_with_pairs": int(np.count_nonzero(counts)),
                          "mfma_row_tiles_of_32": int(sum((min(64, c - j) + 31) // 32 for c in counts.tolist() for j in range(0, c, 64)))})
     quoted = sorted(by_layer, key=lambda r: r["us"])[len(by_layer) // 2]
