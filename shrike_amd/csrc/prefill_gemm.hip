@@ -504,39 +504,47 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
         const uint32_t gate_up_blocks = (a.f + 127u) / 128u;
         bool chosen = false;
         if (tile_total <= 256u && tile_total * gate_up_blocks <= a.resident_workgroups) {
-            uint4 rec[4];
-            uint64_t larger[4], smaller[4];
-            uint32_t larger_total = 0;
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) {
-                const uint32_t idx = lane + 64u * j;
-                rec[j] = idx < tile_total ? reinterpret_cast<const uint4 *>(a.tiles)[idx] : zero4();
-                larger[j] = __ballot(idx < tile_total && rec[j].z > 32u);
-                smaller[j] = __ballot(idx < tile_total && rec[j].z <= 32u);
-                larger_total += uint32_t(__popcll(larger[j]));
-            }
+            // (four named records, not an array: the compiler kept an array of them in private memory)
+            const uint4 *table = reinterpret_cast<const uint4 *>(a.tiles);
+            const uint4 rec0 = lane < tile_total ? table[lane] : zero4();
+            const uint4 rec1 = lane + 64u < tile_total ? table[lane + 64u] : zero4();
+            const uint4 rec2 = lane + 128u < tile_total ? table[lane + 128u] : zero4();
+            const uint4 rec3 = lane + 192u < tile_total ? table[lane + 192u] : zero4();
+            const bool in0 = lane < tile_total, in1 = lane + 64u < tile_total, in2 = lane + 128u < tile_total, in3 = lane + 192u < tile_total;
+            const uint64_t larger0 = __ballot(in0 && rec0.z > 32u), larger1 = __ballot(in1 && rec1.z > 32u);
+            const uint64_t larger2 = __ballot(in2 && rec2.z > 32u), larger3 = __ballot(in3 && rec3.z > 32u);
+            const uint64_t smaller0 = __ballot(in0 && rec0.z <= 32u), smaller1 = __ballot(in1 && rec1.z <= 32u);
+            const uint64_t smaller2 = __ballot(in2 && rec2.z <= 32u), smaller3 = __ballot(in3 && rec3.z <= 32u);
+            const uint32_t larger_total = uint32_t(__popcll(larger0) + __popcll(larger1) + __popcll(larger2) + __popcll(larger3));
             const uint32_t lq = larger_total / 8u, lr = larger_total % 8u;
             if (lq + 1u <= tile_total / 8u) {  // every XCD's share of the larger tiles fits its eighth
                 const uint32_t mine_larger = lq + (xcd < lr ? 1u : 0u), larger_first = xcd * lq + min(xcd, lr);
                 const bool take_larger = place < mine_larger;
                 uint32_t want = take_larger ? larger_first + place : (first - larger_first) + (place - mine_larger);
-                uint64_t set = 0;
-                uint32_t block = 0;
-#pragma unroll
-                for (uint32_t j = 0; j < 4; ++j) {
-                    const uint64_t m = take_larger ? larger[j] : smaller[j];
-                    const uint32_t c = uint32_t(__popcll(m));
-                    if (!chosen && want < c) { set = m; block = j; chosen = true; }
-                    else if (!chosen) want -= c;
-                }
+                const uint64_t m0 = take_larger ? larger0 : smaller0, m1 = take_larger ? larger1 : smaller1;
+                const uint64_t m2 = take_larger ? larger2 : smaller2, m3 = take_larger ? larger3 : smaller3;
+                const uint32_t c0 = uint32_t(__popcll(m0)), c1 = uint32_t(__popcll(m1)), c2 = uint32_t(__popcll(m2)), c3 = uint32_t(__popcll(m3));
+                uint64_t set;
+                uint32_t block;
+                if (want < c0) { set = m0; block = 0; }
+                else if (want < c0 + c1) { set = m1; block = 1; want -= c0; }
+                else if (want < c0 + c1 + c2) { set = m2; block = 2; want -= c0 + c1; }
+                else { set = m3; block = 3; want -= c0 + c1 + c2; }
+                chosen = want < uint32_t(__popcll(set));
                 if (chosen) {
                     const bool me = ((set >> lane) & 1ull) != 0ull && uint32_t(__popcll(set & ((1ull << lane) - 1ull))) == want;
                     const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)__ballot(me)) - 1);
-                    const uint4 pick = block == 0 ? rec[0] : block == 1 ? rec[1] : block == 2 ? rec[2] : rec[3];
-                    tile.cell = uint32_t(__builtin_amdgcn_readlane(int(pick.x), src));
-                    tile.pair_start = uint32_t(__builtin_amdgcn_readlane(int(pick.y), src));
-                    tile.rows = uint32_t(__builtin_amdgcn_readlane(int(pick.z), src));
-                    tile.expert = uint32_t(__builtin_amdgcn_readlane(int(pick.w), src));
+                    auto take = [&](const uint4 &r) {  // (a branch a block, uniform: a select between the four records became an
+                                                       // indexed load from private memory)
+                        tile.cell = uint32_t(__builtin_amdgcn_readlane(int(r.x), src));
+                        tile.pair_start = uint32_t(__builtin_amdgcn_readlane(int(r.y), src));
+                        tile.rows = uint32_t(__builtin_amdgcn_readlane(int(r.z), src));
+                        tile.expert = uint32_t(__builtin_amdgcn_readlane(int(r.w), src));
+                    };
+                    if (block == 0) take(rec0);
+                    else if (block == 1) take(rec1);
+                    else if (block == 2) take(rec2);
+                    else take(rec3);
                     tile_index = 64u * block + uint32_t(src);
                 }
             }
