@@ -41,6 +41,26 @@ __global__ __launch_bounds__(256) void k_prefill_logits(RouterArgs a, uint32_t q
 // step's in flight while one is multiplied) for the four waves to read, and the TPS * ROWS sums of a step
 // go through the butterfly side by side. Every logit is summed in the decode router's order (lane l:
 // chunks l, l+64, ..., xor butterfly).
+// One stage of the split butterfly over LIVE sums (a power of two above 1) at lane distance 32 >> STAGE: the partner with
+// the distance's bit set keeps the upper half of the sums and sends the lower, the other the reverse; each adds the
+// partner's copy of what it keeps. LIVE / 2 sums are left in v[0 .. LIVE / 2).
+template <uint32_t LIVE, uint32_t STAGE>
+__device__ __forceinline__ void split_stage(float *v, uint32_t lane) {
+    constexpr int kDistance = 32 >> STAGE;
+    const bool upper = (lane & uint32_t(kDistance)) != 0u;
+#pragma unroll
+    for (uint32_t j = 0; j < LIVE / 2u; ++j) {
+        const float keep = upper ? v[j + LIVE / 2u] : v[j], send = upper ? v[j] : v[j + LIVE / 2u];
+        v[j] = __fadd_rn(keep, __shfl_xor(send, kDistance));
+    }
+}
+template <uint32_t SUMS, uint32_t STAGES>
+__device__ __forceinline__ void split_stages(float *v, uint32_t lane) {
+    if constexpr (STAGES >= 1u) split_stage<SUMS, 0>(v, lane);
+    if constexpr (STAGES >= 2u) split_stage<SUMS / 2u, 1>(v, lane);
+    if constexpr (STAGES >= 3u) split_stage<SUMS / 4u, 2>(v, lane);
+}
+
 template <int MAXI, int ROWS, uint32_t TOKENS, uint32_t TPS>
 __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weights, const uint16_t *hidden, uint32_t stride,
                                                             const uint16_t *eff, float *logits, uint32_t query_count,
@@ -142,23 +162,11 @@ __global__ __launch_bounds__(256) void k_prefill_logits_f16(const uint16_t *weig
         for (uint32_t u = 0; u < TPS; ++u)
 #pragma unroll
             for (int r = 0; r < ROWS; ++r) v[u * ROWS + r] = acc[u][r];
-        uint32_t live = kSums;  // sums this lane still carries: v[0 .. live)
+        // (every index below is a constant: with the number of live sums in a variable the compiler kept v in private memory)
+        constexpr uint32_t kSplitStages = kSums == 8u ? 3u : kSums == 4u ? 2u : kSums == 2u ? 1u : 0u;
+        split_stages<kSums, kSplitStages>(v, lane);
 #pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) {
-            if (live > 1u) {
-                const bool upper = (lane & uint32_t(o)) != 0u;  // the upper partner keeps the upper half of the sums
-                live >>= 1;
-#pragma unroll
-                for (uint32_t j = 0; j < kSums / 2u; ++j) {
-                    if (j < live) {
-                        const float keep = upper ? v[j + live] : v[j], send = upper ? v[j] : v[j + live];
-                        v[j] = __fadd_rn(keep, __shfl_xor(send, o));
-                    }
-                }
-            } else {
-                v[0] = __fadd_rn(v[0], __shfl_xor(v[0], o));
-            }
-        }
+        for (int o = 32 >> kSplitStages; o >= 1; o >>= 1) v[0] = __fadd_rn(v[0], __shfl_xor(v[0], o));
         // which sum this lane holds: one bit a split, from the first split (xor 32) down
         constexpr uint32_t kSplits = kSums == 8u ? 3u : kSums == 4u ? 2u : kSums == 2u ? 1u : 0u;
         const uint32_t mine = kSplits ? lane >> (6u - kSplits) : 0u;
