@@ -10,9 +10,11 @@ addresses (18 GB, far past the 256 MB Infinity Cache), and the activation vector
 over four variants so that a layer picks other experts from one pass to the next: every
 step streams its experts from HBM. Runs of layers are captured in HIP graphs.
 
-Timing: W warm-up steps, then REGIONS regions of exactly K steps each, every region
-bracketed by HIP events on the launch stream; `ms_per_step` is the median region / K
-(minimum and maximum are reported beside it).
+Timing: W warm-up steps, then REGIONS regions of exactly K steps each in one captured
+graph, the device clock stored by a one-thread kernel between regions (HIP events on the
+launch stream bracket the whole graph as the cross-check, and bracket every region where
+the clock is not to be had); `ms_per_step` is the median region / K (minimum and maximum
+are reported beside it, and what two stamps with nothing between them measure).
 
 Prints ONE JSON line. `value` is expert bytes read per second (8 routed + 1 shared
 expert = 15,925,248 B per step) with all inputs resident in HBM. `roofline` prices the
@@ -675,7 +677,7 @@ def decode_workload(args, rt, capi, S, meta):
     walk = LayerWalk(rt, capi, moe, stream, layers)
     walk.plan(warm, 1)
     walk.enqueue(warm)
-    region_ms, timing_method, whole_graph_us = None, None, None
+    region_ms, timing_method, whole_graph_us, empty_region_us = None, None, None, None
     from harness import probes as _probes
     clock_khz = _probes.load().shrike_probe_wall_clock_khz()
     if args.timing == "graph" and clock_khz > 0:
@@ -684,13 +686,16 @@ def decode_workload(args, rt, capi, S, meta):
         # graph launch per region bills every region a launch boundary of its own (about 19 us on this part, which a
         # 20-layer region feels). HIP events cannot do this: an event recorded by a captured graph cannot be timed
         # (hipEventElapsedTime: invalid resource handle). Events still bracket the whole graph as the cross-check.
-        stamps = rt.empty(8 * (REGIONS + 1)).fill(0)
+        # One more stamp follows the last region's at once: the two bracket nothing, which is what a region holds besides
+        # its K layers (reported as "empty_region_us", not subtracted).
+        stamps = rt.empty(8 * (REGIONS + 2)).fill(0)
 
         def regions_body():
             _probes.check(_probes.load().shrike_probe_timestamp(stream.handle, stamps.ptr), "probe_timestamp")
             for r in range(REGIONS):
                 walk.encode(steps)
                 _probes.check(_probes.load().shrike_probe_timestamp(stream.handle, stamps.ptr + 8 * (r + 1)), "probe_timestamp")
+            _probes.check(_probes.load().shrike_probe_timestamp(stream.handle, stamps.ptr + 8 * (REGIONS + 1)), "probe_timestamp")
         timed = capture(rt, capi, stream, regions_body)
         first, last = rt.Event(), rt.Event()
         stream.synchronize()
@@ -700,8 +705,9 @@ def decode_workload(args, rt, capi, S, meta):
         last.record(stream)
         last.synchronize()
         rt.synchronize()
-        ticks = stamps.download(np.uint64, REGIONS + 1).astype(np.int64)
+        ticks = stamps.download(np.uint64, REGIONS + 2).astype(np.int64)
         region_ms = [float(ticks[r + 1] - ticks[r]) / clock_khz for r in range(REGIONS)]
+        empty_region_us = float(ticks[REGIONS + 1] - ticks[REGIONS]) / clock_khz * 1e3
         whole_graph_us = first.elapsed_ms(last) * 1e3 / (REGIONS * steps)
         capi.check(capi.load().shrike_hip_graph_destroy(timed), "graph_destroy")
         timing_method = (f"one captured graph of {REGIONS} regions of K layers, the device clock ({clock_khz} kHz) stored by a "
@@ -864,7 +870,8 @@ def decode_workload(args, rt, capi, S, meta):
         "timing": {"regions": REGIONS, "steps_per_region": steps, "statistic": "median", "method": timing_method,
                    "us_per_layer_min": round(min(region_ms) / steps * 1e3, 3),
                    "us_per_layer_max": round(max(region_ms) / steps * 1e3, 3),
-                   **({"us_per_layer_by_hip_events_round_all_regions": round(whole_graph_us, 3)} if whole_graph_us else {})},
+                   **({"us_per_layer_by_hip_events_round_all_regions": round(whole_graph_us, 3)} if whole_graph_us else {}),
+                   **({"empty_region_us": round(empty_region_us, 3)} if empty_region_us is not None else {})},
         "hbm_peak_frac_on_expert_bytes": round(value / HBM_PEAK_GBPS, 4),
         "expert_bytes_per_step": expert_bytes, "total_bytes_per_step": total_bytes,
         "kernel_us_per_layer": {k: round(v, 3) for k, v in parts.items()},
