@@ -392,14 +392,17 @@ def prefill_workload(args, rt, capi, S, meta):
     by_layer = []
     for lay in layers:
         router(lay); group(lay)
-        us = timed(lambda _, lay=lay: ffn(lay), max(6, steps // 2), regions=3) * 1e3
+        # these routes over every layer's pool in turn (an expert sits in the same cell of each), so that the experts
+        # come from HBM as in the chunk above and not from the Infinity Cache, which holds one layer's experts whole
+        us = timed(ffn, max(6, steps // 2), regions=3) * 1e3
+        us_one_pool = timed(lambda _, lay=lay: ffn(lay), max(6, steps // 2), regions=3) * 1e3
         counts = routes.counts.download(np.uint32, NE)
         # the table's eighths (the first tiles mod 8 of them one tile longer): what an XCD takes where the launch does not fit the
         # chip at once; where it does, the kernels even out the tiles of more than 32 rows over the XCDs
         tile_rows = routes.download()["row_tiles"][:, 2]
         q, r = divmod(len(tile_rows), 8)
         starts = [x * q + min(x, r) for x in range(9)]
-        by_layer.append({"us": round(us, 2), "row_tiles": int(routes.row_tile_count.download(np.uint32, 1)[0]),
+        by_layer.append({"us": round(us, 2), "us_on_one_pool_over_and_over": round(us_one_pool, 2), "row_tiles": int(routes.row_tile_count.download(np.uint32, 1)[0]),
                          "tiles_by_table_eighth": [starts[x + 1] - starts[x] for x in range(8)],
                          "tiles_over_32_rows_by_table_eighth": [int(np.count_nonzero(tile_rows[starts[x]:starts[x + 1]] > 32)) for x in range(8)],
                          "experts_with_pairs": int(np.count_nonzero(counts)),
