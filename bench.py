@@ -959,7 +959,7 @@ def main():
             gc.collect()
             r = run()
             secondary[name] = {k: r[k] for k in r if k in ("metric", "value", "unit", "ms_per_step", "us_per_layer", "config",
-                                                           "kernel_us_per_chunk", "roofline", "GBps_on_pair_bytes",
+                                                           "kernel_us_per_chunk", "grouped_ffn_by_layer_routes", "roofline", "GBps_on_pair_bytes",
                                                            "hbm_peak_frac_on_expert_bytes", "miss_rate", "host_to_device_GBps", "hit_only_kernel_ms", "hit_only",
                                                            "timeline_ms_per_step", "copy_ms_hidden_behind_compute", "miss_rate_by_policy", "miss_rate_floor",
                                                            "bytes_copied_per_step", "experts_requested_per_step", "steps", "dtype", "cpu_baseline")}
