@@ -910,7 +910,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=80)
     ap.add_argument("--layers", type=int, default=40, help="stacked layers with their own pools (40 x 453 MB)")
     ap.add_argument("--meta", choices=["f16", "bf16"], default="f16")
-    ap.add_argument("--cpu-sample", type=int, default=60, help="layer evaluations timed on the CPU (0 = skip)")
+    ap.add_argument("--cpu-sample", type=int, default=3000, help="layer evaluations timed on the CPU, about ten seconds of host work (0 = skip)")
     ap.add_argument("--no-shared", action="store_true", help="diagnostic: leave the shared expert out of the layer")
     ap.add_argument("--no-secondary", action="store_true", help="the headline workload alone")
     ap.add_argument("--timing", choices=["graph", "launches"], default="graph",
