@@ -148,7 +148,10 @@ int shrike_hip_pool_fetch_experts(shrike_hip_pool *pool, void *stream, shrike_ex
 
 /* ------------------------------------------------------------ MoE operators */
 
-/* MoE.init, sources/Shrike/Kernels/MoE/MoE.swift:94-216. */
+/* MoE.init, sources/Shrike/Kernels/MoE/MoE.swift:94-216.
+ * Sizes the decode operators take (anything else is EINVAL with a message, never a launch): d and f multiples of 64,
+ * d <= SHRIKE_MAX_HIDDEN, and a row of f codes at most 4,096 bytes (f <= 8,192 at 4 bits, f <= 4,096 at 8 bits);
+ * num_experts <= SHRIKE_MAX_ROUTER_EXPERTS, top_k <= SHRIKE_MAX_TOP_K. */
 typedef struct {
     uint32_t d, f, num_experts, top_k;
     uint32_t routed_weight_bits;   /* 4 | 8 */
