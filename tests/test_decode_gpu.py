@@ -223,12 +223,12 @@ def test_phase1_phase2_against_oracle(gpu, bits, meta, d, f):
 
 
 def _swept_shapes():
-    """Sixteen shapes drawn once from a fixed seed: hidden and intermediate sizes any multiple of 64 up to 2,560
+    """Ninety-six shapes drawn once from a fixed seed: hidden and intermediate sizes any multiple of 64 up to 2,560
     (rows of 1 to 160 sixteen-byte chunks: every chunks-per-lane count, whole and ragged waves, rows shorter than
     a wave load), 1 to 8 routed positions, both code widths and both metadata types."""
     rng = np.random.default_rng(0x5EED5EED)
     out = []
-    for _ in range(16):
+    for _ in range(96):
         d, f = (int(64 * rng.integers(1, 41)) for _ in range(2))
         out.append((d, f, int(rng.integers(1, 9)), int(rng.choice([4, 8])), int(rng.choice([S.META_BF16, S.META_F16]))))
     return out
@@ -505,6 +505,29 @@ def test_decode_layer_matches_oracle_and_split_calls(gpu, cfg):
     dl.moe.encode_spec_phase2(dl.pool, dl.resolved, dl.off, dl.acts, dl.out_w, residual, dl.y, dl.hidden, d, f, k)
     assert np.array_equal(dl.acts.download(np.uint16, k * f), acts_fused)
     assert np.array_equal(dl.y.download(np.uint16, d), y_fused)
+
+
+def _swept_layer_configs():
+    """Forty configurations of the fused layer drawn once from a fixed seed: 4 to 256 experts, 1 to 8 positions, sizes any
+    multiple of 64 up to 2,048, the three router widths, with and without a shared expert, both code widths and both
+    metadata types."""
+    rng = np.random.default_rng(0x5EED7A7E)
+    out = []
+    for i in range(40):
+        d, f = (int(64 * rng.integers(1, 33)) for _ in range(2))
+        ne = int(rng.choice([4, 8, 16, 24, 32, 40, 64, 100, 128, 160, 256]))
+        k = int(rng.integers(1, min(ne, 8) + 1))
+        bits, meta = int(rng.choice([4, 8])), int(rng.choice([S.META_BF16, S.META_F16]))
+        rbits, fs = int(rng.choice([0, 4, 8])), int(rng.choice([0, 64, 256, 512, 1024]))
+        if d * f * ne > 150_000_000:  # keep the synthetic pool small: the routes then go over eight experts
+            ne = max(k, 8)
+        out.append((f"sweep-{i}-d{d}-f{f}-e{ne}-k{k}", d, f, ne, k, bits, meta, rbits, fs))
+    return out
+
+
+@pytest.mark.parametrize("cfg", _swept_layer_configs(), ids=[c[0] for c in _swept_layer_configs()])
+def test_decode_layer_config_sweep(gpu, cfg):
+    test_decode_layer_matches_oracle_and_split_calls(gpu, cfg)
 
 
 @pytest.mark.parametrize("ne,k,same", [(32, 4, 32), (64, 8, 64), (64, 8, 5), (256, 8, 256), (256, 8, 11), (40, 8, 40)])

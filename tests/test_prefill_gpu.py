@@ -206,12 +206,12 @@ def test_grouped_ffn_against_oracle(gpu, case):
 
 
 def _swept_ffn_cases():
-    """Ten chunks drawn once from a fixed seed: hidden and intermediate sizes any multiple of 64 up to 1,536 (column blocks
+    """Sixty chunks drawn once from a fixed seed: hidden and intermediate sizes any multiple of 64 up to 1,536 (column blocks
     that end inside a workgroup's 128 or 256 columns, k that ends inside a staged chunk of 256, group counts that are not
     multiples of four), 1 to 150 tokens over 2 to 20 experts (row tiles of one row, of 32, of 33, of 64 and more)."""
     rng = np.random.default_rng(0x5EEDFF)
     out = []
-    for i in range(10):
+    for i in range(60):
         d, f = (int(64 * rng.integers(1, 25)) for _ in range(2))
         ne = int(rng.integers(2, 21))
         k = int(rng.integers(1, min(ne, 8) + 1))
