@@ -354,14 +354,19 @@ def prefill_workload(args, rt, capi, S, meta):
     partials, h2 = rt.empty(2 * T * K * D), rt.empty(2 * T * D)
     work = rt.empty(pf.ffn_workspace_bytes(T, routes.max_row_tiles))
 
+    # the router's pass over `hidden` also leaves the group sums that the FFN's bias term needs (one launch fewer a chunk);
+    # --prefill-two-passes: each of the two reads `hidden` for itself, as the reference's operators do
+    fused_sums = not getattr(args, "prefill_two_passes", False)
+
     def router(lay):
-        pf.encode_block(lay["router"], None, None, hidden, ones_d, ones_e, d_bias, idx, w, logits, T, NE, D, K, D)
+        pf.encode_block(lay["router"], None, None, hidden, ones_d, ones_e, d_bias, idx, w, logits, T, NE, D, K, D,
+                        ffn_workspace=work if fused_sums else None)
 
     def group(lay):
         pf.group_pairs(idx, w, T, K, NE, routes, residency=lay["pool"].table)
 
     def ffn(lay):
-        pf.encode_grouped_expert_gemms(lay["pool"], off, routes, hidden, D, partials, work, T, K)
+        pf.encode_grouped_expert_gemms(lay["pool"], off, routes, hidden, D, partials, work, T, K, presummed=fused_sums)
 
     def reduce(lay):
         pf.encode_reduce_token_major(partials, w, h2, T, K, D)
@@ -408,13 +413,14 @@ def prefill_workload(args, rt, capi, S, meta):
                          "experts_with_pairs": int(np.count_nonzero(counts)),
                          "mfma_row_tiles_of_32": int(sum((min(64, c - j) + 31) // 32 for c in counts.tolist() for j in range(0, c, 64)))})
     quoted = sorted(by_layer, key=lambda r: r["us"])[len(by_layer) // 2]
+    ffn_name = "grouped FFN (2 launches)" if fused_sums else "grouped FFN (3 launches)"
     parts = {"router (2 launches)": parts["router (2 launches)"], "grouping (1 launch)": parts["grouping (1 launch)"],
-             "grouped FFN (3 launches)": quoted["us"], "reduce": parts["reduce"]}
+             ffn_name: quoted["us"], "reduce": parts["reduce"]}
     tiles, used, m_tiles = quoted["row_tiles"], quoted["experts_with_pairs"], quoted["mfma_row_tiles_of_32"]
     expert_bytes = used * stride
     algorithmic = expert_bytes + 2 * T * D * 2 + T * K * 16
     flops = T * K * 6 * D * F
-    ffn_us = parts["grouped FFN (3 launches)"]
+    ffn_us = parts[ffn_name]
     traffic = profile_figure("prefill_chunk_q35b_int4_t512.txt", "hbm_bytes_per_chunk_grouped_ffn") if T == 512 else None
     # What a SIMD makes of matrix and vector instructions side by side, at the FFN kernels' two waves a SIMD: a slot of
     # four 32x32x16 matrix instructions, a slot of thirty-two fused multiply-adds, and both (the FFN's main loop issues
@@ -923,6 +929,8 @@ def main():
                          "(config 5) alone")
     ap.add_argument("--bits", type=int, choices=[4, 8], default=4, help="gptoss: code width")
     ap.add_argument("--tokens", type=int, default=512, help="prefill: tokens in the chunk")
+    ap.add_argument("--prefill-two-passes", action="store_true",
+                    help="prefill diagnostic: the router and the grouped FFN each read the hidden rows for themselves")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path is built and measured on a single MI355X "

@@ -448,6 +448,16 @@ struct PrefillRouter {
         check(shrike_hip_prefill_router(moe.handle(), s, weights, scales, biases, hidden, effectiveScale, perExpertScale, logitBias,
                                         outIndices, outWeights, workspace, queryCount, numExperts, d, topK, hiddenStrideElements));
     }
+    // the same, leaving the group sums of `hidden` at the head of the grouped FFN's workspace (no counterpart in the
+    // reference: a runner that hands both operators the same rows reads them once)
+    static void encodeBlockWithGroupSums(MoE &moe, Stream s, const void *weights, const void *scales, const void *biases, const void *hidden,
+                                         const void *effectiveScale, const void *perExpertScale, const void *logitBias, uint32_t *outIndices,
+                                         void *outWeights, float *workspace, uint32_t queryCount, uint32_t numExperts, uint32_t d,
+                                         uint32_t topK, uint32_t hiddenStrideElements, void *ffnWorkspace) {
+        check(shrike_hip_prefill_router_with_group_sums(moe.handle(), s, weights, scales, biases, hidden, effectiveScale, perExpertScale,
+                                                        logitBias, outIndices, outWeights, workspace, queryCount, numExperts, d, topK,
+                                                        hiddenStrideElements, ffnWorkspace));
+    }
     static std::vector<shrike_token_expert_pair> makeTokenExpertPairs(const std::vector<uint32_t> &indices, const std::vector<uint16_t> &weights,
                                                                       uint32_t queryCount, uint32_t topK) {
         if (indices.size() != size_t(queryCount) * topK || weights.size() != indices.size()) throw Error(EINVAL, "indices count mismatch");
@@ -570,6 +580,15 @@ struct PrefillGroupedRoutedMoE {
                                          uint32_t queryCount, uint32_t d, uint32_t f, uint32_t topK) {
         check(shrike_hip_prefill_grouped_ffn(moe.handle(), s, pool.bases(), pool.stride(), &offsets, &routes, maxRowTiles, hidden,
                                              hiddenStrideElements, routePartials, workspace, workspaceSize, queryCount, d, f, topK));
+    }
+    // the same for a workspace whose head holds the group sums PrefillRouter::encodeBlockWithGroupSums left there
+    static void encodeGroupedExpertGEMMsPresummed(MoE &moe, Stream s, const ExpertPool &pool, const shrike_expert_offsets &offsets,
+                                                  const shrike_hip_grouped_routes &routes, uint32_t maxRowTiles, const void *hidden,
+                                                  uint32_t hiddenStrideElements, void *routePartials, void *workspace, size_t workspaceSize,
+                                                  uint32_t queryCount, uint32_t d, uint32_t f, uint32_t topK) {
+        check(shrike_hip_prefill_grouped_ffn_presummed(moe.handle(), s, pool.bases(), pool.stride(), &offsets, &routes, maxRowTiles,
+                                                       hidden, hiddenStrideElements, routePartials, workspace, workspaceSize, queryCount,
+                                                       d, f, topK));
     }
     // encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:846-922): the sorted pairs [pairStart, pairStart + pairCount)
     // against `residency` (device table, or null for the cells recorded at grouping); returns the microbatch count

@@ -388,6 +388,20 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
                               void *d_out_weights, float *d_workspace,
                               uint32_t query_count, uint32_t num_experts, uint32_t d,
                               uint32_t top_k, uint32_t hidden_stride_elements);
+/* The same call, which also leaves at the head of d_ffn_workspace (the grouped FFN's workspace for this chunk, 256-byte
+ * aligned) what that FFN first derives from `hidden`: per token and group of 64 elements the fp32 sum, as the FFN's own
+ * pass forms it bit for bit. The reference has no such pair of calls: its router (PrefillRouter.swift:75-152) and its
+ * grouped GEMMs (PrefillGroupedRoutedMoE.swift:925-1126) each read `hidden` for themselves, and so do the two entry
+ * points above and below; this one and shrike_hip_prefill_grouped_ffn_presummed let a runner that hands both the same
+ * `hidden` read it once (one launch fewer a chunk). Routes and logits are those of shrike_hip_prefill_router. */
+int shrike_hip_prefill_router_with_group_sums(shrike_hip_moe *moe, void *stream, const void *d_weights,
+                                              const void *d_scales, const void *d_biases, const void *d_hidden,
+                                              const void *d_effective_scale, const void *d_per_expert_scale,
+                                              const void *d_logit_bias, uint32_t *d_out_indices,
+                                              void *d_out_weights, float *d_workspace,
+                                              uint32_t query_count, uint32_t num_experts, uint32_t d,
+                                              uint32_t top_k, uint32_t hidden_stride_elements,
+                                              void *d_ffn_workspace);
 
 /* One 64-row tile of one expert's pairs: the unit the grouped FFN's workgroups take
  * (the device form of PrefillRoutedExpertBlock + rowTileTable,
@@ -439,6 +453,15 @@ int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shri
                                    const void *d_hidden, uint32_t hidden_stride_elements,
                                    void *d_route_partials, void *d_workspace, size_t workspace_bytes,
                                    uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k);
+/* shrike_hip_prefill_grouped_ffn for a d_workspace whose head already holds the group sums of these query_count rows of
+ * `hidden` (shrike_hip_prefill_router_with_group_sums on the same stream, same hidden, same d): the same bytes out, without
+ * the pass over `hidden` that forms them. */
+int shrike_hip_prefill_grouped_ffn_presummed(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                             uint64_t pool_slot_stride, const shrike_expert_offsets *offsets,
+                                             const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles,
+                                             const void *d_hidden, uint32_t hidden_stride_elements,
+                                             void *d_route_partials, void *d_workspace, size_t workspace_bytes,
+                                             uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k);
 
 /* PrefillGroupedRoutedMoE.encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:846-922; kernels
  * prefill_moe_affine_gemv_row_dev and its batched phases, prefill.metal:318-363, :647-728): the

@@ -363,6 +363,8 @@ SIGNATURES = {
     # prefill operators
     "shrike_hip_prefill_router": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                             _U32, _U32, _U32, _U32, _U32]),
+    "shrike_hip_prefill_router_with_group_sums": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
+                                                            _U32, _U32, _U32, _U32, _U32, _VP]),
     "shrike_hip_prefill_router_workspace_bytes": (C.c_size_t, [_U32, _U32, _U32]),
     "shrike_hip_group_max_row_tiles": (_U32, [_U64, _U32]),
     "shrike_hip_group_pairs": (C.c_int, [_VP, _VP, _VP, _U32, _U32, _U32, _VP, _VP, C.POINTER(HipGroupedRoutes)]),
@@ -370,6 +372,9 @@ SIGNATURES = {
     "shrike_hip_prefill_grouped_ffn": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, C.POINTER(ExpertOffsets),
                                                  C.POINTER(HipGroupedRoutes), _U32, _VP, _U32, _VP, _VP, C.c_size_t,
                                                  _U32, _U32, _U32, _U32]),
+    "shrike_hip_prefill_grouped_ffn_presummed": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, C.POINTER(ExpertOffsets),
+                                                           C.POINTER(HipGroupedRoutes), _U32, _VP, _U32, _VP, _VP, C.c_size_t,
+                                                           _U32, _U32, _U32, _U32]),
     "shrike_hip_prefill_streamed_batched": (C.c_int, [_VP, _VP, C.POINTER(PoolBases), _U64, C.POINTER(ExpertOffsets),
                                                       C.POINTER(HipGroupedRoutes), _U32, _VP, _U32, _U32, _U32, _VP, _U32,
                                                       _VP, _VP, C.c_size_t, _U32, _U32, _U32, _U32, C.POINTER(C.c_uint32)]),

@@ -202,19 +202,52 @@ static void launch_prefill_logits_f16(const uint16_t *weights, const uint16_t *h
 }
 
 // prefill.metal:441-563: one wave selects for one token.
+// group_sums (may be null): the wave also leaves, for its token's row of `hidden`, the sum of every group of 64 of its fp16
+// elements, exactly as k_row_group_sums forms it (a lane takes an 8-element chunk: its eight values in order, then eight
+// neighbouring lanes fold pairwise), as (hi, lo) halves at [token][group]. The launch is a chain of dependent steps on half the
+// chip's compute units: the row's loads go out ahead of the selection and are summed behind it.
+template <bool SUMS>
 __global__ __launch_bounds__(256) void k_prefill_select(SelectArgs sel, const float *ws, uint32_t *out_indices,
-                                                        uint16_t *out_weights, uint32_t query_count) {
+                                                        uint16_t *out_weights, uint32_t query_count, const uint16_t *hidden,
+                                                        uint32_t stride, uint32_t d, uint32_t *group_sums) {
     warm_kernel_arguments(sel);
     __shared__ RouteScratch s_route[4];
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t t = blockIdx.x * 4u + wave;
     if (t >= query_count) return;
+    constexpr uint32_t kAhead = SHRIKE_MAX_HIDDEN / 8u / 64u;  // chunks a lane can own
+    uint4 mine[SUMS ? kAhead : 1u];
+    const uint32_t chunks = d / 8u;
+    if (SUMS) {
+        const uint4 *row = reinterpret_cast<const uint4 *>(hidden + size_t(t) * stride);
+#pragma unroll
+        for (uint32_t i = 0; i < kAhead; ++i)
+            if (64u * i < chunks) mine[i] = row[min(lane + 64u * i, chunks - 1u)];  // past the row: a copy, never stored
+    }
     sel.logits = ws + size_t(t) * sel.num_experts;
     RouteLists lists = {};
     lists.out_indices = out_indices + size_t(t) * sel.top_k;
     lists.out_weights = out_weights + size_t(t) * sel.top_k;
     uint32_t cell;
     route_wave<false>(sel, lists, lane, true, cell, s_route[wave]);
+    if (SUMS) {
+#pragma unroll
+        for (uint32_t i = 0; i < kAhead; ++i) {
+            if (64u * i >= chunks) break;
+            const uint32_t c = lane + 64u * i;
+            const uint32_t xw[4] = {mine[i].x, mine[i].y, mine[i].z, mine[i].w};
+            float sum = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                sum = __fadd_rn(sum, f16_to_f32(uint16_t(xw[q])));
+                sum = __fadd_rn(sum, f16_to_f32(uint16_t(xw[q] >> 16)));
+            }
+            sum = __fadd_rn(sum, __shfl_xor(sum, 1));
+            sum = __fadd_rn(sum, __shfl_xor(sum, 2));
+            sum = __fadd_rn(sum, __shfl_xor(sum, 4));
+            if (c < chunks && (c & 7u) == 0u) group_sums[size_t(t) * (d / 64u) + (c >> 3)] = split_hi_lo(sum);  // d % 64 == 0: whole groups
+        }
+    }
 }
 
 // ---- grouping ---------------------------------------------------------------------------
@@ -523,13 +556,12 @@ int launch_row_group_sums(const uint16_t *src, size_t stride, uint32_t rows, uin
 
 using namespace shrike;
 
-extern "C" {
-
-int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_weights, const void *d_scales,
-                              const void *d_biases, const void *d_hidden, const void *d_effective_scale,
-                              const void *d_per_expert_scale, const void *d_logit_bias, uint32_t *d_out_indices,
-                              void *d_out_weights, float *d_logits_workspace, uint32_t query_count, uint32_t num_experts,
-                              uint32_t d, uint32_t top_k, uint32_t hidden_stride_elements) {
+// d_group_sums (may be null): where the group sums of hidden's rows go as well, for the grouped FFN's bias term
+static int prefill_router(shrike_hip_moe *moe, void *stream, const void *d_weights, const void *d_scales, const void *d_biases,
+                          const void *d_hidden, const void *d_effective_scale, const void *d_per_expert_scale,
+                          const void *d_logit_bias, uint32_t *d_out_indices, void *d_out_weights, float *d_logits_workspace,
+                          uint32_t query_count, uint32_t num_experts, uint32_t d, uint32_t top_k, uint32_t hidden_stride_elements,
+                          uint32_t *d_group_sums) {
     SHRIKE_REQUIRE(moe != nullptr, "moe handle is NULL");
     SHRIKE_REQUIRE(query_count > 0, "queryCount must be positive");  // PrefillRouter.swift:99
     if (int rc = check_router(moe, num_experts, d, top_k)) return rc;
@@ -564,7 +596,8 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
         a.lists.out_weights = static_cast<uint16_t *>(d_out_weights);
         a.counter = moe->d_counter + kRouterTokenCounters;
         a.token_stride = hidden_stride_elements;
-        return launch_router_tokens(a, moe->desc.router_weight_bits, query_count, s);
+        if (int rc = launch_router_tokens(a, moe->desc.router_weight_bits, query_count, s)) return rc;
+        return d_group_sums ? launch_row_group_sums(a.hidden, hidden_stride_elements, query_count, d, d_group_sums, nullptr, s) : 0;
     }
     const dim3 grid((num_experts + 3u) / 4u, (query_count + kRouterTokenBlock - 1u) / kRouterTokenBlock);
     switch (moe->desc.router_weight_bits) {
@@ -583,10 +616,42 @@ int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_w
         default: hipLaunchKernelGGL(k_prefill_logits<4>, grid, dim3(256), 0, s, a, query_count, hidden_stride_elements, d_logits_workspace); break;
     }
     SHRIKE_HIP(hipGetLastError());
-    hipLaunchKernelGGL(k_prefill_select, dim3((query_count + 3u) / 4u), dim3(256), 0, s, a.sel, d_logits_workspace, d_out_indices,
-                       static_cast<uint16_t *>(d_out_weights), query_count);
+    if (d_group_sums)  // the selection's waves form them on the side
+        hipLaunchKernelGGL(k_prefill_select<true>, dim3((query_count + 3u) / 4u), dim3(256), 0, s, a.sel, d_logits_workspace,
+                           d_out_indices, static_cast<uint16_t *>(d_out_weights), query_count, a.hidden, hidden_stride_elements, d,
+                           d_group_sums);
+    else
+        hipLaunchKernelGGL(k_prefill_select<false>, dim3((query_count + 3u) / 4u), dim3(256), 0, s, a.sel, d_logits_workspace,
+                           d_out_indices, static_cast<uint16_t *>(d_out_weights), query_count, a.hidden, hidden_stride_elements, d,
+                           nullptr);
     SHRIKE_HIP(hipGetLastError());
     return 0;
+}
+
+extern "C" {
+
+int shrike_hip_prefill_router(shrike_hip_moe *moe, void *stream, const void *d_weights, const void *d_scales,
+                              const void *d_biases, const void *d_hidden, const void *d_effective_scale,
+                              const void *d_per_expert_scale, const void *d_logit_bias, uint32_t *d_out_indices,
+                              void *d_out_weights, float *d_logits_workspace, uint32_t query_count, uint32_t num_experts,
+                              uint32_t d, uint32_t top_k, uint32_t hidden_stride_elements) {
+    return prefill_router(moe, stream, d_weights, d_scales, d_biases, d_hidden, d_effective_scale, d_per_expert_scale, d_logit_bias,
+                          d_out_indices, d_out_weights, d_logits_workspace, query_count, num_experts, d, top_k,
+                          hidden_stride_elements, nullptr);
+}
+
+int shrike_hip_prefill_router_with_group_sums(shrike_hip_moe *moe, void *stream, const void *d_weights, const void *d_scales,
+                                              const void *d_biases, const void *d_hidden, const void *d_effective_scale,
+                                              const void *d_per_expert_scale, const void *d_logit_bias,
+                                              uint32_t *d_out_indices, void *d_out_weights, float *d_logits_workspace,
+                                              uint32_t query_count, uint32_t num_experts, uint32_t d, uint32_t top_k,
+                                              uint32_t hidden_stride_elements, void *d_ffn_workspace) {
+    SHRIKE_REQUIRE(d_ffn_workspace != nullptr, "prefill router: the FFN workspace that takes the group sums is NULL");
+    SHRIKE_REQUIRE(reinterpret_cast<uintptr_t>(d_ffn_workspace) % 256u == 0, "prefill router: the FFN workspace must be 256-byte aligned");
+    SHRIKE_REQUIRE(d % kGroup == 0, "prefill router: group sums need d to be a multiple of 64, got %u", d);
+    return prefill_router(moe, stream, d_weights, d_scales, d_biases, d_hidden, d_effective_scale, d_per_expert_scale, d_logit_bias,
+                          d_out_indices, d_out_weights, d_logits_workspace, query_count, num_experts, d, top_k,
+                          hidden_stride_elements, static_cast<uint32_t *>(d_ffn_workspace));
 }
 
 size_t shrike_hip_prefill_router_workspace_bytes(uint32_t query_count, uint32_t num_experts, uint32_t d) {

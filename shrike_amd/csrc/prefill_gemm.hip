@@ -523,7 +523,7 @@ __global__ __launch_bounds__(256, 2) void k_grouped_ffn(FfnArgs a) {
                 uint32_t want = take_larger ? larger_first + place : (first - larger_first) + (place - mine_larger);
                 const uint64_t m0 = take_larger ? larger0 : smaller0, m1 = take_larger ? larger1 : smaller1;
                 const uint64_t m2 = take_larger ? larger2 : smaller2, m3 = take_larger ? larger3 : smaller3;
-                const uint32_t c0 = uint32_t(__popcll(m0)), c1 = uint32_t(__popcll(m1)), c2 = uint32_t(__popcll(m2)), c3 = uint32_t(__popcll(m3));
+                const uint32_t c0 = uint32_t(__popcll(m0)), c1 = uint32_t(__popcll(m1)), c2 = uint32_t(__popcll(m2));
                 uint64_t set;
                 uint32_t block;
                 if (want < c0) { set = m0; block = 0; }
@@ -633,7 +633,7 @@ static int grouped_ffn(shrike_hip_moe *moe, void *stream, const shrike_pool_base
                        const shrike_expert_offsets *offsets, const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles,
                        const uint64_t *d_residency, uint32_t pair_lo, uint32_t pair_hi, const void *d_hidden,
                        uint32_t hidden_stride_elements, void *d_route_partials, void *d_workspace, size_t workspace_bytes,
-                       uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k) {
+                       uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k, bool presummed = false) {
     SHRIKE_REQUIRE(moe && pool && offsets && routes, "grouped FFN: NULL argument");
     SHRIKE_REQUIRE(d == moe->desc.d && f == moe->desc.f, "grouped FFN: shape %ux%u differs from the handle's %ux%u", d, f, moe->desc.d, moe->desc.f);
     SHRIKE_REQUIRE(d % kGroup == 0 && f % kGroup == 0 && d > 0 && f > 0, "D and F must be positive multiples of 64");
@@ -670,7 +670,8 @@ static int grouped_ffn(shrike_hip_moe *moe, void *stream, const shrike_pool_base
     a.ebias = moe->desc.expert_additive_biases;
     a.resident_workgroups = resident_ffn_workgroups();
     hipStream_t s = as_stream(stream);
-    if (int rc = launch_row_group_sums(a.hidden, hidden_stride_elements, query_count, d, const_cast<uint32_t *>(a.hidden_sums), nullptr, s)) return rc;
+    if (!presummed)
+        if (int rc = launch_row_group_sums(a.hidden, hidden_stride_elements, query_count, d, const_cast<uint32_t *>(a.hidden_sums), nullptr, s)) return rc;
     return moe->desc.routed_weight_bits == 8 ? launch_ffn<8, false>(a, max_row_tiles, s) : launch_ffn<4, false>(a, max_row_tiles, s);
 }
 
@@ -681,6 +682,16 @@ int shrike_hip_prefill_grouped_ffn(shrike_hip_moe *moe, void *stream, const shri
                                    size_t workspace_bytes, uint32_t query_count, uint32_t d, uint32_t f, uint32_t top_k) {
     return grouped_ffn(moe, stream, pool, pool_slot_stride, offsets, routes, max_row_tiles, nullptr, 0u, 0xffffffffu, d_hidden,
                        hidden_stride_elements, d_route_partials, d_workspace, workspace_bytes, query_count, d, f, top_k);
+}
+
+int shrike_hip_prefill_grouped_ffn_presummed(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,
+                                             uint64_t pool_slot_stride, const shrike_expert_offsets *offsets,
+                                             const shrike_hip_grouped_routes *routes, uint32_t max_row_tiles,
+                                             const void *d_hidden, uint32_t hidden_stride_elements, void *d_route_partials,
+                                             void *d_workspace, size_t workspace_bytes, uint32_t query_count, uint32_t d,
+                                             uint32_t f, uint32_t top_k) {
+    return grouped_ffn(moe, stream, pool, pool_slot_stride, offsets, routes, max_row_tiles, nullptr, 0u, 0xffffffffu, d_hidden,
+                       hidden_stride_elements, d_route_partials, d_workspace, workspace_bytes, query_count, d, f, top_k, true);
 }
 
 int shrike_hip_prefill_streamed_batched(shrike_hip_moe *moe, void *stream, const shrike_pool_bases *pool,

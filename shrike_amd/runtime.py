@@ -441,7 +441,16 @@ class Prefill:
 
     def encode_block(self, weights, scales, biases, hidden, effective_scale, per_expert_scale, logit_bias,
                      out_indices, out_weights, logits_workspace, query_count, num_experts, d, top_k,
-                     hidden_stride_elements):
+                     hidden_stride_elements, ffn_workspace=None):
+        """ffn_workspace: the grouped FFN's workspace, which then also takes the group sums of `hidden`
+        (encode_grouped_expert_gemms(..., presummed=True) uses them instead of forming them again)."""
+        if ffn_workspace is not None:
+            check(capi.load().shrike_hip_prefill_router_with_group_sums(
+                self.moe.handle, self._s(), ptr(weights), ptr(scales), ptr(biases), ptr(hidden), ptr(effective_scale),
+                ptr(per_expert_scale), ptr(logit_bias), ptr(out_indices), ptr(out_weights), ptr(logits_workspace),
+                query_count, num_experts, d, top_k, hidden_stride_elements, ptr(ffn_workspace)),
+                "shrike_hip_prefill_router_with_group_sums")
+            return
         check(capi.load().shrike_hip_prefill_router(
             self.moe.handle, self._s(), ptr(weights), ptr(scales), ptr(biases), ptr(hidden), ptr(effective_scale),
             ptr(per_expert_scale), ptr(logit_bias), ptr(out_indices), ptr(out_weights), ptr(logits_workspace),
@@ -459,12 +468,13 @@ class Prefill:
 
     def encode_grouped_expert_gemms(self, pool: ExpertPool, offsets, routes: GroupedRoutesDevice, hidden,
                                     hidden_stride_elements, route_partials, workspace: DeviceBuffer, query_count,
-                                    top_k, max_row_tiles=None):
-        check(capi.load().shrike_hip_prefill_grouped_ffn(
+                                    top_k, max_row_tiles=None, presummed=False):
+        fn = capi.load().shrike_hip_prefill_grouped_ffn_presummed if presummed else capi.load().shrike_hip_prefill_grouped_ffn
+        check(fn(
             self.moe.handle, self._s(), pool.bases, pool.stride, C.byref(offsets), C.byref(routes.c),
             routes.max_row_tiles if max_row_tiles is None else max_row_tiles, ptr(hidden), hidden_stride_elements,
             ptr(route_partials), ptr(workspace), workspace.nbytes, query_count, self.moe.desc.d, self.moe.desc.f, top_k),
-            "shrike_hip_prefill_grouped_ffn")
+            "shrike_hip_prefill_grouped_ffn_presummed" if presummed else "shrike_hip_prefill_grouped_ffn")
 
     def encode_streamed_batched(self, pool: ExpertPool, offsets, routes: GroupedRoutesDevice, hidden,
                                 hidden_stride_elements, route_partials, workspace: DeviceBuffer, query_count, top_k,

@@ -61,6 +61,52 @@ def test_prefill_router_bit_exact_and_equal_to_decode(gpu, router_bits, ne, d, k
         assert np.array_equal(dl.out_w.download(np.uint16, k), got_w[tok * k:(tok + 1) * k])
 
 
+@pytest.mark.parametrize("router_bits,ne,d,f,k,t,pad,bits", [
+    (0, 64, 2048, 512, 8, 70, 0, 4),     # the fp16 logits kernel with four packed rows a wave forms the sums itself
+    (0, 24, 2880, 384, 4, 21, 8, 8),     # the instance for longer rows; an odd token count, padded rows
+    (0, 16, 192, 320, 3, 50, 24, 4),     # a row shorter than one wave load
+    (8, 32, 512, 256, 4, 40, 0, 4),      # an affine router: the sums come from the pass of their own
+    (0, 16, 512, 128, 2, 3, 0, 4)])      # a handful of tokens: the decode router's kernel, and the pass of their own
+def test_router_with_group_sums_feeds_the_presummed_ffn(gpu, router_bits, ne, d, f, k, t, pad, bits):
+    """shrike_hip_prefill_router_with_group_sums + shrike_hip_prefill_grouped_ffn_presummed against the two calls that
+    each read `hidden` for themselves: the same logits, routes and weights, the same group sums at the head of the FFN's
+    workspace, and the same partial rows, all bit for bit."""
+    L = Layer(0x5EED0610 + router_bits + t, d, f, ne, k, bits=bits, router_bits=router_bits)
+    L.logit_bias = S.f32_to_bf16_bits(L.tree.key("bias").normal(ne, std=0.01))
+    dl = DeviceLayer(gpu, L)
+    stride = d + pad
+    x = token_rows(L, t, stride)
+    hidden = gpu.dev(x)
+    pf, idx, w, logits = run_router(gpu, dl, L, hidden, t, stride)
+    routes = gpu.GroupedRoutesDevice(t * k, ne)
+    pf.group_pairs(idx, w, t, k, ne, routes, residency=dl.pool.table)
+    ws_bytes = pf.ffn_workspace_bytes(t, routes.max_row_tiles)
+    ws, ws2 = gpu.empty(ws_bytes).fill(0xA5), gpu.empty(ws_bytes).fill(0x5A)
+    partials, partials2 = (gpu.dev(np.full(t * k * d, 0xD4D0, np.uint16)) for _ in range(2))
+    pf.encode_grouped_expert_gemms(dl.pool, dl.off, routes, hidden, stride, partials, ws, t, k)
+    gpu.synchronize()
+    # the fused pair, into buffers of its own
+    idx2, w2 = gpu.empty(4 * t * k).fill(0xA5), gpu.empty(2 * t * k).fill(0xA5)
+    logits2 = gpu.empty(pf.router_workspace_bytes(t, ne, d)).fill(0xA5)
+    pf.encode_block(dl.router_w, dl.router_s, dl.router_b, hidden, dl.eff_scale, dl.expert_scale, dl.logit_bias,
+                    idx2, w2, logits2, t, ne, d, k, stride, ffn_workspace=ws2)
+    gpu.synchronize()
+    assert np.array_equal(logits2.download(np.uint32, t * ne), logits.download(np.uint32, t * ne))
+    assert np.array_equal(idx2.download(np.uint32, t * k), idx.download(np.uint32, t * k))
+    assert np.array_equal(w2.download(np.uint16, t * k), w.download(np.uint16, t * k))
+    sums = t * (d // 64)
+    assert np.array_equal(ws2.download(np.uint32, sums), ws.download(np.uint32, sums)), "group sums differ from the FFN's own pass"
+    pf.encode_grouped_expert_gemms(dl.pool, dl.off, routes, hidden, stride, partials2, ws2, t, k, presummed=True)
+    gpu.synchronize()
+    assert np.array_equal(partials2.download(np.uint16, t * k * d), partials.download(np.uint16, t * k * d))
+    # what the entry point refuses
+    lib = capi.load()
+    assert lib.shrike_hip_prefill_router_with_group_sums(dl.moe.handle, None, dl.router_w.ptr, None, None, hidden.ptr, dl.eff_scale.ptr,
+                                                         dl.expert_scale.ptr, dl.logit_bias.ptr, idx2.ptr, w2.ptr, logits2.ptr,
+                                                         t, ne, d, k, stride, None) != 0
+    assert "workspace" in capi.last_error()
+
+
 def random_routes(seed, t, k, ne, skew=1.2):
     rng = np.random.default_rng(seed)
     p = 1.0 / np.arange(1, ne + 1) ** skew
