@@ -453,7 +453,10 @@ def prefill_workload(args, rt, capi, S, meta):
         "config": {"workload": f"config 3: ragged prefill, {T} tokens, top-8 of 256 int4 experts (hidden 2048, intermediate 512), "
                                "router + device grouping + grouped FFN + reduce, all slots resident",
                    "stacked_layers": n_layers, "meta_dtype": args.meta, "experts_with_pairs": used, "row_tiles": tiles,
-                   "mfma_row_tiles_of_32": m_tiles},
+                   "mfma_row_tiles_of_32": m_tiles,
+                   "hidden_group_sums": "left by the router's select launch (shrike_hip_prefill_router_with_group_sums + "
+                                        "shrike_hip_prefill_grouped_ffn_presummed)" if fused_sums else
+                                        "formed by the grouped FFN's own first launch (the two-pass entry points)"},
         "kernel_us_per_chunk": {k: round(v, 2) for k, v in parts.items()},
         "grouped_ffn_by_layer_routes": by_layer,
         "roofline": {"bound": "hbm", "kernel": "k_grouped_ffn<4,0> + k_grouped_ffn<4,1> (gate/up + down of every row tile)",
